@@ -1,0 +1,101 @@
+// Row gathers and elementwise ops: embedding lookup, row gather, residual add,
+// SwiGLU.  Arithmetic is done in float32 and rounded once on store.
+#include "zi_common.h"
+
+// out[i,:] = table[ids[i],:]   (reference: src/backend/ops/embedding/cpu/embedding_cpu.cpp:10-23).
+// An id outside [0, V) writes NaN into the row so that the fault shows.
+template <typename TW, typename TO>
+__global__ void embedding_kernel(TO* __restrict__ out, const TW* __restrict__ table,
+                                 const int32_t* __restrict__ ids, int H, int V) {
+    const int64_t row = blockIdx.x;
+    const int id = ids[row];
+    const bool ok = id >= 0 && id < V;
+    const TW* src = table + (int64_t)(ok ? id : 0) * H;
+    TO* dst = out + row * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) zi_store(dst + j, ok ? zi_load(src + j) : NAN);
+}
+
+extern "C" int zi_embedding(void* out, int out_dt, const void* table, int table_dt, const int32_t* ids,
+                            int n, int hidden, int vocab, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && hidden > 0 && vocab > 0, "embedding: bad sizes n=%d hidden=%d vocab=%d", n, hidden, vocab);
+    if (n == 0) return 0;
+    ZI_DISPATCH_DTYPE(table_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
+        embedding_kernel<TW, TO><<<n, 256, 0, stream>>>((TO*)out, (const TW*)table, ids, hidden, vocab);
+    }));
+    return zi_check_launch("embedding");
+}
+
+// out[i,:] = in[idx[i],:]
+template <typename T>
+__global__ void gather_rows_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                   const int32_t* __restrict__ idx, int H, int n_in) {
+    const int64_t row = blockIdx.x;
+    const int s = idx[row];
+    const bool ok = s >= 0 && s < n_in;
+    const T* src = in + (int64_t)(ok ? s : 0) * H;
+    T* dst = out + row * H;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) zi_store(dst + j, ok ? zi_load(src + j) : NAN);
+}
+
+extern "C" int zi_gather_rows(void* out, const void* in, int dt, const int32_t* idx, int n_out, int n_in,
+                              int hidden, hipStream_t stream) {
+    ZI_REQUIRE(n_out >= 0 && n_in >= 0 && hidden > 0, "gather_rows: bad sizes");
+    if (n_out == 0) return 0;
+    ZI_DISPATCH_DTYPE(dt, T, {
+        gather_rows_kernel<T><<<n_out, 256, 0, stream>>>((T*)out, (const T*)in, idx, hidden, n_in);
+    });
+    return zi_check_launch("gather_rows");
+}
+
+// c = a + b, added in float32 (reference: src/backend/ops/add/cpu/add_cpu_opt.cpp:22-24,57-59).
+template <typename TA, typename TB, typename TC>
+__global__ void add_kernel(TC* __restrict__ c, const TA* __restrict__ a, const TB* __restrict__ b, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        zi_store(c + i, zi_load(a + i) + zi_load(b + i));
+}
+
+extern "C" int zi_add(void* c, int c_dt, const void* a, int a_dt, const void* b, int b_dt, int64_t n,
+                      hipStream_t stream) {
+    ZI_REQUIRE(n >= 0, "add: negative size");
+    if (n == 0) return 0;
+    const int blocks = (int)((n + 255) / 256 > 65535 ? 65535 : (n + 255) / 256);
+    ZI_DISPATCH_DTYPE(a_dt, TA, ZI_DISPATCH_DTYPE(b_dt, TB, ZI_DISPATCH_DTYPE(c_dt, TC, {
+        add_kernel<TA, TB, TC><<<blocks, 256, 0, stream>>>((TC*)c, (const TA*)a, (const TB*)b, n);
+    })));
+    return zi_check_launch("add");
+}
+
+// out[i,j] = up[i,j] * gate[i,j] / (1 + exp(-gate[i,j]))
+// (reference: src/backend/ops/swiglu/cpu/swiglu_cpu.cpp:9-23).  gate and up are
+// read with their own row strides, so both halves of one fused [N, 2I] product can be passed.
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gate, const T* __restrict__ up,
+                              int inter, int64_t ld_gate, int64_t ld_up) {
+    const int64_t row = blockIdx.y;
+    const T* g = gate + row * ld_gate;
+    const T* u = up + row * ld_up;
+    T* o = out + row * (int64_t)inter;
+    for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < inter; j += gridDim.x * blockDim.x) {
+        const float gv = zi_load(g + j), uv = zi_load(u + j);
+        zi_store(o + j, uv * (gv / (1.f + expf(-gv))));
+    }
+}
+
+extern "C" int zi_swiglu(void* out, const void* gate, const void* up, int dt, int n, int inter, int64_t ld_gate,
+                         int64_t ld_up, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && inter > 0 && ld_gate >= inter && ld_up >= inter, "swiglu: bad sizes n=%d inter=%d", n, inter);
+    if (n == 0) return 0;
+    ZI_REQUIRE(n <= 65535 * 1024, "swiglu: too many rows");
+    int bx = (inter + 255) / 256;
+    if (bx > 64) bx = 64;
+    // gridDim.y is limited to 65535: fold larger batches.
+    for (int r0 = 0; r0 < n; r0 += 65535) {
+        const int rows = n - r0 < 65535 ? n - r0 : 65535;
+        ZI_DISPATCH_DTYPE(dt, T, {
+            swiglu_kernel<T><<<dim3(bx, rows), 256, 0, stream>>>(
+                (T*)out + (int64_t)r0 * inter, (const T*)gate + (int64_t)r0 * ld_gate,
+                (const T*)up + (int64_t)r0 * ld_up, inter, ld_gate, ld_up);
+        });
+    }
+    return zi_check_launch("swiglu");
+}

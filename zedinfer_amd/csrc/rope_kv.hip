@@ -1,0 +1,132 @@
+// Rotary position encoding (split-half, "NeoX" pairing) fused with the write of
+// keys and values into the paged cache.
+//
+// For k < R/2 (R = rotary dims, R = head_dim for full rotation):
+//   angle = float(pos) * inv_freq[k]          (float32; inv_freq[k] = theta^(-2k/R), made on the host)
+//   out[k]       = a cos(angle) - b sin(angle)
+//   out[k + R/2] = b cos(angle) + a sin(angle)     with a = in[k], b = in[k + R/2]
+// (reference: src/backend/ops/rope/cpu/rope_cpu.cpp:33,47-52,62-65).  Queries are
+// rotated in place; keys are rotated on their way into the cache, values copied
+// (reference: K is stored after rotation, V raw, src/frontend/models/transformer_forward.cpp:99-104).
+//
+// Cache layout of one layer: [page][kv_head][slot_in_page][head_dim]; token slot
+// s lives in page s / page_size at offset s % page_size.  A negative slot skips the write.
+#include "zi_common.h"
+
+template <typename T>
+__global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                                     int64_t ldq, int64_t ldk, int64_t ldv, const int32_t* __restrict__ pos,
+                                     const int32_t* __restrict__ slots, const float* __restrict__ inv_freq,
+                                     T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int d,
+                                     int rot, int page_size, int write_kv, int64_t cache_slots) {
+    extern __shared__ float cs[];  // cos[rot/2], sin[rot/2]
+    const int64_t t = blockIdx.x;
+    const int half = rot / 2;
+    const float p = (float)pos[t];
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float s, c;
+        sincosf(p * inv_freq[i], &s, &c);
+        cs[i] = c;
+        cs[half + i] = s;
+    }
+    __syncthreads();
+    // queries, in place
+    T* qr = q + t * ldq;
+    for (int i = threadIdx.x; i < nh * half; i += blockDim.x) {
+        const int h = i / half, j = i % half;
+        T* base = qr + (int64_t)h * d;
+        const float a = zi_load(base + j), b = zi_load(base + j + half);
+        const float c = cs[j], s = cs[half + j];
+        zi_store(base + j, a * c - b * s);
+        zi_store(base + j + half, b * c + a * s);
+    }
+    if (!write_kv) return;
+    const int slot = slots[t];
+    if (slot < 0 || slot >= cache_slots) return;  // the host checks the range; never write outside the pool
+    const int64_t page = slot / page_size, off = slot % page_size;
+    const T* kr = k + t * ldk;
+    const T* vr = v + t * ldv;
+    for (int i = threadIdx.x; i < nkv * d; i += blockDim.x) {
+        const int h = i / d, j = i % d;
+        const int64_t dst = ((page * nkv + h) * page_size + off) * d + j;
+        float kv;
+        if (j < half) {
+            kv = zi_load(kr + h * d + j) * cs[j] - zi_load(kr + h * d + j + half) * cs[half + j];
+        } else if (j < rot) {
+            const int jj = j - half;
+            kv = zi_load(kr + h * d + j) * cs[jj] + zi_load(kr + h * d + jj) * cs[half + jj];
+        } else {
+            kv = zi_load(kr + h * d + j);
+        }
+        zi_store(kcache + dst, kv);
+        vcache[dst] = vr[h * d + j];
+    }
+}
+
+extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, int n, int64_t ldq, int64_t ldk,
+                                int64_t ldv, const int32_t* pos, const int32_t* slots, const float* inv_freq,
+                                void* kcache, void* vcache, int64_t cache_slots, int nh, int nkv, int d, int rot,
+                                int page_size, int write_kv, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && nh > 0 && nkv >= 0 && d > 0, "rope_kv_store: bad sizes");
+    ZI_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "rope_kv_store: rotary dims %d must be even and <= head_dim %d", rot, d);
+    ZI_REQUIRE(ldq >= (int64_t)nh * d, "rope_kv_store: query row stride %lld < heads*head_dim", (long long)ldq);
+    if (write_kv) {
+        ZI_REQUIRE(page_size > 0 && cache_slots > 0 && cache_slots % page_size == 0,
+                   "rope_kv_store: cache of %lld slots is not a whole number of pages of %d", (long long)cache_slots, page_size);
+        ZI_REQUIRE(ldk >= (int64_t)nkv * d && ldv >= (int64_t)nkv * d, "rope_kv_store: key/value row stride too small");
+        ZI_REQUIRE(k && v && kcache && vcache && slots, "rope_kv_store: null cache or key/value pointer");
+    }
+    ZI_REQUIRE(rot * sizeof(float) <= 48 * 1024, "rope_kv_store: rotary dims %d too large", rot);
+    if (n == 0) return 0;
+    ZI_DISPATCH_DTYPE(dt, T, {
+        rope_kv_store_kernel<T><<<n, 256, rot * sizeof(float), stream>>>(
+            (T*)q, (const T*)k, (const T*)v, ldq, ldk, ldv, pos, slots, inv_freq, (T*)kcache, (T*)vcache, nh, nkv, d,
+            rot, page_size, write_kv, cache_slots);
+    });
+    return zi_check_launch("rope_kv_store");
+}
+
+// Rotation alone, out of place: out[t,h,:] = rotate(in[t,h,:], pos[t])  (op-level entry, and the
+// form a layer uses that reads another layer's cache and therefore stores nothing).
+template <typename T>
+__global__ void rope_kernel(T* __restrict__ out, const T* __restrict__ in, int64_t ld_in, int64_t ld_out,
+                            const int32_t* __restrict__ pos, const float* __restrict__ inv_freq, int nh, int d,
+                            int rot) {
+    extern __shared__ float cs[];
+    const int64_t t = blockIdx.x;
+    const int half = rot / 2;
+    const float p = (float)pos[t];
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float s, c;
+        sincosf(p * inv_freq[i], &s, &c);
+        cs[i] = c;
+        cs[half + i] = s;
+    }
+    __syncthreads();
+    const T* ir = in + t * ld_in;
+    T* orow = out + t * ld_out;
+    for (int i = threadIdx.x; i < nh * half; i += blockDim.x) {
+        const int h = i / half, j = i % half;
+        const float a = zi_load(ir + (int64_t)h * d + j), b = zi_load(ir + (int64_t)h * d + j + half);
+        zi_store(orow + (int64_t)h * d + j, a * cs[j] - b * cs[half + j]);
+        zi_store(orow + (int64_t)h * d + j + half, b * cs[j] + a * cs[half + j]);
+    }
+    for (int i = threadIdx.x; i < nh * (d - rot); i += blockDim.x) {
+        const int h = i / (d - rot), j = rot + i % (d - rot);
+        orow[(int64_t)h * d + j] = ir[(int64_t)h * d + j];
+    }
+}
+
+extern "C" int zi_rope(void* out, const void* in, int dt, int n, int64_t ld_in, int64_t ld_out, const int32_t* pos,
+                       const float* inv_freq, int nh, int d, int rot, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && nh > 0 && d > 0, "rope: bad sizes");
+    ZI_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "rope: rotary dims %d must be even and <= head_dim %d", rot, d);
+    ZI_REQUIRE(ld_in >= (int64_t)nh * d && ld_out >= (int64_t)nh * d, "rope: row stride too small");
+    ZI_REQUIRE(rot * sizeof(float) <= 48 * 1024, "rope: rotary dims %d too large", rot);
+    if (n == 0) return 0;
+    ZI_DISPATCH_DTYPE(dt, T, {
+        rope_kernel<T><<<n, 256, rot * sizeof(float), stream>>>((T*)out, (const T*)in, ld_in, ld_out, pos, inv_freq, nh,
+                                                                d, rot);
+    });
+    return zi_check_launch("rope");
+}

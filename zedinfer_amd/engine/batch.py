@@ -1,0 +1,130 @@
+"""One step's batch: what the caller asks for, and its flattened device form.
+
+A step takes, for each request in it, that request's next tokens (a portion of
+its prompt, or one decoded token) and the places among them whose logits are
+wanted.  All entries are flattened into one token list without padding
+(reference: src/zedinfer/batch_context.cpp:21-85 builds the same flattened
+ids/positions; there decode rows must come first, here any order works).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, SequenceCache
+
+
+@dataclass
+class StepEntry:
+    """``tokens`` continue the sequence whose cache is ``seq`` at position ``seq.length``;
+    ``want`` lists the places among ``tokens`` whose logits are returned."""
+
+    seq: SequenceCache
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class GroupView:
+    slots: torch.Tensor          # [n] int32: where each token's keys and values go
+    block_tables: torch.Tensor   # [entries, max_pages] int32, -1 where no page is held
+
+
+@dataclass
+class DeviceBatch:
+    """The step as the parts see it.  Everything is int32 on the device."""
+
+    num_tokens: int
+    num_entries: int
+    num_logit_rows: int
+    token_ids: torch.Tensor      # [n]
+    positions: torch.Tensor      # [n] absolute position of each token in its sequence
+    tok_seq: torch.Tensor        # [n] entry index of each token
+    logit_rows: torch.Tensor     # [rows] flat token indices
+    entry_start: torch.Tensor    # [entries] first flat token index of the entry
+    entry_len: torch.Tensor      # [entries] tokens of the entry in this step
+    entry_past: torch.Tensor     # [entries] tokens of the entry already in the cache
+    entry_slot: torch.Tensor     # [entries] state slot of the entry
+    groups: List[GroupView] = field(default_factory=list)
+    # host copies, for parts that plan their launches on the host
+    host_start: Optional[np.ndarray] = None
+    host_len: Optional[np.ndarray] = None
+    host_past: Optional[np.ndarray] = None
+    host_slot: Optional[np.ndarray] = None
+
+
+def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
+                       device: torch.device) -> DeviceBatch:
+    """Check the entries, then pack every index array into one host buffer and copy it over once."""
+    if not entries:
+        raise ValueError("a step needs at least one entry")
+    seen = set()
+    lens = []
+    for e in entries:
+        if id(e.seq) in seen:
+            raise ValueError(f"request {e.seq.request_id!r} appears twice in one step")
+        seen.add(id(e.seq))
+        if e.seq.closed:
+            raise ValueError(f"request {e.seq.request_id!r} is closed")
+        n = len(e.tokens)
+        if n == 0:
+            raise ValueError(f"request {e.seq.request_id!r} brings no tokens")
+        for w in e.want:
+            if not (0 <= w < n):
+                raise ValueError(f"request {e.seq.request_id!r}: wanted place {w} is outside its {n} tokens")
+        lens.append(n)
+    E = len(entries)
+    N = int(sum(lens))
+    starts = np.zeros(E, dtype=np.int32)
+    starts[1:] = np.cumsum(lens)[:-1]
+    past = np.array([e.seq.length for e in entries], dtype=np.int32)
+    slot = np.array([e.seq.slot for e in entries], dtype=np.int32)
+    lens_a = np.array(lens, dtype=np.int32)
+
+    token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+    if token_ids.min() < 0 or token_ids.max() >= vocab_size:
+        bad = token_ids[(token_ids < 0) | (token_ids >= vocab_size)][0]
+        raise ValueError(f"token id {int(bad)} is outside the vocabulary of {vocab_size}")
+    positions = np.concatenate([np.arange(p, p + n, dtype=np.int32) for p, n in zip(past, lens)])
+    tok_seq = np.repeat(np.arange(E, dtype=np.int32), lens)
+    rows = [starts[i] + w for i, e in enumerate(entries) for w in e.want]
+    logit_rows = np.asarray(rows, dtype=np.int32)
+    R = len(rows)
+
+    G = len(cache.groups)
+    group_slots, group_tables, widths = [], [], []
+    for g in range(G):
+        group_slots.append(np.concatenate(
+            [cache.token_slots(e.seq, g, int(p), n) for e, p, n in zip(entries, past, lens)]))
+        width = max(1, max(len(e.seq.pages[g]) for e in entries))
+        t = np.full((E, width), -1, dtype=np.int32)
+        for i, e in enumerate(entries):
+            pg = e.seq.pages[g]
+            t[i, :len(pg)] = pg
+        group_tables.append(t)
+        widths.append(width)
+
+    pieces = [token_ids.astype(np.int32), positions, tok_seq, logit_rows, starts, lens_a, past, slot]
+    for g in range(G):
+        pieces += [group_slots[g], group_tables[g].reshape(-1)]
+    sizes = [p.size for p in pieces]
+    host = torch.empty((max(1, sum(sizes)),), dtype=torch.int32, pin_memory=device.type == "cuda")
+    hv = host.numpy()
+    off = 0
+    for p in pieces:
+        hv[off:off + p.size] = p
+        off += p.size
+    dev = host.to(device, non_blocking=True)
+    views = []
+    off = 0
+    for s in sizes:
+        views.append(dev[off:off + s])
+        off += s
+    groups = [GroupView(views[8 + 2 * g], views[9 + 2 * g].view(E, widths[g])) for g in range(G)]
+    return DeviceBatch(num_tokens=N, num_entries=E, num_logit_rows=R, token_ids=views[0], positions=views[1],
+                       tok_seq=views[2], logit_rows=views[3], entry_start=views[4], entry_len=views[5],
+                       entry_past=views[6], entry_slot=views[7], groups=groups, host_start=starts,
+                       host_len=lens_a, host_past=past, host_slot=slot)

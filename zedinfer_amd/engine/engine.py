@@ -1,0 +1,123 @@
+"""The engine: a model, its cache and the one step function.
+
+``Engine.step(entries)`` runs exactly the tokens it is given, as one batch, from
+the cache that earlier steps left, and returns float32 logits at the wanted
+places (the reference returns logits for all rows and lets the caller slice,
+reference: src/zedinfer/serving_loop.cpp:182-422,
+src/frontend/models/transformer_forward.cpp:155-159).  It grows each request's
+block tables before the run and commits the new lengths after it.
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from .. import ops
+from ..cache.manager import CacheManager, SequenceCache
+from ..cache.pages import OutOfPages
+from ..config import ModelConfig, ModelForwardConfig, SchedulerConfig, load_config
+from ..models import DecoderModel, expected_weights
+from ..parts import Runtime
+from ..weights import load_weights, random_weights
+from .batch import DeviceBatch, StepEntry, build_device_batch
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           "f32": torch.float32}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"engine dtype must be float32 or bfloat16, got {name}")
+        return name
+    if str(name) not in _DTYPES:
+        raise ValueError(f"unknown dtype {name!r}; choose bfloat16 or float32")
+    return _DTYPES[str(name)]
+
+
+def require_gpu() -> torch.device:
+    """The engine runs on the GPU only; there is no CPU path."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("zedinfer_amd needs a GPU (torch.cuda.is_available() is False); "
+                           "there is no CPU fallback")
+    ops.load()
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+class Engine:
+    def __init__(self, fc: ModelForwardConfig, weights: Dict[str, torch.Tensor], dtype: torch.dtype,
+                 sched: Optional[SchedulerConfig] = None, device: Optional[torch.device] = None):
+        self.device = device or require_gpu()
+        self.dtype = parse_dtype(dtype)
+        self.sched = sched or SchedulerConfig()
+        self.sched.validate()
+        self.fc = fc
+        self.rt = Runtime(self.device, self.dtype)
+        self.model = DecoderModel(fc, weights, self.rt)
+        kv = self.model.cache_requests()
+        num_pages = self.sched.num_kv_blocks or self._pages_from_free_memory(kv)
+        self.cache = CacheManager(kv, self.model.state_requests(), num_pages, self.sched.kv_block_size,
+                                  self.sched.max_batch_requests, self.dtype, self.device,
+                                  max_step_tokens=self.sched.max_batch_tokens)
+        self.memories = self.cache.memories(fc.schedule)
+        self.vocab_size = fc.vocab_size
+        self.steps_run = 0
+
+    # ---- construction ------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", sched: Optional[SchedulerConfig] = None) -> "Engine":
+        """Load config.json and the safetensors of ``folder``; the model class comes from config.json."""
+        device = require_gpu()
+        arch, cfg = load_config(folder)
+        fc = arch.forward_config(cfg)
+        dt = parse_dtype(dtype)
+        weights = load_weights(folder, expected_weights(fc), dt, device)
+        return cls(fc, weights, dt, sched, device)
+
+    @classmethod
+    def from_config(cls, cfg: ModelConfig, arch_name: Optional[str] = None, dtype="bfloat16", seed: int = 0,
+                    sched: Optional[SchedulerConfig] = None, noisy_norms: bool = False) -> "Engine":
+        """A model with seeded random weights made on the device (no files)."""
+        from ..config.registry import find_architecture
+        device = require_gpu()
+        arch = find_architecture({"architectures": [arch_name] if arch_name else list(cfg.architectures),
+                                  "model_type": cfg.model_type})
+        fc = arch.forward_config(cfg)
+        dt = parse_dtype(dtype)
+        weights = random_weights(expected_weights(fc), seed, dt, device, noisy_norms=noisy_norms)
+        return cls(fc, weights, dt, sched, device)
+
+    def _pages_from_free_memory(self, kv) -> int:
+        """Pool size from free device memory (reference: src/zedinfer/engine.cpp:949-995), capped by
+        what max_batch_requests sequences of max_seq_len tokens could ever use."""
+        per_page = max(1, CacheManager.bytes_per_page(kv, self.sched.kv_block_size, self.dtype))
+        free, total = torch.cuda.mem_get_info(self.device)
+        budget = int(free - (1.0 - self.sched.gpu_memory_utilization) * total)
+        pages = max(16, budget // per_page)
+        cap = self.sched.max_batch_requests * (-(-self.sched.max_seq_len // self.sched.kv_block_size))
+        return int(min(pages, cap))
+
+    # ---- requests ------------------------------------------------------------------
+    def open(self, request_id, expected_tokens: int = 0) -> SequenceCache:
+        return self.cache.open(request_id, expected_tokens)
+
+    def close(self, seq: SequenceCache) -> None:
+        self.cache.close(seq)
+
+    # ---- the step ------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry], copy: bool = True) -> Optional[torch.Tensor]:
+        """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
+        of each entry's ``want`` (None when nothing is wanted).  With ``copy`` False the result is
+        a view of a workspace that the next step overwrites.  Raises OutOfPages, with no
+        request's length changed, when the pool cannot hold the new tokens."""
+        for e in entries:
+            self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
+        batch = build_device_batch(entries, self.cache, self.vocab_size, self.device)
+        logits = self.model.run(batch, self.memories)
+        for e in entries:
+            self.cache.commit(e.seq, e.seq.length + len(e.tokens))
+        self.steps_run += 1
+        return logits.clone() if (copy and logits is not None) else logits

@@ -1,0 +1,124 @@
+"""Building a decoder from its description and running one step through it.
+
+``DecoderModel`` knows parts and the schedule, nothing about architectures: it
+collects the tensors every part asks for, binds them by name, builds the parts
+through the registries and runs ``schedule`` in order (reference: the dense loop
+of src/frontend/models/transformer_forward.cpp:63-156).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .. import ops
+from ..config.forward_config import LayerSpec, ModelForwardConfig, PartSpec
+from ..parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, KVCacheRequest, LayerMemory,
+                     Runtime, StateRequest)
+from ..weights.loader import WeightSpec
+
+
+def _part_weights(registry, spec: PartSpec) -> Dict[str, WeightSpec]:
+    """tensor name -> spec, for one part."""
+    cls = registry.get(spec.kind)
+    out: Dict[str, WeightSpec] = {}
+    for param, ws in cls.weight_specs(spec).items():
+        if param not in spec.weights:
+            raise ValueError(f"part '{spec.kind}' needs parameter '{param}' but its spec names no tensor for it")
+        out[spec.weights[param]] = ws
+    return out
+
+
+def expected_weights(fc: ModelForwardConfig) -> Dict[str, WeightSpec]:
+    """Every checkpoint tensor the model needs, with its shape."""
+    exp: Dict[str, WeightSpec] = {}
+
+    def merge(d: Dict[str, WeightSpec]):
+        for name, ws in d.items():
+            if name in exp and exp[name].shape != ws.shape:
+                raise ValueError(f"tensor '{name}' is asked for with shapes {exp[name].shape} and {ws.shape}")
+            # a part that can live without the tensor does not make it optional for another
+            if name not in exp or exp[name].fallback is not None:
+                exp[name] = ws
+    merge(_part_weights(EMBEDDINGS, fc.embedding))
+    for layer in fc.layers:
+        merge(_part_weights(MIXERS, layer.mixer))
+        merge(_part_weights(FEED_FORWARDS, layer.feed_forward))
+        for n in layer.norms.values():
+            merge(_part_weights(NORMS, n))
+    merge(_part_weights(NORMS, fc.final_norm))
+    merge(_part_weights(HEADS, fc.lm_head))
+    return exp
+
+
+def _build(registry, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+    cls = registry.get(spec.kind)
+    local = {param: weights[name] for param, name in spec.weights.items() if param in cls.weight_specs(spec)}
+    return cls(spec, local, rt)
+
+
+class DecoderModel:
+    def __init__(self, fc: ModelForwardConfig, weights: Dict[str, torch.Tensor], rt: Runtime):
+        fc.validate()
+        self.fc = fc
+        self.rt = rt
+        self.embedding = _build(EMBEDDINGS, fc.embedding, weights, rt)
+        self.blocks = []
+        for layer in fc.layers:
+            block_cls = BLOCKS.get(layer.block)
+            missing = [n for n in block_cls.norm_names if n not in layer.norms]
+            if missing:
+                raise ValueError(f"block '{layer.block}' needs norms {missing}")
+            norms = {n: _build(NORMS, layer.norms[n], weights, rt) for n in block_cls.norm_names}
+            mixer = _build(MIXERS, layer.mixer, weights, rt)
+            ffn = _build(FEED_FORWARDS, layer.feed_forward, weights, rt)
+            self.blocks.append(block_cls(norms, mixer, ffn, rt))
+        self.final_norm = _build(NORMS, fc.final_norm, weights, rt)
+        self.lm_head = _build(HEADS, fc.lm_head, weights, rt)
+        self.vocab_size = fc.vocab_size
+        self.hidden_size = fc.hidden_size
+
+    # ---- what the cache manager has to provide ------------------------------
+    def cache_requests(self) -> Dict[int, KVCacheRequest]:
+        """cache id -> what the step that writes it needs."""
+        out: Dict[int, KVCacheRequest] = {}
+        for st in self.fc.schedule:
+            req = self.blocks[st.layer].mixer.cache_request()
+            if req is None:
+                continue
+            if st.cache in out and (out[st.cache].num_kv_heads, out[st.cache].head_dim) != (req.num_kv_heads, req.head_dim):
+                raise ValueError(f"cache {st.cache} is shared by layers with different key/value shapes")
+            if st.writes_cache or st.cache not in out:
+                out[st.cache] = req
+        return out
+
+    def state_requests(self) -> Dict[int, StateRequest]:
+        out: Dict[int, StateRequest] = {}
+        for st in self.fc.schedule:
+            req = self.blocks[st.layer].mixer.state_request()
+            if req is not None:
+                out[st.cache] = req
+        return out
+
+    # ---- one step -------------------------------------------------------------
+    def run(self, batch, memories: Sequence[LayerMemory]) -> Optional[torch.Tensor]:
+        """Run the tokens of ``batch`` through the schedule; float32 logits [wanted, vocab]
+        at ``batch.logit_rows``, or None when no row is wanted."""
+        resid = self.embedding.forward(batch.token_ids)
+        delta = None
+        for st, mem in zip(self.fc.schedule, memories):
+            delta = self.blocks[st.layer].forward(resid, delta, batch, mem)
+        if batch.num_logit_rows == 0:
+            if delta is not None:
+                pass  # the last feed-forward's output is not needed when no logits are
+            return None
+        rows = batch.logit_rows
+        r = self.rt.buffer("resid_rows", (batch.num_logit_rows, self.hidden_size), torch.float32)
+        ops.gather_rows(resid, rows, out=r)
+        if delta is not None:
+            dsel = self.rt.buffer("delta_rows", (batch.num_logit_rows, self.hidden_size), delta.dtype)
+            ops.gather_rows(delta, rows, out=dsel)
+            x = self.final_norm.add_forward(r, dsel)
+        else:
+            x = self.final_norm.forward(r)
+        return self.lm_head.forward(x)

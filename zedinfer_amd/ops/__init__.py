@@ -1,0 +1,17 @@
+"""The operators: thin, checked Python entries over the HIP kernels.
+
+Each function checks devices, storage types, shapes and strides on the host,
+then launches on torch's current stream.  The op-level names follow the
+reference's Python module (reference: python/bindings/zedinfer_ops.cpp:257-291:
+add, argmax, embedding, linear, rms_norm, rope, swiglu).
+"""
+from .functional import (add, add_rms_norm, argmax, attention, embedding, gather_rows, has_gpu,
+                         linear, rms_norm, rope, rope_kv_store, rope_inv_freq, sample, swiglu,
+                         device_synchronize)
+from ._lib import KernelLibraryError, library_path, load
+
+__all__ = [
+    "add", "add_rms_norm", "argmax", "attention", "embedding", "gather_rows", "has_gpu", "linear",
+    "rms_norm", "rope", "rope_kv_store", "rope_inv_freq", "sample", "swiglu", "device_synchronize",
+    "KernelLibraryError", "library_path", "load",
+]

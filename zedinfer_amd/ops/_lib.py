@@ -1,0 +1,75 @@
+"""Loading the HIP kernel library and declaring its entry points.
+
+There is no fallback: when the library cannot be loaded, every op raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+from typing import Optional
+
+_lock = threading.Lock()
+_lib: Optional[ctypes.CDLL] = None
+_lib_path: Optional[str] = None
+
+P, I, L, F = c_void_p, c_int, c_int64, c_float
+
+_PROTOTYPES = {
+    "zi_abi_version": [],
+    "zi_embedding": [P, I, P, I, P, I, I, I, P],
+    "zi_gather_rows": [P, P, I, P, I, I, I, P],
+    "zi_add": [P, I, P, I, P, I, L, P],
+    "zi_swiglu": [P, P, P, I, I, I, L, L, P],
+    "zi_rmsnorm": [P, I, P, I, P, I, I, I, L, L, F, I, P],
+    "zi_add_rmsnorm": [P, I, P, P, I, P, I, I, I, F, I, P],
+    "zi_rope_kv_store": [P, P, P, I, I, L, L, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
+    "zi_rope": [P, P, I, I, L, L, P, P, I, I, I, P],
+    "zi_attention_generic": [P, P, I, I, L, L, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
+    "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
+    "zi_argmax": [P, P, P, I, I, I, L, P],
+    "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],
+}
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+def library_path() -> Optional[str]:
+    return _lib_path
+
+
+def load() -> ctypes.CDLL:
+    """The loaded library; builds it first when nothing built matches the sources."""
+    global _lib, _lib_path
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        import torch  # noqa: F401  (loads the HIP runtime the library links against)
+        from ..csrc.build import ensure_library
+        try:
+            path = ensure_library()
+            lib = ctypes.CDLL(path)
+        except (OSError, RuntimeError) as e:
+            raise KernelLibraryError(f"cannot load the HIP kernel library: {e}") from e
+        lib.zi_last_error.restype = c_char_p
+        lib.zi_last_error.argtypes = []
+        for name, args in _PROTOTYPES.items():
+            try:
+                fn = getattr(lib, name)
+            except AttributeError as e:
+                raise KernelLibraryError(f"{path} lacks entry point {name}; rebuild it") from e
+            fn.argtypes = args
+            fn.restype = c_int
+        _lib, _lib_path = lib, path
+        return lib
+
+
+def call(name: str, *args) -> None:
+    lib = load()
+    rc = getattr(lib, name)(*args)
+    if rc != 0:
+        raise KernelLibraryError(lib.zi_last_error().decode("utf-8", "replace"))

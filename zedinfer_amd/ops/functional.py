@@ -1,0 +1,364 @@
+"""Checked launches of the HIP kernels on torch tensors."""
+from __future__ import annotations
+
+from ctypes import c_void_p
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def has_gpu() -> bool:
+    return torch.cuda.is_available()
+
+
+def device_synchronize() -> None:
+    torch.cuda.synchronize()
+
+
+def _code(t: torch.Tensor, what: str) -> int:
+    if t.dtype not in _CODES:
+        raise TypeError(f"{what}: dtype {t.dtype} is not supported (float32 and bfloat16 are)")
+    return _CODES[t.dtype]
+
+
+def _gpu(what: str, *tensors: Optional[torch.Tensor]) -> None:
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError(f"{what}: every tensor must live on the GPU; got one on {t.device}")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise ValueError(f"{what}: tensors on different devices ({dev} and {t.device})")
+
+
+def _rows(t: torch.Tensor, what: str) -> Tuple[int, int]:
+    """(row stride, width) of a 2-D tensor whose rows are dense."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise ValueError(f"{what}: expected a 2-D tensor with dense rows, got shape {tuple(t.shape)} "
+                         f"strides {t.stride()}")
+    ld = t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    if ld < t.shape[1]:
+        raise ValueError(f"{what}: rows overlap (stride {ld} < width {t.shape[1]})")
+    return ld, t.shape[1]
+
+
+def _p(t: Optional[torch.Tensor]) -> c_void_p:
+    return c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream() -> c_void_p:
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _i32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise TypeError(f"{what}: expected a contiguous int32 tensor, got {t.dtype}")
+    if n is not None and t.numel() < n:
+        raise ValueError(f"{what}: {t.numel()} entries, {n} needed")
+
+
+# ---------------------------------------------------------------------------
+def embedding(ids: torch.Tensor, table: torch.Tensor, out: Optional[torch.Tensor] = None,
+              out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """out[i,:] = table[ids[i],:] for int32 ids."""
+    _gpu("embedding", ids, table, out)
+    n = ids.numel()
+    _i32(ids, "embedding ids")
+    if table.dim() != 2 or not table.is_contiguous():
+        raise ValueError("embedding: table must be a contiguous [vocab, hidden] tensor")
+    V, H = table.shape
+    if out is None:
+        out = torch.empty((n, H), dtype=out_dtype or table.dtype, device=table.device)
+    if tuple(out.shape) != (n, H) or not out.is_contiguous():
+        raise ValueError(f"embedding: out must be contiguous [{n}, {H}], got {tuple(out.shape)}")
+    _lib.call("zi_embedding", _p(out), _code(out, "embedding out"), _p(table), _code(table, "embedding table"),
+              _p(ids), n, H, V, _stream())
+    return out
+
+
+def gather_rows(x: torch.Tensor, idx: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    _gpu("gather_rows", x, idx, out)
+    _i32(idx, "gather_rows idx")
+    if x.dim() != 2 or not x.is_contiguous():
+        raise ValueError("gather_rows: x must be contiguous 2-D")
+    n = idx.numel()
+    if out is None:
+        out = torch.empty((n, x.shape[1]), dtype=x.dtype, device=x.device)
+    if tuple(out.shape) != (n, x.shape[1]) or out.dtype != x.dtype or not out.is_contiguous():
+        raise ValueError("gather_rows: out has the wrong shape or dtype")
+    _lib.call("zi_gather_rows", _p(out), _p(x), _code(x, "gather_rows"), _p(idx), n, x.shape[0], x.shape[1],
+              _stream())
+    return out
+
+
+def add(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """c = a + b, added in float32."""
+    _gpu("add", a, b, out)
+    if a.shape != b.shape or not a.is_contiguous() or not b.is_contiguous():
+        raise ValueError(f"add: shapes {tuple(a.shape)} and {tuple(b.shape)} must match and be contiguous")
+    if out is None:
+        out = torch.empty_like(a)
+    if out.shape != a.shape or not out.is_contiguous():
+        raise ValueError("add: out has the wrong shape")
+    _lib.call("zi_add", _p(out), _code(out, "add out"), _p(a), _code(a, "add a"), _p(b), _code(b, "add b"),
+              a.numel(), _stream())
+    return out
+
+
+def swiglu(gate: torch.Tensor, up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = up * gate / (1 + exp(-gate)); gate and up may be column slices of one tensor."""
+    _gpu("swiglu", gate, up, out)
+    ldg, I = _rows(gate, "swiglu gate")
+    ldu, I2 = _rows(up, "swiglu up")
+    if gate.shape != up.shape or gate.dtype != up.dtype:
+        raise ValueError(f"swiglu: gate {tuple(gate.shape)} {gate.dtype} and up {tuple(up.shape)} {up.dtype} differ")
+    n = gate.shape[0]
+    if out is None:
+        out = torch.empty((n, I), dtype=gate.dtype, device=gate.device)
+    if tuple(out.shape) != (n, I) or out.dtype != gate.dtype or not out.is_contiguous():
+        raise ValueError("swiglu: out has the wrong shape or dtype")
+    _lib.call("zi_swiglu", _p(out), _p(gate), _p(up), _code(gate, "swiglu"), n, I, ldg, ldu, _stream())
+    return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
+             out_dtype: Optional[torch.dtype] = None, add_one: bool = False) -> torch.Tensor:
+    """y = (w [+1]) * x * rsqrt(mean(x^2) + eps) over the last dimension of a 2-D x."""
+    _gpu("rms_norm", x, weight, out)
+    ldx, H = _rows(x, "rms_norm x")
+    if weight.dim() != 1 or weight.numel() != H or not weight.is_contiguous():
+        raise ValueError(f"rms_norm: weight must be [{H}], got {tuple(weight.shape)}")
+    n = x.shape[0]
+    if out is None:
+        out = torch.empty((n, H), dtype=out_dtype or x.dtype, device=x.device)
+    ldo, Ho = _rows(out, "rms_norm out")
+    if tuple(out.shape) != (n, H):
+        raise ValueError("rms_norm: out has the wrong shape")
+    if not eps > 0:
+        raise ValueError("rms_norm: eps must be positive")
+    _lib.call("zi_rmsnorm", _p(out), _code(out, "rms_norm out"), _p(x), _code(x, "rms_norm x"), _p(weight),
+              _code(weight, "rms_norm weight"), n, H, ldx, ldo, float(eps), int(add_one), _stream())
+    return out
+
+
+def add_rms_norm(resid: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float,
+                 out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
+                 add_one: bool = False) -> torch.Tensor:
+    """resid (float32, changed in place) += delta; returns norm(resid) * w."""
+    _gpu("add_rms_norm", resid, delta, weight, out)
+    if resid.dtype != torch.float32 or resid.dim() != 2 or not resid.is_contiguous():
+        raise ValueError("add_rms_norm: the residual stream must be a contiguous float32 [n, hidden] tensor")
+    if delta.shape != resid.shape or not delta.is_contiguous():
+        raise ValueError("add_rms_norm: delta must match the residual's shape and be contiguous")
+    n, H = resid.shape
+    if weight.dim() != 1 or weight.numel() != H or not weight.is_contiguous():
+        raise ValueError(f"add_rms_norm: weight must be [{H}]")
+    if out is None:
+        out = torch.empty((n, H), dtype=out_dtype or delta.dtype, device=resid.device)
+    if tuple(out.shape) != (n, H) or not out.is_contiguous():
+        raise ValueError("add_rms_norm: out has the wrong shape")
+    _lib.call("zi_add_rmsnorm", _p(out), _code(out, "add_rms_norm out"), _p(resid), _p(delta),
+              _code(delta, "add_rms_norm delta"), _p(weight), _code(weight, "add_rms_norm weight"), n, H,
+              float(eps), int(add_one), _stream())
+    return out
+
+
+def rope_inv_freq(rotary_dim: int, theta: float, device) -> torch.Tensor:
+    """inv_freq[k] = 1 / theta^(2k / rotary_dim) in float32
+    (reference: src/backend/ops/rope/cpu/rope_cpu.cpp:62-65)."""
+    k = np.arange(rotary_dim // 2, dtype=np.float32)
+    expo = (2.0 * k / np.float32(rotary_dim)).astype(np.float32)
+    inv = (np.float32(1.0) / np.power(np.float32(theta), expo)).astype(np.float32)
+    return torch.from_numpy(inv).to(device)
+
+
+def rope(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, out: Optional[torch.Tensor] = None
+         ) -> torch.Tensor:
+    """Split-half rotation of x [n, heads, head_dim] by int32 positions [n]."""
+    _gpu("rope", x, pos, inv_freq, out)
+    if x.dim() != 3 or not x.is_contiguous():
+        raise ValueError("rope: x must be a contiguous [n, heads, head_dim] tensor")
+    n, nh, d = x.shape
+    _i32(pos, "rope positions", n)
+    rot = 2 * inv_freq.numel()
+    if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous() or rot > d:
+        raise ValueError("rope: inv_freq must be float32 with at most head_dim/2 entries")
+    if out is None:
+        out = torch.empty_like(x)
+    if out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous():
+        raise ValueError("rope: out has the wrong shape or dtype")
+    _lib.call("zi_rope", _p(out), _p(x), _code(x, "rope"), n, nh * d, nh * d, _p(pos), _p(inv_freq), nh, d, rot,
+              _stream())
+    return out
+
+
+def _check_cache(kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int, dtype, what: str) -> Tuple[int, int]:
+    """A layer's cache is [pages, kv_heads, page_size, head_dim]; returns (pages, page_size)."""
+    for c in (kcache, vcache):
+        if c.dim() != 4 or not c.is_contiguous() or c.shape[1] != nkv or c.shape[3] != d or c.dtype != dtype:
+            raise ValueError(f"{what}: cache must be contiguous [pages, {nkv}, page_size, {d}] of {dtype}, "
+                             f"got {tuple(c.shape)} {c.dtype}")
+    if kcache.shape != vcache.shape:
+        raise ValueError(f"{what}: key and value caches differ in shape")
+    return kcache.shape[0], kcache.shape[2]
+
+
+def rope_kv_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], pos: torch.Tensor,
+                  slots: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor], kcache: Optional[torch.Tensor],
+                  vcache: Optional[torch.Tensor], nh: int, nkv: int, d: int) -> None:
+    """Rotate q [n, nh*d] in place; rotate k and copy v [n, nkv*d] into the cache at ``slots``.
+    q, k and v may be column slices of one tensor.  With ``k`` None nothing is stored;
+    with ``inv_freq`` None nothing is rotated."""
+    _gpu("rope_kv_store", q, k, v, pos, slots, inv_freq, kcache, vcache)
+    ldq, wq = _rows(q, "rope_kv_store q")
+    n = q.shape[0]
+    if wq != nh * d:
+        raise ValueError(f"rope_kv_store: q has width {wq}, expected {nh}*{d}")
+    _i32(pos, "rope_kv_store positions", n)
+    write = k is not None
+    ldk = ldv = 0
+    pages = ps = 0
+    if write:
+        ldk, wk = _rows(k, "rope_kv_store k")
+        ldv, wv = _rows(v, "rope_kv_store v")
+        if wk != nkv * d or wv != nkv * d or k.shape[0] != n or v.shape[0] != n or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise ValueError("rope_kv_store: k and v must be [n, kv_heads*head_dim] of q's dtype")
+        pages, ps = _check_cache(kcache, vcache, nkv, d, q.dtype, "rope_kv_store")
+        _i32(slots, "rope_kv_store slots", n)
+    if inv_freq is not None:
+        rot = 2 * inv_freq.numel()
+        if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous() or rot > d:
+            raise ValueError("rope_kv_store: inv_freq must be float32 with at most head_dim/2 entries")
+    else:
+        rot = 0
+    _lib.call("zi_rope_kv_store", _p(q), _p(k), _p(v), _code(q, "rope_kv_store"), n, ldq, ldk, ldv, _p(pos),
+              _p(slots), _p(inv_freq), _p(kcache), _p(vcache), pages * ps, nh, nkv, d, rot, max(ps, 1), int(write),
+              _stream())
+
+
+def attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
+              tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
+              window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal grouped-query attention of q [n, nh*d] over the paged cache.
+
+    Token i belongs to row ``tok_seq[i]`` of ``block_tables`` [seqs, max_pages] and sits at
+    absolute position ``tok_pos[i]``; it sees the cached keys at positions
+    [max(0, pos - window + 1), pos] (window 0: all of them).  Returns [n, nh*d]."""
+    _gpu("attention", q, kcache, vcache, tok_seq, tok_pos, block_tables, out)
+    ldq, wq = _rows(q, "attention q")
+    n = q.shape[0]
+    if wq != nh * d:
+        raise ValueError(f"attention: q has width {wq}, expected {nh}*{d}")
+    if nkv <= 0 or nh % nkv:
+        raise ValueError(f"attention: {nh} query heads are not a multiple of {nkv} key/value heads")
+    pages, ps = _check_cache(kcache, vcache, nkv, d, q.dtype, "attention")
+    _i32(tok_seq, "attention tok_seq", n)
+    _i32(tok_pos, "attention tok_pos", n)
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("attention: block_tables must be a contiguous int32 [seqs, max_pages] tensor")
+    if out is None:
+        out = torch.empty((n, nh * d), dtype=q.dtype, device=q.device)
+    ldo, wo = _rows(out, "attention out")
+    if tuple(out.shape) != (n, nh * d) or out.dtype != q.dtype:
+        raise ValueError("attention: out has the wrong shape or dtype")
+    _lib.call("zi_attention_generic", _p(out), _p(q), _code(q, "attention"), n, ldq, ldo, _p(kcache), _p(vcache),
+              _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps,
+              int(window), float(scale), _stream())
+    return out
+
+
+def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+           out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """out[M,N] = x[M,K] . weight[N,K]^T + bias[N], accumulated in float32
+    (reference: src/backend/ops/linear/op.cpp:57-58).
+
+    bfloat16 inputs with bfloat16 weights and output go to the library matrix product, as
+    the reference sends them to its vendor library (reference:
+    src/backend/ops/linear/nvidia/linear_cublas.cu:134-231); every other pairing, and all of
+    the float32 path, runs the plain FMA kernel, which has no reduced-precision mode."""
+    _gpu("linear", x, weight, bias, out)
+    ldx, K = _rows(x, "linear x")
+    ldw, Kw = _rows(weight, "linear weight")
+    M, N = x.shape[0], weight.shape[0]
+    if K != Kw:
+        raise ValueError(f"linear: x has {K} columns, weight has {Kw}")
+    if bias is not None and (bias.dim() != 1 or bias.numel() != N or not bias.is_contiguous()):
+        raise ValueError(f"linear: bias must be [{N}]")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or x.dtype, device=x.device)
+    ldo, No = _rows(out, "linear out")
+    if tuple(out.shape) != (M, N):
+        raise ValueError(f"linear: out must be [{M}, {N}], got {tuple(out.shape)}")
+    if M == 0:
+        return out
+    bf = torch.bfloat16
+    if (x.dtype == bf and weight.dtype == bf and out.dtype == bf and (bias is None or bias.dtype == bf)
+            and out.is_contiguous()):
+        if bias is not None:
+            torch.addmm(bias, x, weight.t(), out=out)
+        else:
+            torch.mm(x, weight.t(), out=out)
+        return out
+    _lib.call("zi_gemm_generic", _p(out), _code(out, "linear out"), _p(x), _code(x, "linear x"), _p(weight),
+              _code(weight, "linear weight"), _p(bias), _code(bias, "linear bias") if bias is not None else F32,
+              M, N, K, ldx, ldw, ldo, _stream())
+    return out
+
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None, return_values: bool = False):
+    """Index of the highest value of each row (lowest index among equals) as int32."""
+    _gpu("argmax", logits, out)
+    if logits.dim() == 1:
+        logits = logits.unsqueeze(0)
+    ld, V = _rows(logits, "argmax logits")
+    R = logits.shape[0]
+    if out is None:
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _i32(out, "argmax out", R)
+    vals = torch.empty((R,), dtype=torch.float32, device=logits.device) if return_values else None
+    _lib.call("zi_argmax", _p(out), _p(vals), _p(logits), _code(logits, "argmax"), R, V, ld, _stream())
+    return (out, vals) if return_values else out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           penalty: torch.Tensor, uniform: torch.Tensor, recent: Optional[torch.Tensor] = None,
+           recent_len: Optional[torch.Tensor] = None, work: Optional[torch.Tensor] = None,
+           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of float32 logits [R, V]; per-row parameters are device tensors [R].
+    A row with temperature <= 0 takes the argmax."""
+    _gpu("sample", logits, temperature, top_k, top_p, penalty, uniform, recent, recent_len, work, out)
+    if logits.dtype != torch.float32:
+        raise TypeError("sample: logits must be float32")
+    ld, V = _rows(logits, "sample logits")
+    R = logits.shape[0]
+    for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                        ("top_p", top_p, torch.float32), ("penalty", penalty, torch.float32),
+                        ("uniform", uniform, torch.float32)):
+        if t.dtype != dt or t.numel() < R or not t.is_contiguous():
+            raise ValueError(f"sample: {name} must be a contiguous {dt} tensor with {R} entries")
+    max_recent = 0
+    if recent is not None:
+        if recent.dim() != 2 or recent.shape[0] < R or recent.dtype != torch.int32 or not recent.is_contiguous():
+            raise ValueError("sample: recent must be a contiguous int32 [R, max_recent] tensor")
+        _i32(recent_len, "sample recent_len", R)
+        max_recent = recent.shape[1]
+    if work is None:
+        work = torch.empty((R, V), dtype=torch.float32, device=logits.device)
+    if work.dtype != torch.float32 or work.numel() < R * V or not work.is_contiguous():
+        raise ValueError("sample: work must be a contiguous float32 buffer of R*V entries")
+    if out is None:
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+    _i32(out, "sample out", R)
+    _lib.call("zi_sample", _p(out), _p(logits), ld, _p(work), R, V, _p(temperature), _p(top_k), _p(top_p),
+              _p(penalty), _p(uniform), _p(recent), _p(recent_len) if recent is not None else c_void_p(0),
+              max_recent, _stream())
+    return out

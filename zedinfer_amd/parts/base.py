@@ -1,0 +1,184 @@
+"""What every part shares: the registries by kind, the runtime a part is built
+with, and the interfaces a new part has to meet.
+
+A part is a class registered under a kind.  It states the checkpoint tensors it
+needs from its spec alone (``weight_specs``), is built from (spec, weights,
+runtime) and never learns which model it sits in.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, Optional, Tuple, Type
+
+import torch
+
+from ..config.forward_config import PartSpec
+from ..weights.loader import WeightSpec
+
+
+class Runtime:
+    """Device, activation type and reusable workspaces.
+
+    ``buffer(name, shape)`` hands out a view into a named allocation that only
+    ever grows, so that steady-state steps allocate nothing and buffers keep
+    their addresses (what a captured graph needs).
+    """
+
+    def __init__(self, device: torch.device | str, dtype: torch.dtype):
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+
+    def buffer(self, name: str, shape: Tuple[int, ...], dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        dtype = dtype or self.dtype
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty((max(n, 1),), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+        return buf[:n].view(shape)
+
+    def reserve(self, name: str, numel: int, dtype: Optional[torch.dtype] = None) -> None:
+        self.buffer(name, (numel,), dtype)
+
+
+class Registry:
+    def __init__(self, what: str):
+        self.what = what
+        self._kinds: Dict[str, type] = {}
+
+    def register(self, kind: str) -> Callable[[type], type]:
+        def deco(cls: type) -> type:
+            self._kinds[kind] = cls
+            cls.kind = kind
+            return cls
+        return deco
+
+    def get(self, kind: str) -> type:
+        if kind not in self._kinds:
+            raise KeyError(f"no {self.what} registered as '{kind}'; registered: {', '.join(sorted(self._kinds))}")
+        return self._kinds[kind]
+
+    def kinds(self) -> Tuple[str, ...]:
+        return tuple(sorted(self._kinds))
+
+
+MIXERS = Registry("mixer")
+FEED_FORWARDS = Registry("feed-forward")
+NORMS = Registry("norm")
+POSITION_ENCODINGS = Registry("position encoding")
+BLOCKS = Registry("block arrangement")
+EMBEDDINGS = Registry("embedding")
+HEADS = Registry("output head")
+
+register_mixer = MIXERS.register
+register_feed_forward = FEED_FORWARDS.register
+register_norm = NORMS.register
+register_position_encoding = POSITION_ENCODINGS.register
+register_block = BLOCKS.register
+register_embedding = EMBEDDINGS.register
+register_head = HEADS.register
+
+
+@dataclass(frozen=True)
+class KVCacheRequest:
+    """What a mixer needs from the paged cache: keys of all positions ("full") or of the
+    last ``window`` positions ("window"), for ``num_kv_heads`` heads of ``head_dim``."""
+
+    kind: str
+    num_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+
+@dataclass(frozen=True)
+class StateRequest:
+    """Fixed-size state a mixer keeps per request: one tensor of ``shape`` per slot."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerMemory:
+    """What the cache manager binds to one run of a layer."""
+
+    group: int = -1                       # cache group whose slots and block tables apply
+    k: Optional[torch.Tensor] = None      # [pages, kv_heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None
+    writes: bool = True
+    state: Optional[torch.Tensor] = None  # [slots, *StateRequest.shape]
+
+
+class Part:
+    """Base of all parts."""
+
+    kind: str = ""
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        """parameter name -> what the checkpoint must hold for it."""
+        return {}
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        self.spec = spec
+        self.rt = rt
+
+
+class Mixer(Part):
+    """Mixes information across the tokens of a sequence.
+
+    ``forward(x, batch, memory)`` takes the normed hidden states [n, hidden] of all tokens
+    of the step and returns [n, hidden].  ``batch`` is the step's device-side description
+    (``engine.batch.DeviceBatch``); ``memory`` is this run's ``LayerMemory``."""
+
+    def cache_request(self) -> Optional[KVCacheRequest]:
+        return None
+
+    def state_request(self) -> Optional[StateRequest]:
+        return None
+
+    def forward(self, x: torch.Tensor, batch, memory: LayerMemory) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """``forward(x)``: [n, hidden] -> [n, hidden], token by token."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    """``forward(x)`` normalises rows; ``add_forward(resid, delta)`` first adds ``delta`` into
+    the float32 residual stream in place and returns the normalised sum."""
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        raise NotImplementedError
+
+    def add_forward(self, resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Encodes positions into queries and keys on their way into the cache."""
+
+    def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
+        raise NotImplementedError
+
+
+class Block:
+    """Arranges norms, a mixer and a feed-forward around the residual stream.  Built from
+    (norms by name, mixer, feed_forward, runtime); ``norm_names`` lists the norms it needs.
+
+    ``forward(resid, delta, batch, memory)``: ``resid`` is the float32 residual stream
+    [n, hidden], ``delta`` a pending addition to it (or None); returns the next pending
+    addition.  The add is folded into the following norm."""
+
+    norm_names: Tuple[str, ...] = ()
+
+    def forward(self, resid, delta, batch, memory: LayerMemory):
+        raise NotImplementedError

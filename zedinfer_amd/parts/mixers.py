@@ -1,0 +1,86 @@
+"""Token mixers."""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..config.forward_config import PartSpec
+from ..weights.loader import WeightSpec
+from .base import (KVCacheRequest, LayerMemory, Mixer, POSITION_ENCODINGS, Runtime, register_mixer)
+from .feed_forward import stack_rows
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    """Causal grouped-query attention over the paged cache.
+
+    q/k/v projections (with biases when ``qkv_bias``), position encoding of q and k, keys
+    and values stored to the cache, attention of every token over the cached positions it
+    may see, output projection without bias (reference:
+    src/frontend/models/transformer_forward.cpp:71-112; the scale 1/sqrt(head_dim) at :31).
+    The three projections are stacked into one [Qd + 2 KVd, H] matrix at load.
+
+    params: hidden_size, num_heads, num_kv_heads, head_dim, qkv_bias, window (0: all keys),
+    scale (default 1/sqrt(head_dim)), position (a PartSpec of a position encoding)."""
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        p = spec.params
+        H, nh, nkv, d = int(p["hidden_size"]), int(p["num_heads"]), int(p["num_kv_heads"]), int(p["head_dim"])
+        w = {"q": WeightSpec((nh * d, H)), "k": WeightSpec((nkv * d, H)), "v": WeightSpec((nkv * d, H)),
+             "o": WeightSpec((H, nh * d))}
+        if p.get("qkv_bias", False):
+            w.update({"q_bias": WeightSpec((nh * d,)), "k_bias": WeightSpec((nkv * d,)),
+                      "v_bias": WeightSpec((nkv * d,))})
+        return w
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.nh, self.nkv, self.d = int(p["num_heads"]), int(p["num_kv_heads"]), int(p["head_dim"])
+        if self.nh % self.nkv:
+            raise ValueError(f"attention: {self.nh} heads are not a multiple of {self.nkv} key/value heads")
+        if self.d % 16:
+            raise ValueError(f"attention: head_dim {self.d} must be a multiple of 16")
+        self.window = int(p.get("window", 0) or 0)
+        self.scale = float(p.get("scale") or 1.0 / math.sqrt(self.d))
+        self.qd, self.kvd = self.nh * self.d, self.nkv * self.d
+        pos_spec: PartSpec = p["position"]
+        self.position = POSITION_ENCODINGS.get(pos_spec.kind)(pos_spec, {}, rt)
+        mats = [weights["q"], weights["k"], weights["v"]]
+        self.qkv = stack_rows(mats)
+        self.mats = None if self.qkv is not None else mats
+        self.bias = self.biases = None
+        if p.get("qkv_bias", False):
+            bs = [weights["q_bias"], weights["k_bias"], weights["v_bias"]]
+            if self.qkv is not None and all(b.dtype == self.qkv.dtype for b in bs):
+                self.bias = torch.cat(bs).contiguous()
+            elif self.qkv is not None:
+                self.bias = torch.cat([b.float() for b in bs]).contiguous()
+            else:
+                self.biases = bs
+        self.o = weights["o"]
+
+    def cache_request(self) -> Optional[KVCacheRequest]:
+        return KVCacheRequest("window" if self.window > 0 else "full", self.nkv, self.d, self.window)
+
+    def forward(self, x: torch.Tensor, batch, memory: LayerMemory) -> torch.Tensor:
+        n = x.shape[0]
+        qkv = self.rt.buffer("attn_qkv", (n, self.qd + 2 * self.kvd))
+        q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
+        if self.qkv is not None:
+            ops.linear(x, self.qkv, self.bias, out=qkv)
+        else:
+            for dst, m, b in zip((q, k, v), self.mats, self.biases or (None, None, None)):
+                ops.linear(x, m, b, out=dst)
+        view = batch.groups[memory.group]
+        self.position.rotate_and_store(q, k, v, batch.positions, view.slots, memory, self.nh, self.nkv, self.d)
+        att = self.rt.buffer("attn_out", (n, self.qd))
+        ops.attention(q, memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh,
+                      self.nkv, self.d, self.scale, self.window, out=att)
+        out = self.rt.buffer("attn_proj", (n, self.hidden))
+        return ops.linear(att, self.o, out=out)

@@ -1,0 +1,43 @@
+"""Position encodings.  They act where queries and keys leave the projection:
+queries are encoded in place, keys on their way into the paged cache."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .. import ops
+from ..config.forward_config import PartSpec
+from .base import LayerMemory, PositionEncoding, Runtime, register_position_encoding
+
+
+@register_position_encoding("rope_neox")
+class RopeNeox(PositionEncoding):
+    """Split-half rotary encoding: pairs (k, k + R/2) of the first R = ``rotary_dim`` dims of
+    each head turn by pos * theta^(-2k/R) (reference: src/backend/ops/rope/cpu/rope_cpu.cpp:12-66;
+    the reference rotates the whole head, no scaling: rope_nvidia.cu:50).
+    params: head_dim, theta, rotary_dim (default head_dim)."""
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        self.head_dim = int(spec.params["head_dim"])
+        self.rotary_dim = int(spec.params.get("rotary_dim", self.head_dim))
+        self.theta = float(spec.params["theta"])
+        if self.rotary_dim % 2 or not (0 < self.rotary_dim <= self.head_dim):
+            raise ValueError(f"rope_neox: rotary_dim {self.rotary_dim} must be even and within head_dim {self.head_dim}")
+        self.inv_freq = ops.rope_inv_freq(self.rotary_dim, self.theta, rt.device)
+
+    def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
+        if memory.writes:
+            ops.rope_kv_store(q, k, v, positions, slots, self.inv_freq, memory.k, memory.v, nh, nkv, d)
+        else:
+            ops.rope_kv_store(q, None, None, positions, None, self.inv_freq, None, None, nh, nkv, d)
+
+
+@register_position_encoding("none")
+class NoPosition(PositionEncoding):
+    """No encoding: keys and values are stored as they are."""
+
+    def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
+        if memory.writes:
+            ops.rope_kv_store(q, k, v, positions, slots, None, memory.k, memory.v, nh, nkv, d)
