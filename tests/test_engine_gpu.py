@@ -1,0 +1,72 @@
+"""The engine against the plain implementation: each request alone and whole; most of it in one
+step and the last 32 tokens one by one; portions of changing size; and mixed batches with so few
+pages that they are used again.  In float32 and in bfloat16, on three tiny configurations."""
+import os
+
+import pytest
+import torch
+
+import tiny_configs
+import traces
+from plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {"A": [5, 17, 33, 100, 70, 64, 90, 41, 128, 77], "B": [1, 31, 64, 100, 47, 90, 120, 66, 35, 80],
+           "C": [1, 31, 64, 100, 47, 90, 120, 66, 35, 80]}
+# float32: rounding of a few hundred float32 operations; bfloat16: activations are rounded to 8 bits
+# of mantissa after every op.
+F32_TOL = 2e-4
+BF16_REL_WORST, BF16_REL_MEAN = 0.06, 0.012
+
+
+@pytest.fixture(scope="module", params=["A", "B", "C"])
+def tiny(request, tmp_path_factory):
+    name = request.param
+    folder = tiny_configs.write_tiny(str(tmp_path_factory.mktemp(f"tiny{name}")), name)
+    cfg, w = plain.load_folder(folder)
+    reqs = {f"r{i}": traces.random_tokens(cfg["vocab_size"], n, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
+    ref = {rid: plain.forward(cfg, w, toks) for rid, toks in reqs.items()}
+    return dict(name=name, folder=folder, cfg=cfg, weights=w, requests=reqs, reference=ref)
+
+
+def make_engine(tiny, dtype, pages):
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    return Engine.from_folder(tiny["folder"], dtype,
+                              SchedulerConfig(num_kv_blocks=pages, kv_block_size=ps, max_batch_requests=4))
+
+
+def check(tiny, dtype, steps, outputs):
+    worst, mean, scale, rows, where = traces.compare(steps, outputs, tiny["reference"], tiny["requests"])
+    print(f"[{tiny['name']} {dtype}] rows={rows} worst={worst:.3e} mean={mean:.3e} scale={scale:.3e} at {where}")
+    assert rows > 0
+    if dtype == "float32":
+        assert worst <= F32_TOL * max(1.0, scale), f"first/worst difference at (step, request, position) {where}"
+    else:
+        assert worst <= BF16_REL_WORST * scale, f"worst difference at {where}"
+        assert mean <= BF16_REL_MEAN * scale
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", ["whole", "last32", "portions", "mixed"])
+def test_engine_matches_plain(tiny, dtype, shape):
+    steps = {"whole": traces.whole, "last32": traces.last_decoded, "portions": traces.portions,
+             "mixed": traces.mixed}[shape](tiny["requests"])
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    pages = traces.max_live_tokens(steps) // ps      # as few pages as the replay tool would have
+    engine = make_engine(tiny, dtype, pages)
+    out = traces.run_in_process(engine, steps)
+    if shape == "mixed":
+        # pages were given back and taken again: more pages handed out than the pool has
+        assert all(g.pool.takes > g.pool.total for g in engine.cache.groups)
+    check(tiny, dtype, steps, out)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_tool(tiny, dtype, tmp_path):
+    """The same mixed trace through bin/trace_run as a child process."""
+    steps = traces.mixed(tiny["requests"], seed=3)
+    out = traces.run_tool(tiny["folder"], dtype, steps, str(tmp_path / "out"), traces.max_live_tokens(steps))
+    check(tiny, dtype, steps, out)

@@ -1,0 +1,259 @@
+"""Each HIP kernel alone against a plain float32 torch reference of the same op, at sizes other
+than the tiny models' (widths that are no power of two, odd head counts, several page sizes)."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DT = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype, f32=1e-5, bf16=2e-2):
+    return dict(atol=f32, rtol=f32) if dtype == torch.float32 else dict(atol=bf16, rtol=bf16)
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from zedinfer_amd import ops as o
+    o.load()
+    assert o.library_path() is not None
+    return o
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).cuda()
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("n,H,V", [(1, 48, 100), (37, 1536, 3000), (5, 200, 77)])
+def test_embedding(ops, dtype, n, H, V):
+    table = rnd(V, H, dtype=dtype)
+    ids = torch.randint(0, V, (n,), dtype=torch.int32, device="cuda")
+    out = ops.embedding(ids, table, out_dtype=torch.float32)
+    assert torch.equal(out, table[ids.long()].float())
+    out2 = ops.embedding(ids, table)
+    assert torch.equal(out2, table[ids.long()])
+
+
+def test_embedding_bad_id_is_loud(ops):
+    table = rnd(10, 32)
+    ids = torch.tensor([3, 11], dtype=torch.int32, device="cuda")
+    out = ops.embedding(ids, table)
+    assert torch.isnan(out[1]).all() and not torch.isnan(out[0]).any()
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_gather_rows(ops, dtype):
+    x = rnd(50, 72, dtype=dtype)
+    idx = torch.tensor([49, 0, 7, 7], dtype=torch.int32, device="cuda")
+    assert torch.equal(ops.gather_rows(x, idx), x[idx.long()])
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_add(ops, dtype):
+    a, b = rnd(33, 100, dtype=dtype, seed=1), rnd(33, 100, dtype=dtype, seed=2)
+    ref = (a.float() + b.float()).to(dtype)
+    assert torch.equal(ops.add(a, b), ref)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("n,I", [(1, 176), (9, 8960), (70000, 8)])
+def test_swiglu(ops, dtype, n, I):
+    gu = rnd(n, 2 * I, dtype=dtype, scale=3.0)
+    g, u = gu[:, :I], gu[:, I:]
+    ref = (torch.nn.functional.silu(g.float()) * u.float())
+    out = ops.swiglu(g, u)
+    torch.testing.assert_close(out.float(), ref.to(dtype).float(), **tol(dtype, 1e-6, 1e-2))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("n,H,eps", [(1, 1536, 1e-6), (7, 100, 1e-5), (3, 5120, 1e-6), (2, 33, 0.1)])
+def test_rms_norm(ops, dtype, n, H, eps):
+    x = rnd(n, H, dtype=dtype, scale=2.0)
+    w = (1 + 0.1 * torch.randn(H)).to(dtype).cuda()
+    xf = x.float()
+    ref = w.float() * xf / torch.sqrt((xf * xf).mean(-1, keepdim=True) + eps)
+    out = ops.rms_norm(x, w, eps)
+    torch.testing.assert_close(out.float(), ref, **tol(dtype))
+    # w = 1 reduces to the library routine
+    one = torch.ones(H, dtype=dtype, device="cuda")
+    lib = torch.nn.functional.rms_norm(xf, (H,), eps=eps)
+    torch.testing.assert_close(ops.rms_norm(x, one, eps).float(), lib, **tol(dtype))
+    # (1 + w) form
+    out1 = ops.rms_norm(x, w, eps, add_one=True)
+    torch.testing.assert_close(out1.float(), ref / w.float() * (w.float() + 1), **tol(dtype, 1e-4, 3e-2))
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_add_rms_norm(ops, dtype):
+    n, H, eps = 6, 200, 1e-6
+    resid = rnd(n, H, seed=3)
+    delta = rnd(n, H, dtype=dtype, seed=4)
+    w = rnd(H, dtype=dtype, seed=5)
+    s = resid + delta.float()
+    ref = w.float() * s / torch.sqrt((s * s).mean(-1, keepdim=True) + eps)
+    r = resid.clone()
+    out = ops.add_rms_norm(r, delta, w, eps)
+    assert torch.equal(r, s)
+    torch.testing.assert_close(out.float(), ref, **tol(dtype))
+
+
+def torch_rope(x, pos, theta):
+    """python/tests/ops/rope.py:7-30 of the reference."""
+    d = x.shape[-1]
+    a, b = x[..., : d // 2], x[..., d // 2:]
+    i = torch.arange(0, d // 2, dtype=torch.float32, device=x.device)
+    freqs = pos.float().unsqueeze(1) / (theta ** (2 * i / d))
+    sin, cos = freqs.sin().unsqueeze(1), freqs.cos().unsqueeze(1)
+    return torch.cat([a * cos - b * sin, b * cos + a * sin], -1)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("n,nh,d,start,theta", [(5, 3, 16, 0, 10000.0), (33, 12, 128, 1024, 1e6), (4, 7, 80, 300, 5e4)])
+def test_rope(ops, dtype, n, nh, d, start, theta):
+    x = rnd(n, nh, d, dtype=dtype)
+    pos = torch.arange(start, start + n, dtype=torch.int32, device="cuda")
+    ref = torch_rope(x.float(), pos, theta)
+    out = ops.rope(x, pos, ops.rope_inv_freq(d, theta, "cuda"))
+    torch.testing.assert_close(out.float(), ref, **tol(dtype, 5e-4, 2e-2))
+
+
+def make_paged(k, v, page_size, num_pages, perm_seed=0):
+    """Scatter k, v [T, nkv, d] into caches [pages, nkv, page_size, d] through a shuffled table."""
+    T, nkv, d = k.shape
+    need = (T + page_size - 1) // page_size
+    g = torch.Generator().manual_seed(perm_seed)
+    table = torch.randperm(num_pages, generator=g)[:need].to(torch.int32)
+    kc = torch.full((num_pages, nkv, page_size, d), float("nan"), dtype=k.dtype, device="cuda")
+    vc = torch.full_like(kc, float("nan"))
+    for t in range(T):
+        p, o = int(table[t // page_size]), t % page_size
+        kc[p, :, o] = k[t]
+        vc[p, :, o] = v[t]
+    return kc, vc, table.cuda()
+
+
+def ref_attention(q, k, v, pos, scale, window):
+    """q [n, nh, d] at absolute positions pos over k, v [T, nkv, d]; float32."""
+    n, nh, d = q.shape
+    nkv = k.shape[1]
+    out = torch.empty_like(q)
+    j = torch.arange(k.shape[0], device=q.device)
+    for h in range(nh):
+        g = h // (nh // nkv)
+        s = (q[:, h] @ k[:, g].t()) * scale
+        vis = j[None, :] <= pos[:, None]
+        if window:
+            vis &= (pos[:, None] - j[None, :]) < window
+        s = s.masked_fill(~vis, float("-inf"))
+        out[:, h] = torch.softmax(s, -1) @ v[:, g]
+    return out
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("nh,nkv,d,ps,T,window", [
+    (4, 2, 16, 16, 49, 0), (12, 2, 128, 16, 300, 0), (3, 1, 32, 8, 100, 0), (6, 2, 48, 8, 90, 20),
+    (5, 5, 80, 4, 70, 0), (28, 4, 128, 32, 130, 64), (2, 1, 256, 16, 65, 0)])
+def test_attention_generic(ops, dtype, nh, nkv, d, ps, T, window):
+    k, v = rnd(T, nkv, d, dtype=dtype, seed=1), rnd(T, nkv, d, dtype=dtype, seed=2)
+    kc, vc, table = make_paged(k, v, ps, 64)
+    # queries: a prompt portion at the end plus scattered single positions, in two "sequences"
+    # that share the same pages through two identical table rows
+    pos = torch.tensor(list(range(T - 7, T)) + [0, 1, ps - 1, ps, T // 2], dtype=torch.int32, device="cuda")
+    n = pos.numel()
+    q = rnd(n, nh, d, dtype=dtype, seed=3)
+    seq = torch.tensor([0] * 7 + [1] * (n - 7), dtype=torch.int32, device="cuda")
+    bt = torch.stack([table, table]).contiguous()
+    scale = 1 / math.sqrt(d)
+    out = ops.attention(q.view(n, nh * d), kc, vc, seq, pos, bt, nh, nkv, d, scale, window)
+    ref = ref_attention(q.float(), k.float(), v.float(), pos.long(), scale, window)
+    torch.testing.assert_close(out.view(n, nh, d).float(), ref, **tol(dtype, 2e-5, 2e-2))
+
+
+def test_attention_far_key_stands_out(ops):
+    """One far key among hundreds is made to dominate: its value must come through."""
+    nh, nkv, d, ps, T = 4, 1, 64, 16, 700
+    k, v = rnd(T, nkv, d, seed=1) * 0.1, rnd(T, nkv, d, seed=2)
+    q = rnd(1, nh, d, seed=3)
+    far = 37
+    k[far, 0] = q[0, 2] * 50.0 / q[0, 2].norm() ** 2 * math.sqrt(d)   # score 50 for head 2
+    kc, vc, table = make_paged(k, v, ps, 64)
+    pos = torch.tensor([T - 1], dtype=torch.int32, device="cuda")
+    out = ops.attention(q.view(1, nh * d), kc, vc, torch.zeros(1, dtype=torch.int32, device="cuda"), pos,
+                        table[None].contiguous(), nh, nkv, d, 1 / math.sqrt(d))
+    torch.testing.assert_close(out.view(nh, d)[2], v[far, 0], atol=1e-4, rtol=1e-4)
+    # and with a window that ends just after it, it is gone
+    out_w = ops.attention(q.view(1, nh * d), kc, vc, torch.zeros(1, dtype=torch.int32, device="cuda"), pos,
+                          table[None].contiguous(), nh, nkv, d, 1 / math.sqrt(d), window=T - 1 - far)
+    assert (out_w.view(nh, d)[2] - v[far, 0]).abs().max() > 0.1
+    out_w2 = ops.attention(q.view(1, nh * d), kc, vc, torch.zeros(1, dtype=torch.int32, device="cuda"), pos,
+                           table[None].contiguous(), nh, nkv, d, 1 / math.sqrt(d), window=T - far)
+    torch.testing.assert_close(out_w2.view(nh, d)[2], v[far, 0], atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_rope_kv_store(ops, dtype):
+    n, nh, nkv, d, ps, pages, theta = 11, 6, 2, 48, 8, 10, 5e4
+    qkv = rnd(n, (nh + 2 * nkv) * d, dtype=dtype)
+    q, k, v = qkv[:, :nh * d], qkv[:, nh * d:(nh + nkv) * d], qkv[:, (nh + nkv) * d:]
+    pos = torch.arange(100, 100 + n, dtype=torch.int32, device="cuda")
+    slots = torch.randperm(pages * ps)[:n].to(torch.int32).cuda()
+    kc = torch.zeros(pages, nkv, ps, d, dtype=dtype, device="cuda")
+    vc = torch.zeros_like(kc)
+    q_ref = torch_rope(q.float().reshape(n, nh, d), pos, theta)
+    k_ref = torch_rope(k.float().reshape(n, nkv, d), pos, theta)
+    v_ref = v.clone().reshape(n, nkv, d)
+    ops.rope_kv_store(q, k, v, pos, slots, ops.rope_inv_freq(d, theta, "cuda"), kc, vc, nh, nkv, d)
+    torch.testing.assert_close(q.float().reshape(n, nh, d), q_ref, **tol(dtype, 5e-4, 2e-2))
+    for t in range(n):
+        p, o = int(slots[t]) // ps, int(slots[t]) % ps
+        torch.testing.assert_close(kc[p, :, o].float(), k_ref[t], **tol(dtype, 5e-4, 2e-2))
+        assert torch.equal(vc[p, :, o], v_ref[t])
+    # untouched slots stay zero
+    assert int((kc != 0).any(-1).any(1).sum()) == n
+
+
+@pytest.mark.parametrize("xdt,wdt,odt", [(torch.float32,) * 3, (torch.bfloat16,) * 3,
+                                          (torch.bfloat16, torch.float32, torch.bfloat16),
+                                          (torch.bfloat16, torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("M,N,K", [(1, 100, 64), (5, 1000, 96), (70, 130, 176), (128, 1536, 8960), (3, 151, 33)])
+def test_linear(ops, xdt, wdt, odt, M, N, K):
+    x, w, b = rnd(M, K, dtype=xdt, seed=1), rnd(N, K, dtype=wdt, scale=0.05, seed=2), rnd(N, dtype=wdt, seed=3)
+    ref = torch.nn.functional.linear(x.double(), w.double(), b.double()).float()
+    out = ops.linear(x, w, b, out_dtype=odt)
+    assert out.dtype == odt
+    t = tol(odt, 5e-5, 2e-2)
+    torch.testing.assert_close(out.float(), ref, **t)
+    out_nb = ops.linear(x, w, out_dtype=odt)
+    torch.testing.assert_close(out_nb.float(), torch.nn.functional.linear(x.double(), w.double()).float(), **t)
+    # into a column slice of a wider buffer
+    wide = torch.zeros(M, N + 8, dtype=odt, device="cuda")
+    ops.linear(x, w, b, out=wide[:, 4:N + 4])
+    torch.testing.assert_close(wide[:, 4:N + 4].float(), ref, **t)
+    assert float(wide[:, :4].abs().max()) == 0 and float(wide[:, N + 4:].abs().max()) == 0
+
+
+def test_linear_f32_row_does_not_depend_on_batch(ops):
+    """The float32 product sums over k in one fixed order: a row's result is bit-identical whatever M is."""
+    x, w = rnd(70, 176, seed=1), rnd(130, 176, seed=2)
+    full = ops.linear(x, w)
+    one = ops.linear(x[17:18].contiguous(), w)
+    assert torch.equal(full[17], one[0])
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_argmax(ops, dtype):
+    x = rnd(5, 1000, dtype=dtype)
+    idx, val = ops.argmax(x, return_values=True)
+    assert torch.equal(idx.long(), torch.argmax(x.float(), -1))
+    torch.testing.assert_close(val, x.float().max(-1).values)
+    # ties: the lowest index wins (reference: tests/sampler/test_sampler.cpp:85-122)
+    t = torch.zeros(2, 151936, dtype=dtype, device="cuda")
+    t[0, 70000] = 3.0
+    t[0, 1234] = 3.0
+    t[1, -1] = 1.0
+    assert ops.argmax(t).tolist() == [1234, 151935]
+    assert ops.argmax(torch.zeros(1, 77, device="cuda")).tolist() == [0]

@@ -29,6 +29,7 @@ class IdPool:
         self.what = what
         self._free: List[int] = list(range(self.total - 1, -1, -1))  # id 0 is handed out first
         self._held = bytearray(self.total)
+        self.takes = 0      # ids handed out so far; more than `total` means ids were used again
 
     @property
     def num_free(self) -> int:
@@ -43,6 +44,7 @@ class IdPool:
             raise (OutOfPages if self.what == "page" else OutOfSlots)(f"no free {self.what} (pool of {self.total})")
         i = self._free.pop()
         self._held[i] = 1
+        self.takes += 1
         return i
 
     def give_back(self, i: int) -> None:
