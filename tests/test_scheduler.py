@@ -1,0 +1,187 @@
+"""The scheduler's decisions, with the cache manager's host bookkeeping and made-up tokens (CPU).
+Cases follow the reference's tests/zedinfer/test_scheduler_sampling.cpp."""
+import pytest
+import torch
+
+from zedinfer_amd.cache import CacheManager
+from zedinfer_amd.config import SchedulerConfig
+from zedinfer_amd.engine.request import GenerationConfig, InferenceRequest, RequestPhase, resolve_max_new_tokens
+from zedinfer_amd.engine.scheduler import QueueFull, Scheduler
+from zedinfer_amd.parts import KVCacheRequest
+
+
+def make(pages=64, page_size=4, **kw):
+    cfg = SchedulerConfig(num_kv_blocks=pages, kv_block_size=page_size, **kw)
+    cache = CacheManager({0: KVCacheRequest("full", 1, 16)}, {}, pages, page_size, cfg.max_batch_requests,
+                         torch.float32, None, cfg.max_batch_tokens)
+    return Scheduler(cfg, cache, stop_token_ids=[99]), cache
+
+
+def run_step(sched, cache, token=7):
+    """What the serving loop does around a model step, with a constant 'sampled' token."""
+    batch = sched.schedule()
+    if batch.empty():
+        return batch
+    for e in batch.entries():
+        cache.ensure(e.seq, e.seq.length + len(e.tokens))
+        cache.commit(e.seq, e.seq.length + len(e.tokens))
+    toks = token if isinstance(token, list) else [token] * len(batch.sampled_requests())
+    sched.process_results(batch, toks)
+    cache.check()
+    return batch
+
+
+def req(n, max_new=4, **kw):
+    return InferenceRequest(list(range(1, n + 1)), GenerationConfig(max_new_tokens=max_new, **kw))
+
+
+def test_mixed_batch_decode_rows_first_and_last_row_of_prompt():
+    # reference: test_scheduler_sampling.cpp:64-102
+    s, c = make()
+    a = req(5)
+    s.submit(a)
+    b1 = run_step(s, c)
+    assert b1.prefill_requests == [a] and b1.prefill_chunk_sizes == [5] and not b1.decode_requests
+    assert a.phase == RequestPhase.DECODE and a.output_ids == [7] and a.generated_count == 1
+    b = req(6)
+    s.submit(b)
+    batch = s.schedule()
+    assert batch.decode_requests == [a] and batch.prefill_requests == [b]
+    entries = batch.entries()
+    assert entries[0].tokens == [7] and list(entries[0].want) == [0]           # the decode row comes first
+    assert entries[1].tokens == [1, 2, 3, 4, 5, 6] and list(entries[1].want) == [5]   # last row of the prompt
+    assert batch.sampled_requests() == [a, b]
+
+
+def test_chunked_prefill_under_the_budget():
+    s, c = make(max_batch_tokens=16, max_prefill_tokens=8)
+    a, b = req(20, max_new=3), req(3, max_new=3)
+    s.submit(a)
+    s.submit(b)
+    sizes = []
+    for _ in range(3):
+        batch = run_step(s, c)
+        sizes.append((list(batch.prefill_chunk_starts), list(batch.prefill_chunk_sizes), len(batch.decode_requests)))
+        assert batch.num_tokens() <= 16
+    # a is cut 8 + 8 + 4; only when a's prompt completes does b get the rest of the budget (3 of 4 left)
+    assert sizes == [([0], [8], 0), ([8], [8], 0), ([16, 0], [4, 3], 0)]
+    assert a.output_ids == [7] and b.output_ids == [7]
+    batch = run_step(s, c)
+    assert len(batch.decode_requests) == 2 and not batch.prefill_requests
+    # an unfinished prompt yields no token and stays at the head of the queue
+    s2, c2 = make(max_prefill_tokens=4)
+    x = req(10)
+    s2.submit(x)
+    b2 = s2.schedule()
+    assert b2.sampled_requests() == [] and list(b2.entries()[0].want) == [] and s2.waiting[0] is x
+    assert x.phase == RequestPhase.PREFILL
+
+
+def test_decode_budget_and_request_cap():
+    s, c = make(max_batch_requests=2)
+    rs = [req(2, max_new=8) for _ in range(3)]
+    for r in rs:
+        s.submit(r)
+    run_step(s, c)
+    assert [r.phase for r in rs] == [RequestPhase.DECODE, RequestPhase.DECODE, RequestPhase.QUEUED]
+    batch = run_step(s, c)
+    assert len(batch.decode_requests) == 2 and not batch.prefill_requests       # the cap keeps the third out
+
+
+def test_finish_reasons_and_release():
+    s, c = make()
+    a, b, d = req(3, max_new=2), req(3, max_new=5), req(3, max_new=1)
+    for r in (a, b, d):
+        s.submit(r)
+    run_step(s, c, token=[7, 99, 7])
+    assert b.done and b.finish_reason == "stop" and b.result.output_ids == [99]
+    assert d.done and d.finish_reason == "length"                  # max_new_tokens == 1 ends at the prompt
+    run_step(s, c)
+    assert a.done and a.finish_reason == "length" and a.output_ids == [7, 7]
+    assert not c.live and c.groups[0].pool.num_free == 64 and not s.has_work()
+    e = req(3, max_new=3, ignore_eos=True)
+    s.submit(e)
+    for _ in range(3):
+        run_step(s, c, token=99)
+    assert e.finish_reason == "length" and e.output_ids == [99, 99, 99]
+
+
+def test_request_that_can_never_fit_fails_instead_of_waiting():
+    # reference: test_scheduler_sampling.cpp:104-131
+    s, c = make(pages=4, page_size=4)
+    big, small = req(40, max_new=4), req(4, max_new=2)
+    s.submit(big)
+    s.submit(small)
+    batch = s.schedule()
+    assert big.done and big.finish_reason == "error" and "Cannot admit" in big.error
+    assert batch.prefill_requests == [small]                       # the queue moves on
+
+
+def test_head_of_queue_waits_while_others_run():
+    s, c = make(pages=8, page_size=4, generation_reserve=4)
+    a = req(20, max_new=4)                                         # 24 tokens: 6 of 8 pages
+    b = req(12, max_new=4)                                         # 16 tokens: 4 pages, does not fit beside a
+    s.submit(a)
+    run_step(s, c)
+    s.submit(b)
+    for _ in range(2):
+        batch = run_step(s, c)
+        assert batch.decode_requests == [a] and not batch.prefill_requests and b.phase == RequestPhase.QUEUED
+    run_step(s, c)                                                 # a reaches its 4 tokens and frees its pages
+    assert a.done
+    batch = run_step(s, c)
+    assert batch.prefill_requests == [b] and not b.error
+
+
+def test_decode_exhaustion_fails_only_that_request():
+    # reference: test_scheduler_sampling.cpp:133-170
+    s, c = make(pages=4, page_size=4, generation_reserve=0)
+    a, b = req(8, max_new=20), req(7, max_new=20)                  # promised 2 + 2 pages, all 4
+    s.submit(a)
+    s.submit(b)
+    run_step(s, c)
+    batch = run_step(s, c)                                         # a needs a third page: none unpromised
+    assert a.done and a.finish_reason == "error" and "KV cache exhausted during decode" in a.error
+    assert batch.decode_requests == [b]
+    for _ in range(4):
+        run_step(s, c)
+    assert not b.done and b.generated_count == 6                   # b took over the pages a gave back
+    c.check()
+
+
+def test_queue_limit_and_limits_resolution():
+    s, c = make(max_queue_size=2)
+    s.submit(req(2))
+    s.submit(req(2))
+    with pytest.raises(QueueFull):
+        s.submit(req(2))
+    # reference: src/zedinfer/generation_types.cpp:39-61
+    assert resolve_max_new_tokens(0, 100, 512) == 412
+    assert resolve_max_new_tokens(1000, 100, 512) == 412
+    assert resolve_max_new_tokens(5, 100, 512) == 5
+    with pytest.raises(ValueError, match="no room"):
+        resolve_max_new_tokens(5, 512, 512)
+    s3, _ = make(max_seq_len=16)
+    r = req(10, max_new=0)
+    s3.submit(r)
+    assert r.config.max_new_tokens == 6
+
+
+def test_failed_step_fails_its_batch_and_frees():
+    s, c = make()
+    a = req(5)
+    s.submit(a)
+    batch = s.schedule()
+    s.fail_batch(batch, "step failed: boom")
+    assert a.done and a.error == "step failed: boom" and not c.live and not s.has_work()
+
+
+def test_sampling_options_are_validated():
+    # reference: tests/sampler/test_sampler.cpp:39-67
+    s, _ = make()
+    for bad in (dict(top_p=0.0), dict(top_p=1.5), dict(top_k=-1), dict(repetition_penalty=0.0),
+                dict(temperature=-1.0)):
+        with pytest.raises(ValueError):
+            s.submit(req(2, **bad))
+    with pytest.raises(ValueError, match="stream_callback"):
+        s.submit(req(2, stream=True))

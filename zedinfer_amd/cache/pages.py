@@ -95,5 +95,3 @@ class PagePool(IdPool):
         super().check()
         if not (0 <= self.committed <= self.total):
             raise AssertionError("page pool: promised pages out of range")
-        if self.num_held > self.committed:
-            raise AssertionError("page pool: more pages held than promised")

@@ -1,0 +1,128 @@
+"""The serving loop and the engine object users hold.
+
+``InferenceEngine.create(model_path, ...)`` builds model, cache, scheduler and sampler;
+``serving_loop().submit_async`` queues requests, ``step()`` runs one scheduled batch,
+``run_loop()`` runs until nothing is left, ``generate_tokens`` does all of it for one prompt
+(reference: include/zedinfer/serving_loop.hpp:36-56, src/zedinfer/serving_loop.cpp:182-422;
+include/zedinfer/engine.hpp:96-166, src/zedinfer/engine.cpp:338-522).
+"""
+from __future__ import annotations
+
+import time
+from typing import Iterable, List, Optional, Sequence
+
+import torch
+
+from ..config import SchedulerConfig
+from ..sampling.sampler import Sampler
+from .engine import Engine
+from .request import GenerationConfig, GenerationResult, InferenceRequest, RequestPhase
+from .scheduler import ScheduledBatch, Scheduler
+
+
+class ServingLoop:
+    def __init__(self, engine: Engine, stop_token_ids: Iterable[int] = ()):
+        self.engine = engine
+        self.scheduler = Scheduler(engine.sched, engine.cache, stop_token_ids)
+        self.sampler = Sampler(engine.device, engine.vocab_size)
+        self._running = False
+
+    def submit_async(self, request: InferenceRequest) -> InferenceRequest:
+        """Queue a request; its ``result`` is set when it completes."""
+        self.scheduler.submit(request)
+        return request
+
+    def pending_count(self) -> int:
+        return self.scheduler.pending_count()
+
+    def active_count(self) -> int:
+        return self.scheduler.active_count()
+
+    def step(self) -> bool:
+        """One scheduled batch through the model.  Returns False when there was nothing to run."""
+        batch = self.scheduler.schedule()
+        if batch.empty():
+            return False
+        t0 = time.perf_counter()
+        try:
+            logits = self.engine.step(batch.entries(), copy=False)
+            sampled = batch.sampled_requests()
+            tokens: List[int] = []
+            if sampled:
+                tokens = self.sampler.sample(logits, [r.sampler for r in sampled], [r.output_ids for r in sampled])
+            else:
+                torch.cuda.synchronize(self.engine.device)
+        except Exception as e:  # noqa: BLE001  (a failed step fails its batch, not the loop)
+            self.scheduler.fail_batch(batch, f"step failed: {type(e).__name__}: {e}")
+            return True
+        ms = (time.perf_counter() - t0) * 1000.0
+        # time is split like the reference's: a step's time goes to prefill for prompt portions and is
+        # shared evenly among the decoding requests (reference: serving_loop.cpp:287-305)
+        n_dec, n_pre = len(batch.decode_requests), len(batch.prefill_requests)
+        for r in batch.prefill_requests:
+            r.stats.prefill_time_ms += ms / n_pre if not n_dec else ms * 0.5 / n_pre
+        for r in batch.decode_requests:
+            r.stats.decode_time_ms += ms / n_dec if not n_pre else ms * 0.5 / n_dec
+        self.scheduler.process_results(batch, tokens)
+        return True
+
+    def run_loop(self) -> None:
+        """Run until every queued and running request is done (reference: run_loop, offline mode)."""
+        while self.scheduler.has_work():
+            if not self.step() and not self.scheduler.has_work():
+                break
+
+    def run_serving(self) -> None:
+        """Run until ``stop()``; sleeps while idle."""
+        self._running = True
+        while self._running:
+            if not self.step():
+                self.scheduler.wait_for_work(timeout=0.05)
+
+    def stop(self) -> None:
+        self._running = False
+
+    def generate_tokens(self, input_ids: Sequence[int], config: Optional[GenerationConfig] = None) -> GenerationResult:
+        req = InferenceRequest(input_ids, config)
+        self.submit_async(req)
+        while not req.done:
+            self.step()
+        if req.error:
+            raise RuntimeError(req.error)
+        return req.result
+
+
+class InferenceEngine:
+    """Everything for generation from one model folder."""
+
+    def __init__(self, engine: Engine):
+        self.engine = engine
+        self._loop = ServingLoop(engine, engine.fc.eos_token_ids)
+
+    @classmethod
+    def create(cls, model_path: str, dtype="bfloat16", scheduler_config: Optional[SchedulerConfig] = None
+               ) -> "InferenceEngine":
+        return cls(Engine.from_folder(model_path, dtype, scheduler_config))
+
+    def serving_loop(self) -> ServingLoop:
+        return self._loop
+
+    def stop_token_ids(self) -> List[int]:
+        return sorted(self._loop.scheduler.stop_token_ids)
+
+    def block_pool(self):
+        return self.engine.cache
+
+    def generate_tokens(self, input_ids: Sequence[int], config: Optional[GenerationConfig] = None) -> GenerationResult:
+        return self._loop.generate_tokens(input_ids, config)
+
+    def generate(self, prompts: Sequence[Sequence[int]], config: Optional[GenerationConfig] = None
+                 ) -> List[GenerationResult]:
+        """Token ids in, token ids out, for several prompts batched continuously."""
+        import copy
+        reqs = [self._loop.submit_async(InferenceRequest(p, copy.copy(config) if config else None)) for p in prompts]
+        self._loop.run_loop()
+        for r in reqs:
+            if r.error:
+                raise RuntimeError(r.error)
+        return [r.result for r in reqs]

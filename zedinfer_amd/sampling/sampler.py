@@ -1,0 +1,95 @@
+"""Choosing the next token: argmax, and temperature / top-k / top-p / repetition-penalty
+sampling, one kernel launch for all rows of a step.
+
+Options and their meanings are the reference's (reference: include/frontend/sampler/sampler.hpp:27-40
+SamplerParams; validation src/frontend/sampler/sampler.cpp:24-38; the order of the steps
+:195-265).  The uniform draw comes from the host, as in the reference's GPU path
+(sampler.cpp:400-407), but from a generator kept per request, so that what a request samples
+does not depend on what else is in the batch (the reference shares one generator,
+src/zedinfer/scheduler.cpp:584-600).
+"""
+from __future__ import annotations
+
+import random
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+
+
+@dataclass
+class SamplingParams:
+    """temperature <= 0 or ``use_argmax`` means greedy (reference: scheduler.cpp:581-583)."""
+
+    temperature: float = 0.0
+    top_k: int = 0                   # 0: off
+    top_p: float = 1.0               # 1: off
+    repetition_penalty: float = 1.0  # 1: off; applied to generated tokens only
+    seed: int = 0                    # 0: seeded from the system
+    use_argmax: bool = False
+
+    @property
+    def greedy(self) -> bool:
+        return self.use_argmax or self.temperature <= 0.0
+
+    def validate(self) -> None:
+        if self.top_k < 0:
+            raise ValueError("top_k must be non-negative")
+        if not (0.0 < self.top_p <= 1.0):
+            raise ValueError("top_p must be in (0, 1]")
+        if not (self.repetition_penalty > 0.0):
+            raise ValueError("repetition_penalty must be positive")
+        if not self.use_argmax and self.temperature < 0.0:
+            raise ValueError("temperature must be non-negative (0 means greedy)")
+
+
+class RequestSampler:
+    """The sampling state of one request: its parameters and its own generator."""
+
+    def __init__(self, params: SamplingParams):
+        params.validate()
+        self.params = params
+        self.rng = random.Random(params.seed) if params.seed != 0 else random.Random()
+
+    def draw(self) -> float:
+        u = np.float32(self.rng.random())
+        return float(min(u, np.float32(0.99999994)))     # stays below 1 after rounding to float32
+
+
+class Sampler:
+    """Samples one token for each row of float32 logits [rows, vocab] on the device."""
+
+    def __init__(self, device: torch.device, vocab_size: int):
+        self.device = device
+        self.vocab_size = vocab_size
+
+    def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler],
+               histories: Optional[Sequence[Sequence[int]]] = None) -> List[int]:
+        """``samplers[i]`` and ``histories[i]`` (the tokens generated so far) belong to row i."""
+        R = logits.shape[0]
+        if R != len(samplers):
+            raise ValueError(f"{R} rows of logits for {len(samplers)} requests")
+        if all(s.params.greedy and s.params.repetition_penalty == 1.0 for s in samplers):
+            return ops.argmax(logits).tolist()
+        temp = np.array([0.0 if s.params.greedy else s.params.temperature for s in samplers], dtype=np.float32)
+        top_k = np.array([s.params.top_k for s in samplers], dtype=np.int32)
+        top_p = np.array([s.params.top_p for s in samplers], dtype=np.float32)
+        pen = np.array([s.params.repetition_penalty for s in samplers], dtype=np.float32)
+        u = np.array([0.0 if s.params.greedy else s.draw() for s in samplers], dtype=np.float32)
+        recent = recent_len = None
+        if histories is not None and any(p != 1.0 for p in pen):
+            width = max(1, max(len(h) if pen[i] != 1.0 else 0 for i, h in enumerate(histories)))
+            rc = np.zeros((R, width), dtype=np.int32)
+            rl = np.zeros((R,), dtype=np.int32)
+            for i, h in enumerate(histories):
+                if pen[i] != 1.0 and len(h):
+                    rc[i, :len(h)] = h
+                    rl[i] = len(h)
+            recent = torch.from_numpy(rc).to(self.device)
+            recent_len = torch.from_numpy(rl).to(self.device)
+        dev = lambda a: torch.from_numpy(a).to(self.device)  # noqa: E731
+        out = ops.sample(logits, dev(temp), dev(top_k), dev(top_p), dev(pen), dev(u), recent, recent_len)
+        return out.tolist()
