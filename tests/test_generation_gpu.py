@@ -1,0 +1,189 @@
+"""Generation through the entry points: greedy tokens against the plain implementation, continuous
+batching with chunked prefill, sampling against the plain sampler, the command lines."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+import tiny_configs
+import traces
+from plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def tiny(request, tmp_path_factory):
+    name = request.param
+    folder = tiny_configs.write_tiny(str(tmp_path_factory.mktemp(f"gen{name}")), name)
+    cfg, w = plain.load_folder(folder)
+    return dict(name=name, folder=folder, cfg=cfg, weights=w)
+
+
+def engine(tiny, dtype="float32", **kw):
+    from zedinfer_amd import InferenceEngine, SchedulerConfig
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    sc = dict(num_kv_blocks=64, kv_block_size=ps, max_batch_requests=4)
+    sc.update(kw)
+    return InferenceEngine.create(tiny["folder"], dtype, SchedulerConfig(**sc))
+
+
+def test_greedy_generation_matches_plain(tiny):
+    """BASELINE's tiny workloads: prompts 5/17/33 (A) and 1/31/64/100 (B), 16 greedy tokens each."""
+    from zedinfer_amd import GenerationConfig
+    lens = [5, 17, 33] if tiny["name"] == "A" else [1, 31, 64, 100]
+    V = tiny["cfg"]["vocab_size"]
+    ie = engine(tiny)
+    for i, n in enumerate(lens):
+        prompt = traces.random_tokens(V, n, seed=i)
+        want = plain.greedy_generate(tiny["cfg"], tiny["weights"], prompt, 16)
+        res = ie.generate_tokens(prompt, GenerationConfig(max_new_tokens=16, ignore_eos=True))
+        assert res.output_ids == want and res.finish_reason == "length"
+        assert res.stats.prompt_tokens == n and res.stats.generated_tokens == 16
+    assert not ie.engine.cache.live
+
+
+def test_continuous_batching_equals_one_by_one(tiny):
+    """Chunked prefill (24 tokens a step) mixed with decoding of earlier requests gives every request
+    the tokens it gets alone."""
+    from zedinfer_amd import GenerationConfig
+    lens = [1, 31, 64, 100, 7, 50]
+    V = tiny["cfg"]["vocab_size"]
+    prompts = [traces.random_tokens(V, n, seed=10 + i) for i, n in enumerate(lens)]
+    ie = engine(tiny, max_prefill_tokens=24, max_batch_tokens=32, max_batch_requests=3)
+    results = ie.generate(prompts, GenerationConfig(max_new_tokens=12, ignore_eos=True))
+    for prompt, res in zip(prompts, results):
+        assert res.output_ids == plain.greedy_generate(tiny["cfg"], tiny["weights"], prompt, 12)
+    ie.engine.cache.check()
+    assert not ie.engine.cache.live and ie.engine.steps_run > 12
+
+
+def test_long_decoding(tiny):
+    """200 tokens decoded one by one from a short prompt: logits at every step against the plain run
+    of the final sequence."""
+    from zedinfer_amd.engine import StepEntry
+    V = tiny["cfg"]["vocab_size"]
+    toks = traces.random_tokens(V, 230, seed=5)
+    ref = plain.forward(tiny["cfg"], tiny["weights"], toks)
+    ie = engine(tiny)
+    e = ie.engine
+    s = e.open("long")
+    got = [e.step([StepEntry(s, toks[:30], list(range(30)))])]
+    for t in toks[30:]:
+        got.append(e.step([StepEntry(s, [t], [0])]))
+    e.close(s)
+    got = torch.cat(got).cpu()
+    assert float((got - ref).abs().max()) < 2e-4
+
+
+def test_first_tokens_of_a_sequence(tiny):
+    """Position 0 alone, then position 1 alone: the smallest cases of the cache."""
+    from zedinfer_amd.engine import StepEntry
+    toks = [7, 9, 11]
+    ref = plain.forward(tiny["cfg"], tiny["weights"], toks)
+    e = engine(tiny).engine
+    s = e.open("first")
+    for i, t in enumerate(toks):
+        lg = e.step([StepEntry(s, [t], [0])]).cpu()
+        assert float((lg[0] - ref[i]).abs().max()) < 1e-4
+    e.close(s)
+
+
+def test_stop_token_ends_generation(tiny):
+    from zedinfer_amd import GenerationConfig
+    prompt = traces.random_tokens(tiny["cfg"]["vocab_size"], 9, seed=3)
+    free = plain.greedy_generate(tiny["cfg"], tiny["weights"], prompt, 8)
+    ie = engine(tiny)
+    ie.serving_loop().scheduler.stop_token_ids = {free[3]}
+    res = ie.generate_tokens(prompt, GenerationConfig(max_new_tokens=8))
+    first = free.index(free[3])
+    assert res.finish_reason == "stop" and res.output_ids == free[:first + 1]
+
+
+def test_out_of_pages_fails_the_request_not_the_engine(tiny):
+    from zedinfer_amd import GenerationConfig
+    ie = engine(tiny, num_kv_blocks=4)
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    with pytest.raises(RuntimeError, match="Cannot admit"):
+        ie.generate_tokens(list(range(1, 5 * ps)), GenerationConfig(max_new_tokens=4))
+    res = ie.generate_tokens([1, 2, 3], GenerationConfig(max_new_tokens=4, ignore_eos=True))
+    assert len(res.output_ids) == 4
+
+
+def test_sampling_kernel_against_plain_sampler():
+    """Same logits, same uniform draw: the kernel picks the token the plain sorted-order sampler picks."""
+    from zedinfer_amd import ops
+    g = torch.Generator().manual_seed(0)
+    V = 1000
+    cases = [(1.0, 0, 1.0, 1.0), (0.7, 0, 1.0, 1.0), (0.7, 5, 1.0, 1.0), (1.3, 0, 0.8, 1.0), (0.9, 50, 0.5, 1.0),
+             (1.0, 1, 1.0, 1.0), (0.01, 0, 1.0, 1.0), (1.0, 0, 0.05, 1.0), (0.8, 20, 0.9, 1.7)]
+    rows, params, us, hist = [], [], [], []
+    for ci, c in enumerate(cases):
+        for r in range(12):
+            rows.append(torch.randn(V, generator=g) * 2.5)
+            params.append(c)
+            us.append(float(torch.rand((), generator=g)))
+            hist.append([int(x) for x in torch.randint(0, V, (6,), generator=g)] + [int(rows[-1].argmax())] * 2)
+    logits = torch.stack(rows).cuda()
+    R = len(rows)
+    dev = lambda v, dt: torch.tensor(v, dtype=dt, device="cuda")  # noqa: E731
+    recent = torch.tensor(hist, dtype=torch.int32, device="cuda")
+    out = ops.sample(logits, dev([p[0] for p in params], torch.float32), dev([p[1] for p in params], torch.int32),
+                     dev([p[2] for p in params], torch.float32), dev([p[3] for p in params], torch.float32),
+                     dev(us, torch.float32), recent, dev([len(h) for h in hist], torch.int32)).tolist()
+    mismatches = 0
+    for i in range(R):
+        T, k, p, pen = params[i]
+        probs, idx = plain.truncated_distribution(rows[i], T, k, p, pen, hist[i])
+        c = torch.cumsum(probs, 0)
+        hit = (us[i] < c).nonzero()
+        want = int(idx[int(hit[0])] if len(hit) else idx[-1])
+        assert out[i] in idx.tolist(), f"row {i}: token {out[i]} is outside the kept set"
+        mismatches += out[i] != want
+    assert mismatches == 0
+    # top_k = 1, a tiny top_p and a tiny temperature are all argmax (reference: tests/sampler/test_sampler.cpp:157-202)
+    am = torch.argmax(logits, -1).tolist()
+    for i, c in enumerate(params):
+        if c in [(1.0, 1, 1.0, 1.0), (0.01, 0, 1.0, 1.0)]:
+            assert out[i] == am[i]
+
+
+def test_sampling_in_the_engine_is_seeded_per_request(tiny):
+    """Temperature 0.7 with a fixed seed: the same request samples the same tokens alone and in a
+    mixed batch with chunked prefill; another seed gives other tokens."""
+    from zedinfer_amd import GenerationConfig, InferenceRequest
+    V = tiny["cfg"]["vocab_size"]
+    prompts = [traces.random_tokens(V, n, seed=20 + i) for i, n in enumerate([1, 31, 64, 100])]
+    cfg = lambda s: GenerationConfig(max_new_tokens=10, temperature=0.7, seed=s, ignore_eos=True)  # noqa: E731
+    alone = [engine(tiny).generate_tokens(p, cfg(100 + i)).output_ids for i, p in enumerate(prompts)]
+    ie = engine(tiny, max_prefill_tokens=24, max_batch_tokens=40)
+    loop = ie.serving_loop()
+    reqs = [loop.submit_async(InferenceRequest(p, cfg(100 + i))) for i, p in enumerate(prompts)]
+    loop.run_loop()
+    assert [r.output_ids for r in reqs] == alone
+    other = engine(tiny).generate_tokens(prompts[3], cfg(999)).output_ids
+    assert other != alone[3]
+    greedy = engine(tiny).generate_tokens(prompts[3], GenerationConfig(max_new_tokens=10, ignore_eos=True)).output_ids
+    assert greedy == plain.greedy_generate(tiny["cfg"], tiny["weights"], prompts[3], 10)
+
+
+def test_command_lines(tiny, tmp_path):
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    run = lambda *a: subprocess.run([sys.executable, *a], capture_output=True, text=True, env=env, timeout=300)  # noqa: E731
+    ps = str(tiny_configs.PAGE_SIZES[tiny["name"]])
+    prompt = traces.random_tokens(tiny["cfg"]["vocab_size"], 9, seed=3)
+    r = run(os.path.join(ROOT, "bin", "ping"), tiny["folder"], "--dtype", "fp32", "--prompt-ids",
+            ",".join(map(str, prompt)), "--max-new-tokens", "5", "--ignore-eos", "--num-kv-blocks", "32",
+            "--kv-block-size", ps)
+    assert r.returncode == 0, r.stderr
+    want = plain.greedy_generate(tiny["cfg"], tiny["weights"], prompt, 5)
+    assert "output_ids: " + ",".join(map(str, want)) in r.stdout and "finish_reason: length" in r.stdout
+    r = run(os.path.join(ROOT, "bin", "bench"), tiny["folder"], "-p", "32", "-d", "8", "-r", "1",
+            "--num-kv-blocks", "32", "--kv-block-size", ps)
+    assert r.returncode == 0 and "Prefill:" in r.stdout and "tok/s" in r.stdout, r.stderr
+    r = run(os.path.join(ROOT, "bin", "batch_bench"), tiny["folder"], "-b", "3", "-p", "20", "-d", "6",
+            "--num-kv-blocks", "64", "--kv-block-size", ps, "--random-weights", "--seed", "4")
+    assert r.returncode == 0 and "Throughput" in r.stdout and "18 tokens generated" in r.stdout, r.stderr + r.stdout
