@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""The headline benchmark: decode tokens a second of the Qwen2.5-1.5B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+A step is one decode step of the serving loop (schedule, model, sampling) with ``batch`` running
+requests that each hold a 2,048-token prompt.  Prints ONE JSON line.  Besides the decode speed it
+reports a 2,048-token prefill (tokens a second and the fraction of the bf16 matrix peak), the
+decode step against the HBM roofline (bytes that must be read: every weight once and the cache of
+the live requests), and decode at batch 1 and 64.  Weights are seeded random, token ids seeded
+uniform random in [100, vocab-100] as in the reference's own benchmark
+(reference: src/zedinfer/profiler.cpp:79-84, docs/perf/benchmark_v0.1.0.md:3-11).
+"""
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# Qwen2.5-1.5B: the benchmark model
+SHAPE = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_size=1536, intermediate_size=8960,
+             vocab_size=151936, max_position_embeddings=32768, num_hidden_layers=28, num_attention_heads=12,
+             num_key_value_heads=2, head_dim=128, rope_theta=1000000.0, rms_norm_eps=1e-6,
+             tie_word_embeddings=True, use_sliding_window=False, torch_dtype="bfloat16")
+FULL_LAYERS = 28
+PROMPT = 2048
+CONTEXT = 4096
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def matmul_params_per_layer(c):
+    H, I = c["hidden_size"], c["intermediate_size"]
+    qd, kvd = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
+    return H * (qd + 2 * kvd) + qd * H + 3 * H * I
+
+
+def decode_bytes(c, layers, batch, ctx_tokens_total, el):
+    """Bytes one decode step has to read: every weight it uses once (layers, norms, biases, the output
+    head) and the keys and values of all live tokens."""
+    H = c["hidden_size"]
+    qd, kvd = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
+    per_layer = matmul_params_per_layer(c) + (qd + 2 * kvd) + 2 * H
+    weights = (layers * per_layer + c["vocab_size"] * H + H) * el
+    kv = ctx_tokens_total * 2 * layers * kvd * el
+    return weights + kv
+
+
+def prefill_flops(c, layers, T):
+    lin = 2 * T * layers * matmul_params_per_layer(c) + 2 * c["vocab_size"] * c["hidden_size"]
+    att = 4 * c["num_attention_heads"] * c["head_dim"] * (T * (T + 1) // 2) * layers
+    return lin + att
+
+
+def rand_ids(rng, n, vocab):
+    return [rng.randrange(100, vocab - 100) for _ in range(n)]
+
+
+def measure_decode(engine_factory, batch, steps, warmup, vocab):
+    """tokens a second and ms a step of `steps` decode steps with `batch` running requests."""
+    import torch
+    from zedinfer_amd import GenerationConfig, InferenceRequest
+    from zedinfer_amd.engine import InferenceEngine
+    ie = InferenceEngine(engine_factory())
+    loop = ie.serving_loop()
+    rng = random.Random(1234 + batch)
+    reqs = [loop.submit_async(InferenceRequest(rand_ids(rng, PROMPT, vocab),
+                                               GenerationConfig(max_new_tokens=warmup + steps + 2 * batch + 8,
+                                                                ignore_eos=True)))
+            for _ in range(batch)]
+    while loop.pending_count() or any(r.phase.value != "decode" for r in reqs):
+        loop.step()
+    for _ in range(warmup):
+        loop.step()
+    ctx0 = sum(r.seq.length for r in reqs)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loop.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ctx1 = sum(r.seq.length for r in reqs)
+    assert all(not r.error for r in reqs), [r.error for r in reqs if r.error][:1]
+    assert ctx1 - ctx0 == batch * steps
+    for r in reqs:
+        r.cancelled = True
+    loop.step()
+    return batch * steps / dt, dt / steps * 1000.0, (ctx0 + ctx1) / 2.0
+
+
+def measure_prefill(engine_factory, vocab, rounds=3):
+    import torch
+    from zedinfer_amd import ops
+    from zedinfer_amd.engine import StepEntry
+    eng = engine_factory()
+    rng = random.Random(77)
+    times = []
+    for i in range(rounds + 1):
+        seq = eng.open(("prefill", i), PROMPT)
+        ids = rand_ids(rng, PROMPT, vocab)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = eng.step([StepEntry(seq, ids, [PROMPT - 1])], copy=False)
+        ops.argmax(logits).tolist()
+        times.append(time.perf_counter() - t0)
+        eng.close(seq)
+    return sum(times[1:]) / rounds * 1000.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (reported)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    from zedinfer_amd.config import Qwen2Config, SchedulerConfig
+    from zedinfer_amd.engine import Engine
+
+    shape = dict(SHAPE, num_hidden_layers=args.layers)
+    cfg = Qwen2Config.from_dict(shape)
+    el = 2 if args.dtype == "bf16" else 4
+    weights_cache = {}
+
+    def factory(batch):
+        def make():
+            pages = batch * (CONTEXT // 16) + 16
+            sched = SchedulerConfig(num_kv_blocks=pages, kv_block_size=16, max_batch_requests=max(batch, 1),
+                                    max_batch_tokens=PROMPT + batch, max_prefill_tokens=PROMPT, max_seq_len=CONTEXT)
+            if "w" not in weights_cache:
+                e = Engine.from_config(cfg, "Qwen2ForCausalLM", args.dtype, seed=0, sched=sched)
+                weights_cache["w"] = e
+                return e
+            # share the first engine's weights: same model, another cache pool
+            e0 = weights_cache["w"]
+            e = Engine.__new__(Engine)
+            e.__dict__.update(e0.__dict__)
+            from zedinfer_amd.cache.manager import CacheManager
+            e.sched = sched
+            e.cache = CacheManager(e.model.cache_requests(), e.model.state_requests(), pages, 16,
+                                   sched.max_batch_requests, e.dtype, e.device, sched.max_batch_tokens)
+            e.memories = e.cache.memories(e.fc.schedule)
+            return e
+        return make
+
+    V = cfg.vocab_size
+    tps, ms_step, ctx_mid = measure_decode(factory(args.batch), args.batch, args.steps, args.warmup, V)
+    need = decode_bytes(shape, args.layers, args.batch, ctx_mid, el)
+    achieved = need / (ms_step / 1000.0) / 1e9
+    out = {
+        "metric": "decode tok/s at batch 8, 2,048-token prompts (Qwen2.5-1.5B shape)",
+        "value": round(tps, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: seeded random weights, seeded uniform-random token ids",
+        "config": {"model": "Qwen2.5-1.5B shape", "global_batch": args.batch, "seq_len": PROMPT,
+                   "context_len": CONTEXT, "parallelism": "single GPU", "num_layers": FULL_LAYERS,
+                   "layers_run": args.layers, "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
+                   "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                   "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": True,
+                   "kv_page_tokens": 16, "sampling": "greedy"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        torch.cuda.empty_cache()
+        pms = measure_prefill(factory(1), V)
+        fl = prefill_flops(shape, args.layers, PROMPT)
+        out["prefill"] = {"value": round(PROMPT / pms * 1000.0, 1), "tokens": PROMPT, "ms": round(pms, 3),
+                          "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}
+        points = {}
+        for b, st in ((1, min(args.steps, 64)), (64, min(args.steps, 32))):
+            torch.cuda.empty_cache()
+            t, _, _ = measure_decode(factory(b), b, st, min(args.warmup, 8), V)
+            points[f"decode_b{b}"] = round(t, 2)
+        out["points"] = points
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

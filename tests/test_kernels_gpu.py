@@ -122,17 +122,18 @@ def test_rope(ops, dtype, n, nh, d, start, theta):
 
 
 def make_paged(k, v, page_size, num_pages, perm_seed=0):
-    """Scatter k, v [T, nkv, d] into caches [pages, nkv, page_size, d] through a shuffled table."""
+    """Scatter k, v [T, nkv, d] into the key cache [pages, nkv, page_size, d] and the transposed value
+    cache [pages, nkv, d, page_size] through a shuffled table."""
     T, nkv, d = k.shape
     need = (T + page_size - 1) // page_size
     g = torch.Generator().manual_seed(perm_seed)
     table = torch.randperm(num_pages, generator=g)[:need].to(torch.int32)
     kc = torch.full((num_pages, nkv, page_size, d), float("nan"), dtype=k.dtype, device="cuda")
-    vc = torch.full_like(kc, float("nan"))
+    vc = torch.full((num_pages, nkv, d, page_size), float("nan"), dtype=k.dtype, device="cuda")
     for t in range(T):
         p, o = int(table[t // page_size]), t % page_size
         kc[p, :, o] = k[t]
-        vc[p, :, o] = v[t]
+        vc[p, :, :, o] = v[t]
     return kc, vc, table.cuda()
 
 
@@ -202,7 +203,7 @@ def test_rope_kv_store(ops, dtype):
     pos = torch.arange(100, 100 + n, dtype=torch.int32, device="cuda")
     slots = torch.randperm(pages * ps)[:n].to(torch.int32).cuda()
     kc = torch.zeros(pages, nkv, ps, d, dtype=dtype, device="cuda")
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(pages, nkv, d, ps, dtype=dtype, device="cuda")
     q_ref = torch_rope(q.float().reshape(n, nh, d), pos, theta)
     k_ref = torch_rope(k.float().reshape(n, nkv, d), pos, theta)
     v_ref = v.clone().reshape(n, nkv, d)
@@ -211,7 +212,7 @@ def test_rope_kv_store(ops, dtype):
     for t in range(n):
         p, o = int(slots[t]) // ps, int(slots[t]) % ps
         torch.testing.assert_close(kc[p, :, o].float(), k_ref[t], **tol(dtype, 5e-4, 2e-2))
-        assert torch.equal(vc[p, :, o], v_ref[t])
+        assert torch.equal(vc[p, :, :, o], v_ref[t])
     # untouched slots stay zero
     assert int((kc != 0).any(-1).any(1).sum()) == n
 
@@ -219,7 +220,8 @@ def test_rope_kv_store(ops, dtype):
 @pytest.mark.parametrize("xdt,wdt,odt", [(torch.float32,) * 3, (torch.bfloat16,) * 3,
                                           (torch.bfloat16, torch.float32, torch.bfloat16),
                                           (torch.bfloat16, torch.bfloat16, torch.float32)])
-@pytest.mark.parametrize("M,N,K", [(1, 100, 64), (5, 1000, 96), (70, 130, 176), (128, 1536, 8960), (3, 151, 33)])
+@pytest.mark.parametrize("M,N,K", [(1, 100, 64), (5, 1000, 96), (70, 130, 176), (128, 1536, 8960), (3, 151, 33),
+                                   (8, 2048, 1536), (1, 1536, 8960), (64, 1000, 176), (17, 17920, 1536), (33, 77, 40)])
 def test_linear(ops, xdt, wdt, odt, M, N, K):
     x, w, b = rnd(M, K, dtype=xdt, seed=1), rnd(N, K, dtype=wdt, scale=0.05, seed=2), rnd(N, dtype=wdt, seed=3)
     ref = torch.nn.functional.linear(x.double(), w.double(), b.double()).float()
@@ -234,6 +236,18 @@ def test_linear(ops, xdt, wdt, odt, M, N, K):
     ops.linear(x, w, b, out=wide[:, 4:N + 4])
     torch.testing.assert_close(wide[:, 4:N + 4].float(), ref, **t)
     assert float(wide[:, :4].abs().max()) == 0 and float(wide[:, N + 4:].abs().max()) == 0
+
+
+def test_linear_skinny_row_does_not_depend_on_batch(ops):
+    """The decode-time product cuts k by the weight's shape alone: a row's result is bit-identical
+    whether 1, 8 or 64 rows ride along."""
+    x, w = rnd(64, 1536, dtype=torch.bfloat16, seed=1), rnd(2048, 1536, dtype=torch.bfloat16, scale=0.05, seed=2)
+    full = ops.linear(x, w)
+    for m in (1, 8, 17):
+        part = ops.linear(x[:m].contiguous(), w)
+        assert torch.equal(full[:m], part)
+    x2, w2 = rnd(64, 8960, dtype=torch.bfloat16, seed=3), rnd(1536, 8960, dtype=torch.bfloat16, scale=0.02, seed=4)
+    assert torch.equal(ops.linear(x2, w2, out_dtype=torch.float32)[5:6], ops.linear(x2[5:6].contiguous(), w2, out_dtype=torch.float32))
 
 
 def test_linear_f32_row_does_not_depend_on_batch(ops):
@@ -257,3 +271,72 @@ def test_argmax(ops, dtype):
     t[1, -1] = 1.0
     assert ops.argmax(t).tolist() == [1234, 151935]
     assert ops.argmax(torch.zeros(1, 77, device="cuda")).tolist() == [0]
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps,T,window", [
+    (12, 2, 128, 16, 2100, 0), (12, 2, 128, 16, 70, 0), (28, 4, 128, 16, 5000, 0), (3, 1, 64, 8, 200, 0),
+    (8, 1, 64, 16, 300, 37), (5, 5, 256, 32, 150, 0), (4, 2, 128, 8, 260, 100), (14, 2, 128, 16, 9, 0)])
+def test_attention_decode(ops, nh, nkv, d, ps, T, window):
+    """The split-keys kernel against the same float32 reference, with a listed subset of the tokens."""
+    dtype = torch.bfloat16
+    assert ops.attention_decode_supported(dtype, nh, nkv, d, ps)
+    k, v = rnd(T, nkv, d, dtype=dtype, seed=1), rnd(T, nkv, d, dtype=dtype, seed=2)
+    pages = (T + ps - 1) // ps + 3
+    kc, vc, table = make_paged(k, v, ps, pages)
+    pos_list = sorted(p for p in {T - 1, T - 2, 0, 1, 7, 8, 63, 64, 65, 127, 128, T // 2, T // 3} if p < T)
+    pos = torch.tensor(pos_list, dtype=torch.int32, device="cuda")
+    n = pos.numel()
+    q = rnd(n, nh, d, dtype=dtype, seed=3)
+    seq = torch.zeros(n, dtype=torch.int32, device="cuda")
+    bt = table[None].contiguous()
+    scale = 1 / math.sqrt(d)
+    ref = ref_attention(q.float(), k.float(), v.float(), pos.long(), scale, window)
+    out = ops.attention_decode(q.view(n, nh * d), kc, vc, seq, pos, bt, nh, nkv, d, scale, T, window)
+    torch.testing.assert_close(out.view(n, nh, d).float(), ref, atol=2e-2, rtol=2e-2)
+    # a listed subset leaves the other rows alone
+    idx = torch.tensor([n - 1, 0, 3], dtype=torch.int32, device="cuda")
+    assert n > 4
+    out2 = torch.full((n, nh * d), 7.0, dtype=dtype, device="cuda")
+    ops.attention_decode(q.view(n, nh * d), kc, vc, seq, pos, bt, nh, nkv, d, scale, T, window, out=out2, tok_index=idx)
+    sel = idx.long()
+    assert torch.equal(out2[sel], out[sel])
+    rest = torch.ones(n, dtype=torch.bool)
+    rest[sel.cpu()] = False
+    assert bool((out2[rest.cuda()] == 7.0).all())
+    # against the plain kernel on the same inputs: both round the same float32 result
+    plain_out = ops.attention(q.view(n, nh * d), kc, vc, seq, pos, bt, nh, nkv, d, scale, window)
+    torch.testing.assert_close(out.float(), plain_out.float(), atol=1e-2, rtol=1e-2)
+
+
+def test_attention_decode_ignores_stale_slots(ops):
+    """Slots of a page beyond the token's position may hold anything, NaN included."""
+    nh, nkv, d, ps, T = 4, 2, 128, 16, 37
+    k, v = rnd(T, nkv, d, dtype=torch.bfloat16, seed=1), rnd(T, nkv, d, dtype=torch.bfloat16, seed=2)
+    kc, vc, table = make_paged(k, v, ps, 8)        # unused slots are NaN
+    pos = torch.tensor([T - 1, 20], dtype=torch.int32, device="cuda")
+    q = rnd(2, nh, d, dtype=torch.bfloat16, seed=3)
+    out = ops.attention_decode(q.view(2, nh * d), kc, vc, torch.zeros(2, dtype=torch.int32, device="cuda"), pos,
+                               table[None].contiguous(), nh, nkv, d, 0.1, T)
+    assert not torch.isnan(out).any()
+    ref = ref_attention(q.float(), k.float(), v.float(), pos.long(), 0.1, 0)
+    torch.testing.assert_close(out.view(2, nh, d).float(), ref, atol=2e-2, rtol=2e-2)
+
+
+def test_unsupported_shapes_are_refused(ops):
+    assert not ops.attention_decode_supported(torch.float32, 12, 2, 128, 16)
+    assert not ops.attention_decode_supported(torch.bfloat16, 12, 2, 48, 16)
+    assert not ops.attention_decode_supported(torch.bfloat16, 12, 1, 128, 16)       # group of 12
+    assert not ops.attention_decode_supported(torch.bfloat16, 12, 2, 128, 4)
+    q = rnd(1, 12 * 48, dtype=torch.bfloat16)
+    kc = torch.zeros(4, 2, 16, 48, dtype=torch.bfloat16, device="cuda")
+    vc = torch.zeros(4, 2, 48, 16, dtype=torch.bfloat16, device="cuda")
+    z = torch.zeros(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(ops.KernelLibraryError, match="unsupported shape"):
+        ops.attention_decode(q, kc, vc, z, z, torch.zeros(1, 4, dtype=torch.int32, device="cuda"), 12, 2, 48, 0.1, 1)
+    with pytest.raises(ValueError, match="multiple"):
+        ops.attention(q, kc, vc, z, z, torch.zeros(1, 4, dtype=torch.int32, device="cuda"), 12, 5, 48, 0.1)
+    with pytest.raises(ops.KernelLibraryError, match="larger than"):
+        big = torch.zeros(1, 1024, dtype=torch.bfloat16, device="cuda")
+        ops.attention(big, torch.zeros(1, 1, 16, 1024, dtype=torch.bfloat16, device="cuda"),
+                      torch.zeros(1, 1, 1024, 16, dtype=torch.bfloat16, device="cuda"), z, z,
+                      torch.zeros(1, 1, dtype=torch.int32, device="cuda"), 1, 1, 1024, 0.1)

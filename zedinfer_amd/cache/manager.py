@@ -8,8 +8,10 @@ page ids, so one table serves every layer of the group (the reference keeps a
 page list per layer, reference: src/backend/kvcache/block_pool.hpp:73-103).
 Pages go back to the pool when the request ends, or, in a window group, as soon
 as no later token can see them.  A page holds ``page_size`` tokens of one layer:
-[kv_head][slot][head_dim] (reference layout [slot][kv_head][head_dim],
-block_pool.hpp:16-25; keys of one head are contiguous here).
+keys as [kv_head][slot][head_dim], values transposed as [kv_head][head_dim][slot]
+(reference layout [slot][kv_head][head_dim], block_pool.hpp:16-25; here one head's
+keys are contiguous, and so is a run of positions of one value dimension, which is
+the order the matrix cores read P.V in).
 
 Admission works on promises: ``open`` promises a sequence the pages its prompt
 and a reserve of generated tokens need (reference: prompt + min(max_new, 256),
@@ -105,9 +107,10 @@ class CacheManager:
         self.state_requests = dict(state_requests)
         if self.device is not None:
             for cid, rq in kv_requests.items():
-                shape = (self.num_pages, rq.num_kv_heads, self.page_size, rq.head_dim)
-                self.k[cid] = torch.zeros(shape, dtype=dtype, device=self.device)
-                self.v[cid] = torch.zeros(shape, dtype=dtype, device=self.device)
+                self.k[cid] = torch.zeros((self.num_pages, rq.num_kv_heads, self.page_size, rq.head_dim),
+                                          dtype=dtype, device=self.device)
+                self.v[cid] = torch.zeros((self.num_pages, rq.num_kv_heads, rq.head_dim, self.page_size),
+                                          dtype=dtype, device=self.device)
             for cid, sr in state_requests.items():
                 self.state[cid] = torch.zeros((self.max_requests,) + tuple(sr.shape), dtype=sr.dtype,
                                               device=self.device)

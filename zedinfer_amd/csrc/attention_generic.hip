@@ -1,6 +1,7 @@
 // Causal grouped-query attention over the paged cache: the plain kernel.
 //
-// One wavefront per (token, query head).  The token at absolute position p of
+// One wavefront per (token, query head); with a token list only the listed tokens are done
+// (n counts the list then).  The token at absolute position p of
 // its sequence sees the keys at positions [lo, p], lo = 0, or p - window + 1
 // for a windowed layer; keys and values are found through the sequence's block
 // table.  s_j = (q . k_j) * scale, softmax with the running maximum subtracted,
@@ -22,13 +23,14 @@ template <typename T>
 __global__ void __launch_bounds__(ZI_WAVE)
 attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t ldq, int64_t ldo,
                          const T* __restrict__ kcache, const T* __restrict__ vcache,
-                         const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos,
-                         const int32_t* __restrict__ block_tables, int max_pages, int num_pages, int nh, int nkv,
-                         int d, int page_size, int window, float scale) {
+                         const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
+                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
+                         int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
+                         float scale) {
     __shared__ float qs[ATTN_MAX_D];
     __shared__ float ps[ZI_WAVE];
     __shared__ int64_t vbase[ZI_WAVE];
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int t = tok_index ? tok_index[blockIdx.x] : blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int g = h / (nh / nkv);
     const int p = tok_pos[t];
     const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
@@ -47,7 +49,7 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
         const int j = base + lane;
         bool valid = j <= p;
         float s = -INFINITY;
-        int64_t row = -1;
+        int64_t row = -1, vrow = -1;
         if (valid) {
             const int pi = j / page_size;
             const int page = pi < max_pages ? bt[pi] : -1;
@@ -55,6 +57,7 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
                 valid = false;  // a hole in the table: the host never schedules this; stay in bounds
             } else {
                 row = (((int64_t)page * nkv + g) * page_size + (j % page_size)) * d;
+                vrow = ((int64_t)page * nkv + g) * page_size * d + (j % page_size);
                 const T* kr = kcache + row;
                 float dot = 0.f;
                 for (int x = 0; x < d; ++x) dot += qs[x] * zi_load(kr + x);
@@ -67,7 +70,7 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
         const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
         l = l * corr + zi_wave_sum(pj);
         ps[lane] = pj;
-        vbase[lane] = row;
+        vbase[lane] = vrow;
         __syncthreads();
         const int cnt = (p - base + 1 < ZI_WAVE) ? p - base + 1 : ZI_WAVE;
 #pragma unroll
@@ -79,7 +82,7 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
 #pragma unroll
             for (int i = 0; i < ATTN_ACC; ++i) {
                 const int x = lane + i * ZI_WAVE;
-                if (x < d) acc[i] += pw * zi_load(vcache + vr + x);
+                if (x < d) acc[i] += pw * zi_load(vcache + vr + (int64_t)x * page_size);
             }
         }
         m = m_new;
@@ -95,8 +98,8 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
 }
 
 extern "C" int zi_attention_generic(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,
-                                    const void* kcache, const void* vcache, const int32_t* tok_seq,
-                                    const int32_t* tok_pos, const int32_t* block_tables, int max_pages,
+                                    const void* kcache, const void* vcache, const int32_t* tok_index,
+                                    const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables, int max_pages,
                                     int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
                                     hipStream_t stream) {
     ZI_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0 && max_pages > 0 && num_pages > 0,
@@ -109,7 +112,7 @@ extern "C" int zi_attention_generic(void* out, const void* q, int dt, int n, int
     if (n == 0) return 0;
     ZI_DISPATCH_DTYPE(dt, T, {
         attention_generic_kernel<T><<<dim3(n, nh), ZI_WAVE, 0, stream>>>(
-            (T*)out, (const T*)q, ldq, ldo, (const T*)kcache, (const T*)vcache, tok_seq, tok_pos, block_tables,
+            (T*)out, (const T*)q, ldq, ldo, (const T*)kcache, (const T*)vcache, tok_index, tok_seq, tok_pos, block_tables,
             max_pages, num_pages, nh, nkv, d, page_size, window, scale);
     });
     return zi_check_launch("attention_generic");

@@ -9,8 +9,11 @@
 // rotated in place; keys are rotated on their way into the cache, values copied
 // (reference: K is stored after rotation, V raw, src/frontend/models/transformer_forward.cpp:99-104).
 //
-// Cache layout of one layer: [page][kv_head][slot_in_page][head_dim]; token slot
-// s lives in page s / page_size at offset s % page_size.  A negative slot skips the write.
+// Cache layout of one layer.  Keys: [page][kv_head][slot_in_page][head_dim].  Values are
+// stored transposed: [page][kv_head][head_dim][slot_in_page], so that a run of consecutive
+// positions of one dimension is contiguous, which is the order the matrix cores want for
+// the P.V product.  Token slot s lives in page s / page_size at offset s % page_size.
+// A negative slot skips the write.
 #include "zi_common.h"
 
 template <typename T>
@@ -59,7 +62,7 @@ __global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k,
             kv = zi_load(kr + h * d + j);
         }
         zi_store(kcache + dst, kv);
-        vcache[dst] = vr[h * d + j];
+        vcache[((page * nkv + h) * d + j) * page_size + off] = vr[h * d + j];
     }
 }
 

@@ -17,6 +17,9 @@ import torch
 from ..cache.manager import CacheManager, SequenceCache
 
 
+SHORT_ENTRY = 4     # entries of up to this many tokens are attended token by token, split over the keys
+
+
 @dataclass
 class StepEntry:
     """``tokens`` continue the sequence whose cache is ``seq`` at position ``seq.length``;
@@ -49,6 +52,14 @@ class DeviceBatch:
     entry_past: torch.Tensor     # [entries] tokens of the entry already in the cache
     entry_slot: torch.Tensor     # [entries] state slot of the entry
     groups: List[GroupView] = field(default_factory=list)
+    # Tokens of entries that bring at most SHORT_ENTRY tokens ("decode" tokens) and the rest, as
+    # lists of flat token indices; None when the list would be all tokens or is empty.
+    short_idx: Optional[torch.Tensor] = None
+    long_idx: Optional[torch.Tensor] = None
+    num_short: int = 0
+    num_long: int = 0
+    max_short_keys: int = 0      # largest position + 1 among the short entries' tokens
+    max_long_keys: int = 0
     # host copies, for parts that plan their launches on the host
     host_start: Optional[np.ndarray] = None
     host_len: Optional[np.ndarray] = None
@@ -107,7 +118,16 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
         group_tables.append(t)
         widths.append(width)
 
-    pieces = [token_ids.astype(np.int32), positions, tok_seq, logit_rows, starts, lens_a, past, slot]
+    short_tok = np.repeat(lens_a <= SHORT_ENTRY, lens)
+    flat = np.arange(N, dtype=np.int32)
+    short_idx, long_idx = flat[short_tok], flat[~short_tok]
+    n_short, n_long = int(short_idx.size), int(long_idx.size)
+    ends = past + lens_a
+    max_short = int(ends[lens_a <= SHORT_ENTRY].max()) if n_short else 0
+    max_long = int(ends[lens_a > SHORT_ENTRY].max()) if n_long else 0
+
+    pieces = [token_ids.astype(np.int32), positions, tok_seq, logit_rows, starts, lens_a, past, slot,
+              short_idx, long_idx]
     for g in range(G):
         pieces += [group_slots[g], group_tables[g].reshape(-1)]
     sizes = [p.size for p in pieces]
@@ -123,8 +143,11 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     for s in sizes:
         views.append(dev[off:off + s])
         off += s
-    groups = [GroupView(views[8 + 2 * g], views[9 + 2 * g].view(E, widths[g])) for g in range(G)]
+    groups = [GroupView(views[10 + 2 * g], views[11 + 2 * g].view(E, widths[g])) for g in range(G)]
     return DeviceBatch(num_tokens=N, num_entries=E, num_logit_rows=R, token_ids=views[0], positions=views[1],
                        tok_seq=views[2], logit_rows=views[3], entry_start=views[4], entry_len=views[5],
-                       entry_past=views[6], entry_slot=views[7], groups=groups, host_start=starts,
+                       entry_past=views[6], entry_slot=views[7], groups=groups,
+                       short_idx=views[8] if 0 < n_short < N else None,
+                       long_idx=views[9] if 0 < n_long < N else None, num_short=n_short, num_long=n_long,
+                       max_short_keys=max_short, max_long_keys=max_long, host_start=starts,
                        host_len=lens_a, host_past=past, host_slot=slot)

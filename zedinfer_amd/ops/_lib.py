@@ -25,8 +25,12 @@ _PROTOTYPES = {
     "zi_add_rmsnorm": [P, I, P, P, I, P, I, I, I, F, I, P],
     "zi_rope_kv_store": [P, P, P, I, I, L, L, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_rope": [P, P, I, I, L, L, P, P, I, I, I, P],
-    "zi_attention_generic": [P, P, I, I, L, L, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
+    "zi_attention_generic": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
+    "zi_attention_decode": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P],
+    "zi_attention_decode_supported": [I, I, I, I, I],
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
+    "zi_gemm_skinny": [P, I, P, P, P, I, I, I, L, L, L, P, L, P],
+    "zi_gemm_skinny_supported": [I, I, I, L, L],
     "zi_argmax": [P, P, P, I, I, I, L, P],
     "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],
 }
@@ -64,6 +68,8 @@ def load() -> ctypes.CDLL:
                 raise KernelLibraryError(f"{path} lacks entry point {name}; rebuild it") from e
             fn.argtypes = args
             fn.restype = c_int
+        lib.zi_gemm_skinny_workspace.argtypes = [I, I, I]
+        lib.zi_gemm_skinny_workspace.restype = c_int64
         _lib, _lib_path = lib, path
         return lib
 

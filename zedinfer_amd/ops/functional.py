@@ -202,14 +202,17 @@ def rope(x: torch.Tensor, pos: torch.Tensor, inv_freq: torch.Tensor, out: Option
 
 
 def _check_cache(kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int, dtype, what: str) -> Tuple[int, int]:
-    """A layer's cache is [pages, kv_heads, page_size, head_dim]; returns (pages, page_size)."""
-    for c in (kcache, vcache):
-        if c.dim() != 4 or not c.is_contiguous() or c.shape[1] != nkv or c.shape[3] != d or c.dtype != dtype:
-            raise ValueError(f"{what}: cache must be contiguous [pages, {nkv}, page_size, {d}] of {dtype}, "
-                             f"got {tuple(c.shape)} {c.dtype}")
-    if kcache.shape != vcache.shape:
-        raise ValueError(f"{what}: key and value caches differ in shape")
-    return kcache.shape[0], kcache.shape[2]
+    """A layer's key cache is [pages, kv_heads, page_size, head_dim], its value cache is stored
+    transposed, [pages, kv_heads, head_dim, page_size]; returns (pages, page_size)."""
+    if (kcache.dim() != 4 or not kcache.is_contiguous() or kcache.shape[1] != nkv or kcache.shape[3] != d
+            or kcache.dtype != dtype):
+        raise ValueError(f"{what}: key cache must be contiguous [pages, {nkv}, page_size, {d}] of {dtype}, "
+                         f"got {tuple(kcache.shape)} {kcache.dtype}")
+    pages, ps = kcache.shape[0], kcache.shape[2]
+    if tuple(vcache.shape) != (pages, nkv, d, ps) or not vcache.is_contiguous() or vcache.dtype != dtype:
+        raise ValueError(f"{what}: value cache must be contiguous [{pages}, {nkv}, {d}, {ps}] of {dtype}, "
+                         f"got {tuple(vcache.shape)} {vcache.dtype}")
+    return pages, ps
 
 
 def rope_kv_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], pos: torch.Tensor,
@@ -245,34 +248,84 @@ def rope_kv_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
               _stream())
 
 
+def _attention_args(what, q, kcache, vcache, tok_seq, tok_pos, block_tables, nh, nkv, d, tok_index, out):
+    _gpu(what, q, kcache, vcache, tok_seq, tok_pos, block_tables, tok_index, out)
+    ldq, wq = _rows(q, f"{what} q")
+    n = q.shape[0]
+    if wq != nh * d:
+        raise ValueError(f"{what}: q has width {wq}, expected {nh}*{d}")
+    if nkv <= 0 or nh % nkv:
+        raise ValueError(f"{what}: {nh} query heads are not a multiple of {nkv} key/value heads")
+    pages, ps = _check_cache(kcache, vcache, nkv, d, q.dtype, what)
+    _i32(tok_seq, f"{what} tok_seq", n)
+    _i32(tok_pos, f"{what} tok_pos", n)
+    if tok_index is not None:
+        _i32(tok_index, f"{what} tok_index")
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError(f"{what}: block_tables must be a contiguous int32 [seqs, max_pages] tensor")
+    if out is None:
+        out = torch.empty((n, nh * d), dtype=q.dtype, device=q.device)
+    ldo, wo = _rows(out, f"{what} out")
+    if tuple(out.shape) != (n, nh * d) or out.dtype != q.dtype:
+        raise ValueError(f"{what}: out has the wrong shape or dtype")
+    count = tok_index.numel() if tok_index is not None else n
+    return out, n, count, ldq, ldo, pages, ps
+
+
 def attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
               tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
-              window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Causal grouped-query attention of q [n, nh*d] over the paged cache.
+              window: int = 0, out: Optional[torch.Tensor] = None, tok_index: Optional[torch.Tensor] = None
+              ) -> torch.Tensor:
+    """Causal grouped-query attention of q [n, nh*d] over the paged cache: the plain kernel, for
+    every shape and both storage types.
 
     Token i belongs to row ``tok_seq[i]`` of ``block_tables`` [seqs, max_pages] and sits at
     absolute position ``tok_pos[i]``; it sees the cached keys at positions
-    [max(0, pos - window + 1), pos] (window 0: all of them).  Returns [n, nh*d]."""
-    _gpu("attention", q, kcache, vcache, tok_seq, tok_pos, block_tables, out)
-    ldq, wq = _rows(q, "attention q")
-    n = q.shape[0]
-    if wq != nh * d:
-        raise ValueError(f"attention: q has width {wq}, expected {nh}*{d}")
-    if nkv <= 0 or nh % nkv:
-        raise ValueError(f"attention: {nh} query heads are not a multiple of {nkv} key/value heads")
-    pages, ps = _check_cache(kcache, vcache, nkv, d, q.dtype, "attention")
-    _i32(tok_seq, "attention tok_seq", n)
-    _i32(tok_pos, "attention tok_pos", n)
-    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
-        raise ValueError("attention: block_tables must be a contiguous int32 [seqs, max_pages] tensor")
-    if out is None:
-        out = torch.empty((n, nh * d), dtype=q.dtype, device=q.device)
-    ldo, wo = _rows(out, "attention out")
-    if tuple(out.shape) != (n, nh * d) or out.dtype != q.dtype:
-        raise ValueError("attention: out has the wrong shape or dtype")
-    _lib.call("zi_attention_generic", _p(out), _p(q), _code(q, "attention"), n, ldq, ldo, _p(kcache), _p(vcache),
-              _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps,
-              int(window), float(scale), _stream())
+    [max(0, pos - window + 1), pos] (window 0: all of them).  With ``tok_index`` only the listed
+    tokens are computed (the other rows of ``out`` are left alone).  Returns [n, nh*d]."""
+    out, n, count, ldq, ldo, pages, ps = _attention_args("attention", q, kcache, vcache, tok_seq, tok_pos,
+                                                         block_tables, nh, nkv, d, tok_index, out)
+    _lib.call("zi_attention_generic", _p(out), _p(q), _code(q, "attention"), count, ldq, ldo, _p(kcache), _p(vcache),
+              _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages, nh, nkv, d,
+              ps, int(window), float(scale), _stream())
+    return out
+
+
+DECODE_MAX_SPLITS = 64
+DECODE_SPLIT_KEYS = 64
+
+
+def attention_decode_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, page_size: int) -> bool:
+    if dtype not in _CODES:
+        return False
+    return bool(_lib.load().zi_attention_decode_supported(_CODES[dtype], nh, nkv, d, page_size))
+
+
+def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
+                     tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
+                     max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
+                     tok_index: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None
+                     ) -> torch.Tensor:
+    """The same attention for single query tokens, split over the keys (bfloat16, head_dim
+    64/128/256, group size <= 8, page size a multiple of 8).  ``max_keys`` is an upper bound of
+    the keys any listed token sees (its position + 1, or the window), known on the host."""
+    out, n, count, ldq, ldo, pages, ps = _attention_args("attention_decode", q, kcache, vcache, tok_seq, tok_pos,
+                                                         block_tables, nh, nkv, d, tok_index, out)
+    if window > 0:
+        max_keys = min(max_keys, window)
+    # a token's key range is widened down to a multiple of 8 and cut into splits of 64 keys (more
+    # beyond 4096 keys, never more than 64 splits); this bound only sizes the launch
+    max_splits = max(1, min(DECODE_MAX_SPLITS, -(-(max_keys + 7) // DECODE_SPLIT_KEYS)))
+    need = count * nh * DECODE_MAX_SPLITS * (d + 2)
+    if max_splits > 1:
+        if workspace is None:
+            workspace = torch.empty((need,), dtype=torch.float32, device=q.device)
+        if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
+            raise ValueError(f"attention_decode: workspace must be a contiguous float32 buffer of {need} entries")
+    _lib.call("zi_attention_decode", _p(out), _p(q), _code(q, "attention_decode"), count, ldq, ldo, _p(kcache),
+              _p(vcache), _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages,
+              nh, nkv, d, ps, int(window), float(scale), max_splits, _p(workspace),
+              workspace.numel() if workspace is not None else 0, _stream())
     return out
 
 
@@ -301,8 +354,18 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     if M == 0:
         return out
     bf = torch.bfloat16
-    if (x.dtype == bf and weight.dtype == bf and out.dtype == bf and (bias is None or bias.dtype == bf)
-            and out.is_contiguous()):
+    all_bf = x.dtype == bf and weight.dtype == bf and (bias is None or bias.dtype == bf)
+    if all_bf and (M <= SKINNY_MAX_ROWS or out.dtype == torch.float32) and _skinny_ok(x, weight, K, ldx, ldw):
+        # few rows (decoding), or float32 output (logits): the hand-written matrix-core kernel
+        lib = _lib.load()
+        for m0 in range(0, M, SKINNY_MAX_ROWS):
+            m = min(SKINNY_MAX_ROWS, M - m0)
+            need = lib.zi_gemm_skinny_workspace(m, N, K)
+            ws = _workspace(x.device, need) if need else None
+            _lib.call("zi_gemm_skinny", _p(out[m0:m0 + m]), _code(out, "linear out"), _p(x[m0:m0 + m]), _p(weight),
+                      _p(bias), m, N, K, ldx, ldw, ldo, _p(ws), need, _stream())
+        return out
+    if all_bf and out.dtype == bf and out.is_contiguous():
         if bias is not None:
             torch.addmm(bias, x, weight.t(), out=out)
         else:
@@ -312,6 +375,24 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
               _code(weight, "linear weight"), _p(bias), _code(bias, "linear bias") if bias is not None else F32,
               M, N, K, ldx, ldw, ldo, _stream())
     return out
+
+
+SKINNY_MAX_ROWS = 64
+_WORKSPACES = {}
+
+
+def _workspace(device: torch.device, floats: int) -> torch.Tensor:
+    """A float32 scratch buffer per device that only grows (split partial sums live in it)."""
+    ws = _WORKSPACES.get(device)
+    if ws is None or ws.numel() < floats:
+        ws = torch.empty((max(floats, 1 << 20),), dtype=torch.float32, device=device)
+        _WORKSPACES[device] = ws
+    return ws
+
+
+def _skinny_ok(x: torch.Tensor, w: torch.Tensor, K: int, ldx: int, ldw: int) -> bool:
+    return (K >= 8 and K % 8 == 0 and ldx % 8 == 0 and ldw % 8 == 0 and x.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
 
 
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None, return_values: bool = False):

@@ -108,7 +108,7 @@ class LayerMemory:
 
     group: int = -1                       # cache group whose slots and block tables apply
     k: Optional[torch.Tensor] = None      # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None      # [pages, kv_heads, head_dim, page_size] (transposed)
     writes: bool = True
     state: Optional[torch.Tensor] = None  # [slots, *StateRequest.shape]
 

@@ -65,6 +65,25 @@ class Attention(Mixer):
                 self.biases = bs
         self.o = weights["o"]
 
+    def attend(self, q, att, batch, view, memory: LayerMemory) -> None:
+        """Tokens of short entries (decoded tokens) go to the kernel that splits one query's keys over
+        many wavefronts; longer portions, and every shape that kernel does not take, go to the plain one."""
+        args = (memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
+                self.scale)
+        n_long = batch.num_long
+        if batch.num_short:
+            if ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
+                ws = self.rt.buffer("attn_split", (batch.num_short * self.nh * ops.functional.DECODE_MAX_SPLITS
+                                                   * (self.d + 2),), torch.float32)
+                ops.attention_decode(q, *args, batch.max_short_keys, self.window, out=att,
+                                     tok_index=batch.short_idx, workspace=ws)
+            else:
+                n_long = -1      # everything through the plain kernel
+        if n_long < 0:
+            ops.attention(q, *args, self.window, out=att)
+        elif n_long > 0:
+            ops.attention(q, *args, self.window, out=att, tok_index=batch.long_idx)
+
     def cache_request(self) -> Optional[KVCacheRequest]:
         return KVCacheRequest("window" if self.window > 0 else "full", self.nkv, self.d, self.window)
 
@@ -80,7 +99,6 @@ class Attention(Mixer):
         view = batch.groups[memory.group]
         self.position.rotate_and_store(q, k, v, batch.positions, view.slots, memory, self.nh, self.nkv, self.d)
         att = self.rt.buffer("attn_out", (n, self.qd))
-        ops.attention(q, memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh,
-                      self.nkv, self.d, self.scale, self.window, out=att)
+        self.attend(q, att, batch, view, memory)
         out = self.rt.buffer("attn_proj", (n, self.hidden))
         return ops.linear(att, self.o, out=out)
