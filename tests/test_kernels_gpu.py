@@ -340,3 +340,95 @@ def test_unsupported_shapes_are_refused(ops):
         ops.attention(big, torch.zeros(1, 1, 16, 1024, dtype=torch.bfloat16, device="cuda"),
                       torch.zeros(1, 1, 1024, 16, dtype=torch.bfloat16, device="cuda"), z, z,
                       torch.zeros(1, 1, dtype=torch.int32, device="cuda"), 1, 1, 1024, 0.1)
+
+
+def prefill_tiles(entries, tile=64):
+    """entries: [(start, len, past)] -> (tile_entry, tile_off) with the heaviest tile first."""
+    tiles = [(past + off + min(tile, n - off), e, off) for e, (s, n, past) in enumerate(entries)
+             for off in range(0, n, tile)]
+    tiles.sort(key=lambda t: -t[0])
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")  # noqa: E731
+    return dev([t[1] for t in tiles]), dev([t[2] for t in tiles])
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps,window,portions", [
+    (12, 2, 128, 16, 0, [(0, 300), (300, 77)]),          # a prompt from the start, then a portion on top of it
+    (4, 2, 16, 16, 0, [(0, 49), (49, 5), (54, 130)]),
+    (3, 1, 32, 8, 0, [(0, 100), (100, 64), (164, 65)]),
+    (6, 2, 48, 8, 20, [(0, 90), (90, 40)]),              # head_dim that is no multiple of 32, window
+    (5, 5, 80, 32, 0, [(3, 70)]),
+    (28, 4, 128, 64, 64, [(0, 130), (130, 200)]),
+    (2, 1, 112, 128, 0, [(17, 129)]),
+    (14, 2, 64, 16, 150, [(0, 1000)]),
+])
+def test_attention_prefill(ops, nh, nkv, d, ps, window, portions):
+    """The matrix-core prompt kernel against the float32 reference: portions at several pasts, two
+    sequences in one launch that share pages through identical table rows."""
+    dtype = torch.bfloat16
+    assert ops.attention_prefill_supported(dtype, nh, nkv, d, ps)
+    T = max(p + n for p, n in portions)
+    k, v = rnd(T, nkv, d, dtype=dtype, seed=1), rnd(T, nkv, d, dtype=dtype, seed=2)
+    kc, vc, table = make_paged(k, v, ps, (T + ps - 1) // ps + 3)      # unused slots are NaN
+    entries, pos = [], []
+    for past, n in portions:
+        entries.append((len(pos), n, past))
+        pos += list(range(past, past + n))
+    n_tok = len(pos)
+    pos_t = torch.tensor(pos, dtype=torch.int32, device="cuda")
+    q = rnd(n_tok, nh, d, dtype=dtype, seed=3)
+    bt = torch.stack([table] * len(entries)).contiguous()
+    te, to = prefill_tiles(entries)
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")  # noqa: E731
+    scale = 1 / math.sqrt(d)
+    out = torch.full((n_tok, nh * d), 7.0, dtype=dtype, device="cuda")
+    ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, te, to, dev([e[0] for e in entries]),
+                          dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale, window,
+                          out=out)
+    assert not torch.isnan(out).any()
+    ref = ref_attention(q.float(), k.float(), v.float(), pos_t.long(), scale, window)
+    torch.testing.assert_close(out.view(n_tok, nh, d).float(), ref, atol=2e-2, rtol=2e-2)
+    # against the plain kernel on the same inputs
+    seq = torch.tensor([e for e, (s, n, p) in enumerate(entries) for _ in range(n)], dtype=torch.int32, device="cuda")
+    plain_out = ops.attention(q.view(n_tok, nh * d), kc, vc, seq, pos_t, bt, nh, nkv, d, scale, window)
+    torch.testing.assert_close(out.float(), plain_out.float(), atol=1.5e-2, rtol=1.5e-2)
+    # a tile list that leaves an entry out leaves its rows alone
+    if len(entries) > 1:
+        out2 = torch.full((n_tok, nh * d), 7.0, dtype=dtype, device="cuda")
+        keep = te != 0
+        ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, te[keep].contiguous(), to[keep].contiguous(),
+                              dev([e[0] for e in entries]), dev([e[1] for e in entries]),
+                              dev([e[2] for e in entries]), bt, nh, nkv, d, scale, window, out=out2)
+        n0 = entries[0][1]
+        assert bool((out2[:n0] == 7.0).all()) and torch.equal(out2[n0:], out[n0:])
+
+
+def test_attention_prefill_far_key_stands_out(ops):
+    """One far key among a thousand is made to dominate one query of a late tile."""
+    nh, nkv, d, ps, T = 4, 1, 64, 16, 1100
+    dtype = torch.bfloat16
+    k, v = rnd(T, nkv, d, seed=1) * 0.1, rnd(T, nkv, d, seed=2)
+    q = rnd(T, nh, d, seed=3) * 0.1
+    far, who = 37, 1003
+    q[who, 2] = rnd(d, seed=9)
+    k[far, 0] = q[who, 2] * 60.0 / q[who, 2].norm() ** 2 * math.sqrt(d)
+    k, v, q = k.to(dtype), v.to(dtype), q.to(dtype)
+    kc, vc, table = make_paged(k, v, ps, 80)
+    te, to = prefill_tiles([(0, T, 0)])
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    out = ops.attention_prefill(q.view(T, nh * d), kc, vc, te, to, dev([0]), dev([T]), dev([0]), table[None].contiguous(),
+                                nh, nkv, d, 1 / math.sqrt(d))
+    torch.testing.assert_close(out.view(T, nh, d)[who, 2].float(), v[far, 0].float(), atol=2e-2, rtol=2e-2)
+    # with a window that ends just after the far key it is gone; one key wider and it is back
+    for window, seen in ((who - far, False), (who - far + 1, True)):
+        o = ops.attention_prefill(q.view(T, nh * d), kc, vc, te, to, dev([0]), dev([T]), dev([0]),
+                                  table[None].contiguous(), nh, nkv, d, 1 / math.sqrt(d), window)
+        diff = float((o.view(T, nh, d)[who, 2].float() - v[far, 0].float()).abs().max())
+        assert (diff < 2e-2) == seen, (window, diff)
+
+
+def test_attention_prefill_refuses_other_shapes(ops):
+    assert not ops.attention_prefill_supported(torch.float32, 12, 2, 128, 16)
+    assert not ops.attention_prefill_supported(torch.bfloat16, 12, 2, 256, 16)
+    assert not ops.attention_prefill_supported(torch.bfloat16, 12, 2, 40, 16)
+    assert not ops.attention_prefill_supported(torch.bfloat16, 12, 2, 128, 24)
+    assert not ops.attention_prefill_supported(torch.bfloat16, 12, 5, 128, 16)

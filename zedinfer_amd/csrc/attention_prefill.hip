@@ -1,0 +1,260 @@
+// Paged causal grouped-query attention for prompt portions on the matrix cores.
+//
+// A workgroup of four wavefronts owns a tile of 64 consecutive query tokens of one
+// entry (16 a wavefront) and one query head.  It walks the keys the tile can see in
+// blocks of 64, aligned to absolute multiples of 64, so a query's blocks do not
+// depend on how its prompt was cut into steps.  Each block of keys and values is
+// staged once in LDS for the four wavefronts; scores and the P.V product run on
+// v_mfma_f32_16x16x32_bf16 with float32 accumulation, the running softmax
+// (maximum, sum, rescaling) is float32, and s_j = (q . k_j) * scale is scaled after
+// the dot product (reference formulas:
+// src/backend/ops/self_attention/cpu/paged_attention_cpu.cpp:106-162).
+//
+// Operand layout.  Scores are computed transposed: the A operand is a 16-key tile of
+// K, the B operand the 16 queries, so a lane ends up with the scores of ONE query
+// (lane % 16) and four keys per tile.  Keys are placed in LDS rows in a permuted
+// order (row t*16 + j*4 + e holds key (t/2)*32 + j*8 + (t%2)*4 + e of the block), which
+// makes the eight probabilities a lane holds after two tiles exactly the eight
+// consecutive keys j*8..j*8+7 that the B operand of the P.V product wants from that
+// lane: no data moves between lanes.  Values are cached transposed ([dim][slot]),
+// so the A operand of P.V (16 dims x 32 keys) is read as 16-byte runs of keys.
+// LDS rows are padded by 16 bytes, which spreads a quarter-wave's 16-byte reads over
+// all banks.
+//
+// bfloat16; head_dim a multiple of 16 up to 128 (a head_dim that is no multiple of 32 is
+// padded with zeros for the score product); page size 8, 16, 32 or a multiple of 64.
+// Other shapes are the plain kernel's.
+#include "zi_common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float pf_f32x4_t;
+
+#define PF_WAVES 4
+#define PF_BM 64     // queries per workgroup
+#define PF_BN 64     // keys per block
+
+union pf_pack {
+    uint4 u;
+    pf_bf16x8_t b;
+    uint16_t h[8];
+};
+
+template <int D>
+__global__ void __launch_bounds__(PF_WAVES* ZI_WAVE)
+attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* __restrict__ q, int64_t ldq,
+                         const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,
+                         const int32_t* __restrict__ tile_entry, const int32_t* __restrict__ tile_off,
+                         const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
+                         const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
+                         int max_pages, int num_pages, int nh, int nkv, int ps, int window, float scale) {
+    static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
+    constexpr int DK = (D + 31) / 32;   // k-steps of the score product
+    constexpr int DP = DK * 32;         // head_dim padded to a multiple of 32
+    constexpr int KS = DP + 8;          // LDS row stride of the key tile, in elements
+    constexpr int VS = PF_BN + 8;       // LDS row stride of the transposed value tile
+    constexpr int DT = D / 16;          // output tiles of 16 dims
+    constexpr int CPR = DP / 8;         // 16-byte chunks per (padded) key row
+    __shared__ __attribute__((aligned(16))) uint16_t k_lds[PF_BN * KS];
+    __shared__ __attribute__((aligned(16))) uint16_t v_lds[D * VS];
+
+    const int tile = blockIdx.x, h = blockIdx.y;
+    const int g = h / (nh / nkv);
+    const int e = tile_entry[tile], off = tile_off[tile];
+    const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
+    const int count = (len - off < PF_BM) ? len - off : PF_BM;
+    const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
+    const int r = lane & 15, j = lane >> 4;
+    const int32_t* bt = block_tables + (int64_t)e * max_pages;
+    const int pos0 = past + off;            // position of the tile's first query
+    const int kmax = pos0 + count - 1;      // last key any query of the tile sees
+    const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int kb_begin = (lo_tile / PF_BN) * PF_BN;
+
+    // this wavefront's queries
+    const int row = wave * 16 + r;
+    const bool wave_active = wave * 16 < count;
+    const bool qvalid = row < count;
+    const int qrow = qvalid ? row : count - 1;
+    const int qpos = pos0 + qrow;
+    const int wave_last = pos0 + ((wave * 16 + 15 < count) ? wave * 16 + 15 : count - 1);
+    const int wave_lo = (window > 0 && pos0 + wave * 16 - window + 1 > 0) ? pos0 + wave * 16 - window + 1 : 0;
+    pf_bf16x8_t qop[DK];
+    {
+        const zi_bf16* qr = q + (int64_t)(start + off + qrow) * ldq + (int64_t)h * D + j * 8;
+#pragma unroll
+        for (int dk = 0; dk < DK; ++dk) {
+            pf_pack p;
+            p.u = (dk * 32 + j * 8 < D) ? *reinterpret_cast<const uint4*>(qr + dk * 32) : make_uint4(0, 0, 0, 0);
+            qop[dk] = p.b;
+        }
+    }
+    pf_f32x4_t o[DT];
+#pragma unroll
+    for (int dd = 0; dd < DT; ++dd) o[dd] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, lsum = 0.f;
+
+    const int vpart = ps < PF_BN ? ps : PF_BN;   // keys of one page inside a block
+    const int gpp = vpart / 8;                   // 8-key groups of that part
+
+    for (int kb = kb_begin; kb <= kmax; kb += PF_BN) {
+        __syncthreads();
+        // ---- stage the keys: row rho(kk) of the LDS tile takes key kb + kk
+#pragma unroll
+        for (int pass = 0; pass < PF_BN * CPR / (PF_WAVES * ZI_WAVE); ++pass) {
+            const int idx = pass * (PF_WAVES * ZI_WAVE) + tid;
+            const int kk = idx / CPR, c = idx % CPR;
+            const int key = kb + kk;
+            uint4 val = make_uint4(0, 0, 0, 0);
+            if (key <= kmax && c * 8 < D) {
+                const int pi = key / ps;
+                const int page = pi < max_pages ? bt[pi] : -1;
+                if (page >= 0 && page < num_pages)
+                    val = *reinterpret_cast<const uint4*>(
+                        kcache + (((int64_t)page * nkv + g) * ps + key % ps) * D + c * 8);
+            }
+            const int rho = (2 * (kk / 32) + ((kk % 8) / 4)) * 16 + ((kk % 32) / 8) * 4 + kk % 4;
+            *reinterpret_cast<uint4*>(&k_lds[rho * KS + c * 8]) = val;
+        }
+        // ---- stage the values, transposed: row dim, column key - kb
+        for (int idx = tid; idx < D * (PF_BN / 8); idx += PF_WAVES * ZI_WAVE) {
+            const int part = idx / (D * gpp), rem = idx % (D * gpp);
+            const int dim = rem / gpp, s8 = rem % gpp;
+            const int col = part * vpart + s8 * 8;
+            const int key0 = kb + col;
+            pf_pack val;
+            val.u = make_uint4(0, 0, 0, 0);
+            if (key0 <= kmax) {
+                const int pi = key0 / ps;
+                const int page = pi < max_pages ? bt[pi] : -1;
+                if (page >= 0 && page < num_pages) {
+                    val.u = *reinterpret_cast<const uint4*>(
+                        vcache + (((int64_t)page * nkv + g) * D + dim) * ps + key0 % ps);
+                    if (key0 + 8 > kmax + 1) {   // slots past the last key may hold anything
+#pragma unroll
+                        for (int x = 0; x < 8; ++x)
+                            if (key0 + x > kmax) val.h[x] = 0;
+                    }
+                }
+            }
+            *reinterpret_cast<uint4*>(&v_lds[dim * VS + col]) = val.u;
+        }
+        __syncthreads();
+        if (!wave_active || kb > wave_last || kb + PF_BN <= wave_lo) continue;
+
+        // ---- scores of 64 keys for this lane's query
+        pf_f32x4_t s[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            s[t] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int dk = 0; dk < DK; ++dk) {
+                pf_pack a;
+                a.u = *reinterpret_cast<const uint4*>(&k_lds[(t * 16 + r) * KS + dk * 32 + j * 8]);
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, qop[dk], s[t], 0, 0, 0);
+            }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
+                const bool vis = key <= qpos && (window <= 0 || key > qpos - window);
+                const float v = vis ? s[t][x] * scale : -INFINITY;
+                s[t][x] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = (m == -INFINITY) ? 0.f : __expf(m - m_use);
+        m = m_new;
+        float psum = 0.f;
+        pf_pack pb[2];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const float p = __expf(s[t][x] - m_use);    // exp(-inf) = 0 for masked keys
+                psum += p;
+                pb[t / 2].h[(t % 2) * 4 + x] = zi_float_to_bf16(p);
+            }
+        lsum = lsum * corr + psum;
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd) {
+            o[dd][0] *= corr; o[dd][1] *= corr; o[dd][2] *= corr; o[dd][3] *= corr;
+        }
+        // ---- o^T += V^T . P^T
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                pf_pack a;
+                a.u = *reinterpret_cast<const uint4*>(&v_lds[(dd * 16 + r) * VS + b * 32 + j * 8]);
+                o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[b].b, o[dd], 0, 0, 0);
+            }
+    }
+    if (!qvalid) return;
+    float l = lsum;
+    l += __shfl_xor(l, 16, ZI_WAVE);
+    l += __shfl_xor(l, 32, ZI_WAVE);
+    const float inv = 1.f / l;
+    zi_bf16* orow = out + (int64_t)(start + off + row) * ldo + (int64_t)h * D;
+#pragma unroll
+    for (int dd = 0; dd < DT; ++dd) {
+        uint2 w;
+        w.x = (uint32_t)zi_float_to_bf16(o[dd][0] * inv) | ((uint32_t)zi_float_to_bf16(o[dd][1] * inv) << 16);
+        w.y = (uint32_t)zi_float_to_bf16(o[dd][2] * inv) | ((uint32_t)zi_float_to_bf16(o[dd][3] * inv) << 16);
+        *reinterpret_cast<uint2*>(orow + dd * 16 + j * 4) = w;
+    }
+}
+
+// 1 when the shape is this kernel's, else 0.
+extern "C" int zi_attention_prefill_supported(int dt, int nh, int nkv, int d, int page_size) {
+    if (dt != ZI_BF16 || nkv <= 0 || nh <= 0 || nh % nkv) return 0;
+    if (d < 16 || d > 128 || d % 16) return 0;
+    return page_size == 8 || page_size == 16 || page_size == 32 || (page_size > 0 && page_size % 64 == 0);
+}
+
+extern "C" int zi_attention_prefill_tile() { return PF_BM; }
+
+// Tile i covers the queries [tile_off[i], tile_off[i] + 64) of entry tile_entry[i] (fewer at the
+// entry's end); entry e brings entry_len[e] tokens that start at row entry_start[e] of q and at
+// position entry_past[e] of its sequence, whose block table is row e of block_tables.
+extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
+                                    const void* kcache, const void* vcache, const int32_t* tile_entry,
+                                    const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
+                                    const int32_t* entry_past, const int32_t* block_tables, int max_pages,
+                                    int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
+                                    hipStream_t stream) {
+    ZI_REQUIRE(zi_attention_prefill_supported(dt, nh, nkv, d, page_size),
+               "attention_prefill: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, page size 8/16/32 "
+               "or a multiple of 64): dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
+    ZI_REQUIRE(num_tiles >= 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_prefill: bad sizes");
+    ZI_REQUIRE(ldq >= (int64_t)nh * d && ldo >= (int64_t)nh * d && ldq % 8 == 0 && ldo % 4 == 0,
+               "attention_prefill: bad row stride");
+    ZI_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 && ((uintptr_t)kcache % 16) == 0 &&
+                   ((uintptr_t)vcache % 16) == 0,
+               "attention_prefill: q, out and the caches must be aligned to 16 bytes");
+    ZI_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
+    if (num_tiles == 0) return 0;
+    const dim3 grid(num_tiles, nh);
+#define ZI_PF(DD)                                                                                              \
+    attention_prefill_kernel<DD><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                                     \
+        (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
+        tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, page_size,  \
+        window, scale)
+    switch (d) {
+        case 16: ZI_PF(16); break;
+        case 32: ZI_PF(32); break;
+        case 48: ZI_PF(48); break;
+        case 64: ZI_PF(64); break;
+        case 80: ZI_PF(80); break;
+        case 96: ZI_PF(96); break;
+        case 112: ZI_PF(112); break;
+        default: ZI_PF(128); break;
+    }
+#undef ZI_PF
+    return zi_check_launch("attention_prefill");
+}

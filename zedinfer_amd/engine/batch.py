@@ -18,6 +18,7 @@ from ..cache.manager import CacheManager, SequenceCache
 
 
 SHORT_ENTRY = 4     # entries of up to this many tokens are attended token by token, split over the keys
+LONG_TILE = 64      # longer entries are cut into tiles of this many queries for the prompt kernel
 
 
 @dataclass
@@ -60,6 +61,11 @@ class DeviceBatch:
     num_long: int = 0
     max_short_keys: int = 0      # largest position + 1 among the short entries' tokens
     max_long_keys: int = 0
+    # The long entries cut into tiles of LONG_TILE queries, the tile that sees most keys first:
+    # tile i covers tokens [tile_off[i], tile_off[i] + LONG_TILE) of entry tile_entry[i].
+    tile_entry: Optional[torch.Tensor] = None
+    tile_off: Optional[torch.Tensor] = None
+    num_tiles: int = 0
     # host copies, for parts that plan their launches on the host
     host_start: Optional[np.ndarray] = None
     host_len: Optional[np.ndarray] = None
@@ -126,8 +132,14 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     max_short = int(ends[lens_a <= SHORT_ENTRY].max()) if n_short else 0
     max_long = int(ends[lens_a > SHORT_ENTRY].max()) if n_long else 0
 
+    tiles = [(int(past[i]) + off + min(LONG_TILE, int(lens_a[i]) - off), i, off)
+             for i in range(E) if lens_a[i] > SHORT_ENTRY for off in range(0, int(lens_a[i]), LONG_TILE)]
+    tiles.sort(key=lambda t: -t[0])
+    tile_entry = np.array([t[1] for t in tiles], dtype=np.int32)
+    tile_off = np.array([t[2] for t in tiles], dtype=np.int32)
+
     pieces = [token_ids.astype(np.int32), positions, tok_seq, logit_rows, starts, lens_a, past, slot,
-              short_idx, long_idx]
+              short_idx, long_idx, tile_entry, tile_off]
     for g in range(G):
         pieces += [group_slots[g], group_tables[g].reshape(-1)]
     sizes = [p.size for p in pieces]
@@ -143,11 +155,12 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     for s in sizes:
         views.append(dev[off:off + s])
         off += s
-    groups = [GroupView(views[10 + 2 * g], views[11 + 2 * g].view(E, widths[g])) for g in range(G)]
+    groups = [GroupView(views[12 + 2 * g], views[13 + 2 * g].view(E, widths[g])) for g in range(G)]
     return DeviceBatch(num_tokens=N, num_entries=E, num_logit_rows=R, token_ids=views[0], positions=views[1],
                        tok_seq=views[2], logit_rows=views[3], entry_start=views[4], entry_len=views[5],
                        entry_past=views[6], entry_slot=views[7], groups=groups,
                        short_idx=views[8] if 0 < n_short < N else None,
                        long_idx=views[9] if 0 < n_long < N else None, num_short=n_short, num_long=n_long,
-                       max_short_keys=max_short, max_long_keys=max_long, host_start=starts,
+                       max_short_keys=max_short, max_long_keys=max_long, tile_entry=views[10], tile_off=views[11],
+                       num_tiles=len(tiles), host_start=starts,
                        host_len=lens_a, host_past=past, host_slot=slot)

@@ -28,6 +28,9 @@ _PROTOTYPES = {
     "zi_attention_generic": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
     "zi_attention_decode": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P],
     "zi_attention_decode_supported": [I, I, I, I, I],
+    "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
+    "zi_attention_prefill_supported": [I, I, I, I, I],
+    "zi_attention_prefill_tile": [],
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
     "zi_gemm_skinny": [P, I, P, P, P, I, I, I, L, L, L, P, L, P],
     "zi_gemm_skinny_supported": [I, I, I, L, L],

@@ -329,6 +329,57 @@ def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
     return out
 
 
+PREFILL_TILE = 64     # queries one workgroup of the prompt kernel takes
+
+
+def attention_prefill_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, page_size: int) -> bool:
+    if dtype not in _CODES:
+        return False
+    return bool(_lib.load().zi_attention_prefill_supported(_CODES[dtype], nh, nkv, d, page_size))
+
+
+def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tile_entry: torch.Tensor,
+                      tile_off: torch.Tensor, entry_start: torch.Tensor, entry_len: torch.Tensor,
+                      entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
+                      window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
+    of 16 up to 128, page size 8/16/32 or a multiple of 64).
+
+    Entry e brings ``entry_len[e]`` tokens, rows ``entry_start[e]...`` of q, that continue a sequence
+    holding ``entry_past[e]`` tokens whose block table is row e of ``block_tables``.  Tile i covers the
+    queries [tile_off[i], tile_off[i] + PREFILL_TILE) of entry ``tile_entry[i]``; rows of ``out`` that no
+    tile covers are left alone."""
+    _gpu("attention_prefill", q, kcache, vcache, tile_entry, tile_off, entry_start, entry_len, entry_past,
+         block_tables, out)
+    ldq, wq = _rows(q, "attention_prefill q")
+    n = q.shape[0]
+    if wq != nh * d:
+        raise ValueError(f"attention_prefill: q has width {wq}, expected {nh}*{d}")
+    if nkv <= 0 or nh % nkv:
+        raise ValueError(f"attention_prefill: {nh} query heads are not a multiple of {nkv} key/value heads")
+    pages, ps = _check_cache(kcache, vcache, nkv, d, q.dtype, "attention_prefill")
+    num_tiles = tile_entry.numel()
+    _i32(tile_entry, "attention_prefill tile_entry")
+    _i32(tile_off, "attention_prefill tile_off", num_tiles)
+    E = entry_start.numel()
+    for name, t in (("entry_start", entry_start), ("entry_len", entry_len), ("entry_past", entry_past)):
+        _i32(t, f"attention_prefill {name}", E)
+    if (block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous()
+            or block_tables.shape[0] < E):
+        raise ValueError("attention_prefill: block_tables must be a contiguous int32 [entries, max_pages] tensor")
+    if _lib.load().zi_attention_prefill_tile() != PREFILL_TILE:
+        raise _lib.KernelLibraryError("the kernel library was built for another prompt tile size")
+    if out is None:
+        out = torch.empty((n, nh * d), dtype=q.dtype, device=q.device)
+    ldo, wo = _rows(out, "attention_prefill out")
+    if tuple(out.shape) != (n, nh * d) or out.dtype != q.dtype:
+        raise ValueError("attention_prefill: out has the wrong shape or dtype")
+    _lib.call("zi_attention_prefill", _p(out), _p(q), _code(q, "attention_prefill"), num_tiles, ldq, ldo, _p(kcache),
+              _p(vcache), _p(tile_entry), _p(tile_off), _p(entry_start), _p(entry_len), _p(entry_past),
+              _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), _stream())
+    return out
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """out[M,N] = x[M,K] . weight[N,K]^T + bias[N], accumulated in float32

@@ -67,7 +67,8 @@ class Attention(Mixer):
 
     def attend(self, q, att, batch, view, memory: LayerMemory) -> None:
         """Tokens of short entries (decoded tokens) go to the kernel that splits one query's keys over
-        many wavefronts; longer portions, and every shape that kernel does not take, go to the plain one."""
+        many wavefronts, longer portions to the matrix-core prompt kernel; every shape those kernels do
+        not take goes to the plain one."""
         args = (memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
                 self.scale)
         n_long = batch.num_long
@@ -82,7 +83,12 @@ class Attention(Mixer):
         if n_long < 0:
             ops.attention(q, *args, self.window, out=att)
         elif n_long > 0:
-            ops.attention(q, *args, self.window, out=att, tok_index=batch.long_idx)
+            if ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
+                ops.attention_prefill(q, memory.k, memory.v, batch.tile_entry, batch.tile_off, batch.entry_start,
+                                      batch.entry_len, batch.entry_past, view.block_tables, self.nh, self.nkv,
+                                      self.d, self.scale, self.window, out=att)
+            else:
+                ops.attention(q, *args, self.window, out=att, tok_index=batch.long_idx)
 
     def cache_request(self) -> Optional[KVCacheRequest]:
         return KVCacheRequest("window" if self.window > 0 else "full", self.nkv, self.d, self.window)
