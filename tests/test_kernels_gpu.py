@@ -275,7 +275,8 @@ def test_argmax(ops, dtype):
 
 @pytest.mark.parametrize("nh,nkv,d,ps,T,window", [
     (12, 2, 128, 16, 2100, 0), (12, 2, 128, 16, 70, 0), (28, 4, 128, 16, 5000, 0), (3, 1, 64, 8, 200, 0),
-    (8, 1, 64, 16, 300, 37), (5, 5, 256, 32, 150, 0), (4, 2, 128, 8, 260, 100), (14, 2, 128, 16, 9, 0)])
+    (8, 1, 64, 16, 300, 37), (5, 5, 80, 32, 150, 0), (4, 2, 128, 8, 260, 100), (14, 2, 128, 16, 9, 0),
+    (12, 1, 48, 8, 700, 0), (4, 2, 16, 16, 1000, 300), (32, 2, 112, 64, 530, 0), (12, 2, 128, 16, 17000, 0)])
 def test_attention_decode(ops, nh, nkv, d, ps, T, window):
     """The split-keys kernel against the same float32 reference, with a listed subset of the tokens."""
     dtype = torch.bfloat16
@@ -283,7 +284,7 @@ def test_attention_decode(ops, nh, nkv, d, ps, T, window):
     k, v = rnd(T, nkv, d, dtype=dtype, seed=1), rnd(T, nkv, d, dtype=dtype, seed=2)
     pages = (T + ps - 1) // ps + 3
     kc, vc, table = make_paged(k, v, ps, pages)
-    pos_list = sorted(p for p in {T - 1, T - 2, 0, 1, 7, 8, 63, 64, 65, 127, 128, T // 2, T // 3} if p < T)
+    pos_list = sorted(p for p in {T - 1, T - 2, 0, 1, 7, 8, 63, 64, 65, 127, 128, 255, 256, 257, 511, 512, 16383, 16384, T // 2, T // 3} if p < T)
     pos = torch.tensor(pos_list, dtype=torch.int32, device="cuda")
     n = pos.numel()
     q = rnd(n, nh, d, dtype=dtype, seed=3)
@@ -324,15 +325,19 @@ def test_attention_decode_ignores_stale_slots(ops):
 
 def test_unsupported_shapes_are_refused(ops):
     assert not ops.attention_decode_supported(torch.float32, 12, 2, 128, 16)
-    assert not ops.attention_decode_supported(torch.bfloat16, 12, 2, 48, 16)
-    assert not ops.attention_decode_supported(torch.bfloat16, 12, 1, 128, 16)       # group of 12
+    assert not ops.attention_decode_supported(torch.bfloat16, 12, 2, 40, 16)
+    assert not ops.attention_decode_supported(torch.bfloat16, 12, 2, 256, 16)
+    assert not ops.attention_decode_supported(torch.bfloat16, 34, 2, 128, 16)       # group of 17
     assert not ops.attention_decode_supported(torch.bfloat16, 12, 2, 128, 4)
     q = rnd(1, 12 * 48, dtype=torch.bfloat16)
     kc = torch.zeros(4, 2, 16, 48, dtype=torch.bfloat16, device="cuda")
     vc = torch.zeros(4, 2, 48, 16, dtype=torch.bfloat16, device="cuda")
     z = torch.zeros(1, dtype=torch.int32, device="cuda")
     with pytest.raises(ops.KernelLibraryError, match="unsupported shape"):
-        ops.attention_decode(q, kc, vc, z, z, torch.zeros(1, 4, dtype=torch.int32, device="cuda"), 12, 2, 48, 0.1, 1)
+        ops.attention_decode(rnd(1, 2 * 256, dtype=torch.bfloat16),
+                             torch.zeros(4, 2, 16, 256, dtype=torch.bfloat16, device="cuda"),
+                             torch.zeros(4, 2, 256, 16, dtype=torch.bfloat16, device="cuda"), z, z,
+                             torch.zeros(1, 4, dtype=torch.int32, device="cuda"), 2, 2, 256, 0.1, 1)
     with pytest.raises(ValueError, match="multiple"):
         ops.attention(q, kc, vc, z, z, torch.zeros(1, 4, dtype=torch.int32, device="cuda"), 12, 5, 48, 0.1)
     with pytest.raises(ops.KernelLibraryError, match="larger than"):

@@ -1,297 +1,338 @@
-// Paged grouped-query attention for single query tokens, split over the keys.
+// Paged grouped-query attention for single query tokens, split over the keys, on
+// the matrix cores.
 //
-// One wavefront per (token, key/value head, split of the keys).  It serves all
-// G = heads / kv_heads query heads of its group from one pass over the keys and
-// values, so each cached byte is read once per token.  A token at position p
-// sees keys [lo, p] (lo = 0, or p - window + 1); that range, widened down to a
-// multiple of 8, is cut into at most 64 splits of 64 keys (128, 256, ... when
-// there are more than 4096 keys), which depends on the token alone, never on the
-// rest of the batch.  Each split leaves a partial (running maximum, sum,
-// unnormalised output) and a second kernel merges the splits; a token with one
-// split is finished by the first kernel.
+// One workgroup of four wavefronts per (token, key/value head, chunk of the keys).
+// It serves all G = heads / kv_heads query heads of its group from one pass over
+// the keys and values, so each cached byte is read once per token: the G heads
+// stand in for the 16 "queries" of a v_mfma_f32_16x16x32_bf16 tile (rows beyond G
+// are zero).  A token at position p sees keys [lo, p] (lo = 0, or p - window + 1);
+// that range, widened down to a multiple of 8, is cut into at most 64 chunks of 256
+// keys (512, 1024, ... when there are more than 16384 keys), which depends on the
+// token alone, never on the rest of the batch.  Inside a chunk every wavefront takes
+// a quarter, in blocks of 64 keys: it loads the block's keys and values straight
+// from the cache into matrix-core operands (nothing is shared between wavefronts,
+// so nothing goes through LDS), computes the scores transposed, S^T = K . Q^T, so
+// that a lane holds the scores of one head, runs the softmax on them in float32,
+// and accumulates O^T += V^T . P^T.  The four wavefronts' running (maximum, sum,
+// output) are merged through LDS; a token with one chunk is finished there, else
+// the chunk leaves a partial and a second kernel merges the chunks in rising order.
+// (reference formulas: src/backend/ops/self_attention/cpu/paged_attention_cpu.cpp:15-72;
+// the scale is applied after the dot product, :44.)
 //
-// Keys are read 16 bytes a lane, head_dim/8 lanes a key, and the dot products
-// are finished with a butterfly over those lanes.  Values are stored transposed
-// ([dim][slot]), so a lane owns output dimensions and reads eight consecutive
-// positions of one dimension at a time.  Scores, the softmax and the sums are
-// float32 (reference formulas: src/backend/ops/self_attention/cpu/paged_attention_cpu.cpp:15-72).
+// Operand layout: as in the prompt kernel, the keys of a block are assigned to the
+// rows of the four score tiles in a permuted order (tile t, row j*4 + e <-> key
+// (t/2)*32 + j*8 + (t%2)*4 + e), which makes the eight probabilities a lane holds
+// after two tiles the eight consecutive keys that the P.V product wants from it.
+// Values are cached transposed ([dim][slot]), so a lane reads 16-byte runs of keys.
 //
-// bfloat16 only; head_dim 64, 128 or 256; group size up to 8; page size a multiple
-// of 8.  Other shapes are the plain kernel's.
+// bfloat16 only; head_dim a multiple of 16 up to 128; group size up to 16; page size
+// a multiple of 8.  Other shapes are the plain kernel's.
 #include "zi_common.h"
 
-#define DEC_MAXS 64      // most splits of one token
-#define DEC_TILE 64      // keys a wavefront handles at a time
+typedef __attribute__((ext_vector_type(8))) __bf16 dec_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float dec_f32x4_t;
 
-__device__ __forceinline__ void unpack8(const uint4& r, float* f) {
-    f[0] = __uint_as_float(r.x << 16); f[1] = __uint_as_float(r.x & 0xffff0000u);
-    f[2] = __uint_as_float(r.y << 16); f[3] = __uint_as_float(r.y & 0xffff0000u);
-    f[4] = __uint_as_float(r.z << 16); f[5] = __uint_as_float(r.z & 0xffff0000u);
-    f[6] = __uint_as_float(r.w << 16); f[7] = __uint_as_float(r.w & 0xffff0000u);
-}
+#define DEC_MAXC 64       // most chunks of one token
+#define DEC_CHUNK 256     // keys of the smallest chunk
+#define DEC_WAVES 4
+#define DEC_BLOCK 64      // keys a wavefront handles at a time
 
-// The cut of a token's keys: first key seen, first key of split 0 (a multiple of 8),
-// keys per split, number of splits.
+union dec_pack {
+    uint4 u;
+    dec_bf16x8_t b;
+    uint16_t h[8];
+};
+
+// The cut of a token's keys: first key seen, first key of chunk 0 (a multiple of 8),
+// keys per chunk, number of chunks.
 struct DecSplit {
     int lo, lo_al, len, count;
 };
-__device__ __forceinline__ DecSplit dec_split(int p, int window) {
+__host__ __device__ __forceinline__ DecSplit dec_split(int p, int window) {
     DecSplit s;
     s.lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
     s.lo_al = s.lo & ~7;
     const int nk = p - s.lo_al + 1;
-    s.len = DEC_TILE;
-    while (nk > s.len * DEC_MAXS) s.len *= 2;
+    s.len = DEC_CHUNK;
+    while (nk > s.len * DEC_MAXC) s.len *= 2;
     s.count = (nk + s.len - 1) / s.len;
     return s;
 }
 
-template <int D, int G>
-__global__ void __launch_bounds__(ZI_WAVE)
+template <int D>
+__global__ void __launch_bounds__(DEC_WAVES* ZI_WAVE)
 attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restrict__ part_o,
                         float* __restrict__ part_ml, const zi_bf16* __restrict__ q, int64_t ldq,
                         const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,
                         const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
-                        int max_pages, int num_pages, int nh, int nkv, int ps, int window, float scale,
-                        int max_splits) {
-    constexpr int LPK = D / 8;          // lanes that share one key
-    constexpr int KPI = ZI_WAVE / LPK;  // keys per load instruction
-    constexpr int DV = D / ZI_WAVE;     // output dims per lane
-    static_assert(D % ZI_WAVE == 0 && LPK <= ZI_WAVE, "head_dim must be 64, 128 or 256");
-    __shared__ __attribute__((aligned(16))) float sc[G][DEC_TILE];
+                        int max_pages, int num_pages, int nh, int nkv, int G, int ps, int window, float scale,
+                        int max_chunks) {
+    static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
+    constexpr int DK = (D + 31) / 32;   // k-steps of the score product
+    constexpr int DT = D / 16;          // output tiles of 16 dims
+    __shared__ float sm[DEC_WAVES][16], sl[DEC_WAVES][16];
+    __shared__ dec_f32x4_t so[DEC_WAVES][DT][ZI_WAVE];
 
-    const int x = blockIdx.x, kvh = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+    const int x = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
+    const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
+    const int r = lane & 15, j = lane >> 4;
     const int t = tok_index ? tok_index[x] : x;
     const int p = tok_pos[t];
     const DecSplit sp = dec_split(p, window);
-    if (sp.count > max_splits) {
+    if (sp.count > max_chunks) {
         // The host sized the launch (and the workspace) for fewer keys than this token sees.  Nothing
         // may be written to the workspace then; the token's output is made NaN so that it shows.
-        if (split == 0)
-            for (int i = lane; i < G * D; i += ZI_WAVE)
+        if (chunk == 0)
+            for (int i = tid; i < G * D; i += DEC_WAVES * ZI_WAVE)
                 zi_store(out + (int64_t)t * ldo + (int64_t)kvh * G * D + i, NAN);
         return;
     }
-    if (split >= sp.count) return;
+    if (chunk >= sp.count) return;
     const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
-    const int k_begin = sp.lo_al + split * sp.len;
-    const int k_stop = (k_begin + sp.len < p + 1) ? k_begin + sp.len : p + 1;   // one past the last key
+    const int quarter = sp.len / DEC_WAVES;
+    const int k_begin = sp.lo_al + chunk * sp.len + wave * quarter;
+    const int k_end = (k_begin + quarter < p + 1) ? k_begin + quarter : p + 1;   // one past the wavefront's last key
 
-    const int sub = lane / LPK, chunk = lane % LPK;
-    float qr[G][8];
+    // the group's queries as the B operand: lane (r, j) holds head r, dims dk*32 + j*8 ..
+    dec_bf16x8_t qop[DK];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const uint4 raw = *reinterpret_cast<const uint4*>(q + (int64_t)t * ldq + (int64_t)(kvh * G + g) * D + chunk * 8);
-        unpack8(raw, qr[g]);
+    for (int dk = 0; dk < DK; ++dk) {
+        dec_pack w;
+        w.u = make_uint4(0, 0, 0, 0);
+        if (r < G && dk * 32 + j * 8 < D)
+            w.u = *reinterpret_cast<const uint4*>(q + (int64_t)t * ldq + (int64_t)(kvh * G + r) * D + dk * 32 + j * 8);
+        qop[dk] = w.b;
     }
-    float m[G], l[G], acc[G][DV];
+    dec_f32x4_t o[DT];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        m[g] = -INFINITY;
-        l[g] = 0.f;
-#pragma unroll
-        for (int v = 0; v < DV; ++v) acc[g][v] = 0.f;
-    }
+    for (int dd = 0; dd < DT; ++dd) o[dd] = dec_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, lsum = 0.f;
 
-    for (int base = k_begin; base < k_stop; base += DEC_TILE) {
-        // ---- scores of up to 64 keys
-#pragma unroll 2
-        for (int i = 0; i < DEC_TILE / KPI; ++i) {
-            const int key = base + i * KPI + sub;
-            const bool valid = key >= sp.lo && key < k_stop;
-            float dot[G];
+    for (int base = k_begin; base < k_end; base += DEC_BLOCK) {
+        // ---- all loads of the block first: keys (4 tiles x DK) and values (DT x 2)
+        dec_pack kop[4][DK], vop[DT][2];
 #pragma unroll
-            for (int g = 0; g < G; ++g) dot[g] = 0.f;
-            if (valid) {
+        for (int tt = 0; tt < 4; ++tt) {
+            const int key = base + (tt / 2) * 32 + (r / 4) * 8 + (tt % 2) * 4 + (r % 4);
+            const zi_bf16* kr = nullptr;
+            if (key < k_end && key >= sp.lo) {
                 const int pi = key / ps;
                 const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages) {
-                    const uint4 raw = *reinterpret_cast<const uint4*>(
-                        kcache + (((int64_t)page * nkv + kvh) * ps + key % ps) * D + chunk * 8);
-                    float kf[8];
-                    unpack8(raw, kf);
-#pragma unroll
-                    for (int g = 0; g < G; ++g)
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) dot[g] = fmaf(qr[g][e], kf[e], dot[g]);
-                }
+                if (page >= 0 && page < num_pages) kr = kcache + (((int64_t)page * nkv + kvh) * ps + key % ps) * D + j * 8;
             }
 #pragma unroll
-            for (int g = 0; g < G; ++g) {
-#pragma unroll
-                for (int o = LPK / 2; o > 0; o >>= 1) dot[g] += __shfl_xor(dot[g], o, ZI_WAVE);
-            }
-            if (chunk == 0) {
-#pragma unroll
-                for (int g = 0; g < G; ++g) sc[g][i * KPI + sub] = valid ? dot[g] * scale : -INFINITY;
+            for (int dk = 0; dk < DK; ++dk) {
+                kop[tt][dk].u = make_uint4(0, 0, 0, 0);
+                if (kr && dk * 32 + j * 8 < D) kop[tt][dk].u = *reinterpret_cast<const uint4*>(kr + dk * 32);
             }
         }
-        __syncthreads();
-        // ---- running softmax, one key a lane
-        float corr[G];
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const float s = sc[g][lane];
-            const float m_new = fmaxf(m[g], zi_wave_max(s));
-            const float pj = (s == -INFINITY) ? 0.f : expf(s - m_new);
-            corr[g] = (m[g] == -INFINITY) ? 0.f : expf(m[g] - m_new);
-            l[g] = l[g] * corr[g] + zi_wave_sum(pj);
-            m[g] = m_new;
-            sc[g][lane] = pj;
+        for (int b = 0; b < 2; ++b) {
+            const int key0 = base + b * 32 + j * 8;
+            const zi_bf16* vr = nullptr;
+            if (key0 < k_end && key0 + 8 > sp.lo) {
+                const int pi = key0 / ps;
+                const int page = pi < max_pages ? bt[pi] : -1;
+                if (page >= 0 && page < num_pages) vr = vcache + (((int64_t)page * nkv + kvh) * D + r) * ps + key0 % ps;
+            }
+            const bool edge = key0 < sp.lo || key0 + 8 > k_end;
 #pragma unroll
-            for (int v = 0; v < DV; ++v) acc[g][v] *= corr[g];
-        }
-        __syncthreads();
-        // ---- values: eight positions of one dimension per load
-        for (int grp = 0; grp < DEC_TILE / 8; ++grp) {
-            const int key0 = base + grp * 8;
-            if (key0 >= k_stop || key0 + 8 <= sp.lo) continue;
-            const int pi = key0 / ps;
-            const int page = pi < max_pages ? bt[pi] : -1;
-            if (page < 0 || page >= num_pages) continue;
-            const bool edge = key0 < sp.lo || key0 + 8 > k_stop;
-            const int64_t vb = ((int64_t)page * nkv + kvh) * D * ps + key0 % ps;
+            for (int dd = 0; dd < DT; ++dd) {
+                vop[dd][b].u = make_uint4(0, 0, 0, 0);
+                if (vr) {
+                    vop[dd][b].u = *reinterpret_cast<const uint4*>(vr + (int64_t)dd * 16 * ps);
+                    if (edge) {   // slots outside [lo, p] may hold anything: keep them out of the sum
 #pragma unroll
-            for (int v = 0; v < DV; ++v) {
-                const uint4 raw = *reinterpret_cast<const uint4*>(vcache + vb + (int64_t)(lane + v * ZI_WAVE) * ps);
-                float vf[8];
-                unpack8(raw, vf);
-                if (edge) {   // positions outside [lo, p] may hold anything: keep them out of the sum
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (key0 + e < sp.lo || key0 + e >= k_stop) vf[e] = 0.f;
-                }
-#pragma unroll
-                for (int g = 0; g < G; ++g) {
-                    const float4 p0 = *reinterpret_cast<const float4*>(&sc[g][grp * 8]);
-                    const float4 p1 = *reinterpret_cast<const float4*>(&sc[g][grp * 8 + 4]);
-                    float a = acc[g][v];
-                    a = fmaf(p0.x, vf[0], a); a = fmaf(p0.y, vf[1], a); a = fmaf(p0.z, vf[2], a); a = fmaf(p0.w, vf[3], a);
-                    a = fmaf(p1.x, vf[4], a); a = fmaf(p1.y, vf[5], a); a = fmaf(p1.z, vf[6], a); a = fmaf(p1.w, vf[7], a);
-                    acc[g][v] = a;
+                        for (int e = 0; e < 8; ++e)
+                            if (key0 + e < sp.lo || key0 + e >= k_end) vop[dd][b].h[e] = 0;
+                    }
                 }
             }
         }
-        __syncthreads();
+        // ---- scores of 64 keys for this lane's head
+        dec_f32x4_t s[4];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            s[tt] = dec_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int dk = 0; dk < DK; ++dk)
+                s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[tt][dk].b, qop[dk], s[tt], 0, 0, 0);
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int key = base + (tt / 2) * 32 + j * 8 + (tt % 2) * 4 + e;
+                const float v = (key >= sp.lo && key < k_end) ? s[tt][e] * scale : -INFINITY;
+                s[tt][e] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = (m == -INFINITY) ? 0.f : __expf(m - m_use);
+        m = m_new;
+        float psum = 0.f;
+        dec_pack pb[2];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float pj = __expf(s[tt][e] - m_use);   // exp(-inf) = 0 for keys not seen
+                psum += pj;
+                pb[tt / 2].h[(tt % 2) * 4 + e] = zi_float_to_bf16(pj);
+            }
+        lsum = lsum * corr + psum;
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd) {
+            o[dd][0] *= corr; o[dd][1] *= corr; o[dd][2] *= corr; o[dd][3] *= corr;
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+                o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vop[dd][b].b, pb[b].b, o[dd], 0, 0, 0);
+        }
     }
-
-    if (sp.count == 1) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-            const float inv = 1.f / l[g];
-#pragma unroll
-            for (int v = 0; v < DV; ++v)
-                zi_store(out + (int64_t)t * ldo + (int64_t)(kvh * G + g) * D + lane + v * ZI_WAVE, acc[g][v] * inv);
-        }
-        return;
+    // ---- merge the four wavefronts: head r's (m, l) and this lane's outputs
+    lsum += __shfl_xor(lsum, 16, ZI_WAVE);
+    lsum += __shfl_xor(lsum, 32, ZI_WAVE);
+    if (j == 0) {
+        sm[wave][r] = m;
+        sl[wave][r] = lsum;
     }
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        const int64_t slot = ((int64_t)x * nh + kvh * G + g) * DEC_MAXS + split;
+    for (int dd = 0; dd < DT; ++dd) so[wave][dd][lane] = o[dd];
+    __syncthreads();
+    float M = sm[0][r];
 #pragma unroll
-        for (int v = 0; v < DV; ++v) part_o[slot * D + lane + v * ZI_WAVE] = acc[g][v];
-        if (lane == 0) {
-            part_ml[slot * 2] = m[g];
-            part_ml[slot * 2 + 1] = l[g];
+    for (int w = 1; w < DEC_WAVES; ++w) M = fmaxf(M, sm[w][r]);
+    float a[DEC_WAVES], L = 0.f;
+#pragma unroll
+    for (int w = 0; w < DEC_WAVES; ++w) {
+        a[w] = (sm[w][r] == -INFINITY) ? 0.f : __expf(sm[w][r] - M);
+        L += a[w] * sl[w][r];
+    }
+    const bool final = sp.count == 1;
+    const float inv = final ? 1.f / L : 1.f;
+    const int64_t slot = ((int64_t)x * nh + kvh * G + r) * DEC_MAXC + chunk;
+    for (int dd = wave; dd < DT; dd += DEC_WAVES) {
+        dec_f32x4_t acc = dec_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < DEC_WAVES; ++w) {
+            const dec_f32x4_t v = so[w][dd][lane];
+            acc[0] += a[w] * v[0]; acc[1] += a[w] * v[1]; acc[2] += a[w] * v[2]; acc[3] += a[w] * v[3];
         }
+        if (r >= G) continue;
+        if (final) {
+            uint2 wv;
+            wv.x = (uint32_t)zi_float_to_bf16(acc[0] * inv) | ((uint32_t)zi_float_to_bf16(acc[1] * inv) << 16);
+            wv.y = (uint32_t)zi_float_to_bf16(acc[2] * inv) | ((uint32_t)zi_float_to_bf16(acc[3] * inv) << 16);
+            *reinterpret_cast<uint2*>(out + (int64_t)t * ldo + (int64_t)(kvh * G + r) * D + dd * 16 + j * 4) = wv;
+        } else {
+            *reinterpret_cast<dec_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = acc;
+        }
+    }
+    if (!final && wave == 0 && j == 0 && r < G) {
+        part_ml[slot * 2] = M;
+        part_ml[slot * 2 + 1] = L;
     }
 }
 
-// Merge the splits of one (token, head): out = sum_s e^(m_s - M) o_s / sum_s e^(m_s - M) l_s.
-template <int D>
+// Merge the chunks of one (token, head): out = sum_c e^(m_c - M) o_c / sum_c e^(m_c - M) l_c.
 __global__ void __launch_bounds__(ZI_WAVE)
 attention_decode_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const float* __restrict__ part_o,
                               const float* __restrict__ part_ml, const int32_t* __restrict__ tok_index,
-                              const int32_t* __restrict__ tok_pos, int nh, int window, int max_splits) {
-    constexpr int DV = D / ZI_WAVE;
+                              const int32_t* __restrict__ tok_pos, int nh, int D, int window, int max_chunks) {
     const int x = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int t = tok_index ? tok_index[x] : x;
     const DecSplit sp = dec_split(tok_pos[t], window);
-    if (sp.count == 1 || sp.count > max_splits) return;
-    const int64_t slot0 = ((int64_t)x * nh + h) * DEC_MAXS;
-    float M = -INFINITY;
-    for (int s = 0; s < sp.count; ++s) M = fmaxf(M, part_ml[(slot0 + s) * 2]);
-    float L = 0.f, acc[DV];
+    if (sp.count == 1 || sp.count > max_chunks) return;
+    const int64_t slot0 = ((int64_t)x * nh + h) * DEC_MAXC;
+    // chunk c's (m, l) sit in lane c
+    const float mc = lane < sp.count ? part_ml[(slot0 + lane) * 2] : -INFINITY;
+    const float lc = lane < sp.count ? part_ml[(slot0 + lane) * 2 + 1] : 0.f;
+    const float M = zi_wave_max(mc);
+    const float wc = (mc == -INFINITY) ? 0.f : __expf(mc - M);
+    float L = 0.f, acc[2] = {0.f, 0.f};
+    for (int c = 0; c < sp.count; ++c) {
+        const float w = __shfl(wc, c, ZI_WAVE);
+        L += w * __shfl(lc, c, ZI_WAVE);
 #pragma unroll
-    for (int v = 0; v < DV; ++v) acc[v] = 0.f;
-    for (int s = 0; s < sp.count; ++s) {
-        const float ms = part_ml[(slot0 + s) * 2];
-        const float w = (ms == -INFINITY) ? 0.f : expf(ms - M);
-        L += w * part_ml[(slot0 + s) * 2 + 1];
-#pragma unroll
-        for (int v = 0; v < DV; ++v) acc[v] += w * part_o[(slot0 + s) * D + lane + v * ZI_WAVE];
+        for (int v = 0; v < 2; ++v)
+            if (lane + v * ZI_WAVE < D) acc[v] += w * part_o[(slot0 + c) * D + lane + v * ZI_WAVE];
     }
     const float inv = 1.f / L;
 #pragma unroll
-    for (int v = 0; v < DV; ++v) zi_store(out + (int64_t)t * ldo + (int64_t)h * D + lane + v * ZI_WAVE, acc[v] * inv);
-}
-
-template <int D>
-static int launch_decode(int G, dim3 grid, hipStream_t stream, zi_bf16* out, int64_t ldo, float* po, float* pml,
-                         const zi_bf16* q, int64_t ldq, const zi_bf16* kc, const zi_bf16* vc, const int32_t* ti,
-                         const int32_t* ts, const int32_t* tp, const int32_t* bt, int max_pages, int num_pages,
-                         int nh, int nkv, int ps, int window, float scale, int max_splits) {
-#define ZI_DEC_CASE(GG)                                                                                          \
-    case GG:                                                                                                     \
-        attention_decode_kernel<D, GG><<<grid, ZI_WAVE, 0, stream>>>(out, ldo, po, pml, q, ldq, kc, vc, ti, ts, \
-                                                                     tp, bt, max_pages, num_pages, nh, nkv, ps, \
-                                                                     window, scale, max_splits);                \
-        break;
-    switch (G) {
-        ZI_DEC_CASE(1) ZI_DEC_CASE(2) ZI_DEC_CASE(3) ZI_DEC_CASE(4) ZI_DEC_CASE(5) ZI_DEC_CASE(6) ZI_DEC_CASE(7)
-        ZI_DEC_CASE(8)
-        default: return zi_fail("attention_decode: group size %d is not supported (1..8)", G);
-    }
-#undef ZI_DEC_CASE
-    return 0;
+    for (int v = 0; v < 2; ++v)
+        if (lane + v * ZI_WAVE < D) zi_store(out + (int64_t)t * ldo + (int64_t)h * D + lane + v * ZI_WAVE, acc[v] * inv);
 }
 
 // Floats of workspace the split kernel needs for n tokens.
 extern "C" int64_t zi_attention_decode_workspace(int n, int nh, int d) {
-    return (int64_t)n * nh * DEC_MAXS * (d + 2);
+    return (int64_t)n * nh * DEC_MAXC * (d + 2);
+}
+
+// Chunks the launch must cover when no token sees more than `keys` keys (position + 1, or the window).
+extern "C" int zi_attention_decode_chunks(int keys) {
+    if (keys < 1) keys = 1;
+    // the range is widened down to a multiple of 8: up to 7 more keys.  Past DEC_CHUNK * DEC_MAXC keys
+    // the chunks grow and their number drops again, but a token with fewer keys may still need them all.
+    if (keys + 7 > DEC_CHUNK * DEC_MAXC) return DEC_MAXC;
+    return dec_split(keys - 1 + 7, 0).count;
 }
 
 // 1 when the shape is this kernel's, else 0.
 extern "C" int zi_attention_decode_supported(int dt, int nh, int nkv, int d, int page_size) {
-    if (dt != ZI_BF16 || nkv <= 0 || nh % nkv) return 0;
+    if (dt != ZI_BF16 || nkv <= 0 || nh <= 0 || nh % nkv) return 0;
     const int G = nh / nkv;
-    return (d == 64 || d == 128 || d == 256) && G >= 1 && G <= 8 && page_size % 8 == 0;
+    return d >= 16 && d <= 128 && d % 16 == 0 && G <= 16 && page_size > 0 && page_size % 8 == 0;
 }
 
 extern "C" int zi_attention_decode(void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo,
                                    const void* kcache, const void* vcache, const int32_t* tok_index,
                                    const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
                                    int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
-                                   float scale, int max_splits, float* workspace, int64_t workspace_floats,
+                                   float scale, int max_chunks, float* workspace, int64_t workspace_floats,
                                    hipStream_t stream) {
     ZI_REQUIRE(zi_attention_decode_supported(dt, nh, nkv, d, page_size),
-               "attention_decode: unsupported shape (bfloat16, head_dim 64/128/256, group <= 8, page size %% 8 == 0): "
-               "dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
+               "attention_decode: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, group <= 16, "
+               "page size %% 8 == 0): dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
     ZI_REQUIRE(n_idx >= 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_decode: bad sizes");
-    ZI_REQUIRE(max_splits >= 1 && max_splits <= DEC_MAXS, "attention_decode: max_splits %d outside 1..%d", max_splits, DEC_MAXS);
-    ZI_REQUIRE(ldq >= (int64_t)nh * d && ldo >= (int64_t)nh * d && ldq % 8 == 0, "attention_decode: bad row stride");
-    ZI_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)kcache % 16) == 0 && ((uintptr_t)vcache % 16) == 0,
-               "attention_decode: q and the caches must be 16-byte aligned");
-    ZI_REQUIRE(nkv <= 65535, "attention_decode: too many kv heads");
+    ZI_REQUIRE(max_chunks >= 1 && max_chunks <= DEC_MAXC, "attention_decode: max_chunks %d outside 1..%d", max_chunks,
+               DEC_MAXC);
+    ZI_REQUIRE(ldq >= (int64_t)nh * d && ldo >= (int64_t)nh * d && ldq % 8 == 0 && ldo % 4 == 0,
+               "attention_decode: bad row stride");
+    ZI_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 && ((uintptr_t)kcache % 16) == 0 &&
+                   ((uintptr_t)vcache % 16) == 0,
+               "attention_decode: q, out and the caches must be aligned to 16 bytes");
+    ZI_REQUIRE(nkv <= 65535 && nh <= 65535, "attention_decode: too many heads");
     if (n_idx == 0) return 0;
-    ZI_REQUIRE(max_splits == 1 || workspace_floats >= zi_attention_decode_workspace(n_idx, nh, d),
-               "attention_decode: workspace of %lld floats is too small", (long long)workspace_floats);
+    ZI_REQUIRE(max_chunks == 1 || (workspace && workspace_floats >= zi_attention_decode_workspace(n_idx, nh, d) &&
+                                   ((uintptr_t)workspace % 16) == 0),
+               "attention_decode: workspace of %lld floats is too small or not aligned", (long long)workspace_floats);
     float* po = workspace;
-    float* pml = workspace ? workspace + (int64_t)n_idx * nh * DEC_MAXS * d : nullptr;
-    const dim3 grid(n_idx, nkv, max_splits);
-    int rc = 0;
+    float* pml = workspace ? workspace + (int64_t)n_idx * nh * DEC_MAXC * d : nullptr;
+    const dim3 grid(n_idx, nkv, max_chunks);
     const int G = nh / nkv;
-#define ZI_DEC_D(DD)                                                                                               \
-    rc = launch_decode<DD>(G, grid, stream, (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq,                   \
-                           (const zi_bf16*)kcache, (const zi_bf16*)vcache, tok_index, tok_seq, tok_pos,            \
-                           block_tables, max_pages, num_pages, nh, nkv, page_size, window, scale, max_splits);     \
-    if (!rc && max_splits > 1)                                                                                     \
-        attention_decode_merge_kernel<DD><<<dim3(n_idx, nh), ZI_WAVE, 0, stream>>>((zi_bf16*)out, ldo, po, pml,    \
-                                                                                   tok_index, tok_pos, nh, window,  \
-                                                                                   max_splits);
-    if (d == 64) { ZI_DEC_D(64) } else if (d == 128) { ZI_DEC_D(128) } else { ZI_DEC_D(256) }
-#undef ZI_DEC_D
-    if (rc) return rc;
+#define ZI_DEC(DD)                                                                                                   \
+    attention_decode_kernel<DD><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                            \
+        (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,         \
+        tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,       \
+        max_chunks)
+    switch (d) {
+        case 16: ZI_DEC(16); break;
+        case 32: ZI_DEC(32); break;
+        case 48: ZI_DEC(48); break;
+        case 64: ZI_DEC(64); break;
+        case 80: ZI_DEC(80); break;
+        case 96: ZI_DEC(96); break;
+        case 112: ZI_DEC(112); break;
+        default: ZI_DEC(128); break;
+    }
+#undef ZI_DEC
+    if (max_chunks > 1)
+        attention_decode_merge_kernel<<<dim3(n_idx, nh), ZI_WAVE, 0, stream>>>((zi_bf16*)out, ldo, po, pml, tok_index,
+                                                                              tok_pos, nh, d, window, max_chunks);
     return zi_check_launch("attention_decode");
 }

@@ -5,14 +5,14 @@ then launches on torch's current stream.  The op-level names follow the
 reference's Python module (reference: python/bindings/zedinfer_ops.cpp:257-291:
 add, argmax, embedding, linear, rms_norm, rope, swiglu).
 """
-from .functional import (add, add_rms_norm, argmax, attention, attention_decode, attention_decode_supported, attention_prefill,
+from .functional import (add, add_rms_norm, argmax, attention, attention_decode, attention_decode_supported, attention_decode_workspace, attention_prefill,
                          attention_prefill_supported, embedding, gather_rows, has_gpu,
                          linear, rms_norm, rope, rope_kv_store, rope_inv_freq, sample, swiglu,
                          device_synchronize)
 from ._lib import KernelLibraryError, library_path, load
 
 __all__ = [
-    "add", "add_rms_norm", "argmax", "attention", "attention_decode", "attention_decode_supported", "attention_prefill",
+    "add", "add_rms_norm", "argmax", "attention", "attention_decode", "attention_decode_supported", "attention_decode_workspace", "attention_prefill",
     "attention_prefill_supported", "embedding", "gather_rows", "has_gpu", "linear",
     "rms_norm", "rope", "rope_kv_store", "rope_inv_freq", "sample", "swiglu", "device_synchronize",
     "KernelLibraryError", "library_path", "load",

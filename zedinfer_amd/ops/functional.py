@@ -291,8 +291,7 @@ def attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_s
     return out
 
 
-DECODE_MAX_SPLITS = 64
-DECODE_SPLIT_KEYS = 64
+DECODE_MAX_CHUNKS = 64
 
 
 def attention_decode_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, page_size: int) -> bool:
@@ -301,30 +300,34 @@ def attention_decode_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, pa
     return bool(_lib.load().zi_attention_decode_supported(_CODES[dtype], nh, nkv, d, page_size))
 
 
+def attention_decode_workspace(tokens: int, nh: int, d: int) -> int:
+    """Floats of workspace for the chunk partials of ``tokens`` tokens."""
+    return tokens * nh * DECODE_MAX_CHUNKS * (d + 2)
+
+
 def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
                      tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                      max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
                      tok_index: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None
                      ) -> torch.Tensor:
-    """The same attention for single query tokens, split over the keys (bfloat16, head_dim
-    64/128/256, group size <= 8, page size a multiple of 8).  ``max_keys`` is an upper bound of
-    the keys any listed token sees (its position + 1, or the window), known on the host."""
+    """The same attention for single query tokens, split over the keys, on the matrix cores
+    (bfloat16, head_dim a multiple of 16 up to 128, group size <= 16, page size a multiple of 8).
+    ``max_keys`` is an upper bound of the keys any listed token sees (its position + 1), known on
+    the host; it only sizes the launch."""
     out, n, count, ldq, ldo, pages, ps = _attention_args("attention_decode", q, kcache, vcache, tok_seq, tok_pos,
                                                          block_tables, nh, nkv, d, tok_index, out)
     if window > 0:
         max_keys = min(max_keys, window)
-    # a token's key range is widened down to a multiple of 8 and cut into splits of 64 keys (more
-    # beyond 4096 keys, never more than 64 splits); this bound only sizes the launch
-    max_splits = max(1, min(DECODE_MAX_SPLITS, -(-(max_keys + 7) // DECODE_SPLIT_KEYS)))
-    need = count * nh * DECODE_MAX_SPLITS * (d + 2)
-    if max_splits > 1:
+    max_chunks = int(_lib.load().zi_attention_decode_chunks(int(max_keys)))
+    need = attention_decode_workspace(count, nh, d)
+    if max_chunks > 1:
         if workspace is None:
             workspace = torch.empty((need,), dtype=torch.float32, device=q.device)
         if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
             raise ValueError(f"attention_decode: workspace must be a contiguous float32 buffer of {need} entries")
     _lib.call("zi_attention_decode", _p(out), _p(q), _code(q, "attention_decode"), count, ldq, ldo, _p(kcache),
               _p(vcache), _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages,
-              nh, nkv, d, ps, int(window), float(scale), max_splits, _p(workspace),
+              nh, nkv, d, ps, int(window), float(scale), max_chunks, _p(workspace),
               workspace.numel() if workspace is not None else 0, _stream())
     return out
 

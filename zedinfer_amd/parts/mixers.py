@@ -74,8 +74,8 @@ class Attention(Mixer):
         n_long = batch.num_long
         if batch.num_short:
             if ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
-                ws = self.rt.buffer("attn_split", (batch.num_short * self.nh * ops.functional.DECODE_MAX_SPLITS
-                                                   * (self.d + 2),), torch.float32)
+                ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(batch.num_short, self.nh, self.d),),
+                                    torch.float32)
                 ops.attention_decode(q, *args, batch.max_short_keys, self.window, out=att,
                                      tok_index=batch.short_idx, workspace=ws)
             else:
