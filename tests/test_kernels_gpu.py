@@ -437,3 +437,86 @@ def test_attention_prefill_refuses_other_shapes(ops):
     assert not ops.attention_prefill_supported(torch.bfloat16, 12, 2, 40, 16)
     assert not ops.attention_prefill_supported(torch.bfloat16, 12, 2, 128, 24)
     assert not ops.attention_prefill_supported(torch.bfloat16, 12, 5, 128, 16)
+
+
+# ---- the few-rows product's partial sums and the kernels that consume them ------------------------
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 1536), (8, 1536, 8960), (16, 17920, 1536), (17, 1536, 1536),
+                                   (64, 2048, 1536), (5, 176, 64), (33, 1000, 96), (3, 48, 520)])
+def test_linear_sums(ops, M, N, K):
+    bf = torch.bfloat16
+    x, w = rnd(M, K, dtype=bf, seed=1), rnd(N, K, dtype=bf, scale=0.05, seed=2)
+    b = rnd(N, dtype=bf, seed=3)
+    sums = ops.linear_sums(x, w)
+    assert sums.shape == (ops.linear_splits(N, K), M, N) and sums.dtype == torch.float32
+    ref = x.float() @ w.float().t()
+    torch.testing.assert_close(sums.sum(0), ref, atol=2e-3, rtol=2e-3)
+    # the consumer-side sum is what linear() itself gives, bit for bit
+    assert torch.equal(ops.reduce_sums(sums, b), ops.linear(x, w, b))
+    # a row's sums do not depend on the rows that ride along
+    if M > 1:
+        alone = ops.linear_sums(x[M - 1:M].contiguous(), w)
+        assert torch.equal(alone[:, 0], sums[:, M - 1])
+
+
+@pytest.mark.parametrize("M,I,K", [(1, 8960, 1536), (8, 8960, 1536), (40, 176, 64), (16, 256, 96), (2, 208, 80)])
+def test_linear_swiglu(ops, M, I, K):
+    from zedinfer_amd.parts.feed_forward import interleave_rows
+    bf = torch.bfloat16
+    x = rnd(M, K, dtype=bf, seed=1)
+    g, u = rnd(I, K, dtype=bf, scale=0.08, seed=2), rnd(I, K, dtype=bf, scale=0.08, seed=3)
+    w = interleave_rows(g, u, 8)
+    assert torch.equal(w[:8], g[:8]) and torch.equal(w[8:16], u[:8]) and torch.equal(w[16:24], g[8:16])
+    gf, uf = x.float() @ g.float().t(), x.float() @ u.float().t()
+    ref = uf * torch.nn.functional.silu(gf)
+    if ops.linear_swiglu_supported(x, w):
+        out = ops.linear_swiglu(x, w)
+        torch.testing.assert_close(out.float(), ref, atol=2e-2, rtol=2e-2)
+    else:
+        assert ops.linear_splits(2 * I, K) > 1
+    # the same through partial sums and the SwiGLU kernel, and through the interleaved 2-D form
+    sums = ops.linear_sums(x, w)
+    out2 = ops.swiglu(sums, interleave=8, out_dtype=bf)
+    torch.testing.assert_close(out2.float(), ref, atol=2e-2, rtol=2e-2)
+    gu = ops.linear(x, w)
+    out3 = ops.swiglu(gu, interleave=8)
+    torch.testing.assert_close(out3.float(), ref, atol=3e-2, rtol=3e-2)
+
+
+def test_add_rms_norm_from_sums(ops):
+    n, H, S = 9, 200, 3
+    resid = rnd(n, H, seed=1)
+    sums = rnd(S, n, H, seed=2)
+    w = (1 + rnd(H, seed=3) * 0.1).to(torch.bfloat16)
+    total = resid + sums[0] + sums[1] + sums[2]
+    out = ops.add_rms_norm(resid, sums, w, 1e-5, out_dtype=torch.bfloat16)
+    torch.testing.assert_close(resid, total, atol=1e-6, rtol=1e-6)
+    ref = w.float() * total * torch.rsqrt((total * total).mean(-1, keepdim=True) + 1e-5)
+    torch.testing.assert_close(out.float(), ref, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_rope_kv_store_sums(ops, dtype, with_bias):
+    n, nh, nkv, d, ps, pages, theta, S = 7, 6, 2, 48, 8, 10, 5e4, 3
+    width = (nh + 2 * nkv) * d
+    sums = rnd(S, n, width, seed=1)
+    bias = rnd(width, seed=2).to(dtype) if with_bias else None
+    total = sums.sum(0) + (bias.float() if with_bias else 0)
+    q, k, v = total[:, :nh * d], total[:, nh * d:(nh + nkv) * d], total[:, (nh + nkv) * d:]
+    pos = torch.arange(100, 100 + n, dtype=torch.int32, device="cuda")
+    slots = torch.randperm(pages * ps)[:n].to(torch.int32).cuda()
+    kc = torch.zeros(pages, nkv, ps, d, dtype=dtype, device="cuda")
+    vc = torch.zeros(pages, nkv, d, ps, dtype=dtype, device="cuda")
+    q_out = torch.empty(n, nh * d, dtype=dtype, device="cuda")
+    ops.rope_kv_store_sums(sums, bias, q_out, pos, slots, ops.rope_inv_freq(d, theta, "cuda"), kc, vc, nh, nkv, d)
+    q_ref = torch_rope(q.reshape(n, nh, d), pos, theta)
+    k_ref = torch_rope(k.reshape(n, nkv, d), pos, theta)
+    torch.testing.assert_close(q_out.float().reshape(n, nh, d), q_ref, **tol(dtype, 5e-4, 3e-2))
+    for t in range(n):
+        p, o = int(slots[t]) // ps, int(slots[t]) % ps
+        torch.testing.assert_close(kc[p, :, o].float(), k_ref[t], **tol(dtype, 5e-4, 3e-2))
+        torch.testing.assert_close(vc[p, :, :, o].float(), v[t].reshape(nkv, d), **tol(dtype, 1e-6, 2e-2))
+    # queries alone (a layer that reads another layer's cache)
+    q2 = torch.empty_like(q_out)
+    ops.rope_kv_store_sums(sums, bias, q2, pos, None, ops.rope_inv_freq(d, theta, "cuda"), None, None, nh, nkv, d)
+    assert torch.equal(q2, q_out)

@@ -28,6 +28,11 @@ def assert_close_to_scale(got, ref, dtype, f32=2e-5, bf16=0.02):
     assert worst <= (f32 if dtype == torch.float32 else bf16) * max(scale, 1e-6), (worst, scale)
 
 
+def as_rows(t):
+    """A part may return its addition as a stack [S, n, H] of float32 partial sums."""
+    return t.float().sum(0) if t.dim() == 3 else t.float()
+
+
 def rnd(*shape, seed=0, scale=1.0):
     g = torch.Generator().manual_seed(seed + 7 * len(shape) + sum(shape))
     return torch.randn(*shape, generator=g) * scale
@@ -83,7 +88,7 @@ def test_swiglu_part(dtype, n):
     x = rnd(n, H, seed=4)
     part = FEED_FORWARDS.get("swiglu")(spec("swiglu", {"hidden_size": H, "intermediate_size": I}),
                                        {k: v.to(dtype).cuda() for k, v in w.items()}, runtime(dtype))
-    got = part.forward(x.to(dtype).cuda()).float().cpu()
+    got = as_rows(part.forward(x.to(dtype).cuda())).cpu()
     wf = {k: v.to(dtype).float() for k, v in w.items()}
     xf = x.to(dtype).float()
     ref = plain.linear(plain.swiglu(plain.linear(xf, wf["gate"]), plain.linear(xf, wf["up"])), wf["down"])
@@ -168,7 +173,7 @@ def test_attention_part_in_portions(dtype, nh, nkv, d, window, bias):
     got, i = [], 0
     for n in [23, 2, 1, 9, 1, 1, 3, 20, 1]:
         batch = one_sequence_batch(cache, seq, n)
-        got.append(mixer.forward(x[i:i + n].cuda(), batch, mem).float().cpu())
+        got.append(as_rows(mixer.forward(x[i:i + n].cuda(), batch, mem)).cpu())
         cache.commit(seq, seq.length + n)
         i += n
     assert i == T

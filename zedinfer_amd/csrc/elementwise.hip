@@ -66,24 +66,38 @@ extern "C" int zi_add(void* c, int c_dt, const void* a, int a_dt, const void* b,
 }
 
 // out[i,j] = up[i,j] * gate[i,j] / (1 + exp(-gate[i,j]))
-// (reference: src/backend/ops/swiglu/cpu/swiglu_cpu.cpp:9-23).  gate and up are
-// read with their own row strides, so both halves of one fused [N, 2I] product can be passed.
-template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gate, const T* __restrict__ up,
-                              int inter, int64_t ld_gate, int64_t ld_up) {
+// (reference: src/backend/ops/swiglu/cpu/swiglu_cpu.cpp:9-23).  gate and up are read with their
+// own row strides, so both halves of one fused [n, 2I] product can be passed.  With
+// `interleave` = B > 0 they are columns of ONE matrix in blocks of B: gate column j sits at
+// (j / B) * 2B + j % B of `gate`, up column j another B further (`up` is not used).  The input
+// may come as `splits` partial sums (split s at + s * split_stride), added in rising order.
+template <typename TI, typename TO>
+__global__ void swiglu_kernel(TO* __restrict__ out, const TI* __restrict__ gate, const TI* __restrict__ up,
+                              int inter, int64_t ld_gate, int64_t ld_up, int interleave, int splits,
+                              int64_t split_stride) {
     const int64_t row = blockIdx.y;
-    const T* g = gate + row * ld_gate;
-    const T* u = up + row * ld_up;
-    T* o = out + row * (int64_t)inter;
+    const TI* g = gate + row * ld_gate;
+    const TI* u = interleave > 0 ? g + interleave : up + row * ld_up;
+    TO* o = out + row * (int64_t)inter;
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < inter; j += gridDim.x * blockDim.x) {
-        const float gv = zi_load(g + j), uv = zi_load(u + j);
+        const int64_t c = interleave > 0 ? (int64_t)(j / interleave) * 2 * interleave + j % interleave : j;
+        float gv = zi_load(g + c), uv = zi_load(u + c);
+        for (int s = 1; s < splits; ++s) {
+            gv += zi_load(g + s * split_stride + c);
+            uv += zi_load(u + s * split_stride + c);
+        }
         zi_store(o + j, uv * (gv / (1.f + expf(-gv))));
     }
 }
 
-extern "C" int zi_swiglu(void* out, const void* gate, const void* up, int dt, int n, int inter, int64_t ld_gate,
-                         int64_t ld_up, hipStream_t stream) {
-    ZI_REQUIRE(n >= 0 && inter > 0 && ld_gate >= inter && ld_up >= inter, "swiglu: bad sizes n=%d inter=%d", n, inter);
+extern "C" int zi_swiglu(void* out, int out_dt, const void* gate, const void* up, int dt, int n, int inter,
+                         int64_t ld_gate, int64_t ld_up, int interleave, int splits, int64_t split_stride,
+                         hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && inter > 0 && ld_gate >= inter, "swiglu: bad sizes n=%d inter=%d", n, inter);
+    ZI_REQUIRE(interleave >= 0 && (interleave == 0 ? (up != nullptr && ld_up >= inter)
+                                                   : (inter % interleave == 0 && ld_gate >= 2 * (int64_t)inter)),
+               "swiglu: bad layout (interleave %d)", interleave);
+    ZI_REQUIRE(splits >= 1, "swiglu: bad number of partial sums");
     if (n == 0) return 0;
     ZI_REQUIRE(n <= 65535 * 1024, "swiglu: too many rows");
     int bx = (inter + 255) / 256;
@@ -91,11 +105,12 @@ extern "C" int zi_swiglu(void* out, const void* gate, const void* up, int dt, in
     // gridDim.y is limited to 65535: fold larger batches.
     for (int r0 = 0; r0 < n; r0 += 65535) {
         const int rows = n - r0 < 65535 ? n - r0 : 65535;
-        ZI_DISPATCH_DTYPE(dt, T, {
-            swiglu_kernel<T><<<dim3(bx, rows), 256, 0, stream>>>(
-                (T*)out + (int64_t)r0 * inter, (const T*)gate + (int64_t)r0 * ld_gate,
-                (const T*)up + (int64_t)r0 * ld_up, inter, ld_gate, ld_up);
-        });
+        ZI_DISPATCH_DTYPE(dt, TI, ZI_DISPATCH_DTYPE(out_dt, TO, {
+            swiglu_kernel<TI, TO><<<dim3(bx, rows), 256, 0, stream>>>(
+                (TO*)out + (int64_t)r0 * inter, (const TI*)gate + (int64_t)r0 * ld_gate,
+                up ? (const TI*)up + (int64_t)r0 * ld_up : nullptr, inter, ld_gate, ld_up, interleave, splits,
+                split_stride);
+        }));
     }
     return zi_check_launch("swiglu");
 }

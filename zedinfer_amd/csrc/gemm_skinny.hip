@@ -2,13 +2,22 @@
 // matrix product, bound by the one pass over the weights.
 //
 // bfloat16 x and w, float32 accumulation on the matrix cores
-// (v_mfma_f32_16x16x32_bf16), output bfloat16 or float32.  A workgroup of four
-// wavefronts owns a tile of 16 weight rows; the wavefronts take the k-blocks of 128
-// in turn and their sums are added through LDS in a fixed order.  Small weight
-// matrices are additionally cut along k over several workgroups (gridDim.y) so
-// that enough loads are in flight to fill HBM; those write float32 partials that a
-// second kernel adds, again in a fixed order.  The cut depends on N and K only, so
-// a row's result does not depend on how many rows ride along.
+// (v_mfma_f32_16x16x32_bf16).  A workgroup of four wavefronts owns tiles of 16 weight
+// rows and a range of k: each wavefront takes KPW consecutive k-blocks of 128, the
+// four sums are added through LDS in the order of the wavefronts.  When the weight
+// matrix is small the k dimension is additionally cut over several workgroups
+// (gridDim.y "splits") so that enough loads are in flight to fill HBM; those write
+// float32 partial sums [split][M][N] that the consumer adds in rising order (the next
+// norm, the rotary kernel, the SwiGLU kernel, or the reduce kernel here).  The cut
+// depends on N and K only, so a row's result does not depend on how many rows ride
+// along.  With up to 16 rows of x a workgroup keeps its slice of x in registers and
+// walks several weight tiles, prefetching the next tile's rows while the matrix
+// cores work on the current one.
+//
+// Epilogues: plain (bias, bfloat16 or float32 out), partial sums, and SwiGLU: when the
+// weight rows are gate and up rows interleaved in blocks of 8 (tile = 8 gate rows, then
+// the 8 up rows of the same columns), the tile's lanes exchange halves and write
+// act = up * gate / (1 + exp(-gate)) (reference: src/backend/ops/swiglu/cpu/swiglu_cpu.cpp:9-23).
 //
 // Operand layout.  For one MFMA the A operand is a 16 x 32 tile of w (lane l: row
 // l%16, eight consecutive k) and the B operand the matching 32 x 16 tile of x^T
@@ -24,6 +33,13 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 #define SK_ROWS 16
 #define SK_KB 128
 #define SK_WAVES 4
+#define SK_MAX_KPW 4
+#define SK_TARGET_WGS 512
+#define SK_MAX_TPW 16
+
+#define SK_MODE_PLAIN 0
+#define SK_MODE_PARTIAL 1
+#define SK_MODE_SWIGLU 2
 
 __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4& v) {
     union { uint4 u; bf16x8_t b; } c;
@@ -31,81 +47,128 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4& v) {
     return c.b;
 }
 
-template <int MT>
+// The 64 bytes of row `row` this lane owns in k-block `kb` (zeros past K; K % 8 == 0).
+__device__ __forceinline__ void sk_load_row(uint4 (&dst)[4], const zi_bf16* row, int kb, int j, int K) {
+    const int k0 = kb * SK_KB + j * 32;
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+        dst[c] = (k0 + c * 8 < K) ? *reinterpret_cast<const uint4*>(row + k0 + c * 8) : make_uint4(0, 0, 0, 0);
+}
+
+template <int MT, int KPW>
 __global__ void __launch_bounds__(SK_WAVES* ZI_WAVE)
-gemm_skinny_kernel(void* __restrict__ out, int out_f32, float* __restrict__ partial,
-                   const zi_bf16* __restrict__ x, const zi_bf16* __restrict__ w, const zi_bf16* __restrict__ bias,
-                   int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int kb_per_split) {
-    __shared__ f32x4_t red[SK_WAVES][MT][ZI_WAVE];
+gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* x, const zi_bf16* __restrict__ w,
+                   const zi_bf16* __restrict__ bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
+                   int tiles_per_wg) {
+    constexpr bool XRES = (MT == 1);   // the slice of x stays in registers over the workgroup's tiles
+    __shared__ f32x4_t red[2][SK_WAVES][MT][ZI_WAVE];
     const int lane = threadIdx.x & (ZI_WAVE - 1), wave = threadIdx.x / ZI_WAVE;
     const int r = lane & 15, j = lane >> 4;
-    const int n0 = blockIdx.x * SK_ROWS;
-    const int nrow = (n0 + r < N) ? n0 + r : N - 1;
-    const zi_bf16* wrow = w + (int64_t)nrow * ldw + j * 32;
+    const int split = blockIdx.y;
+    const int kb_total = (K + SK_KB - 1) / SK_KB;
+    const int kb0 = split * (SK_WAVES * KPW) + wave * KPW;
+    const int n_tiles = (N + SK_ROWS - 1) / SK_ROWS;
+    const int tile_lo = blockIdx.x * tiles_per_wg;
+    const int tile_hi = (tile_lo + tiles_per_wg < n_tiles) ? tile_lo + tiles_per_wg : n_tiles;
+
     const zi_bf16* xrow[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         const int m = t * 16 + r;
-        xrow[t] = x + (int64_t)(m < M ? m : M - 1) * ldx + j * 32;
+        xrow[t] = x + (int64_t)(m < M ? m : M - 1) * ldx;
     }
-    f32x4_t acc[MT];
+    uint4 xr[XRES ? KPW : 1][4];
+    if (XRES) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-    const int kb_total = (K + SK_KB - 1) / SK_KB;
-    const int kb_lo = blockIdx.y * kb_per_split;
-    const int kb_hi = (kb_lo + kb_per_split < kb_total) ? kb_lo + kb_per_split : kb_total;
-    const uint4 zero = make_uint4(0, 0, 0, 0);
-    for (int kb = kb_lo + wave; kb < kb_hi; kb += SK_WAVES) {
-        const int k0 = kb * SK_KB;
-        uint4 a[4], b[MT][4];
-        if (k0 + SK_KB <= K) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const uint4*>(wrow + k0 + i * 8);
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) b[t][i] = *reinterpret_cast<const uint4*>(xrow[t] + k0 + i * 8);
-        } else {   // the last, partial k-block (K is a multiple of 8)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const bool in = k0 + j * 32 + i * 8 < K;
-                a[i] = in ? *reinterpret_cast<const uint4*>(wrow + k0 + i * 8) : zero;
-#pragma unroll
-                for (int t = 0; t < MT; ++t) b[t][i] = in ? *reinterpret_cast<const uint4*>(xrow[t] + k0 + i * 8) : zero;
-            }
+        for (int i = 0; i < KPW; ++i) {
+            if (kb0 + i < kb_total) sk_load_row(xr[i], xrow[0], kb0 + i, j, K);
+            else xr[i][0] = xr[i][1] = xr[i][2] = xr[i][3] = make_uint4(0, 0, 0, 0);
         }
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int t = 0; t < MT; ++t)
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[i]), as_bf16x8(b[t][i]), acc[t], 0, 0, 0);
     }
+    uint4 a_next[KPW][4];
+    {
+        const int nrow = (tile_lo * SK_ROWS + r < N) ? tile_lo * SK_ROWS + r : N - 1;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
-    __syncthreads();
-    // wave t of the workgroup finishes row tile t of x: C[n = (lane/16)*4 + e][m = lane%16]
-    for (int t = wave; t < MT; t += SK_WAVES) {
-        f32x4_t s = red[0][t][lane];
-#pragma unroll
-        for (int q = 1; q < SK_WAVES; ++q) {
-            const f32x4_t o = red[q][t][lane];
-            s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
+        for (int i = 0; i < KPW; ++i) {
+            if (kb0 + i < kb_total) sk_load_row(a_next[i], w + (int64_t)nrow * ldw, kb0 + i, j, K);
+            else a_next[i][0] = a_next[i][1] = a_next[i][2] = a_next[i][3] = make_uint4(0, 0, 0, 0);
         }
-        const int m = t * 16 + r;
-        if (m >= M) continue;
+    }
+    int buf = 0;
+    for (int tile = tile_lo; tile < tile_hi; ++tile) {
+        uint4 a[KPW][4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int n = n0 + j * 4 + e;
-            if (n >= N) continue;
-            if (partial) {
-                partial[((int64_t)blockIdx.y * M + m) * N + n] = s[e];
+        for (int i = 0; i < KPW; ++i)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) a[i][c] = a_next[i][c];
+        if (tile + 1 < tile_hi) {
+            const int nrow = ((tile + 1) * SK_ROWS + r < N) ? (tile + 1) * SK_ROWS + r : N - 1;
+#pragma unroll
+            for (int i = 0; i < KPW; ++i)
+                if (kb0 + i < kb_total) sk_load_row(a_next[i], w + (int64_t)nrow * ldw, kb0 + i, j, K);
+        }
+        f32x4_t acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < KPW; ++i) {
+            if (kb0 + i >= kb_total) break;
+            if (XRES) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[i][c]), as_bf16x8(xr[i][c]), acc[0], 0, 0, 0);
             } else {
-                const float v = s[e] + (bias ? zi_load(bias + n) : 0.f);
-                if (out_f32) ((float*)out)[(int64_t)m * ldo + n] = v;
-                else zi_store((zi_bf16*)out + (int64_t)m * ldo + n, v);
+                uint4 b[MT][4];
+#pragma unroll
+                for (int t = 0; t < MT; ++t) sk_load_row(b[t], xrow[t], kb0 + i, j, K);
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+#pragma unroll
+                    for (int t = 0; t < MT; ++t)
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[i][c]), as_bf16x8(b[t][c]), acc[t], 0, 0, 0);
             }
         }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) red[buf][wave][t][lane] = acc[t];
+        __syncthreads();
+        // wave t of the workgroup finishes row tile t of x: C[n = (lane/16)*4 + e][m = lane%16]
+        const int n0 = tile * SK_ROWS;
+        for (int t = wave; t < MT; t += SK_WAVES) {
+            f32x4_t s = red[buf][0][t][lane];
+#pragma unroll
+            for (int q = 1; q < SK_WAVES; ++q) {
+                const f32x4_t o = red[buf][q][t][lane];
+                s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
+            }
+            const int m = t * 16 + r;
+            if (mode == SK_MODE_SWIGLU) {
+                // lanes j = 0,1 hold gate rows j*4 + e, lanes j = 2,3 the up rows of the same columns
+                f32x4_t up;
+                up[0] = __shfl_xor(s[0], 32, ZI_WAVE); up[1] = __shfl_xor(s[1], 32, ZI_WAVE);
+                up[2] = __shfl_xor(s[2], 32, ZI_WAVE); up[3] = __shfl_xor(s[3], 32, ZI_WAVE);
+                if (j >= 2 || m >= M) continue;
+                const int col = tile * 8 + j * 4;     // N / 2 columns of output
+                zi_bf16* dst = (zi_bf16*)out + (int64_t)m * ldo + col;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (col + e < N / 2) zi_store(dst + e, up[e] * (s[e] / (1.f + expf(-s[e]))));
+                continue;
+            }
+            if (m >= M) continue;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = n0 + j * 4 + e;
+                if (n >= N) continue;
+                if (mode == SK_MODE_PARTIAL) {
+                    ((float*)out)[((int64_t)split * M + m) * N + n] = s[e];
+                } else {
+                    const float v = s[e] + (bias ? zi_load(bias + n) : 0.f);
+                    if (out_f32) ((float*)out)[(int64_t)m * ldo + n] = v;
+                    else zi_store((zi_bf16*)out + (int64_t)m * ldo + n, v);
+                }
+            }
+        }
+        buf ^= 1;
     }
 }
 
@@ -122,65 +185,125 @@ __global__ void gemm_skinny_reduce_kernel(void* __restrict__ out, int out_f32, c
     else zi_store((zi_bf16*)out + (int64_t)m * ldo + n, s);
 }
 
-// How the k dimension is cut for a weight matrix [N, K]: (splits, k-blocks per split).
-static void skinny_plan(int N, int K, int* splits, int* kb_per_split) {
+// How the product with a weight matrix [N, K] is cut: k-blocks per wavefront, splits of k over
+// workgroups, and weight tiles per workgroup.  A function of N and K alone.
+static void skinny_plan(int N, int K, int* kpw, int* splits, int* tiles_per_wg) {
     const int tiles = (N + SK_ROWS - 1) / SK_ROWS;
     const int kb_total = (K + SK_KB - 1) / SK_KB;
-    int s = (2048 + tiles * SK_WAVES - 1) / (tiles * SK_WAVES);      // aim at 2048 wavefronts
-    const int most = kb_total / SK_WAVES > 0 ? kb_total / SK_WAVES : 1;   // keep every wavefront busy
-    if (s > most) s = most;
-    if (s < 1) s = 1;
-    int per = (kb_total + s - 1) / s;
-    s = (kb_total + per - 1) / per;
-    *splits = s;
-    *kb_per_split = per;
+    int best = 1;
+    for (int c = SK_MAX_KPW; c >= 1; --c) {
+        const int s = (kb_total + SK_WAVES * c - 1) / (SK_WAVES * c);
+        if ((int64_t)s * tiles >= SK_TARGET_WGS) { best = c; break; }
+    }
+    while (best > 1 && (kb_total + SK_WAVES * (best - 1) - 1) / (SK_WAVES * (best - 1)) ==
+                           (kb_total + SK_WAVES * best - 1) / (SK_WAVES * best))
+        --best;   // fewer k-blocks a wavefront for the same number of splits: more wavefronts busy
+    *kpw = best;
+    *splits = (kb_total + SK_WAVES * best - 1) / (SK_WAVES * best);
+    int64_t tpw = (int64_t)(*splits) * tiles / SK_TARGET_WGS;
+    if (tpw < 1) tpw = 1;
+    if (tpw > SK_MAX_TPW) tpw = SK_MAX_TPW;
+    *tiles_per_wg = (int)tpw;
 }
 
 extern "C" int zi_gemm_skinny_supported(int M, int N, int K, int64_t ldx, int64_t ldw) {
     return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
 
+// Splits of k for a weight matrix [N, K]: the leading dimension of the partial sums.
+extern "C" int zi_gemm_skinny_splits(int N, int K) {
+    int kpw, s, tpw;
+    skinny_plan(N, K, &kpw, &s, &tpw);
+    return s;
+}
+
 // Floats of workspace for the split partials (0 when the product is not split).
 extern "C" int64_t zi_gemm_skinny_workspace(int M, int N, int K) {
-    int s, per;
-    skinny_plan(N, K, &s, &per);
+    const int s = zi_gemm_skinny_splits(N, K);
     return s > 1 ? (int64_t)s * M * N : 0;
 }
 
-extern "C" int zi_gemm_skinny(void* out, int out_dt, const void* x, const void* w, const void* bias, int M, int N,
-                              int K, int64_t ldx, int64_t ldw, int64_t ldo, float* workspace,
-                              int64_t workspace_floats, hipStream_t stream) {
-    ZI_REQUIRE(zi_gemm_skinny_supported(M, N, K, ldx, ldw),
-               "gemm_skinny: unsupported sizes M=%d N=%d K=%d (1 <= M <= 64, K and row strides multiples of 8)", M, N, K);
-    ZI_REQUIRE(out_dt == ZI_F32 || out_dt == ZI_BF16, "gemm_skinny: unknown output dtype %d", out_dt);
-    ZI_REQUIRE(ldx >= K && ldw >= K && ldo >= N, "gemm_skinny: leading dimension too small");
-    ZI_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny: x and w must be 16-byte aligned");
-    int splits, per;
-    skinny_plan(N, K, &splits, &per);
-    float* partial = nullptr;
-    if (splits > 1) {
-        ZI_REQUIRE(workspace && workspace_floats >= (int64_t)splits * M * N,
-                   "gemm_skinny: workspace of %lld floats is too small (%lld needed)", (long long)workspace_floats,
-                   (long long)splits * M * N);
-        partial = workspace;
-    }
-    const dim3 grid((N + SK_ROWS - 1) / SK_ROWS, splits);
-    const int mt = (M + 15) / 16;
-#define ZI_SK(MT)                                                                                                   \
-    gemm_skinny_kernel<MT><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(out, out_dt == ZI_F32, partial, (const zi_bf16*)x, \
-                                                                    (const zi_bf16*)w, (const zi_bf16*)bias, M, N, K, \
-                                                                    ldx, ldw, ldo, per)
-    switch (mt) {
+template <int MT>
+static void sk_launch(int kpw, dim3 grid, hipStream_t stream, void* out, int mode, int out_f32, const zi_bf16* x,
+                      const zi_bf16* w, const zi_bf16* bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
+                      int tpw) {
+#define ZI_SK(KPW)                                                                                                  \
+    gemm_skinny_kernel<MT, KPW><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, \
+                                                                         ldw, ldo, tpw)
+    switch (kpw) {
         case 1: ZI_SK(1); break;
         case 2: ZI_SK(2); break;
         case 3: ZI_SK(3); break;
         default: ZI_SK(4); break;
     }
 #undef ZI_SK
-    if (splits > 1) {
+}
+
+// mode 0: out[M,N] (+ bias), reduced through `workspace` when the product is split.
+// mode 1: out = float32 partial sums [splits][M][N] (no bias; splits from zi_gemm_skinny_splits).
+// mode 2: w holds gate and up rows interleaved in blocks of 8; out[M, N/2] (bfloat16) =
+//         up * silu(gate); only for products that are not split.
+extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, const void* w, const void* bias, int M,
+                              int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, float* workspace,
+                              int64_t workspace_floats, hipStream_t stream) {
+    ZI_REQUIRE(zi_gemm_skinny_supported(M, N, K, ldx, ldw),
+               "gemm_skinny: unsupported sizes M=%d N=%d K=%d (1 <= M <= 64, K and row strides multiples of 8)", M, N, K);
+    ZI_REQUIRE(out_dt == ZI_F32 || out_dt == ZI_BF16, "gemm_skinny: unknown output dtype %d", out_dt);
+    ZI_REQUIRE(mode >= 0 && mode <= 2, "gemm_skinny: unknown mode %d", mode);
+    ZI_REQUIRE(ldx >= K && ldw >= K, "gemm_skinny: leading dimension too small");
+    ZI_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny: x and w must be 16-byte aligned");
+    int kpw, splits, tpw;
+    skinny_plan(N, K, &kpw, &splits, &tpw);
+    const int tiles = (N + SK_ROWS - 1) / SK_ROWS;
+    const int mt = (M + 15) / 16;
+    if (mt > 1) tpw = 1;   // more than 16 rows of x do not stay in registers
+    const dim3 grid((tiles + tpw - 1) / tpw, splits);
+    void* dst = out;
+    int kmode = mode;
+    if (mode == SK_MODE_PLAIN) {
+        ZI_REQUIRE(ldo >= N, "gemm_skinny: leading dimension of out too small");
+        if (splits > 1) {
+            ZI_REQUIRE(workspace && workspace_floats >= (int64_t)splits * M * N,
+                       "gemm_skinny: workspace of %lld floats is too small (%lld needed)", (long long)workspace_floats,
+                       (long long)splits * M * N);
+            dst = workspace;
+            kmode = SK_MODE_PARTIAL;
+        }
+    } else if (mode == SK_MODE_PARTIAL) {
+        ZI_REQUIRE(out_dt == ZI_F32, "gemm_skinny: partial sums are float32");
+    } else {
+        ZI_REQUIRE(splits == 1, "gemm_skinny: the SwiGLU epilogue needs a product that is not split (N=%d K=%d has %d)",
+                   N, K, splits);
+        ZI_REQUIRE(N % 16 == 0 && out_dt == ZI_BF16 && ldo >= N / 2,
+                   "gemm_skinny: the SwiGLU epilogue needs N %% 16 == 0 and a bfloat16 out of N/2 columns");
+    }
+    const zi_bf16* b = kmode == SK_MODE_PLAIN ? (const zi_bf16*)bias : nullptr;
+    const int of32 = out_dt == ZI_F32;
+#define ZI_SKM(MT)                                                                                                  \
+    sk_launch<MT>(kpw, grid, stream, dst, kmode, of32, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo, tpw)
+    switch (mt) {
+        case 1: ZI_SKM(1); break;
+        case 2: ZI_SKM(2); break;
+        case 3: ZI_SKM(3); break;
+        default: ZI_SKM(4); break;
+    }
+#undef ZI_SKM
+    if (mode == SK_MODE_PLAIN && splits > 1) {
         const int64_t total = (int64_t)M * N;
-        gemm_skinny_reduce_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(out, out_dt == ZI_F32, partial,
+        gemm_skinny_reduce_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(out, of32, workspace,
                                                                                   (const zi_bf16*)bias, M, N, ldo, splits);
     }
     return zi_check_launch("gemm_skinny");
+}
+
+// out[m,n] = sum_s sums[s,m,n] + bias[n] for float32 sums [splits][M][N], added in rising order.
+extern "C" int zi_reduce_splits(void* out, int out_dt, const float* sums, const void* bias, int M, int N, int64_t ldo,
+                                int splits, hipStream_t stream) {
+    ZI_REQUIRE(M >= 0 && N > 0 && splits >= 1 && ldo >= N, "reduce_splits: bad sizes");
+    ZI_REQUIRE(out_dt == ZI_F32 || out_dt == ZI_BF16, "reduce_splits: unknown output dtype %d", out_dt);
+    if (M == 0) return 0;
+    const int64_t total = (int64_t)M * N;
+    gemm_skinny_reduce_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(out, out_dt == ZI_F32, sums,
+                                                                              (const zi_bf16*)bias, M, N, ldo, splits);
+    return zi_check_launch("reduce_splits");
 }

@@ -38,10 +38,12 @@ extern "C" int zi_rmsnorm(void* out, int out_dt, const void* x, int x_dt, const 
     return zi_check_launch("rmsnorm");
 }
 
-// resid (float32, in place) += delta;  out = norm(resid) * w.
+// resid (float32, in place) += delta;  out = norm(resid) * w.  delta may come as `splits` partial
+// sums (split s at delta + s * split_stride), which are added in rising order.
 template <typename TD, typename TW, typename TO>
 __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ resid, const TD* __restrict__ delta,
-                                   const TW* __restrict__ w, int H, float eps, float w_offset) {
+                                   int splits, int64_t split_stride, const TW* __restrict__ w, int H, float eps,
+                                   float w_offset) {
     __shared__ float red[16];
     const int64_t row = blockIdx.x;
     float* rr = resid + row * H;
@@ -49,7 +51,9 @@ __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ res
     TO* orow = out + row * H;
     float ss = 0.f;
     for (int j = threadIdx.x; j < H; j += blockDim.x) {
-        const float v = rr[j] + zi_load(dr + j);
+        float d = zi_load(dr + j);
+        for (int s = 1; s < splits; ++s) d += zi_load(dr + s * split_stride + j);
+        const float v = rr[j] + d;
         rr[j] = v;
         ss += v * v;
     }
@@ -59,14 +63,18 @@ __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ res
     for (int j = threadIdx.x; j < H; j += blockDim.x) zi_store(orow + j, (zi_load(w + j) + w_offset) * rr[j] * rstd);
 }
 
-extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* delta, int delta_dt, const void* w,
-                              int w_dt, int n, int hidden, float eps, int add_one, hipStream_t stream) {
+extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* delta, int delta_dt, int splits,
+                              int64_t split_stride, const void* w, int w_dt, int n, int hidden, float eps, int add_one,
+                              hipStream_t stream) {
     ZI_REQUIRE(n >= 0 && hidden > 0, "add_rmsnorm: bad sizes n=%d hidden=%d", n, hidden);
     ZI_REQUIRE(eps > 0.f, "add_rmsnorm: eps must be positive");
+    ZI_REQUIRE(splits >= 1 && (splits == 1 || split_stride >= (int64_t)n * hidden),
+               "add_rmsnorm: bad partial sums (splits %d, stride %lld)", splits, (long long)split_stride);
     if (n == 0) return 0;
     ZI_DISPATCH_DTYPE(delta_dt, TD, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
-        add_rmsnorm_kernel<TD, TW, TO><<<n, NORM_THREADS, 0, stream>>>((TO*)out, resid, (const TD*)delta, (const TW*)w,
-                                                                       hidden, eps, add_one ? 1.f : 0.f);
+        add_rmsnorm_kernel<TD, TW, TO><<<n, NORM_THREADS, 0, stream>>>((TO*)out, resid, (const TD*)delta, splits,
+                                                                       split_stride, (const TW*)w, hidden, eps,
+                                                                       add_one ? 1.f : 0.f);
     })));
     return zi_check_launch("add_rmsnorm");
 }

@@ -89,6 +89,96 @@ extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, i
     return zi_check_launch("rope_kv_store");
 }
 
+// The same for q, k, v that arrive as float32 partial sums of one fused projection: columns
+// [0, nh*d) of a row are q, the next nkv*d are k, the last nkv*d are v; split s of row t starts at
+// part + s * split_stride + t * ldp.  The splits are added in rising order, the bias is added, and
+// the row is rotated from float32: q goes to q_out (rounded once), k and v into the cache.
+template <typename T, typename TB>
+__global__ void rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __restrict__ part,
+                                           int splits, int64_t split_stride, int64_t ldp,
+                                           const TB* __restrict__ bias, const int32_t* __restrict__ pos,
+                                           const int32_t* __restrict__ slots, const float* __restrict__ inv_freq,
+                                           T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int d,
+                                           int rot, int page_size, int write_kv, int64_t cache_slots) {
+    extern __shared__ float sh[];  // cos[rot/2], sin[rot/2], then the summed row
+    const int64_t t = blockIdx.x;
+    const int half = rot / 2;
+    const int qd = nh * d, kvd = nkv * d;
+    const int width = qd + (write_kv ? 2 * kvd : 0);
+    float* cs = sh;
+    float* row = sh + rot;
+    const float p = (float)pos[t];
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float s, c;
+        sincosf(p * inv_freq[i], &s, &c);
+        cs[i] = c;
+        cs[half + i] = s;
+    }
+    const float* pr = part + t * ldp;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float v = pr[i];
+        for (int s = 1; s < splits; ++s) v += pr[s * split_stride + i];
+        if (bias) v += zi_load(bias + i);
+        row[i] = v;
+    }
+    __syncthreads();
+    T* qr = q_out + t * ldq;
+    for (int i = threadIdx.x; i < qd; i += blockDim.x) {
+        const int h = i / d, j = i % d;
+        const float* base = row + h * d;
+        float v;
+        if (j < half) v = base[j] * cs[j] - base[j + half] * cs[half + j];
+        else if (j < rot) v = base[j] * cs[j - half] + base[j - half] * cs[j];
+        else v = base[j];
+        zi_store(qr + i, v);
+    }
+    if (!write_kv) return;
+    const int slot = slots[t];
+    if (slot < 0 || slot >= cache_slots) return;  // the host checks the range; never write outside the pool
+    const int64_t page = slot / page_size, off = slot % page_size;
+    for (int i = threadIdx.x; i < kvd; i += blockDim.x) {
+        const int h = i / d, j = i % d;
+        const float* base = row + qd + h * d;
+        float kv;
+        if (j < half) kv = base[j] * cs[j] - base[j + half] * cs[half + j];
+        else if (j < rot) kv = base[j] * cs[j - half] + base[j - half] * cs[j];
+        else kv = base[j];
+        zi_store(kcache + ((page * nkv + h) * page_size + off) * d + j, kv);
+        zi_store(vcache + ((page * nkv + h) * d + j) * page_size + off, row[qd + kvd + i]);
+    }
+}
+
+extern "C" int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const float* part, int splits,
+                                      int64_t split_stride, int64_t ldp, const void* bias, int bias_dt, int n,
+                                      const int32_t* pos, const int32_t* slots, const float* inv_freq, void* kcache,
+                                      void* vcache, int64_t cache_slots, int nh, int nkv, int d, int rot,
+                                      int page_size, int write_kv, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && nh > 0 && nkv >= 0 && d > 0, "rope_kv_store_split: bad sizes");
+    ZI_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "rope_kv_store_split: rotary dims %d must be even and <= head_dim %d",
+               rot, d);
+    const int64_t width = (int64_t)nh * d + (write_kv ? 2 * (int64_t)nkv * d : 0);
+    ZI_REQUIRE(ldq >= (int64_t)nh * d && ldp >= width, "rope_kv_store_split: row stride too small");
+    ZI_REQUIRE(splits >= 1 && (splits == 1 || split_stride >= (int64_t)n * ldp),
+               "rope_kv_store_split: bad partial sums (splits %d, stride %lld)", splits, (long long)split_stride);
+    ZI_REQUIRE(rot == 0 || inv_freq, "rope_kv_store_split: no frequency table");
+    if (write_kv) {
+        ZI_REQUIRE(page_size > 0 && cache_slots > 0 && cache_slots % page_size == 0,
+                   "rope_kv_store_split: cache of %lld slots is not a whole number of pages of %d", (long long)cache_slots,
+                   page_size);
+        ZI_REQUIRE(kcache && vcache && slots, "rope_kv_store_split: null cache pointer");
+    }
+    const size_t lds = (size_t)(rot + width) * sizeof(float);
+    ZI_REQUIRE(lds <= 60 * 1024, "rope_kv_store_split: a row of %lld values does not fit in LDS", (long long)width);
+    if (n == 0) return 0;
+    if (!bias) bias_dt = ZI_F32;
+    ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(bias_dt, TB, {
+        rope_kv_store_split_kernel<T, TB><<<n, 256, lds, stream>>>(
+            (T*)q_out, ldq, part, splits, split_stride, ldp, (const TB*)bias, pos, slots, inv_freq, (T*)kcache,
+            (T*)vcache, nh, nkv, d, rot, page_size, write_kv, cache_slots);
+    }));
+    return zi_check_launch("rope_kv_store_split");
+}
+
 // Rotation alone, out of place: out[t,h,:] = rotate(in[t,h,:], pos[t])  (op-level entry, and the
 // form a layer uses that reads another layer's cache and therefore stores nothing).
 template <typename T>

@@ -113,6 +113,12 @@ class DecoderModel:
                 pass  # the last feed-forward's output is not needed when no logits are
             return None
         rows = batch.logit_rows
+        if delta is not None and delta.dim() == 3:
+            # float32 partial sums (few tokens): norm every row, then pick the wanted ones
+            x_all = self.final_norm.add_forward(resid, delta)
+            x = ops.gather_rows(x_all, rows, out=self.rt.buffer("norm_rows", (batch.num_logit_rows, self.hidden_size),
+                                                               x_all.dtype))
+            return self.lm_head.forward(x)
         r = self.rt.buffer("resid_rows", (batch.num_logit_rows, self.hidden_size), torch.float32)
         ops.gather_rows(resid, rows, out=r)
         if delta is not None:

@@ -7,13 +7,16 @@ add, argmax, embedding, linear, rms_norm, rope, swiglu).
 """
 from .functional import (add, add_rms_norm, argmax, attention, attention_decode, attention_decode_supported, attention_decode_workspace, attention_prefill,
                          attention_prefill_supported, embedding, gather_rows, has_gpu,
-                         linear, rms_norm, rope, rope_kv_store, rope_inv_freq, sample, swiglu,
+                         linear, linear_splits, linear_sums, linear_sums_supported, linear_swiglu,
+                         linear_swiglu_supported, reduce_sums, rms_norm, rope, rope_kv_store, rope_kv_store_sums,
+                         rope_inv_freq, sample, swiglu,
                          device_synchronize)
 from ._lib import KernelLibraryError, library_path, load
 
 __all__ = [
     "add", "add_rms_norm", "argmax", "attention", "attention_decode", "attention_decode_supported", "attention_decode_workspace", "attention_prefill",
     "attention_prefill_supported", "embedding", "gather_rows", "has_gpu", "linear",
-    "rms_norm", "rope", "rope_kv_store", "rope_inv_freq", "sample", "swiglu", "device_synchronize",
+    "linear_splits", "linear_sums", "linear_sums_supported", "linear_swiglu", "linear_swiglu_supported", "reduce_sums",
+    "rms_norm", "rope", "rope_kv_store", "rope_kv_store_sums", "rope_inv_freq", "sample", "swiglu", "device_synchronize",
     "KernelLibraryError", "library_path", "load",
 ]

@@ -20,9 +20,9 @@ _PROTOTYPES = {
     "zi_embedding": [P, I, P, I, P, I, I, I, P],
     "zi_gather_rows": [P, P, I, P, I, I, I, P],
     "zi_add": [P, I, P, I, P, I, L, P],
-    "zi_swiglu": [P, P, P, I, I, I, L, L, P],
+    "zi_swiglu": [P, I, P, P, I, I, I, L, L, I, I, L, P],
     "zi_rmsnorm": [P, I, P, I, P, I, I, I, L, L, F, I, P],
-    "zi_add_rmsnorm": [P, I, P, P, I, P, I, I, I, F, I, P],
+    "zi_add_rmsnorm": [P, I, P, P, I, I, L, P, I, I, I, F, I, P],
     "zi_rope_kv_store": [P, P, P, I, I, L, L, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_rope": [P, P, I, I, L, L, P, P, I, I, I, P],
     "zi_attention_generic": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
@@ -33,7 +33,10 @@ _PROTOTYPES = {
     "zi_attention_prefill_supported": [I, I, I, I, I],
     "zi_attention_prefill_tile": [],
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
-    "zi_gemm_skinny": [P, I, P, P, P, I, I, I, L, L, L, P, L, P],
+    "zi_gemm_skinny": [P, I, I, P, P, P, I, I, I, L, L, L, P, L, P],
+    "zi_gemm_skinny_splits": [I, I],
+    "zi_reduce_splits": [P, I, P, P, I, I, L, I, P],
+    "zi_rope_kv_store_split": [P, I, L, P, I, L, L, P, I, I, P, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_gemm_skinny_supported": [I, I, I, L, L],
     "zi_argmax": [P, P, P, I, I, I, L, P],
     "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],

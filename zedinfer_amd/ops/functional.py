@@ -114,19 +114,38 @@ def add(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None) ->
     return out
 
 
-def swiglu(gate: torch.Tensor, up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = up * gate / (1 + exp(-gate)); gate and up may be column slices of one tensor."""
+def swiglu(gate: torch.Tensor, up: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+           interleave: int = 0, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """out = up * gate / (1 + exp(-gate)).
+
+    ``gate`` and ``up`` [n, I] may be column slices of one tensor.  With ``interleave`` = B, ``gate``
+    is one [n, 2I] matrix that holds B gate columns, then the B up columns of the same places, and so
+    on (``up`` is not given).  A 3-D ``gate`` [S, n, 2I] (interleaved only) is a stack of float32
+    partial sums that are added in rising order first."""
     _gpu("swiglu", gate, up, out)
-    ldg, I = _rows(gate, "swiglu gate")
-    ldu, I2 = _rows(up, "swiglu up")
-    if gate.shape != up.shape or gate.dtype != up.dtype:
-        raise ValueError(f"swiglu: gate {tuple(gate.shape)} {gate.dtype} and up {tuple(up.shape)} {up.dtype} differ")
+    splits, split_stride = 1, 0
+    if gate.dim() == 3:
+        if interleave <= 0 or not gate.is_contiguous():
+            raise ValueError("swiglu: partial sums must be one contiguous interleaved [S, n, 2I] tensor")
+        splits, split_stride = gate.shape[0], gate.shape[1] * gate.shape[2]
+        gate = gate[0]
+    ldg, wg = _rows(gate, "swiglu gate")
     n = gate.shape[0]
+    if interleave > 0:
+        if up is not None or wg % (2 * interleave):
+            raise ValueError(f"swiglu: an interleaved input of width {wg} must hold whole blocks of 2*{interleave}")
+        I, ldu = wg // 2, 0
+    else:
+        ldu, I2 = _rows(up, "swiglu up")
+        if gate.shape != up.shape or gate.dtype != up.dtype:
+            raise ValueError(f"swiglu: gate {tuple(gate.shape)} {gate.dtype} and up {tuple(up.shape)} {up.dtype} differ")
+        I = wg
     if out is None:
-        out = torch.empty((n, I), dtype=gate.dtype, device=gate.device)
-    if tuple(out.shape) != (n, I) or out.dtype != gate.dtype or not out.is_contiguous():
-        raise ValueError("swiglu: out has the wrong shape or dtype")
-    _lib.call("zi_swiglu", _p(out), _p(gate), _p(up), _code(gate, "swiglu"), n, I, ldg, ldu, _stream())
+        out = torch.empty((n, I), dtype=out_dtype or gate.dtype, device=gate.device)
+    if tuple(out.shape) != (n, I) or not out.is_contiguous():
+        raise ValueError("swiglu: out has the wrong shape")
+    _lib.call("zi_swiglu", _p(out), _code(out, "swiglu out"), _p(gate), _p(up), _code(gate, "swiglu"), n, I, ldg, ldu,
+              int(interleave), splits, split_stride, _stream())
     return out
 
 
@@ -153,22 +172,29 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[to
 def add_rms_norm(resid: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float,
                  out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
                  add_one: bool = False) -> torch.Tensor:
-    """resid (float32, changed in place) += delta; returns norm(resid) * w."""
+    """resid (float32, changed in place) += delta; returns norm(resid) * w.  ``delta`` is [n, H], or a
+    stack [S, n, H] of float32 partial sums that are added in rising order."""
     _gpu("add_rms_norm", resid, delta, weight, out)
     if resid.dtype != torch.float32 or resid.dim() != 2 or not resid.is_contiguous():
         raise ValueError("add_rms_norm: the residual stream must be a contiguous float32 [n, hidden] tensor")
-    if delta.shape != resid.shape or not delta.is_contiguous():
-        raise ValueError("add_rms_norm: delta must match the residual's shape and be contiguous")
     n, H = resid.shape
+    splits, split_stride = 1, 0
+    if delta.dim() == 3:
+        if delta.dtype != torch.float32:
+            raise ValueError("add_rms_norm: partial sums must be float32")
+        splits, split_stride = delta.shape[0], n * H
+    if tuple(delta.shape[-2:]) != (n, H) or not delta.is_contiguous():
+        raise ValueError("add_rms_norm: delta must match the residual's shape and be contiguous")
     if weight.dim() != 1 or weight.numel() != H or not weight.is_contiguous():
         raise ValueError(f"add_rms_norm: weight must be [{H}]")
     if out is None:
-        out = torch.empty((n, H), dtype=out_dtype or delta.dtype, device=resid.device)
+        out = torch.empty((n, H), dtype=out_dtype or (delta.dtype if delta.dim() == 2 else torch.bfloat16),
+                          device=resid.device)
     if tuple(out.shape) != (n, H) or not out.is_contiguous():
         raise ValueError("add_rms_norm: out has the wrong shape")
     _lib.call("zi_add_rmsnorm", _p(out), _code(out, "add_rms_norm out"), _p(resid), _p(delta),
-              _code(delta, "add_rms_norm delta"), _p(weight), _code(weight, "add_rms_norm weight"), n, H,
-              float(eps), int(add_one), _stream())
+              _code(delta, "add_rms_norm delta"), splits, split_stride, _p(weight),
+              _code(weight, "add_rms_norm weight"), n, H, float(eps), int(add_one), _stream())
     return out
 
 
@@ -244,6 +270,42 @@ def rope_kv_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
     else:
         rot = 0
     _lib.call("zi_rope_kv_store", _p(q), _p(k), _p(v), _code(q, "rope_kv_store"), n, ldq, ldk, ldv, _p(pos),
+              _p(slots), _p(inv_freq), _p(kcache), _p(vcache), pages * ps, nh, nkv, d, rot, max(ps, 1), int(write),
+              _stream())
+
+
+def rope_kv_store_sums(sums: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.Tensor, pos: torch.Tensor,
+                       slots: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
+                       kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], nh: int, nkv: int, d: int
+                       ) -> None:
+    """The same from the float32 partial sums [S, n, nh*d + 2*nkv*d] of one fused q/k/v projection:
+    adds the splits in rising order and the bias, rotates, writes q to ``q_out`` [n, nh*d] and k, v
+    into the cache.  With ``kcache`` None only q is made (the sums may then be [S, n, nh*d])."""
+    _gpu("rope_kv_store_sums", sums, bias, q_out, pos, slots, inv_freq, kcache, vcache)
+    if sums.dim() != 3 or sums.dtype != torch.float32 or not sums.is_contiguous():
+        raise ValueError("rope_kv_store_sums: sums must be a contiguous float32 [S, n, width] tensor")
+    S, n, width = sums.shape
+    write = kcache is not None
+    need = nh * d + (2 * nkv * d if write else 0)
+    if width < need:
+        raise ValueError(f"rope_kv_store_sums: rows of {width} values, {need} needed")
+    if bias is not None and (bias.dim() != 1 or bias.numel() < need or not bias.is_contiguous()):
+        raise ValueError(f"rope_kv_store_sums: bias must hold {need} values")
+    ldq, wq = _rows(q_out, "rope_kv_store_sums q_out")
+    if q_out.shape[0] != n or wq != nh * d:
+        raise ValueError(f"rope_kv_store_sums: q_out must be [{n}, {nh * d}]")
+    _i32(pos, "rope_kv_store_sums positions", n)
+    pages = ps = 0
+    if write:
+        pages, ps = _check_cache(kcache, vcache, nkv, d, q_out.dtype, "rope_kv_store_sums")
+        _i32(slots, "rope_kv_store_sums slots", n)
+    rot = 0
+    if inv_freq is not None:
+        rot = 2 * inv_freq.numel()
+        if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous() or rot > d:
+            raise ValueError("rope_kv_store_sums: inv_freq must be float32 with at most head_dim/2 entries")
+    _lib.call("zi_rope_kv_store_split", _p(q_out), _code(q_out, "rope_kv_store_sums"), ldq, _p(sums), S, n * width,
+              width, _p(bias), _code(bias, "rope_kv_store_sums bias") if bias is not None else F32, n, _p(pos),
               _p(slots), _p(inv_freq), _p(kcache), _p(vcache), pages * ps, nh, nkv, d, rot, max(ps, 1), int(write),
               _stream())
 
@@ -416,7 +478,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             m = min(SKINNY_MAX_ROWS, M - m0)
             need = lib.zi_gemm_skinny_workspace(m, N, K)
             ws = _workspace(x.device, need) if need else None
-            _lib.call("zi_gemm_skinny", _p(out[m0:m0 + m]), _code(out, "linear out"), _p(x[m0:m0 + m]), _p(weight),
+            _lib.call("zi_gemm_skinny", _p(out[m0:m0 + m]), _code(out, "linear out"), 0, _p(x[m0:m0 + m]), _p(weight),
                       _p(bias), m, N, K, ldx, ldw, ldo, _p(ws), need, _stream())
         return out
     if all_bf and out.dtype == bf and out.is_contiguous():
@@ -428,6 +490,81 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     _lib.call("zi_gemm_generic", _p(out), _code(out, "linear out"), _p(x), _code(x, "linear x"), _p(weight),
               _code(weight, "linear weight"), _p(bias), _code(bias, "linear bias") if bias is not None else F32,
               M, N, K, ldx, ldw, ldo, _stream())
+    return out
+
+
+def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether ``linear_sums`` takes this product: bfloat16, at most SKINNY_MAX_ROWS rows."""
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.dim() != 2 or weight.dim() != 2:
+        return False
+    if not (0 < x.shape[0] <= SKINNY_MAX_ROWS) or x.shape[1] != weight.shape[1]:
+        return False
+    if (x.shape[1] > 1 and x.stride(1) != 1) or (weight.shape[1] > 1 and weight.stride(1) != 1):
+        return False
+    return _skinny_ok(x, weight, x.shape[1], x.stride(0), weight.stride(0))
+
+
+def linear_splits(N: int, K: int) -> int:
+    """Partial sums the few-rows product with a weight matrix [N, K] leaves (a function of N and K alone)."""
+    return int(_lib.load().zi_gemm_skinny_splits(int(N), int(K)))
+
+
+def linear_sums(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[M,K] . weight[N,K]^T for M <= SKINNY_MAX_ROWS as float32 partial sums [S, M, N], S =
+    ``linear_splits(N, K)``, without bias: the consumer adds them in rising order."""
+    _gpu("linear_sums", x, weight, out)
+    if not linear_sums_supported(x, weight):
+        raise ValueError("linear_sums: needs bfloat16 x and weight, at most 64 rows, 16-byte aligned rows")
+    M, K = x.shape
+    N = weight.shape[0]
+    S = linear_splits(N, K)
+    if out is None:
+        out = torch.empty((S, M, N), dtype=torch.float32, device=x.device)
+    if tuple(out.shape) != (S, M, N) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError(f"linear_sums: out must be a contiguous float32 [{S}, {M}, {N}] tensor")
+    _lib.call("zi_gemm_skinny", _p(out), F32, 1, _p(x), _p(weight), c_void_p(0), M, N, K, x.stride(0), weight.stride(0),
+              N, c_void_p(0), 0, _stream())
+    return out
+
+
+def linear_swiglu_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    return (linear_sums_supported(x, weight) and weight.shape[0] % 16 == 0
+            and linear_splits(weight.shape[0], weight.shape[1]) == 1)
+
+
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """up * silu(gate) of x . weight^T in one kernel, for a weight [2I, K] whose rows are 8 gate rows,
+    then the 8 up rows of the same columns, and so on; out [M, I] bfloat16."""
+    _gpu("linear_swiglu", x, weight, out)
+    if not linear_swiglu_supported(x, weight):
+        raise ValueError("linear_swiglu: needs an unsplit bfloat16 few-rows product with 2I a multiple of 16")
+    M, K = x.shape
+    N = weight.shape[0]
+    if out is None:
+        out = torch.empty((M, N // 2), dtype=torch.bfloat16, device=x.device)
+    ldo, wo = _rows(out, "linear_swiglu out")
+    if tuple(out.shape) != (M, N // 2) or out.dtype != torch.bfloat16:
+        raise ValueError(f"linear_swiglu: out must be bfloat16 [{M}, {N // 2}]")
+    _lib.call("zi_gemm_skinny", _p(out), BF16, 2, _p(x), _p(weight), c_void_p(0), M, N, K, x.stride(0), weight.stride(0),
+              ldo, c_void_p(0), 0, _stream())
+    return out
+
+
+def reduce_sums(sums: torch.Tensor, bias: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """out[m,n] = sum_s sums[s,m,n] + bias[n], added in rising order."""
+    _gpu("reduce_sums", sums, bias, out)
+    if sums.dim() != 3 or sums.dtype != torch.float32 or not sums.is_contiguous():
+        raise ValueError("reduce_sums: sums must be a contiguous float32 [S, M, N] tensor")
+    S, M, N = sums.shape
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
+        raise ValueError(f"reduce_sums: bias must be bfloat16 [{N}]")
+    if out is None:
+        out = torch.empty((M, N), dtype=out_dtype or torch.bfloat16, device=sums.device)
+    ldo, wo = _rows(out, "reduce_sums out")
+    if tuple(out.shape) != (M, N):
+        raise ValueError("reduce_sums: out has the wrong shape")
+    _lib.call("zi_reduce_splits", _p(out), _code(out, "reduce_sums out"), _p(sums), _p(bias), M, N, ldo, S, _stream())
     return out
 
 

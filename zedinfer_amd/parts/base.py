@@ -132,8 +132,11 @@ class Mixer(Part):
     """Mixes information across the tokens of a sequence.
 
     ``forward(x, batch, memory)`` takes the normed hidden states [n, hidden] of all tokens
-    of the step and returns [n, hidden].  ``batch`` is the step's device-side description
-    (``engine.batch.DeviceBatch``); ``memory`` is this run's ``LayerMemory``."""
+    of the step and returns the addition to the residual stream: [n, hidden], or a stack
+    [S, n, hidden] of float32 partial sums that the next norm adds in rising order (what
+    the few-rows matrix product leaves when it is cut along k).  ``batch`` is the step's
+    device-side description (``engine.batch.DeviceBatch``); ``memory`` is this run's
+    ``LayerMemory``."""
 
     def cache_request(self) -> Optional[KVCacheRequest]:
         return None
@@ -146,15 +149,17 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
-    """``forward(x)``: [n, hidden] -> [n, hidden], token by token."""
+    """``forward(x)``: [n, hidden] -> [n, hidden] (or a stack [S, n, hidden] of float32 partial
+    sums, as for a mixer), token by token."""
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
 
 
 class Norm(Part):
-    """``forward(x)`` normalises rows; ``add_forward(resid, delta)`` first adds ``delta`` into
-    the float32 residual stream in place and returns the normalised sum."""
+    """``forward(x)`` normalises rows; ``add_forward(resid, delta)`` first adds ``delta`` ([n, hidden],
+    or a stack [S, n, hidden] of float32 partial sums, added in rising order) into the float32
+    residual stream in place and returns the normalised sum."""
 
     def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         raise NotImplementedError
@@ -164,10 +169,25 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """Encodes positions into queries and keys on their way into the cache."""
+    """Encodes positions into queries and keys on their way into the cache.
+
+    ``rotate_and_store`` encodes q [n, nh*d] in place and stores the encoded k and the raw v
+    [n, nkv*d] at ``slots`` of ``memory``'s cache (nothing is stored when ``memory.writes`` is
+    False).  ``rotate_and_store_sums`` does the same from the float32 partial sums [S, n,
+    nh*d + 2*nkv*d] of a fused q/k/v projection plus its bias, and writes q to ``q_out``; the
+    default adds the sums up and calls ``rotate_and_store``."""
 
     def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
         raise NotImplementedError
+
+    def rotate_and_store_sums(self, sums, bias, q_out, positions, slots, memory: LayerMemory, nh: int, nkv: int,
+                              d: int) -> None:
+        from .. import ops
+        qkv = ops.reduce_sums(sums, bias, out_dtype=q_out.dtype)
+        qd, kvd = nh * d, nkv * d
+        q, k, v = qkv[:, :qd], qkv[:, qd:qd + kvd], qkv[:, qd + kvd:]
+        self.rotate_and_store(q, k, v, positions, slots, memory, nh, nkv, d)
+        q_out.copy_(q)
 
 
 class Block:
@@ -175,8 +195,9 @@ class Block:
     (norms by name, mixer, feed_forward, runtime); ``norm_names`` lists the norms it needs.
 
     ``forward(resid, delta, batch, memory)``: ``resid`` is the float32 residual stream
-    [n, hidden], ``delta`` a pending addition to it (or None); returns the next pending
-    addition.  The add is folded into the following norm."""
+    [n, hidden], ``delta`` a pending addition to it (or None; [n, hidden] or a stack
+    [S, n, hidden] of float32 partial sums); returns the next pending addition.  The add is
+    folded into the following norm."""
 
     norm_names: Tuple[str, ...] = ()
 

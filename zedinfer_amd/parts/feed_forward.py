@@ -18,12 +18,23 @@ def stack_rows(tensors):
     return torch.cat(list(tensors), dim=0).contiguous()
 
 
+def interleave_rows(a: torch.Tensor, b: torch.Tensor, block: int) -> torch.Tensor:
+    """[a rows 0..block-1, b rows 0..block-1, a rows block..2*block-1, ...] for two [n, k] matrices."""
+    n, k = a.shape
+    return torch.stack([a.view(n // block, block, k), b.view(n // block, block, k)], dim=1).reshape(2 * n, k).contiguous()
+
+
+GATE_UP_BLOCK = 8    # gate and up rows alternate in blocks of 8: one matrix-core tile holds both for 8 columns
+
+
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
     """down(up(x) * silu(gate(x))), no biases (reference:
     src/frontend/models/transformer_forward.cpp:128-137; src/backend/ops/swiglu/cpu/swiglu_cpu.cpp:9-23).
     gate and up are stacked into one [2I, H] matrix at load: one product instead of two, the same
-    sums per output element.  params: hidden_size, intermediate_size."""
+    sums per output element.  In bfloat16 (and with I a multiple of 8) their rows alternate in
+    blocks of 8, so that the few-rows product can apply the activation in its epilogue.
+    params: hidden_size, intermediate_size."""
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -34,19 +45,40 @@ class SwiGLU(FeedForward):
         super().__init__(spec, weights, rt)
         self.hidden = int(spec.params["hidden_size"])
         self.inter = int(spec.params["intermediate_size"])
-        self.gate_up = stack_rows([weights["gate"], weights["up"]])
-        self.gate, self.up = (None, None) if self.gate_up is not None else (weights["gate"], weights["up"])
+        g, u = weights["gate"], weights["up"]
+        self.interleave = 0
+        self.gate = self.up = None
+        if g.dtype == u.dtype == torch.bfloat16 and self.inter % GATE_UP_BLOCK == 0:
+            self.gate_up = interleave_rows(g, u, GATE_UP_BLOCK)
+            self.interleave = GATE_UP_BLOCK
+        else:
+            self.gate_up = stack_rows([g, u])
+            if self.gate_up is None:
+                self.gate, self.up = g, u
         self.down = weights["down"]
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         n, I = x.shape[0], self.inter
-        gu = self.rt.buffer("ffn_gate_up", (n, 2 * I))
-        if self.gate_up is not None:
-            ops.linear(x, self.gate_up, out=gu)
-        else:
-            ops.linear(x, self.gate, out=gu[:, :I])
-            ops.linear(x, self.up, out=gu[:, I:])
         act = self.rt.buffer("ffn_act", (n, I))
-        ops.swiglu(gu[:, :I], gu[:, I:], out=act)
+        if self.interleave and ops.linear_swiglu_supported(x, self.gate_up):
+            ops.linear_swiglu(x, self.gate_up, out=act)
+        elif self.interleave and ops.linear_sums_supported(x, self.gate_up):
+            S = ops.linear_splits(2 * I, self.hidden)
+            sums = ops.linear_sums(x, self.gate_up, out=self.rt.buffer("ffn_gate_up_sums", (S, n, 2 * I), torch.float32))
+            ops.swiglu(sums, out=act, interleave=self.interleave)
+        else:
+            gu = self.rt.buffer("ffn_gate_up", (n, 2 * I))
+            if self.gate_up is not None:
+                ops.linear(x, self.gate_up, out=gu)
+            else:
+                ops.linear(x, self.gate, out=gu[:, :I])
+                ops.linear(x, self.up, out=gu[:, I:])
+            if self.interleave:
+                ops.swiglu(gu, out=act, interleave=self.interleave)
+            else:
+                ops.swiglu(gu[:, :I], gu[:, I:], out=act)
+        if ops.linear_sums_supported(act, self.down):
+            S = ops.linear_splits(self.hidden, I)
+            return ops.linear_sums(act, self.down, out=self.rt.buffer("ffn_out_sums", (S, n, self.hidden), torch.float32))
         out = self.rt.buffer("ffn_out", (n, self.hidden))
         return ops.linear(act, self.down, out=out)

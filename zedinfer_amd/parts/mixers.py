@@ -95,16 +95,28 @@ class Attention(Mixer):
 
     def forward(self, x: torch.Tensor, batch, memory: LayerMemory) -> torch.Tensor:
         n = x.shape[0]
-        qkv = self.rt.buffer("attn_qkv", (n, self.qd + 2 * self.kvd))
-        q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
-        if self.qkv is not None:
-            ops.linear(x, self.qkv, self.bias, out=qkv)
-        else:
-            for dst, m, b in zip((q, k, v), self.mats, self.biases or (None, None, None)):
-                ops.linear(x, m, b, out=dst)
         view = batch.groups[memory.group]
-        self.position.rotate_and_store(q, k, v, batch.positions, view.slots, memory, self.nh, self.nkv, self.d)
+        if self.qkv is not None and ops.linear_sums_supported(x, self.qkv):
+            # few rows: the projection leaves float32 partial sums; the rotary kernel adds them and the bias
+            S = ops.linear_splits(self.qkv.shape[0], self.hidden)
+            sums = self.rt.buffer("attn_qkv_sums", (S, n, self.qd + 2 * self.kvd), torch.float32)
+            ops.linear_sums(x, self.qkv, out=sums)
+            q = self.rt.buffer("attn_q", (n, self.qd))
+            self.position.rotate_and_store_sums(sums, self.bias, q, batch.positions, view.slots, memory, self.nh,
+                                                self.nkv, self.d)
+        else:
+            qkv = self.rt.buffer("attn_qkv", (n, self.qd + 2 * self.kvd))
+            q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
+            if self.qkv is not None:
+                ops.linear(x, self.qkv, self.bias, out=qkv)
+            else:
+                for dst, m, b in zip((q, k, v), self.mats, self.biases or (None, None, None)):
+                    ops.linear(x, m, b, out=dst)
+            self.position.rotate_and_store(q, k, v, batch.positions, view.slots, memory, self.nh, self.nkv, self.d)
         att = self.rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
+        if ops.linear_sums_supported(att, self.o):
+            S = ops.linear_splits(self.hidden, self.qd)
+            return ops.linear_sums(att, self.o, out=self.rt.buffer("attn_proj_sums", (S, n, self.hidden), torch.float32))
         out = self.rt.buffer("attn_proj", (n, self.hidden))
         return ops.linear(att, self.o, out=out)

@@ -33,6 +33,13 @@ class RopeNeox(PositionEncoding):
         else:
             ops.rope_kv_store(q, None, None, positions, None, self.inv_freq, None, None, nh, nkv, d)
 
+    def rotate_and_store_sums(self, sums, bias, q_out, positions, slots, memory: LayerMemory, nh: int, nkv: int,
+                              d: int) -> None:
+        if memory.writes:
+            ops.rope_kv_store_sums(sums, bias, q_out, positions, slots, self.inv_freq, memory.k, memory.v, nh, nkv, d)
+        else:
+            ops.rope_kv_store_sums(sums, bias, q_out, positions, None, self.inv_freq, None, None, nh, nkv, d)
+
 
 @register_position_encoding("none")
 class NoPosition(PositionEncoding):
@@ -41,3 +48,10 @@ class NoPosition(PositionEncoding):
     def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
         if memory.writes:
             ops.rope_kv_store(q, k, v, positions, slots, None, memory.k, memory.v, nh, nkv, d)
+
+    def rotate_and_store_sums(self, sums, bias, q_out, positions, slots, memory: LayerMemory, nh: int, nkv: int,
+                              d: int) -> None:
+        if memory.writes:
+            ops.rope_kv_store_sums(sums, bias, q_out, positions, slots, None, memory.k, memory.v, nh, nkv, d)
+        else:
+            ops.rope_kv_store_sums(sums, bias, q_out, positions, None, None, None, None, nh, nkv, d)
