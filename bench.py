@@ -144,15 +144,7 @@ def main():
                 weights_cache["w"] = e
                 return e
             # share the first engine's weights: same model, another cache pool
-            e0 = weights_cache["w"]
-            e = Engine.__new__(Engine)
-            e.__dict__.update(e0.__dict__)
-            from zedinfer_amd.cache.manager import CacheManager
-            e.sched = sched
-            e.cache = CacheManager(e.model.cache_requests(), e.model.state_requests(), pages, 16,
-                                   sched.max_batch_requests, e.dtype, e.device, sched.max_batch_tokens)
-            e.memories = e.cache.memories(e.fc.schedule)
-            return e
+            return weights_cache["w"].with_cache(sched)
         return make
 
     V = cfg.vocab_size

@@ -187,3 +187,53 @@ def test_command_lines(tiny, tmp_path):
     r = run(os.path.join(ROOT, "bin", "batch_bench"), tiny["folder"], "-b", "3", "-p", "20", "-d", "6",
             "--num-kv-blocks", "64", "--kv-block-size", ps, "--random-weights", "--seed", "4")
     assert r.returncode == 0 and "Throughput" in r.stdout and "18 tokens generated" in r.stdout, r.stderr + r.stdout
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype):
+    """Steps of single decoded tokens are captured as graphs and replayed.  Every replay is checked
+    against an engine that launches eagerly, with eager prompt portions, closes and new requests
+    (reused pages, other batch sizes) between the replays."""
+    from zedinfer_amd.engine import StepEntry
+    V = tiny["cfg"]["vocab_size"]
+    fast, slow = engine(tiny, dtype).engine, engine(tiny, dtype).engine
+    assert fast.use_graphs
+    slow.use_graphs = False
+    toks = {r: traces.random_tokens(V, 150, seed=60 + i) for i, r in enumerate("abcd")}
+    fed = {r: 0 for r in toks}
+    seqs = {}
+
+    def both(plan):
+        """plan: [(request, number of tokens)]; returns the two engines' logits."""
+        outs = []
+        for eng in (fast, slow):
+            entries = []
+            for r, n in plan:
+                if (eng, r) not in seqs:
+                    seqs[(eng, r)] = eng.open(r)
+                entries.append(StepEntry(seqs[(eng, r)], toks[r][fed[r]:fed[r] + n], list(range(n))))
+            outs.append(eng.step(entries))
+        for r, n in plan:
+            fed[r] += n
+        assert torch.equal(outs[0], outs[1]), plan
+        return outs[0]
+
+    both([("a", 20), ("b", 7)])
+    for _ in range(6):
+        both([("a", 1), ("b", 1)])
+    both([("c", 33), ("a", 1)])                 # a mixed step runs eagerly
+    for _ in range(5):
+        both([("a", 1), ("b", 1), ("c", 1)])
+    for eng in (fast, slow):
+        eng.close(seqs.pop((eng, "b")))
+    both([("d", 40)])                           # takes the pages b gave back
+    for _ in range(30):
+        both([("a", 1), ("c", 1), ("d", 1)])    # crosses page edges; the same graph serves all of them
+    for _ in range(4):
+        both([("d", 1)])
+    assert fast.graph_replays >= 30 and slow.graph_replays == 0
+    # and the replayed logits are the plain implementation's
+    last = both([("d", 1)])
+    ref = plain.forward(tiny["cfg"], tiny["weights"], toks["d"][:fed["d"]])
+    tol = 2e-4 if dtype == "float32" else 0.06 * float(ref.abs().max())
+    assert float((last[0].cpu() - ref[fed["d"] - 1]).abs().max()) < tol

@@ -73,9 +73,46 @@ class DeviceBatch:
     host_slot: Optional[np.ndarray] = None
 
 
+class StagingRing:
+    """A few pinned host buffers used in turn for the step's one copy to the device.  A buffer is
+    written again only after the copy that last read it has finished."""
+
+    def __init__(self, device: torch.device, depth: int = 4):
+        self.device = device
+        self.pinned = device.type == "cuda"
+        self.buffers: List[Optional[torch.Tensor]] = [None] * depth
+        self.events: List[Optional[torch.cuda.Event]] = [None] * depth
+        self.turn = 0
+
+    def acquire(self, n: int) -> torch.Tensor:
+        self.turn = (self.turn + 1) % len(self.buffers)
+        ev = self.events[self.turn]
+        if ev is not None:
+            ev.synchronize()
+        buf = self.buffers[self.turn]
+        if buf is None or buf.numel() < n:
+            buf = torch.empty((max(n, 4096),), dtype=torch.int32, pin_memory=self.pinned)
+            self.buffers[self.turn] = buf
+        return buf[:n]
+
+    def copied(self) -> None:
+        """The copy out of the buffer last acquired has been queued on the current stream."""
+        if self.pinned:
+            ev = self.events[self.turn] or torch.cuda.Event()
+            ev.record()
+            self.events[self.turn] = ev
+
+
 def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
-                       device: torch.device) -> DeviceBatch:
-    """Check the entries, then pack every index array into one host buffer and copy it over once."""
+                       device: torch.device, staging: Optional[StagingRing] = None,
+                       table_widths: Optional[Sequence[int]] = None,
+                       static: Optional[torch.Tensor] = None) -> DeviceBatch:
+    """Check the entries, then pack every index array into one host buffer and copy it over once.
+
+    ``table_widths`` pads each group's block table to a given width; ``static`` is a device buffer
+    the arrays are copied into instead of a fresh one (the layout depends only on the number of
+    tokens, entries, wanted rows and tiles and on the table widths, so a captured graph that reads
+    the arrays finds them at the same addresses every step)."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     seen = set()
@@ -117,6 +154,10 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
         group_slots.append(np.concatenate(
             [cache.token_slots(e.seq, g, int(p), n) for e, p, n in zip(entries, past, lens)]))
         width = max(1, max(len(e.seq.pages[g]) for e in entries))
+        if table_widths is not None:
+            if table_widths[g] < width:
+                raise ValueError(f"block tables of group {g} need {width} columns, {table_widths[g]} given")
+            width = int(table_widths[g])
         t = np.full((E, width), -1, dtype=np.int32)
         for i, e in enumerate(entries):
             pg = e.seq.pages[g]
@@ -143,13 +184,23 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     for g in range(G):
         pieces += [group_slots[g], group_tables[g].reshape(-1)]
     sizes = [p.size for p in pieces]
-    host = torch.empty((max(1, sum(sizes)),), dtype=torch.int32, pin_memory=device.type == "cuda")
+    total = max(1, sum(sizes))
+    host = staging.acquire(total) if staging is not None else torch.empty(
+        (total,), dtype=torch.int32, pin_memory=device.type == "cuda")
     hv = host.numpy()
     off = 0
     for p in pieces:
         hv[off:off + p.size] = p
         off += p.size
-    dev = host.to(device, non_blocking=True)
+    if static is not None:
+        if static.numel() < total or static.dtype != torch.int32:
+            raise ValueError("the static batch buffer is too small")
+        dev = static[:total]
+        dev.copy_(host, non_blocking=True)
+    else:
+        dev = host.to(device, non_blocking=True)
+    if staging is not None:
+        staging.copied()
     views = []
     off = 0
     for s in sizes:

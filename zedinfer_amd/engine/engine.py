@@ -22,7 +22,7 @@ from ..config import ModelConfig, ModelForwardConfig, SchedulerConfig, load_conf
 from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
 from ..weights import load_weights, random_weights
-from .batch import DeviceBatch, StepEntry, build_device_batch
+from .batch import DeviceBatch, StagingRing, StepEntry, build_device_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            "f32": torch.float32}
@@ -65,6 +65,15 @@ class Engine:
         self.memories = self.cache.memories(fc.schedule)
         self.vocab_size = fc.vocab_size
         self.steps_run = 0
+        self.staging = StagingRing(self.device)
+        # Steps of single decoded tokens are captured as HIP graphs and replayed, one graph per
+        # (entries, wanted rows, block-table widths, attention launch size).
+        self.use_graphs = (self.device.type == "cuda" and self.model.graph_safe()
+                           and os.environ.get("ZEDINFER_DISABLE_GRAPHS", "0") in ("", "0"))
+        self.graph_max_entries = 64
+        self.graph_limit = 48
+        self._graphs: Dict[tuple, "_DecodeGraph"] = {}
+        self.graph_replays = 0
 
     # ---- construction ------------------------------------------------------------
     @classmethod
@@ -100,6 +109,23 @@ class Engine:
         cap = self.sched.max_batch_requests * (-(-self.sched.max_seq_len // self.sched.kv_block_size))
         return int(min(pages, cap))
 
+    def with_cache(self, sched: SchedulerConfig) -> "Engine":
+        """Another engine over the same model and weights with a cache pool of its own (``sched``
+        sizes it); the two must not run steps at the same time, they share workspaces."""
+        sched.validate()
+        other = Engine.__new__(Engine)
+        other.__dict__.update(self.__dict__)
+        other.sched = sched
+        kv = self.model.cache_requests()
+        other.cache = CacheManager(kv, self.model.state_requests(), sched.num_kv_blocks or self._pages_from_free_memory(kv),
+                                   sched.kv_block_size, sched.max_batch_requests, self.dtype, self.device,
+                                   max_step_tokens=sched.max_batch_tokens)
+        other.memories = other.cache.memories(self.fc.schedule)
+        other.staging = StagingRing(self.device)
+        other._graphs = {}
+        other.steps_run = other.graph_replays = 0
+        return other
+
     # ---- requests ------------------------------------------------------------------
     def open(self, request_id, expected_tokens: int = 0) -> SequenceCache:
         return self.cache.open(request_id, expected_tokens)
@@ -115,9 +141,67 @@ class Engine:
         request's length changed, when the pool cannot hold the new tokens."""
         for e in entries:
             self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
-        batch = build_device_batch(entries, self.cache, self.vocab_size, self.device)
-        logits = self.model.run(batch, self.memories)
+        if (self.use_graphs and 0 < len(entries) <= self.graph_max_entries
+                and all(len(e.tokens) == 1 for e in entries)):
+            logits = self._graph_step(entries)
+        else:
+            batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging)
+            logits = self.model.run(batch, self.memories)
         for e in entries:
             self.cache.commit(e.seq, e.seq.length + len(e.tokens))
         self.steps_run += 1
         return logits.clone() if (copy and logits is not None) else logits
+
+    # ---- decode steps as graphs ------------------------------------------------------
+    def _graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """A step in which every entry brings one token.  Its launches depend on the number of entries
+        and wanted rows, on the width of the block tables and on the size of the attention launch
+        only: the first step of a kind runs eagerly and is captured, later ones replay the graph
+        after the step's index arrays have been copied into the graph's buffer."""
+        E = len(entries)
+        R = sum(len(e.want) for e in entries)
+        widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
+                       for g in range(len(self.cache.groups)))
+        max_keys = max(e.seq.length for e in entries) + 1
+        keys_bucket = _pow2_at_least(max_keys, 256)
+        key = (E, R, widths, keys_bucket)
+        dg = self._graphs.get(key)
+        if dg is None:
+            if len(self._graphs) >= self.graph_limit:
+                self._graphs.pop(next(iter(self._graphs)))
+            size = 8 * E + 2 * R + sum(E * (w + 1) for w in widths) + 64
+            dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
+            self._graphs[key] = dg
+        batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer)
+        batch.max_short_keys = keys_bucket
+        if dg.graph is not None:
+            dg.graph.replay()
+            self.graph_replays += 1
+            return dg.logits
+        logits = self.model.run(batch, self.memories)      # allocates every workspace; its result is this step's
+        if dg.warm:
+            # the second step of this kind: capture (nothing runs), to be replayed from the third on
+            torch.cuda.synchronize(self.device)
+            first = logits.clone() if logits is not None else None
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                dg.logits = self.model.run(batch, self.memories)
+            dg.graph = g
+            return first
+        dg.warm = True
+        return logits
+
+
+class _DecodeGraph:
+    def __init__(self, buffer: torch.Tensor):
+        self.buffer = buffer
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.warm = False
+
+
+def _pow2_at_least(n: int, floor: int = 1) -> int:
+    v = max(int(floor), 1)
+    while v < n:
+        v *= 2
+    return v

@@ -100,6 +100,10 @@ class DecoderModel:
                 out[st.cache] = req
         return out
 
+    def graph_safe(self) -> bool:
+        """Whether a step's launches can be captured and replayed: every mixer says so."""
+        return all(getattr(b.mixer, "graph_safe", False) for b in self.blocks)
+
     # ---- one step -------------------------------------------------------------
     def run(self, batch, memories: Sequence[LayerMemory]) -> Optional[torch.Tensor]:
         """Run the tokens of ``batch`` through the schedule; float32 logits [wanted, vocab]

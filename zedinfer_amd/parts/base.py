@@ -138,6 +138,11 @@ class Mixer(Part):
     device-side description (``engine.batch.DeviceBatch``); ``memory`` is this run's
     ``LayerMemory``."""
 
+    # A mixer whose forward only launches kernels that read the batch's device arrays (no copies to
+    # the host, no launches that depend on the arrays' contents) may set this: steps of decoded
+    # tokens are then captured as graphs and replayed.
+    graph_safe: bool = False
+
     def cache_request(self) -> Optional[KVCacheRequest]:
         return None
 

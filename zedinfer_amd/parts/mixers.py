@@ -26,6 +26,8 @@ class Attention(Mixer):
     params: hidden_size, num_heads, num_kv_heads, head_dim, qkv_bias, window (0: all keys),
     scale (default 1/sqrt(head_dim)), position (a PartSpec of a position encoding)."""
 
+    graph_safe = True
+
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
         p = spec.params
