@@ -271,6 +271,14 @@ def test_argmax(ops, dtype):
     t[1, -1] = 1.0
     assert ops.argmax(t).tolist() == [1234, 151935]
     assert ops.argmax(torch.zeros(1, 77, device="cuda")).tolist() == [0]
+    # long rows are cut over several workgroups; rows may be slices of a wider matrix
+    big = rnd(7, 50001, dtype=dtype)[:, 3:40004]
+    idx, val = ops.argmax(big, return_values=True)
+    assert torch.equal(idx.long(), torch.argmax(big.float(), -1))
+    torch.testing.assert_close(val, big.float().max(-1).values)
+    z = torch.zeros(3, 20000, dtype=dtype, device="cuda")
+    z[1, 8192] = z[1, 19999] = 2.0
+    assert ops.argmax(z).tolist() == [0, 8192, 0]
 
 
 @pytest.mark.parametrize("nh,nkv,d,ps,T,window", [

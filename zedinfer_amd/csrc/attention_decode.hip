@@ -255,12 +255,21 @@ attention_decode_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const floa
     const float M = zi_wave_max(mc);
     const float wc = (mc == -INFINITY) ? 0.f : __expf(mc - M);
     float L = 0.f, acc[2] = {0.f, 0.f};
-    for (int c = 0; c < sp.count; ++c) {
-        const float w = __shfl(wc, c, ZI_WAVE);
-        L += w * __shfl(lc, c, ZI_WAVE);
+    for (int c0 = 0; c0 < sp.count; c0 += 8) {
+        float po[8][2];   // eight chunks' loads are issued before the first is used
 #pragma unroll
-        for (int v = 0; v < 2; ++v)
-            if (lane + v * ZI_WAVE < D) acc[v] += w * part_o[(slot0 + c) * D + lane + v * ZI_WAVE];
+        for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int v = 0; v < 2; ++v)
+                po[c][v] = (c0 + c < sp.count && lane + v * ZI_WAVE < D)
+                               ? part_o[(slot0 + c0 + c) * D + lane + v * ZI_WAVE] : 0.f;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const float w = __shfl(wc, (c0 + c) & (ZI_WAVE - 1), ZI_WAVE);   // 0 for chunks past the count
+            L += w * __shfl(lc, (c0 + c) & (ZI_WAVE - 1), ZI_WAVE);
+            acc[0] += w * po[c][0];
+            acc[1] += w * po[c][1];
+        }
     }
     const float inv = 1.f / L;
 #pragma unroll

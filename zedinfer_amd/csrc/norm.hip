@@ -63,6 +63,62 @@ __global__ void add_rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ res
     for (int j = threadIdx.x; j < H; j += blockDim.x) zi_store(orow + j, (zi_load(w + j) + w_offset) * rr[j] * rstd);
 }
 
+__device__ __forceinline__ float4 zi_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 zi_load4(const zi_bf16* p) {
+    const uint2 r = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                       __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ __forceinline__ void zi_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void zi_store4(zi_bf16* p, float4 v) {
+    uint2 r;
+    r.x = (uint32_t)zi_float_to_bf16(v.x) | ((uint32_t)zi_float_to_bf16(v.y) << 16);
+    r.y = (uint32_t)zi_float_to_bf16(v.z) | ((uint32_t)zi_float_to_bf16(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = r;
+}
+
+// The same for rows of H = 4 * blockDim.x * IT values at most (H % 4 == 0): a thread owns IT groups of four
+// consecutive values, loads everything it needs at once (up to 16 splits) and keeps the sums in
+// registers, so the row is read once and nothing is read back.
+template <typename TD, typename TW, typename TO, int IT>
+__global__ void add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__ resid, const TD* __restrict__ delta,
+                                       int splits, int64_t split_stride, const TW* __restrict__ w, int H, float eps,
+                                       float w_offset) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    float4 v[IT], wv[IT];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int j = (it * blockDim.x + threadIdx.x) * 4;
+        v[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+        wv[it] = v[it];
+        if (j >= H) continue;
+        v[it] = zi_load4(resid + row * H + j);
+        wv[it] = zi_load4(w + j);
+        const TD* dr = delta + row * H + j;
+        float4 d[16];   // every split's load is issued before the first is used
+#pragma unroll
+        for (int sp = 0; sp < 16; ++sp)
+            d[sp] = (sp < splits) ? zi_load4(dr + (int64_t)sp * split_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+        float4 t = d[0];
+#pragma unroll
+        for (int sp = 1; sp < 16; ++sp) { t.x += d[sp].x; t.y += d[sp].y; t.z += d[sp].z; t.w += d[sp].w; }
+        v[it].x += t.x; v[it].y += t.y; v[it].z += t.z; v[it].w += t.w;
+        zi_store4(resid + row * H + j, v[it]);
+        ss += v[it].x * v[it].x + v[it].y * v[it].y + v[it].z * v[it].z + v[it].w * v[it].w;
+    }
+    ss = zi_block_sum(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int j = (it * blockDim.x + threadIdx.x) * 4;
+        if (j >= H) continue;
+        zi_store4(out + row * H + j, make_float4((wv[it].x + w_offset) * v[it].x * rstd, (wv[it].y + w_offset) * v[it].y * rstd,
+                                                 (wv[it].z + w_offset) * v[it].z * rstd, (wv[it].w + w_offset) * v[it].w * rstd));
+    }
+}
+
 extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* delta, int delta_dt, int splits,
                               int64_t split_stride, const void* w, int w_dt, int n, int hidden, float eps, int add_one,
                               hipStream_t stream) {
@@ -71,6 +127,22 @@ extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* d
     ZI_REQUIRE(splits >= 1 && (splits == 1 || split_stride >= (int64_t)n * hidden),
                "add_rmsnorm: bad partial sums (splits %d, stride %lld)", splits, (long long)split_stride);
     if (n == 0) return 0;
+    const bool aligned = ((uintptr_t)out % 16) == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 &&
+                         ((uintptr_t)w % 16) == 0 && split_stride % 4 == 0;
+    if (hidden % 4 == 0 && hidden <= 8192 && splits <= 16 && aligned) {
+        const int vecs = hidden / 4;
+        const int it = vecs > 1024 ? 2 : 1;
+        int threads = ((vecs + it - 1) / it + ZI_WAVE - 1) / ZI_WAVE * ZI_WAVE;
+        ZI_DISPATCH_DTYPE(delta_dt, TD, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
+            if (it == 1)
+                add_rmsnorm_vec_kernel<TD, TW, TO, 1><<<n, threads, 0, stream>>>(
+                    (TO*)out, resid, (const TD*)delta, splits, split_stride, (const TW*)w, hidden, eps, add_one ? 1.f : 0.f);
+            else
+                add_rmsnorm_vec_kernel<TD, TW, TO, 2><<<n, threads, 0, stream>>>(
+                    (TO*)out, resid, (const TD*)delta, splits, split_stride, (const TW*)w, hidden, eps, add_one ? 1.f : 0.f);
+        })));
+        return zi_check_launch("add_rmsnorm");
+    }
     ZI_DISPATCH_DTYPE(delta_dt, TD, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
         add_rmsnorm_kernel<TD, TW, TO><<<n, NORM_THREADS, 0, stream>>>((TO*)out, resid, (const TD*)delta, splits,
                                                                        split_stride, (const TW*)w, hidden, eps,

@@ -99,14 +99,14 @@ __global__ void rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, c
                                            const TB* __restrict__ bias, const int32_t* __restrict__ pos,
                                            const int32_t* __restrict__ slots, const float* __restrict__ inv_freq,
                                            T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int d,
-                                           int rot, int page_size, int write_kv, int64_t cache_slots) {
-    extern __shared__ float sh[];  // cos[rot/2], sin[rot/2], then the summed row
+                                           int rot, int page_size, int write_kv, int64_t cache_slots, int vec4) {
+    extern __shared__ __attribute__((aligned(16))) float sh[];  // cos[rot/2], sin[rot/2], then the summed row
     const int64_t t = blockIdx.x;
     const int half = rot / 2;
     const int qd = nh * d, kvd = nkv * d;
     const int width = qd + (write_kv ? 2 * kvd : 0);
     float* cs = sh;
-    float* row = sh + rot;
+    float* row = sh + ((rot + 3) & ~3);
     const float p = (float)pos[t];
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
         float s, c;
@@ -115,11 +115,30 @@ __global__ void rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, c
         cs[half + i] = s;
     }
     const float* pr = part + t * ldp;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
-        float v = pr[i];
-        for (int s = 1; s < splits; ++s) v += pr[s * split_stride + i];
-        if (bias) v += zi_load(bias + i);
-        row[i] = v;
+    if (vec4) {
+        // every split's load is issued before the first is used (host: splits <= 16, 16-byte alignment)
+        for (int i = threadIdx.x * 4; i < width; i += blockDim.x * 4) {
+            float4 d[16];
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                d[s] = (s < splits) ? *reinterpret_cast<const float4*>(pr + (int64_t)s * split_stride + i)
+                                    : make_float4(0.f, 0.f, 0.f, 0.f);
+            float4 v = d[0];
+#pragma unroll
+            for (int s = 1; s < 16; ++s) { v.x += d[s].x; v.y += d[s].y; v.z += d[s].z; v.w += d[s].w; }
+            if (bias) {
+                v.x += zi_load(bias + i); v.y += zi_load(bias + i + 1); v.z += zi_load(bias + i + 2);
+                v.w += zi_load(bias + i + 3);
+            }
+            *reinterpret_cast<float4*>(row + i) = v;
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) {
+            float v = pr[i];
+            for (int s = 1; s < splits; ++s) v += pr[s * split_stride + i];
+            if (bias) v += zi_load(bias + i);
+            row[i] = v;
+        }
     }
     __syncthreads();
     T* qr = q_out + t * ldq;
@@ -167,14 +186,15 @@ extern "C" int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const fl
                    page_size);
         ZI_REQUIRE(kcache && vcache && slots, "rope_kv_store_split: null cache pointer");
     }
-    const size_t lds = (size_t)(rot + width) * sizeof(float);
+    const size_t lds = (size_t)(((rot + 3) & ~3) + width + 4) * sizeof(float);
+    const int vec4 = width % 4 == 0 && ldp % 4 == 0 && split_stride % 4 == 0 && ((uintptr_t)part % 16) == 0 && splits <= 16;
     ZI_REQUIRE(lds <= 60 * 1024, "rope_kv_store_split: a row of %lld values does not fit in LDS", (long long)width);
     if (n == 0) return 0;
     if (!bias) bias_dt = ZI_F32;
     ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(bias_dt, TB, {
         rope_kv_store_split_kernel<T, TB><<<n, 256, lds, stream>>>(
             (T*)q_out, ldq, part, splits, split_stride, ldp, (const TB*)bias, pos, slots, inv_freq, (T*)kcache,
-            (T*)vcache, nh, nkv, d, rot, page_size, write_kv, cache_slots);
+            (T*)vcache, nh, nkv, d, rot, page_size, write_kv, cache_slots, vec4);
     }));
     return zi_check_launch("rope_kv_store_split");
 }

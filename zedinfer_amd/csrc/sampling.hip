@@ -60,10 +60,71 @@ argmax_kernel(int32_t* __restrict__ out_idx, float* __restrict__ out_val, const 
     }
 }
 
+// Stage one of the argmax of long rows: part `blockIdx.y` of row `blockIdx.x` leaves its best (value, index).
+template <typename T>
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+argmax_part_kernel(float* __restrict__ part_val, int32_t* __restrict__ part_idx, const T* __restrict__ logits,
+                   int64_t ld, int V, int part_len) {
+    __shared__ float fred[16];
+    __shared__ int ired[16];
+    const int64_t row = blockIdx.x;
+    const int lo = blockIdx.y * part_len;
+    const int n = (lo + part_len < V) ? part_len : V - lo;
+    float bv;
+    const int bi = block_argmax<T>(logits + row * ld + lo, n, &bv, fred, ired);
+    if (threadIdx.x == 0) {
+        part_val[row * gridDim.y + blockIdx.y] = bv;
+        part_idx[row * gridDim.y + blockIdx.y] = lo + bi;
+    }
+}
+
+// Stage two: the best of a row's parts; the lowest index among equals (parts are in rising order of index).
+__global__ void argmax_merge_kernel(int32_t* __restrict__ out_idx, float* __restrict__ out_val,
+                                    const float* __restrict__ part_val, const int32_t* __restrict__ part_idx,
+                                    int parts) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lane; i < parts; i += ZI_WAVE) {
+        const float v = part_val[row * parts + i];
+        const int x = part_idx[row * parts + i];
+        if (v > best || (v == best && x < bi)) { best = v; bi = x; }
+    }
+#pragma unroll
+    for (int o = ZI_WAVE / 2; o > 0; o >>= 1) {
+        const float ob = __shfl_xor(best, o, ZI_WAVE);
+        const int oi = __shfl_xor(bi, o, ZI_WAVE);
+        if (ob > best || (ob == best && oi < bi)) { best = ob; bi = oi; }
+    }
+    if (lane == 0) {
+        out_idx[row] = bi == 0x7fffffff ? 0 : bi;
+        if (out_val) out_val[row] = best;
+    }
+}
+
+#define ARGMAX_PART 8192   // values one workgroup scans when a row is cut
+
+// Floats of workspace that let a row be cut over several workgroups (0: rows are short).
+extern "C" int64_t zi_argmax_workspace(int rows, int vocab) {
+    const int parts = (vocab + ARGMAX_PART - 1) / ARGMAX_PART;
+    return parts > 1 ? 2 * (int64_t)rows * parts : 0;
+}
+
 extern "C" int zi_argmax(int32_t* out_idx, float* out_val, const void* logits, int dt, int rows, int vocab,
-                         int64_t ld, hipStream_t stream) {
+                         int64_t ld, float* workspace, int64_t workspace_floats, hipStream_t stream) {
     ZI_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
     if (rows == 0) return 0;
+    const int parts = (vocab + ARGMAX_PART - 1) / ARGMAX_PART;
+    if (parts > 1 && workspace && workspace_floats >= 2 * (int64_t)rows * parts && rows <= 65535 && parts <= 65535) {
+        float* pv = workspace;
+        int32_t* pi = reinterpret_cast<int32_t*>(workspace + (int64_t)rows * parts);
+        ZI_DISPATCH_DTYPE(dt, T, {
+            argmax_part_kernel<T><<<dim3(rows, parts), SAMPLE_THREADS, 0, stream>>>(pv, pi, (const T*)logits, ld, vocab,
+                                                                                    ARGMAX_PART);
+        });
+        argmax_merge_kernel<<<rows, ZI_WAVE, 0, stream>>>(out_idx, out_val, pv, pi, parts);
+        return zi_check_launch("argmax");
+    }
     ZI_DISPATCH_DTYPE(dt, T, {
         argmax_kernel<T><<<rows, SAMPLE_THREADS, 0, stream>>>(out_idx, out_val, (const T*)logits, ld, vocab);
     });

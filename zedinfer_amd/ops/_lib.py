@@ -38,7 +38,7 @@ _PROTOTYPES = {
     "zi_reduce_splits": [P, I, P, P, I, I, L, I, P],
     "zi_rope_kv_store_split": [P, I, L, P, I, L, L, P, I, I, P, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_gemm_skinny_supported": [I, I, I, L, L],
-    "zi_argmax": [P, P, P, I, I, I, L, P],
+    "zi_argmax": [P, P, P, I, I, I, L, P, L, P],
     "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],
 }
 
@@ -77,6 +77,8 @@ def load() -> ctypes.CDLL:
             fn.restype = c_int
         lib.zi_gemm_skinny_workspace.argtypes = [I, I, I]
         lib.zi_gemm_skinny_workspace.restype = c_int64
+        lib.zi_argmax_workspace.argtypes = [I, I]
+        lib.zi_argmax_workspace.restype = c_int64
         _lib, _lib_path = lib, path
         return lib
 

@@ -597,7 +597,9 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None, return_valu
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
     _i32(out, "argmax out", R)
     vals = torch.empty((R,), dtype=torch.float32, device=logits.device) if return_values else None
-    _lib.call("zi_argmax", _p(out), _p(vals), _p(logits), _code(logits, "argmax"), R, V, ld, _stream())
+    need = _lib.load().zi_argmax_workspace(R, V)      # long rows are cut over several workgroups
+    ws = _workspace(logits.device, need) if need else None
+    _lib.call("zi_argmax", _p(out), _p(vals), _p(logits), _code(logits, "argmax"), R, V, ld, _p(ws), need, _stream())
     return (out, vals) if return_values else out
 
 
