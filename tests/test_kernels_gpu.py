@@ -242,10 +242,13 @@ def test_linear_skinny_row_does_not_depend_on_batch(ops):
     """The decode-time product cuts k by the weight's shape alone: a row's result is bit-identical
     whether 1, 8 or 64 rows ride along."""
     x, w = rnd(64, 1536, dtype=torch.bfloat16, seed=1), rnd(2048, 1536, dtype=torch.bfloat16, scale=0.05, seed=2)
-    full = ops.linear(x, w)
+    full = ops.linear(x, w, out_dtype=torch.float32)
     for m in (1, 8, 17):
-        part = ops.linear(x[:m].contiguous(), w)
+        part = ops.linear(x[:m].contiguous(), w, out_dtype=torch.float32)
         assert torch.equal(full[:m], part)
+    # with bfloat16 output up to 16 rows run on the same kernel (more rows go to the library product)
+    assert torch.equal(ops.linear(x[:16].contiguous(), w)[:3], ops.linear(x[:3].contiguous(), w))
+    assert torch.equal(ops.linear(x[:3].contiguous(), w), full[:3].to(torch.bfloat16))
     x2, w2 = rnd(64, 8960, dtype=torch.bfloat16, seed=3), rnd(1536, 8960, dtype=torch.bfloat16, scale=0.02, seed=4)
     assert torch.equal(ops.linear(x2, w2, out_dtype=torch.float32)[5:6], ops.linear(x2[5:6].contiguous(), w2, out_dtype=torch.float32))
 
@@ -448,10 +451,11 @@ def test_attention_prefill_refuses_other_shapes(ops):
 
 
 # ---- the few-rows product's partial sums and the kernels that consume them ------------------------
-@pytest.mark.parametrize("M,N,K", [(1, 2048, 1536), (8, 1536, 8960), (16, 17920, 1536), (17, 1536, 1536),
-                                   (64, 2048, 1536), (5, 176, 64), (33, 1000, 96), (3, 48, 520)])
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 1536), (8, 1536, 8960), (16, 17920, 1536), (13, 1536, 1536),
+                                   (16, 2048, 1536), (5, 176, 64), (11, 1000, 96), (3, 48, 520), (2, 3584, 18944)])
 def test_linear_sums(ops, M, N, K):
     bf = torch.bfloat16
+    assert not ops.linear_sums_supported(rnd(17, K, dtype=bf), rnd(N, K, dtype=bf))
     x, w = rnd(M, K, dtype=bf, seed=1), rnd(N, K, dtype=bf, scale=0.05, seed=2)
     b = rnd(N, dtype=bf, seed=3)
     sums = ops.linear_sums(x, w)
@@ -466,7 +470,8 @@ def test_linear_sums(ops, M, N, K):
         assert torch.equal(alone[:, 0], sums[:, M - 1])
 
 
-@pytest.mark.parametrize("M,I,K", [(1, 8960, 1536), (8, 8960, 1536), (40, 176, 64), (16, 256, 96), (2, 208, 80)])
+@pytest.mark.parametrize("M,I,K", [(1, 8960, 1536), (8, 8960, 1536), (14, 176, 64), (16, 256, 96), (2, 208, 80),
+                                   (4, 18944, 3584)])
 def test_linear_swiglu(ops, M, I, K):
     from zedinfer_amd.parts.feed_forward import interleave_rows
     bf = torch.bfloat16

@@ -34,8 +34,9 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 #define SK_KB 128
 #define SK_WAVES 4
 #define SK_MAX_KPW 4
-#define SK_TARGET_WGS 512
-#define SK_MAX_TPW 16
+#define SK_RESIDENT_WGS 480   // workgroups that are surely resident at once (256 compute units, two each)
+#define SK_ENOUGH_WGS 256
+#define SK_MAX_TPW 32
 
 #define SK_MODE_PLAIN 0
 #define SK_MODE_PARTIAL 1
@@ -187,23 +188,38 @@ __global__ void gemm_skinny_reduce_kernel(void* __restrict__ out, int out_f32, c
 
 // How the product with a weight matrix [N, K] is cut: k-blocks per wavefront, splits of k over
 // workgroups, and weight tiles per workgroup.  A function of N and K alone.
+//
+// The kernel is bound by memory latency and bandwidth, so what counts is that all its workgroups are
+// resident at once (two per compute unit fit: no second round that runs half empty) and that there are
+// many of them.  Among the cuts with at most SK_RESIDENT_WGS workgroups the one with the fewest splits
+// that still gives SK_ENOUGH_WGS workgroups is taken (fewer partial sums to write and add), then the one
+// with the most workgroups.
 static void skinny_plan(int N, int K, int* kpw, int* splits, int* tiles_per_wg) {
     const int tiles = (N + SK_ROWS - 1) / SK_ROWS;
     const int kb_total = (K + SK_KB - 1) / SK_KB;
-    int best = 1;
+    int best_k = 1, best_s = (kb_total + SK_WAVES - 1) / SK_WAVES, best_t = SK_MAX_TPW;
+    int64_t best_w = -1;
+    bool best_enough = false;
     for (int c = SK_MAX_KPW; c >= 1; --c) {
         const int s = (kb_total + SK_WAVES * c - 1) / (SK_WAVES * c);
-        if ((int64_t)s * tiles >= SK_TARGET_WGS) { best = c; break; }
+        if (c > 1 && (kb_total + SK_WAVES * (c - 1) - 1) / (SK_WAVES * (c - 1)) == s)
+            continue;   // fewer k-blocks a wavefront give the same splits: more wavefronts busy
+        for (int t = 1; t <= SK_MAX_TPW; ++t) {
+            const int64_t w = (int64_t)s * ((tiles + t - 1) / t);
+            if (w > SK_RESIDENT_WGS && t < SK_MAX_TPW) continue;
+            const bool enough = w >= SK_ENOUGH_WGS;
+            bool better;
+            if (best_w < 0) better = true;
+            else if (enough != best_enough) better = enough;
+            else if (enough) better = s < best_s || (s == best_s && w > best_w);
+            else better = w > best_w || (w == best_w && s < best_s);
+            if (better) { best_k = c; best_s = s; best_t = t; best_w = w; best_enough = enough; }
+            break;   // larger t only gives fewer workgroups
+        }
     }
-    while (best > 1 && (kb_total + SK_WAVES * (best - 1) - 1) / (SK_WAVES * (best - 1)) ==
-                           (kb_total + SK_WAVES * best - 1) / (SK_WAVES * best))
-        --best;   // fewer k-blocks a wavefront for the same number of splits: more wavefronts busy
-    *kpw = best;
-    *splits = (kb_total + SK_WAVES * best - 1) / (SK_WAVES * best);
-    int64_t tpw = (int64_t)(*splits) * tiles / SK_TARGET_WGS;
-    if (tpw < 1) tpw = 1;
-    if (tpw > SK_MAX_TPW) tpw = SK_MAX_TPW;
-    *tiles_per_wg = (int)tpw;
+    *kpw = best_k;
+    *splits = best_s;
+    *tiles_per_wg = best_t;
 }
 
 extern "C" int zi_gemm_skinny_supported(int M, int N, int K, int64_t ldx, int64_t ldw) {

@@ -471,7 +471,7 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         return out
     bf = torch.bfloat16
     all_bf = x.dtype == bf and weight.dtype == bf and (bias is None or bias.dtype == bf)
-    if all_bf and (M <= SKINNY_MAX_ROWS or out.dtype == torch.float32) and _skinny_ok(x, weight, K, ldx, ldw):
+    if all_bf and (M <= FEW_ROWS or out.dtype == torch.float32) and _skinny_ok(x, weight, K, ldx, ldw):
         # few rows (decoding), or float32 output (logits): the hand-written matrix-core kernel
         lib = _lib.load()
         for m0 in range(0, M, SKINNY_MAX_ROWS):
@@ -494,10 +494,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
 
 
 def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether ``linear_sums`` takes this product: bfloat16, at most SKINNY_MAX_ROWS rows."""
+    """Whether ``linear_sums`` takes this product: bfloat16, at most FEW_ROWS rows."""
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.dim() != 2 or weight.dim() != 2:
         return False
-    if not (0 < x.shape[0] <= SKINNY_MAX_ROWS) or x.shape[1] != weight.shape[1]:
+    if not (0 < x.shape[0] <= FEW_ROWS) or x.shape[1] != weight.shape[1]:
         return False
     if (x.shape[1] > 1 and x.stride(1) != 1) or (weight.shape[1] > 1 and weight.stride(1) != 1):
         return False
@@ -510,11 +510,11 @@ def linear_splits(N: int, K: int) -> int:
 
 
 def linear_sums(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x[M,K] . weight[N,K]^T for M <= SKINNY_MAX_ROWS as float32 partial sums [S, M, N], S =
+    """x[M,K] . weight[N,K]^T for M <= FEW_ROWS as float32 partial sums [S, M, N], S =
     ``linear_splits(N, K)``, without bias: the consumer adds them in rising order."""
     _gpu("linear_sums", x, weight, out)
     if not linear_sums_supported(x, weight):
-        raise ValueError("linear_sums: needs bfloat16 x and weight, at most 64 rows, 16-byte aligned rows")
+        raise ValueError(f"linear_sums: needs bfloat16 x and weight, at most {FEW_ROWS} rows, 16-byte aligned rows")
     M, K = x.shape
     N = weight.shape[0]
     S = linear_splits(N, K)
@@ -568,7 +568,8 @@ def reduce_sums(sums: torch.Tensor, bias: Optional[torch.Tensor] = None, out: Op
     return out
 
 
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 64   # rows the few-rows kernel takes in one launch
+FEW_ROWS = 16          # up to here it beats the library product (x stays in registers over the weight tiles)
 _WORKSPACES = {}
 
 
