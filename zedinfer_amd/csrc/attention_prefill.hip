@@ -4,7 +4,8 @@
 // entry (16 a wavefront) and one query head.  It walks the keys the tile can see in
 // blocks of 64, aligned to absolute multiples of 64, so a query's blocks do not
 // depend on how its prompt was cut into steps.  Each block of keys and values is
-// staged once in LDS for the four wavefronts; scores and the P.V product run on
+// staged once in LDS for the four wavefronts (two buffers: the next block travels
+// from the cache into registers while the matrix cores work on this one); scores and the P.V product run on
 // v_mfma_f32_16x16x32_bf16 with float32 accumulation, the running softmax
 // (maximum, sum, rescaling) is float32, and s_j = (q . k_j) * scale is scaled after
 // the dot product (reference formulas:
@@ -54,8 +55,8 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     constexpr int VS = PF_BN + 8;       // LDS row stride of the transposed value tile
     constexpr int DT = D / 16;          // output tiles of 16 dims
     constexpr int CPR = DP / 8;         // 16-byte chunks per (padded) key row
-    __shared__ __attribute__((aligned(16))) uint16_t k_lds[PF_BN * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t v_lds[D * VS];
+    __shared__ __attribute__((aligned(16))) uint16_t k_lds[2 * PF_BN * KS];   // two buffers each
+    __shared__ __attribute__((aligned(16))) uint16_t v_lds[2 * D * VS];
 
     const int tile = blockIdx.x, h = blockIdx.y;
     const int g = h / (nh / nkv);
@@ -95,52 +96,87 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 
     const int vpart = ps < PF_BN ? ps : PF_BN;   // keys of one page inside a block
     const int gpp = vpart / 8;                   // 8-key groups of that part
+    constexpr int THREADS = PF_WAVES * ZI_WAVE;
+    constexpr int KPASS = PF_BN * CPR / THREADS;                      // 16-byte pieces of K a thread stages
+    constexpr int VPASS = (D * (PF_BN / 8) + THREADS - 1) / THREADS;  // and of V
+    uint4 kreg[KPASS], vreg[VPASS];
 
-    for (int kb = kb_begin; kb <= kmax; kb += PF_BN) {
-        __syncthreads();
-        // ---- stage the keys: row rho(kk) of the LDS tile takes key kb + kk
+    // global -> registers: the block of keys [kb, kb + 64)
+    auto fetch = [&](int kb) {
 #pragma unroll
-        for (int pass = 0; pass < PF_BN * CPR / (PF_WAVES * ZI_WAVE); ++pass) {
-            const int idx = pass * (PF_WAVES * ZI_WAVE) + tid;
+        for (int pass = 0; pass < KPASS; ++pass) {
+            const int idx = pass * THREADS + tid;
             const int kk = idx / CPR, c = idx % CPR;
             const int key = kb + kk;
-            uint4 val = make_uint4(0, 0, 0, 0);
+            kreg[pass] = make_uint4(0, 0, 0, 0);
             if (key <= kmax && c * 8 < D) {
                 const int pi = key / ps;
                 const int page = pi < max_pages ? bt[pi] : -1;
                 if (page >= 0 && page < num_pages)
-                    val = *reinterpret_cast<const uint4*>(
+                    kreg[pass] = *reinterpret_cast<const uint4*>(
                         kcache + (((int64_t)page * nkv + g) * ps + key % ps) * D + c * 8);
             }
-            const int rho = (2 * (kk / 32) + ((kk % 8) / 4)) * 16 + ((kk % 32) / 8) * 4 + kk % 4;
-            *reinterpret_cast<uint4*>(&k_lds[rho * KS + c * 8]) = val;
         }
-        // ---- stage the values, transposed: row dim, column key - kb
-        for (int idx = tid; idx < D * (PF_BN / 8); idx += PF_WAVES * ZI_WAVE) {
+#pragma unroll
+        for (int pass = 0; pass < VPASS; ++pass) {
+            const int idx = pass * THREADS + tid;
+            vreg[pass] = make_uint4(0, 0, 0, 0);
+            if (idx >= D * (PF_BN / 8)) continue;
+            const int part = idx / (D * gpp), rem = idx % (D * gpp);
+            const int dim = rem / gpp, s8 = rem % gpp;
+            const int key0 = kb + part * vpart + s8 * 8;
+            if (key0 <= kmax) {
+                const int pi = key0 / ps;
+                const int page = pi < max_pages ? bt[pi] : -1;
+                if (page >= 0 && page < num_pages)
+                    vreg[pass] = *reinterpret_cast<const uint4*>(
+                        vcache + (((int64_t)page * nkv + g) * D + dim) * ps + key0 % ps);
+            }
+        }
+    };
+    // registers -> LDS buffer `b`: key kb + kk goes to row rho(kk) of the key tile; values go in
+    // transposed, row dim, column key - kb
+    auto stash = [&](int kb, int b) {
+        uint16_t* kl = k_lds + b * (PF_BN * KS);
+        uint16_t* vl = v_lds + b * (D * VS);
+#pragma unroll
+        for (int pass = 0; pass < KPASS; ++pass) {
+            const int idx = pass * THREADS + tid;
+            const int kk = idx / CPR, c = idx % CPR;
+            const int rho = (2 * (kk / 32) + ((kk % 8) / 4)) * 16 + ((kk % 32) / 8) * 4 + kk % 4;
+            *reinterpret_cast<uint4*>(&kl[rho * KS + c * 8]) = kreg[pass];
+        }
+#pragma unroll
+        for (int pass = 0; pass < VPASS; ++pass) {
+            const int idx = pass * THREADS + tid;
+            if (idx >= D * (PF_BN / 8)) continue;
             const int part = idx / (D * gpp), rem = idx % (D * gpp);
             const int dim = rem / gpp, s8 = rem % gpp;
             const int col = part * vpart + s8 * 8;
             const int key0 = kb + col;
             pf_pack val;
-            val.u = make_uint4(0, 0, 0, 0);
-            if (key0 <= kmax) {
-                const int pi = key0 / ps;
-                const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages) {
-                    val.u = *reinterpret_cast<const uint4*>(
-                        vcache + (((int64_t)page * nkv + g) * D + dim) * ps + key0 % ps);
-                    if (key0 + 8 > kmax + 1) {   // slots past the last key may hold anything
+            val.u = vreg[pass];
+            if (key0 + 8 > kmax + 1) {   // slots past the last key may hold anything
 #pragma unroll
-                        for (int x = 0; x < 8; ++x)
-                            if (key0 + x > kmax) val.h[x] = 0;
-                    }
-                }
+                for (int x = 0; x < 8; ++x)
+                    if (key0 + x > kmax) val.h[x] = 0;
             }
-            *reinterpret_cast<uint4*>(&v_lds[dim * VS + col]) = val.u;
+            *reinterpret_cast<uint4*>(&vl[dim * VS + col]) = val.u;
         }
-        __syncthreads();
-        if (!wave_active || kb > wave_last || kb + PF_BN <= wave_lo) continue;
+    };
 
+    fetch(kb_begin);
+    stash(kb_begin, 0);
+    __syncthreads();
+    int cur = 0;
+    for (int kb = kb_begin; kb <= kmax; kb += PF_BN, cur ^= 1) {
+        // the next block travels from the cache into registers while this one is worked on; it goes
+        // into the other LDS buffer, which everyone has finished reading at the barrier before
+        const bool has_next = kb + PF_BN <= kmax;
+        if (has_next) fetch(kb + PF_BN);
+        const uint16_t* kl = k_lds + cur * (PF_BN * KS);
+        const uint16_t* vl = v_lds + cur * (D * VS);
+        if (wave_active && kb <= wave_last && kb + PF_BN > wave_lo) {
         // ---- scores of 64 keys for this lane's query
         pf_f32x4_t s[4];
 #pragma unroll
@@ -149,7 +185,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 #pragma unroll
             for (int dk = 0; dk < DK; ++dk) {
                 pf_pack a;
-                a.u = *reinterpret_cast<const uint4*>(&k_lds[(t * 16 + r) * KS + dk * 32 + j * 8]);
+                a.u = *reinterpret_cast<const uint4*>(&kl[(t * 16 + r) * KS + dk * 32 + j * 8]);
                 s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, qop[dk], s[t], 0, 0, 0);
             }
         }
@@ -191,9 +227,12 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 pf_pack a;
-                a.u = *reinterpret_cast<const uint4*>(&v_lds[(dd * 16 + r) * VS + b * 32 + j * 8]);
+                a.u = *reinterpret_cast<const uint4*>(&vl[(dd * 16 + r) * VS + b * 32 + j * 8]);
                 o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[b].b, o[dd], 0, 0, 0);
             }
+        }
+        if (has_next) stash(kb + PF_BN, cur ^ 1);
+        __syncthreads();
     }
     if (!qvalid) return;
     float l = lsum;

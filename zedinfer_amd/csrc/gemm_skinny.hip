@@ -19,12 +19,10 @@
 // the 8 up rows of the same columns), the tile's lanes exchange halves and write
 // act = up * gate / (1 + exp(-gate)) (reference: src/backend/ops/swiglu/cpu/swiglu_cpu.cpp:9-23).
 //
-// Operand layout.  For one MFMA the A operand is a 16 x 32 tile of w (lane l: row
-// l%16, eight consecutive k) and the B operand the matching 32 x 16 tile of x^T
-// (lane l: row l%16 of x, the same eight k).  Within a k-block of 128 the lane group
-// j = l/16 reads k in [32j, 32j+32) as four 16-byte loads and MFMA i consumes load i:
-// a permutation of k that both operands share, which turns every row's reads into
-// 256 contiguous bytes per k-block.
+// Operand layout.  For one MFMA the A operand is a 16 x 32 tile of w (lane l: row l%16, the eight
+// consecutive k starting at 8 * (l/16)) and the B operand the matching 32 x 16 tile of x^T (lane l: row
+// l%16 of x, the same eight k).  A k-block of 128 is four such MFMAs; each of a wavefront's load
+// instructions reads 64 contiguous bytes of each of its 16 rows.
 #include "zi_common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -48,19 +46,21 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4& v) {
     return c.b;
 }
 
-// The 64 bytes of row `row` this lane owns in k-block `kb` (zeros past K; K % 8 == 0).
+// The four 16-byte pieces of row `row` this lane owns in k-block `kb` (zeros past K; K % 8 == 0): piece c
+// holds k = kb*128 + c*32 + j*8 .. +8, so that one load instruction reads 64 contiguous bytes of each
+// of the wavefront's 16 rows.
 __device__ __forceinline__ void sk_load_row(uint4 (&dst)[4], const zi_bf16* row, int kb, int j, int K) {
-    const int k0 = kb * SK_KB + j * 32;
+    const int k0 = kb * SK_KB + j * 8;
 #pragma unroll
     for (int c = 0; c < 4; ++c)
-        dst[c] = (k0 + c * 8 < K) ? *reinterpret_cast<const uint4*>(row + k0 + c * 8) : make_uint4(0, 0, 0, 0);
+        dst[c] = (k0 + c * 32 < K) ? *reinterpret_cast<const uint4*>(row + k0 + c * 32) : make_uint4(0, 0, 0, 0);
 }
 
 template <int MT, int KPW>
 __global__ void __launch_bounds__(SK_WAVES* ZI_WAVE)
 gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* x, const zi_bf16* __restrict__ w,
                    const zi_bf16* __restrict__ bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
-                   int tiles_per_wg) {
+                   int tiles_per_wg, int vec_out) {
     constexpr bool XRES = (MT == 1);   // the slice of x stays in registers over the workgroup's tiles
     __shared__ f32x4_t red[2][SK_WAVES][MT][ZI_WAVE];
     const int lane = threadIdx.x & (ZI_WAVE - 1), wave = threadIdx.x / ZI_WAVE;
@@ -150,15 +150,45 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
                 if (j >= 2 || m >= M) continue;
                 const int col = tile * 8 + j * 4;     // N / 2 columns of output
                 zi_bf16* dst = (zi_bf16*)out + (int64_t)m * ldo + col;
+                float act[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (col + e < N / 2) zi_store(dst + e, up[e] * (s[e] / (1.f + expf(-s[e]))));
+                for (int e = 0; e < 4; ++e) act[e] = up[e] * (s[e] / (1.f + expf(-s[e])));
+                if (vec_out) {   // N % 16 == 0: the four columns exist
+                    uint2 pk;
+                    pk.x = (uint32_t)zi_float_to_bf16(act[0]) | ((uint32_t)zi_float_to_bf16(act[1]) << 16);
+                    pk.y = (uint32_t)zi_float_to_bf16(act[2]) | ((uint32_t)zi_float_to_bf16(act[3]) << 16);
+                    *reinterpret_cast<uint2*>(dst) = pk;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (col + e < N / 2) zi_store(dst + e, act[e]);
+                }
                 continue;
             }
             if (m >= M) continue;
+            const int nb = n0 + j * 4;   // this lane's four consecutive columns
+            if (nb + 3 < N && vec_out) {
+                if (mode == SK_MODE_PARTIAL) {
+                    *reinterpret_cast<f32x4_t*>((float*)out + ((int64_t)split * M + m) * N + nb) = s;
+                } else {
+                    if (bias) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) s[e] += zi_load(bias + nb + e);
+                    }
+                    if (out_f32) {
+                        *reinterpret_cast<f32x4_t*>((float*)out + (int64_t)m * ldo + nb) = s;
+                    } else {
+                        uint2 pk;
+                        pk.x = (uint32_t)zi_float_to_bf16(s[0]) | ((uint32_t)zi_float_to_bf16(s[1]) << 16);
+                        pk.y = (uint32_t)zi_float_to_bf16(s[2]) | ((uint32_t)zi_float_to_bf16(s[3]) << 16);
+                        *reinterpret_cast<uint2*>((zi_bf16*)out + (int64_t)m * ldo + nb) = pk;
+                    }
+                }
+                continue;
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int n = n0 + j * 4 + e;
+                const int n = nb + e;
                 if (n >= N) continue;
                 if (mode == SK_MODE_PARTIAL) {
                     ((float*)out)[((int64_t)split * M + m) * N + n] = s[e];
@@ -242,10 +272,10 @@ extern "C" int64_t zi_gemm_skinny_workspace(int M, int N, int K) {
 template <int MT>
 static void sk_launch(int kpw, dim3 grid, hipStream_t stream, void* out, int mode, int out_f32, const zi_bf16* x,
                       const zi_bf16* w, const zi_bf16* bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
-                      int tpw) {
+                      int tpw, int vec_out) {
 #define ZI_SK(KPW)                                                                                                  \
     gemm_skinny_kernel<MT, KPW><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, \
-                                                                         ldw, ldo, tpw)
+                                                                         ldw, ldo, tpw, vec_out)
     switch (kpw) {
         case 1: ZI_SK(1); break;
         case 2: ZI_SK(2); break;
@@ -294,9 +324,15 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
                    "gemm_skinny: the SwiGLU epilogue needs N %% 16 == 0 and a bfloat16 out of N/2 columns");
     }
     const zi_bf16* b = kmode == SK_MODE_PLAIN ? (const zi_bf16*)bias : nullptr;
+    // four columns go out as one store when every row of the destination keeps them aligned
+    int vec_out;
+    if (kmode == SK_MODE_PARTIAL) vec_out = N % 4 == 0 && ((uintptr_t)dst % 16) == 0;
+    else if (kmode == SK_MODE_SWIGLU) vec_out = ldo % 4 == 0 && ((uintptr_t)dst % 8) == 0;
+    else vec_out = ldo % 4 == 0 && ((uintptr_t)dst % (out_dt == ZI_F32 ? 16 : 8)) == 0;
     const int of32 = out_dt == ZI_F32;
 #define ZI_SKM(MT)                                                                                                  \
-    sk_launch<MT>(kpw, grid, stream, dst, kmode, of32, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo, tpw)
+    sk_launch<MT>(kpw, grid, stream, dst, kmode, of32, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo, tpw, \
+                  vec_out)
     switch (mt) {
         case 1: ZI_SKM(1); break;
         case 2: ZI_SKM(2); break;
