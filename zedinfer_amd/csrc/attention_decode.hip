@@ -90,6 +90,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     }
     if (chunk >= sp.count) return;
     const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
+    const int ps_shift = (ps & (ps - 1)) == 0 ? __ffs(ps) - 1 : -1;   // no division for the usual page sizes
     const int quarter = sp.len / DEC_WAVES;
     const int k_begin = sp.lo_al + chunk * sp.len + wave * quarter;
     const int k_end = (k_begin + quarter < p + 1) ? k_begin + quarter : p + 1;   // one past the wavefront's last key
@@ -107,7 +108,8 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     dec_f32x4_t o[DT];
 #pragma unroll
     for (int dd = 0; dd < DT; ++dd) o[dd] = dec_f32x4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, lsum = 0.f;
+    float m = -INFINITY, lsum = 0.f;   // m is in base-2 units: the maximum of s * scale * log2(e)
+    const float scale_log2 = scale * 1.4426950408889634f;
 
     for (int base = k_begin; base < k_end; base += DEC_BLOCK) {
         // ---- all loads of the block first: keys (4 tiles x DK) and values (DT x 2)
@@ -117,9 +119,9 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
             const int key = base + (tt / 2) * 32 + (r / 4) * 8 + (tt % 2) * 4 + (r % 4);
             const zi_bf16* kr = nullptr;
             if (key < k_end && key >= sp.lo) {
-                const int pi = key / ps;
+                const int pi = ps_shift >= 0 ? key >> ps_shift : key / ps;
                 const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages) kr = kcache + (((int64_t)page * nkv + kvh) * ps + key % ps) * D + j * 8;
+                if (page >= 0 && page < num_pages) kr = kcache + (((int64_t)page * nkv + kvh) * ps + (key - pi * ps)) * D + j * 8;
             }
 #pragma unroll
             for (int dk = 0; dk < DK; ++dk) {
@@ -132,9 +134,9 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
             const int key0 = base + b * 32 + j * 8;
             const zi_bf16* vr = nullptr;
             if (key0 < k_end && key0 + 8 > sp.lo) {
-                const int pi = key0 / ps;
+                const int pi = ps_shift >= 0 ? key0 >> ps_shift : key0 / ps;
                 const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages) vr = vcache + (((int64_t)page * nkv + kvh) * D + r) * ps + key0 % ps;
+                if (page >= 0 && page < num_pages) vr = vcache + (((int64_t)page * nkv + kvh) * D + r) * ps + (key0 - pi * ps);
             }
             const bool edge = key0 < sp.lo || key0 + 8 > k_end;
 #pragma unroll
@@ -159,13 +161,15 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
             for (int dk = 0; dk < DK; ++dk)
                 s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop[tt][dk].b, qop[dk], s[tt], 0, 0, 0);
         }
+        // softmax in base 2: t = s * scale * log2(e), p = 2^(t - m)
+        const bool whole = base >= sp.lo && base + DEC_BLOCK <= k_end;
         float mx = -INFINITY;
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int key = base + (tt / 2) * 32 + j * 8 + (tt % 2) * 4 + e;
-                const float v = (key >= sp.lo && key < k_end) ? s[tt][e] * scale : -INFINITY;
+                const float v = (whole || (key >= sp.lo && key < k_end)) ? s[tt][e] * scale_log2 : -INFINITY;
                 s[tt][e] = v;
                 mx = fmaxf(mx, v);
             }
@@ -173,18 +177,24 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = (m == -INFINITY) ? 0.f : __expf(m - m_use);
+        const float corr = __builtin_amdgcn_exp2f(m - m_use);      // 2^(-inf) = 0 before the first key
         m = m_new;
         float psum = 0.f;
-        dec_pack pb[2];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float pj = __expf(s[tt][e] - m_use);   // exp(-inf) = 0 for keys not seen
-                psum += pj;
-                pb[tt / 2].h[(tt % 2) * 4 + e] = zi_float_to_bf16(pj);
+                s[tt][e] = __builtin_amdgcn_exp2f(s[tt][e] - m_use);   // 0 for keys not seen
+                psum += s[tt][e];
             }
+        dec_pack pb[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            pb[b].u.x = zi_pack_bf16x2(s[2 * b][0], s[2 * b][1]);
+            pb[b].u.y = zi_pack_bf16x2(s[2 * b][2], s[2 * b][3]);
+            pb[b].u.z = zi_pack_bf16x2(s[2 * b + 1][0], s[2 * b + 1][1]);
+            pb[b].u.w = zi_pack_bf16x2(s[2 * b + 1][2], s[2 * b + 1][3]);
+        }
         lsum = lsum * corr + psum;
 #pragma unroll
         for (int dd = 0; dd < DT; ++dd) {
@@ -210,7 +220,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     float a[DEC_WAVES], L = 0.f;
 #pragma unroll
     for (int w = 0; w < DEC_WAVES; ++w) {
-        a[w] = (sm[w][r] == -INFINITY) ? 0.f : __expf(sm[w][r] - M);
+        a[w] = (sm[w][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sm[w][r] - M);
         L += a[w] * sl[w][r];
     }
     const bool final = sp.count == 1;
@@ -226,8 +236,8 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         if (r >= G) continue;
         if (final) {
             uint2 wv;
-            wv.x = (uint32_t)zi_float_to_bf16(acc[0] * inv) | ((uint32_t)zi_float_to_bf16(acc[1] * inv) << 16);
-            wv.y = (uint32_t)zi_float_to_bf16(acc[2] * inv) | ((uint32_t)zi_float_to_bf16(acc[3] * inv) << 16);
+            wv.x = zi_pack_bf16x2(acc[0] * inv, acc[1] * inv);
+            wv.y = zi_pack_bf16x2(acc[2] * inv, acc[3] * inv);
             *reinterpret_cast<uint2*>(out + (int64_t)t * ldo + (int64_t)(kvh * G + r) * D + dd * 16 + j * 4) = wv;
         } else {
             *reinterpret_cast<dec_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = acc;
@@ -253,7 +263,7 @@ attention_decode_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const floa
     const float mc = lane < sp.count ? part_ml[(slot0 + lane) * 2] : -INFINITY;
     const float lc = lane < sp.count ? part_ml[(slot0 + lane) * 2 + 1] : 0.f;
     const float M = zi_wave_max(mc);
-    const float wc = (mc == -INFINITY) ? 0.f : __expf(mc - M);
+    const float wc = (mc == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - M);   // maxima are in base-2 units
     float L = 0.f, acc[2] = {0.f, 0.f};
     for (int c0 = 0; c0 < sp.count; c0 += 8) {
         float po[8][2];   // eight chunks' loads are issued before the first is used

@@ -23,7 +23,7 @@
 // all banks.
 //
 // bfloat16; head_dim a multiple of 16 up to 128 (a head_dim that is no multiple of 32 is
-// padded with zeros for the score product); page size 8, 16, 32 or a multiple of 64.
+// padded with zeros for the score product); page size a power of two from 8.
 // Other shapes are the plain kernel's.
 #include "zi_common.h"
 
@@ -47,7 +47,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                          const int32_t* __restrict__ tile_entry, const int32_t* __restrict__ tile_off,
                          const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                          const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
-                         int max_pages, int num_pages, int nh, int nkv, int ps, int window, float scale) {
+                         int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DP = DK * 32;         // head_dim padded to a multiple of 32
@@ -77,7 +77,9 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     const bool qvalid = row < count;
     const int qrow = qvalid ? row : count - 1;
     const int qpos = pos0 + qrow;
+    const int wave_first = pos0 + ((wave * 16 < count) ? wave * 16 : count - 1);
     const int wave_last = pos0 + ((wave * 16 + 15 < count) ? wave * 16 + 15 : count - 1);
+    const float scale_log2 = scale * 1.4426950408889634f;
     const int wave_lo = (window > 0 && pos0 + wave * 16 - window + 1 > 0) ? pos0 + wave * 16 - window + 1 : 0;
     pf_bf16x8_t qop[DK];
     {
@@ -94,43 +96,58 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     for (int dd = 0; dd < DT; ++dd) o[dd] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, lsum = 0.f;
 
+    const int ps = 1 << ps_shift;
     const int vpart = ps < PF_BN ? ps : PF_BN;   // keys of one page inside a block
-    const int gpp = vpart / 8;                   // 8-key groups of that part
+    const int gpp = vpart / 8;                   // 8-key groups of that part (a power of two)
+    const int gshift = __ffs(gpp) - 1;
     constexpr int THREADS = PF_WAVES * ZI_WAVE;
     constexpr int KPASS = PF_BN * CPR / THREADS;                      // 16-byte pieces of K a thread stages
     constexpr int VPASS = (D * (PF_BN / 8) + THREADS - 1) / THREADS;  // and of V
     uint4 kreg[KPASS], vreg[VPASS];
+    // What a thread stages does not change from block to block: key row and 16-byte piece of K, and
+    // (dim, column) of V.  Page sizes are powers of two here: no division in the loop.
+    int k_kk[KPASS], k_c[KPASS], k_dst[KPASS], v_dim[VPASS], v_col[VPASS];
+#pragma unroll
+    for (int pass = 0; pass < KPASS; ++pass) {
+        const int idx = pass * THREADS + tid;
+        const int kk = idx / CPR, c = idx % CPR;
+        k_kk[pass] = kk;
+        k_c[pass] = c;
+        k_dst[pass] = ((2 * (kk / 32) + ((kk % 8) / 4)) * 16 + ((kk % 32) / 8) * 4 + kk % 4) * KS + c * 8;
+    }
+#pragma unroll
+    for (int pass = 0; pass < VPASS; ++pass) {
+        const int idx = pass * THREADS + tid;
+        const int part = (idx / D) >> gshift, rem = idx - part * (D << gshift);
+        v_dim[pass] = idx < D * (PF_BN / 8) ? rem >> gshift : -1;
+        v_col[pass] = part * vpart + (rem & (gpp - 1)) * 8;
+    }
+    const int ps_mask = ps - 1;
 
     // global -> registers: the block of keys [kb, kb + 64)
     auto fetch = [&](int kb) {
 #pragma unroll
         for (int pass = 0; pass < KPASS; ++pass) {
-            const int idx = pass * THREADS + tid;
-            const int kk = idx / CPR, c = idx % CPR;
-            const int key = kb + kk;
+            const int key = kb + k_kk[pass];
             kreg[pass] = make_uint4(0, 0, 0, 0);
-            if (key <= kmax && c * 8 < D) {
-                const int pi = key / ps;
+            if (key <= kmax && k_c[pass] * 8 < D) {
+                const int pi = key >> ps_shift;
                 const int page = pi < max_pages ? bt[pi] : -1;
                 if (page >= 0 && page < num_pages)
                     kreg[pass] = *reinterpret_cast<const uint4*>(
-                        kcache + (((int64_t)page * nkv + g) * ps + key % ps) * D + c * 8);
+                        kcache + ((((int64_t)page * nkv + g) << ps_shift) + (key & ps_mask)) * D + k_c[pass] * 8);
             }
         }
 #pragma unroll
         for (int pass = 0; pass < VPASS; ++pass) {
-            const int idx = pass * THREADS + tid;
             vreg[pass] = make_uint4(0, 0, 0, 0);
-            if (idx >= D * (PF_BN / 8)) continue;
-            const int part = idx / (D * gpp), rem = idx % (D * gpp);
-            const int dim = rem / gpp, s8 = rem % gpp;
-            const int key0 = kb + part * vpart + s8 * 8;
-            if (key0 <= kmax) {
-                const int pi = key0 / ps;
+            const int key0 = kb + v_col[pass];
+            if (v_dim[pass] >= 0 && key0 <= kmax) {
+                const int pi = key0 >> ps_shift;
                 const int page = pi < max_pages ? bt[pi] : -1;
                 if (page >= 0 && page < num_pages)
                     vreg[pass] = *reinterpret_cast<const uint4*>(
-                        vcache + (((int64_t)page * nkv + g) * D + dim) * ps + key0 % ps);
+                        vcache + ((((int64_t)page * nkv + g) * D + v_dim[pass]) << ps_shift) + (key0 & ps_mask));
             }
         }
     };
@@ -140,20 +157,11 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         uint16_t* kl = k_lds + b * (PF_BN * KS);
         uint16_t* vl = v_lds + b * (D * VS);
 #pragma unroll
-        for (int pass = 0; pass < KPASS; ++pass) {
-            const int idx = pass * THREADS + tid;
-            const int kk = idx / CPR, c = idx % CPR;
-            const int rho = (2 * (kk / 32) + ((kk % 8) / 4)) * 16 + ((kk % 32) / 8) * 4 + kk % 4;
-            *reinterpret_cast<uint4*>(&kl[rho * KS + c * 8]) = kreg[pass];
-        }
+        for (int pass = 0; pass < KPASS; ++pass) *reinterpret_cast<uint4*>(&kl[k_dst[pass]]) = kreg[pass];
 #pragma unroll
         for (int pass = 0; pass < VPASS; ++pass) {
-            const int idx = pass * THREADS + tid;
-            if (idx >= D * (PF_BN / 8)) continue;
-            const int part = idx / (D * gpp), rem = idx % (D * gpp);
-            const int dim = rem / gpp, s8 = rem % gpp;
-            const int col = part * vpart + s8 * 8;
-            const int key0 = kb + col;
+            if (v_dim[pass] < 0) continue;
+            const int key0 = kb + v_col[pass];
             pf_pack val;
             val.u = vreg[pass];
             if (key0 + 8 > kmax + 1) {   // slots past the last key may hold anything
@@ -161,7 +169,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                 for (int x = 0; x < 8; ++x)
                     if (key0 + x > kmax) val.h[x] = 0;
             }
-            *reinterpret_cast<uint4*>(&vl[dim * VS + col]) = val.u;
+            *reinterpret_cast<uint4*>(&vl[v_dim[pass] * VS + v_col[pass]]) = val.u;
         }
     };
 
@@ -189,33 +197,52 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                 s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, qop[dk], s[t], 0, 0, 0);
             }
         }
+        // softmax in base 2: t = s * scale * log2(e), p = 2^(t - m).  A block that every query of the
+        // wavefront sees whole (all but those on the diagonal and at a window's edge) needs no mask.
+        const bool whole = kb + PF_BN - 1 <= wave_first && (window <= 0 || kb > wave_last - window);
         float mx = -INFINITY;
+        if (whole) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
-                const bool vis = key <= qpos && (window <= 0 || key > qpos - window);
-                const float v = vis ? s[t][x] * scale : -INFINITY;
-                s[t][x] = v;
-                mx = fmaxf(mx, v);
-            }
+                for (int x = 0; x < 4; ++x) {
+                    s[t][x] *= scale_log2;
+                    mx = fmaxf(mx, s[t][x]);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
+                    const bool vis = key <= qpos && (window <= 0 || key > qpos - window);
+                    const float v = vis ? s[t][x] * scale_log2 : -INFINITY;
+                    s[t][x] = v;
+                    mx = fmaxf(mx, v);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = (m == -INFINITY) ? 0.f : __expf(m - m_use);
+        const float corr = __builtin_amdgcn_exp2f(m - m_use);      // 2^(-inf) = 0 before the first key
         m = m_new;
         float psum = 0.f;
-        pf_pack pb[2];
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                const float p = __expf(s[t][x] - m_use);    // exp(-inf) = 0 for masked keys
-                psum += p;
-                pb[t / 2].h[(t % 2) * 4 + x] = zi_float_to_bf16(p);
+                s[t][x] = __builtin_amdgcn_exp2f(s[t][x] - m_use);    // 0 for masked keys
+                psum += s[t][x];
             }
+        pf_pack pb[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            pb[b].u.x = zi_pack_bf16x2(s[2 * b][0], s[2 * b][1]);
+            pb[b].u.y = zi_pack_bf16x2(s[2 * b][2], s[2 * b][3]);
+            pb[b].u.z = zi_pack_bf16x2(s[2 * b + 1][0], s[2 * b + 1][1]);
+            pb[b].u.w = zi_pack_bf16x2(s[2 * b + 1][2], s[2 * b + 1][3]);
+        }
         lsum = lsum * corr + psum;
 #pragma unroll
         for (int dd = 0; dd < DT; ++dd) {
@@ -243,8 +270,8 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 #pragma unroll
     for (int dd = 0; dd < DT; ++dd) {
         uint2 w;
-        w.x = (uint32_t)zi_float_to_bf16(o[dd][0] * inv) | ((uint32_t)zi_float_to_bf16(o[dd][1] * inv) << 16);
-        w.y = (uint32_t)zi_float_to_bf16(o[dd][2] * inv) | ((uint32_t)zi_float_to_bf16(o[dd][3] * inv) << 16);
+        w.x = zi_pack_bf16x2(o[dd][0] * inv, o[dd][1] * inv);
+        w.y = zi_pack_bf16x2(o[dd][2] * inv, o[dd][3] * inv);
         *reinterpret_cast<uint2*>(orow + dd * 16 + j * 4) = w;
     }
 }
@@ -253,7 +280,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 extern "C" int zi_attention_prefill_supported(int dt, int nh, int nkv, int d, int page_size) {
     if (dt != ZI_BF16 || nkv <= 0 || nh <= 0 || nh % nkv) return 0;
     if (d < 16 || d > 128 || d % 16) return 0;
-    return page_size == 8 || page_size == 16 || page_size == 32 || (page_size > 0 && page_size % 64 == 0);
+    return page_size >= 8 && (page_size & (page_size - 1)) == 0;
 }
 
 extern "C" int zi_attention_prefill_tile() { return PF_BM; }
@@ -268,8 +295,8 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
                                     int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
                                     hipStream_t stream) {
     ZI_REQUIRE(zi_attention_prefill_supported(dt, nh, nkv, d, page_size),
-               "attention_prefill: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, page size 8/16/32 "
-               "or a multiple of 64): dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
+               "attention_prefill: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, page size a power "
+               "of two from 8): dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
     ZI_REQUIRE(num_tiles >= 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_prefill: bad sizes");
     ZI_REQUIRE(ldq >= (int64_t)nh * d && ldo >= (int64_t)nh * d && ldq % 8 == 0 && ldo % 4 == 0,
                "attention_prefill: bad row stride");
@@ -279,10 +306,12 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
     ZI_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
     if (num_tiles == 0) return 0;
     const dim3 grid(num_tiles, nh);
+    int ps_shift = 0;
+    while ((1 << ps_shift) < page_size) ++ps_shift;
 #define ZI_PF(DD)                                                                                              \
     attention_prefill_kernel<DD><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                                     \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
-        tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, page_size,  \
+        tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
         window, scale)
     switch (d) {
         case 16: ZI_PF(16); break;

@@ -25,6 +25,19 @@ __device__ __forceinline__ uint16_t zi_float_to_bf16(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// Two floats to two bfloat16 in one word (first in the low half), rounded to nearest even by the
+// hardware convert (v_cvt_pk_bf16_f32).
+typedef __attribute__((ext_vector_type(2))) __bf16 zi_bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float zi_f32x2_t;
+__device__ __forceinline__ uint32_t zi_pack_bf16x2(float a, float b) {
+    zi_f32x2_t v;
+    v[0] = a;
+    v[1] = b;
+    union { zi_bf16x2_t h; uint32_t u; } c;
+    c.h = __builtin_convertvector(v, zi_bf16x2_t);
+    return c.u;
+}
+
 __device__ __forceinline__ float zi_load(const float* p) { return *p; }
 __device__ __forceinline__ float zi_load(const zi_bf16* p) { return zi_bf16_to_float(p->bits); }
 __device__ __forceinline__ void zi_store(float* p, float v) { *p = v; }

@@ -408,7 +408,7 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
                       entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
-    of 16 up to 128, page size 8/16/32 or a multiple of 64).
+    of 16 up to 128, page size a power of two from 8).
 
     Entry e brings ``entry_len[e]`` tokens, rows ``entry_start[e]...`` of q, that continue a sequence
     holding ``entry_past[e]`` tokens whose block table is row e of ``block_tables``.  Tile i covers the
