@@ -1,9 +1,11 @@
 // Paged causal grouped-query attention for prompt portions on the matrix cores.
 //
-// A workgroup of four wavefronts owns a tile of 64 consecutive query tokens of one
-// entry (16 a wavefront) and one query head.  It walks the keys the tile can see in
-// blocks of 64, aligned to absolute multiples of 64, so a query's blocks do not
-// depend on how its prompt was cut into steps.  Each block of keys and values is
+// A workgroup of eight wavefronts owns a tile of 64 consecutive query tokens of one
+// entry and one query head: four sub-tiles of 16 queries, each shared by two
+// wavefronts that take alternate runs of 64 keys and merge their results at the end
+// (the longest chain of dependent work, a late tile's walk over all earlier keys, is
+// halved that way).  The tile's keys are walked in blocks of 128, aligned to absolute
+// multiples of 128, so a query's blocks do not depend on how its prompt was cut into steps.  Each block of keys and values is
 // staged once in LDS for the four wavefronts (two buffers: the next block travels
 // from the cache into registers while the matrix cores work on this one); scores and the P.V product run on
 // v_mfma_f32_16x16x32_bf16 with float32 accumulation, the running softmax
@@ -30,9 +32,11 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4_t;
 
-#define PF_WAVES 4
-#define PF_BM 64     // queries per workgroup
-#define PF_BN 64     // keys per block
+#define PF_KH 2                  // wavefronts that share a query sub-tile, each with its own 64 keys of a block
+#define PF_WAVES (4 * PF_KH)
+#define PF_BM 64                 // queries per workgroup
+#define PF_BN 64                 // keys per wavefront and block
+#define PF_BS (PF_BN * PF_KH)    // keys per block
 
 union pf_pack {
     uint4 u;
@@ -52,13 +56,14 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DP = DK * 32;         // head_dim padded to a multiple of 32
     constexpr int KS = DP + 8;          // LDS row stride of the key tile, in elements
-    constexpr int VS = PF_BN + 8;       // LDS row stride of the transposed value tile
+    constexpr int VS = PF_BS + 8;       // LDS row stride of the transposed value tile
     constexpr int DT = D / 16;          // output tiles of 16 dims
     constexpr int CPR = DP / 8;         // 16-byte chunks per (padded) key row
-    __shared__ __attribute__((aligned(16))) uint16_t k_lds[2 * PF_BN * KS];   // two buffers each
+    __shared__ __attribute__((aligned(16))) uint16_t k_lds[2 * PF_BS * KS];   // two buffers each
     __shared__ __attribute__((aligned(16))) uint16_t v_lds[2 * D * VS];
 
-    const int tile = blockIdx.x, h = blockIdx.y;
+    // tiles come heaviest first; all heads of a tile are dispatched before the next tile
+    const int tile = blockIdx.x / nh, h = blockIdx.x % nh;
     const int g = h / (nh / nkv);
     const int e = tile_entry[tile], off = tile_off[tile];
     const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
@@ -69,18 +74,19 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     const int pos0 = past + off;            // position of the tile's first query
     const int kmax = pos0 + count - 1;      // last key any query of the tile sees
     const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-    const int kb_begin = (lo_tile / PF_BN) * PF_BN;
+    const int kb_begin = (lo_tile / PF_BS) * PF_BS;
 
-    // this wavefront's queries
-    const int row = wave * 16 + r;
-    const bool wave_active = wave * 16 < count;
+    // this wavefront's queries (sub-tile qs) and its share of every block's keys (kh)
+    const int qs = wave % 4, kh = wave / 4;
+    const int row = qs * 16 + r;
+    const bool wave_active = qs * 16 < count;
     const bool qvalid = row < count;
     const int qrow = qvalid ? row : count - 1;
     const int qpos = pos0 + qrow;
-    const int wave_first = pos0 + ((wave * 16 < count) ? wave * 16 : count - 1);
-    const int wave_last = pos0 + ((wave * 16 + 15 < count) ? wave * 16 + 15 : count - 1);
+    const int wave_first = pos0 + ((qs * 16 < count) ? qs * 16 : count - 1);
+    const int wave_last = pos0 + ((qs * 16 + 15 < count) ? qs * 16 + 15 : count - 1);
     const float scale_log2 = scale * 1.4426950408889634f;
-    const int wave_lo = (window > 0 && pos0 + wave * 16 - window + 1 > 0) ? pos0 + wave * 16 - window + 1 : 0;
+    const int wave_lo = (window > 0 && pos0 + qs * 16 - window + 1 > 0) ? pos0 + qs * 16 - window + 1 : 0;
     pf_bf16x8_t qop[DK];
     {
         const zi_bf16* qr = q + (int64_t)(start + off + qrow) * ldq + (int64_t)h * D + j * 8;
@@ -97,12 +103,12 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     float m = -INFINITY, lsum = 0.f;
 
     const int ps = 1 << ps_shift;
-    const int vpart = ps < PF_BN ? ps : PF_BN;   // keys of one page inside a block
+    const int vpart = ps < PF_BS ? ps : PF_BS;   // keys of one page inside a block
     const int gpp = vpart / 8;                   // 8-key groups of that part (a power of two)
     const int gshift = __ffs(gpp) - 1;
     constexpr int THREADS = PF_WAVES * ZI_WAVE;
-    constexpr int KPASS = PF_BN * CPR / THREADS;                      // 16-byte pieces of K a thread stages
-    constexpr int VPASS = (D * (PF_BN / 8) + THREADS - 1) / THREADS;  // and of V
+    constexpr int KPASS = (PF_BS * CPR + THREADS - 1) / THREADS;      // 16-byte pieces of K a thread stages
+    constexpr int VPASS = (D * (PF_BS / 8) + THREADS - 1) / THREADS;  // and of V
     uint4 kreg[KPASS], vreg[VPASS];
     // What a thread stages does not change from block to block: key row and 16-byte piece of K, and
     // (dim, column) of V.  Page sizes are powers of two here: no division in the loop.
@@ -111,29 +117,32 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     for (int pass = 0; pass < KPASS; ++pass) {
         const int idx = pass * THREADS + tid;
         const int kk = idx / CPR, c = idx % CPR;
-        k_kk[pass] = kk;
+        const int k64 = kk % PF_BN;   // the 64 keys of one wavefront are permuted among themselves
+        k_kk[pass] = idx < PF_BS * CPR ? kk : -1;
         k_c[pass] = c;
-        k_dst[pass] = ((2 * (kk / 32) + ((kk % 8) / 4)) * 16 + ((kk % 32) / 8) * 4 + kk % 4) * KS + c * 8;
+        k_dst[pass] = ((kk / PF_BN) * PF_BN + (2 * (k64 / 32) + ((k64 % 8) / 4)) * 16 + ((k64 % 32) / 8) * 4 + k64 % 4) * KS +
+                      c * 8;
     }
 #pragma unroll
     for (int pass = 0; pass < VPASS; ++pass) {
         const int idx = pass * THREADS + tid;
         const int part = (idx / D) >> gshift, rem = idx - part * (D << gshift);
-        v_dim[pass] = idx < D * (PF_BN / 8) ? rem >> gshift : -1;
+        v_dim[pass] = idx < D * (PF_BS / 8) ? rem >> gshift : -1;
         v_col[pass] = part * vpart + (rem & (gpp - 1)) * 8;
     }
     const int ps_mask = ps - 1;
 
     // global -> registers: the block of keys [kb, kb + 64)
     auto fetch = [&](int kb) {
+        const bool inside = kb + PF_BS - 1 <= kmax;    // every key of the block exists (all blocks but the last)
 #pragma unroll
         for (int pass = 0; pass < KPASS; ++pass) {
             const int key = kb + k_kk[pass];
             kreg[pass] = make_uint4(0, 0, 0, 0);
-            if (key <= kmax && k_c[pass] * 8 < D) {
+            if (k_kk[pass] >= 0 && (inside || key <= kmax) && (D % 32 == 0 || k_c[pass] * 8 < D)) {
                 const int pi = key >> ps_shift;
                 const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages)
+                if ((unsigned)page < (unsigned)num_pages)
                     kreg[pass] = *reinterpret_cast<const uint4*>(
                         kcache + ((((int64_t)page * nkv + g) << ps_shift) + (key & ps_mask)) * D + k_c[pass] * 8);
             }
@@ -142,10 +151,10 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         for (int pass = 0; pass < VPASS; ++pass) {
             vreg[pass] = make_uint4(0, 0, 0, 0);
             const int key0 = kb + v_col[pass];
-            if (v_dim[pass] >= 0 && key0 <= kmax) {
+            if (v_dim[pass] >= 0 && (inside || key0 <= kmax)) {
                 const int pi = key0 >> ps_shift;
                 const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages)
+                if ((unsigned)page < (unsigned)num_pages)
                     vreg[pass] = *reinterpret_cast<const uint4*>(
                         vcache + ((((int64_t)page * nkv + g) * D + v_dim[pass]) << ps_shift) + (key0 & ps_mask));
             }
@@ -154,22 +163,27 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     // registers -> LDS buffer `b`: key kb + kk goes to row rho(kk) of the key tile; values go in
     // transposed, row dim, column key - kb
     auto stash = [&](int kb, int b) {
-        uint16_t* kl = k_lds + b * (PF_BN * KS);
+        uint16_t* kl = k_lds + b * (PF_BS * KS);
         uint16_t* vl = v_lds + b * (D * VS);
 #pragma unroll
-        for (int pass = 0; pass < KPASS; ++pass) *reinterpret_cast<uint4*>(&kl[k_dst[pass]]) = kreg[pass];
+        for (int pass = 0; pass < KPASS; ++pass)
+            if (k_kk[pass] >= 0) *reinterpret_cast<uint4*>(&kl[k_dst[pass]]) = kreg[pass];
+        if (kb + PF_BS - 1 <= kmax) {     // all blocks but the last: nothing to mask
 #pragma unroll
-        for (int pass = 0; pass < VPASS; ++pass) {
-            if (v_dim[pass] < 0) continue;
-            const int key0 = kb + v_col[pass];
-            pf_pack val;
-            val.u = vreg[pass];
-            if (key0 + 8 > kmax + 1) {   // slots past the last key may hold anything
+            for (int pass = 0; pass < VPASS; ++pass)
+                if (v_dim[pass] >= 0) *reinterpret_cast<uint4*>(&vl[v_dim[pass] * VS + v_col[pass]]) = vreg[pass];
+        } else {
+#pragma unroll
+            for (int pass = 0; pass < VPASS; ++pass) {
+                if (v_dim[pass] < 0) continue;
+                const int key0 = kb + v_col[pass];
+                pf_pack val;
+                val.u = vreg[pass];
 #pragma unroll
                 for (int x = 0; x < 8; ++x)
-                    if (key0 + x > kmax) val.h[x] = 0;
+                    if (key0 + x > kmax) val.h[x] = 0;    // slots past the last key may hold anything
+                *reinterpret_cast<uint4*>(&vl[v_dim[pass] * VS + v_col[pass]]) = val.u;
             }
-            *reinterpret_cast<uint4*>(&vl[v_dim[pass] * VS + v_col[pass]]) = val.u;
         }
     };
 
@@ -177,13 +191,14 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     stash(kb_begin, 0);
     __syncthreads();
     int cur = 0;
-    for (int kb = kb_begin; kb <= kmax; kb += PF_BN, cur ^= 1) {
+    for (int kb0 = kb_begin; kb0 <= kmax; kb0 += PF_BS, cur ^= 1) {
         // the next block travels from the cache into registers while this one is worked on; it goes
         // into the other LDS buffer, which everyone has finished reading at the barrier before
-        const bool has_next = kb + PF_BN <= kmax;
-        if (has_next) fetch(kb + PF_BN);
-        const uint16_t* kl = k_lds + cur * (PF_BN * KS);
-        const uint16_t* vl = v_lds + cur * (D * VS);
+        const bool has_next = kb0 + PF_BS <= kmax;
+        if (has_next) fetch(kb0 + PF_BS);
+        const int kb = kb0 + kh * PF_BN;      // this wavefront's 64 keys of the block
+        const uint16_t* kl = k_lds + cur * (PF_BS * KS) + kh * (PF_BN * KS);
+        const uint16_t* vl = v_lds + cur * (D * VS) + kh * PF_BN;
         if (wave_active && kb <= wave_last && kb + PF_BN > wave_lo) {
         // ---- scores of 64 keys for this lane's query
         pf_f32x4_t s[4];
@@ -244,9 +259,11 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
             pb[b].u.w = zi_pack_bf16x2(s[2 * b + 1][2], s[2 * b + 1][3]);
         }
         lsum = lsum * corr + psum;
+        if (__any(corr != 1.f)) {     // the running maximum seldom moves after the first blocks
 #pragma unroll
-        for (int dd = 0; dd < DT; ++dd) {
-            o[dd][0] *= corr; o[dd][1] *= corr; o[dd][2] *= corr; o[dd][3] *= corr;
+            for (int dd = 0; dd < DT; ++dd) {
+                o[dd][0] *= corr; o[dd][1] *= corr; o[dd][2] *= corr; o[dd][3] *= corr;
+            }
         }
         // ---- o^T += V^T . P^T
 #pragma unroll
@@ -258,13 +275,45 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                 o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[b].b, o[dd], 0, 0, 0);
             }
         }
-        if (has_next) stash(kb + PF_BN, cur ^ 1);
+        if (has_next) stash(kb0 + PF_BS, cur ^ 1);
         __syncthreads();
     }
-    if (!qvalid) return;
     float l = lsum;
     l += __shfl_xor(l, 16, ZI_WAVE);
     l += __shfl_xor(l, 32, ZI_WAVE);
+    if (PF_KH > 1) {
+        // the wavefronts of a query sub-tile merge their (maximum, sum, output) through LDS, in the order
+        // of the wavefronts; nobody reads the key tiles any more
+        float* mo = reinterpret_cast<float*>(k_lds);                 // [kh-1][qs][DT][64][4]
+        float* ml = mo + (PF_KH - 1) * 4 * DT * ZI_WAVE * 4;         // [kh-1][qs][64][2]
+        if (kh > 0) {
+            float* dst = mo + ((kh - 1) * 4 + qs) * (DT * ZI_WAVE * 4);
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(dst + (dd * ZI_WAVE + lane) * 4) = o[dd];
+            ml[(((kh - 1) * 4 + qs) * ZI_WAVE + lane) * 2] = m;
+            ml[(((kh - 1) * 4 + qs) * ZI_WAVE + lane) * 2 + 1] = l;
+        }
+        __syncthreads();
+        if (kh > 0) return;
+#pragma unroll
+        for (int k2 = 1; k2 < PF_KH; ++k2) {
+            const float* src = mo + ((k2 - 1) * 4 + qs) * (DT * ZI_WAVE * 4);
+            const float m2 = ml[(((k2 - 1) * 4 + qs) * ZI_WAVE + lane) * 2];
+            const float l2 = ml[(((k2 - 1) * 4 + qs) * ZI_WAVE + lane) * 2 + 1];
+            const float mm = fmaxf(m, m2);
+            const float mu = (mm == -INFINITY) ? 0.f : mm;
+            const float a1 = __builtin_amdgcn_exp2f(m - mu), a2 = __builtin_amdgcn_exp2f(m2 - mu);
+            l = l * a1 + l2 * a2;
+            m = mm;
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) {
+                const pf_f32x4_t v = *reinterpret_cast<const pf_f32x4_t*>(src + (dd * ZI_WAVE + lane) * 4);
+                o[dd][0] = o[dd][0] * a1 + v[0] * a2; o[dd][1] = o[dd][1] * a1 + v[1] * a2;
+                o[dd][2] = o[dd][2] * a1 + v[2] * a2; o[dd][3] = o[dd][3] * a1 + v[3] * a2;
+            }
+        }
+    }
+    if (!qvalid) return;
     const float inv = 1.f / l;
     zi_bf16* orow = out + (int64_t)(start + off + row) * ldo + (int64_t)h * D;
 #pragma unroll
@@ -305,7 +354,8 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
                "attention_prefill: q, out and the caches must be aligned to 16 bytes");
     ZI_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
     if (num_tiles == 0) return 0;
-    const dim3 grid(num_tiles, nh);
+    ZI_REQUIRE((int64_t)num_tiles * nh < (1ll << 31), "attention_prefill: too many tiles");
+    const dim3 grid(num_tiles * nh);
     int ps_shift = 0;
     while ((1 << ps_shift) < page_size) ++ps_shift;
 #define ZI_PF(DD)                                                                                              \
