@@ -120,6 +120,8 @@ def main():
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the 2,048-token prefill (for profiling) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -148,6 +150,12 @@ def main():
         return make
 
     V = cfg.vocab_size
+    if args.prefill_only:
+        pms = measure_prefill(factory(1), V)
+        fl = prefill_flops(shape, args.layers, PROMPT)
+        print(json.dumps({"prefill": {"value": round(PROMPT / pms * 1000.0, 1), "tokens": PROMPT, "ms": round(pms, 3),
+                                      "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}}))
+        return 0
     tps, ms_step, ctx_mid = measure_decode(factory(args.batch), args.batch, args.steps, args.warmup, V)
     need = decode_bytes(shape, args.layers, args.batch, ctx_mid, el)
     achieved = need / (ms_step / 1000.0) / 1e9
