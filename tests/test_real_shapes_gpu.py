@@ -1,0 +1,73 @@
+"""Two layers of the Qwen2.5-1.5B and 7B layer shapes (real widths, head counts and groups; a smaller
+vocabulary and two layers so that the plain implementation stays affordable on the CPU) against the plain
+implementation: a prompt in portions, then decoded tokens, alone and beside a second request."""
+import pytest
+import torch
+
+import traces
+from plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {
+    "1.5B": dict(hidden_size=1536, intermediate_size=8960, num_attention_heads=12, num_key_value_heads=2,
+                 head_dim=128, tie_word_embeddings=True),
+    "7B": dict(hidden_size=3584, intermediate_size=18944, num_attention_heads=28, num_key_value_heads=4,
+               head_dim=128, tie_word_embeddings=False),
+}
+
+
+@pytest.fixture(scope="module", params=list(SHAPES))
+def model(request, tmp_path_factory):
+    from zedinfer_amd.config import Qwen2Config
+    from zedinfer_amd.models import expected_weights
+    from zedinfer_amd.models.qwen2 import qwen2_forward_config
+    from zedinfer_amd.weights import write_model_folder
+    cfgd = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=4099, max_position_embeddings=4096,
+                num_hidden_layers=2, rope_theta=1000000.0, rms_norm_eps=1e-6, use_sliding_window=False,
+                torch_dtype="float32", eos_token_id=4098, **SHAPES[request.param])
+    cfg = Qwen2Config.from_dict(cfgd)
+    folder = str(tmp_path_factory.mktemp("real" + request.param))
+    write_model_folder(folder, cfg, expected_weights(qwen2_forward_config(cfg)), seed=7, dtype=torch.float32,
+                       noisy_norms=True)
+    pcfg, w = plain.load_folder(folder)
+    reqs = {"p": traces.random_tokens(4099, 330, seed=1), "q": traces.random_tokens(4099, 97, seed=2)}
+    ref = {rid: plain.forward(pcfg, w, toks) for rid, toks in reqs.items()}
+    return dict(folder=folder, requests=reqs, reference=ref)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_real_layer_shapes_match_plain(model, dtype):
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    engine = Engine.from_folder(model["folder"], dtype, SchedulerConfig(num_kv_blocks=40, kv_block_size=16,
+                                                                        max_batch_requests=4))
+    reqs = model["requests"]
+    p, q = reqs["p"], reqs["q"]
+    want = lambda n: list(range(n))   # noqa: E731
+    steps = [
+        {"step": 0, "entries": [{"id": "p", "tokens": p[:200], "want": want(200)}], "end": []},
+        {"step": 1, "entries": [{"id": "p", "tokens": p[200:270], "want": want(70)},
+                                {"id": "q", "tokens": q[:65], "want": want(65)}], "end": []},
+        {"step": 2, "entries": [{"id": "p", "tokens": p[270:273], "want": want(3)},
+                                {"id": "q", "tokens": q[65:66], "want": [0]}], "end": []},
+    ]
+    fp, fq = 273, 66
+    while fq < len(q):          # both decode, token by token; q ends first and p goes on alone
+        steps.append({"step": len(steps), "entries": [{"id": "p", "tokens": p[fp:fp + 1], "want": [0]},
+                                                      {"id": "q", "tokens": q[fq:fq + 1], "want": [0]}],
+                      "end": ["q"] if fq == len(q) - 1 else []})
+        fp, fq = fp + 1, fq + 1
+    while fp < len(p):
+        steps.append({"step": len(steps), "entries": [{"id": "p", "tokens": p[fp:fp + 1], "want": [0]}],
+                      "end": ["p"] if fp == len(p) - 1 else []})
+        fp += 1
+    out = traces.run_in_process(engine, steps)
+    worst, mean, scale, rows, where = traces.compare(steps, out, model["reference"], reqs)
+    print(f"[{dtype}] rows={rows} worst={worst:.3e} mean={mean:.3e} scale={scale:.3e} at {where}")
+    assert rows == len(p) + len(q)
+    if dtype == "float32":
+        assert worst <= 3e-4 * max(1.0, scale), where
+    else:
+        assert engine.graph_replays > 10
+        assert worst <= 0.06 * scale and mean <= 0.012 * scale, where
