@@ -35,6 +35,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 #define SK_RESIDENT_WGS 480   // workgroups that are surely resident at once (256 compute units, two each)
 #define SK_ENOUGH_WGS 256
 #define SK_MAX_TPW 32
+#define SK_DEEP_RING 0    // three tiles in flight per workgroup measured slower than two (14.3 -> 16.1 us for 17920 x 1536)
 
 #define SK_MODE_PLAIN 0
 #define SK_MODE_PARTIAL 1
@@ -56,7 +57,7 @@ __device__ __forceinline__ void sk_load_row(uint4 (&dst)[4], const zi_bf16* row,
         dst[c] = (k0 + c * 32 < K) ? *reinterpret_cast<const uint4*>(row + k0 + c * 32) : make_uint4(0, 0, 0, 0);
 }
 
-template <int MT, int KPW>
+template <int MT, int KPW, int NB>
 __global__ void __launch_bounds__(SK_WAVES* ZI_WAVE)
 gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* x, const zi_bf16* __restrict__ w,
                    const zi_bf16* __restrict__ bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
@@ -86,28 +87,20 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
             else xr[i][0] = xr[i][1] = xr[i][2] = xr[i][3] = make_uint4(0, 0, 0, 0);
         }
     }
-    uint4 a_next[KPW][4];
-    {
-        const int nrow = (tile_lo * SK_ROWS + r < N) ? tile_lo * SK_ROWS + r : N - 1;
+    // the weight rows of up to NB tiles are in flight at once: a ring of register buffers
+    uint4 ring[NB][KPW][4];
 #pragma unroll
-        for (int i = 0; i < KPW; ++i) {
-            if (kb0 + i < kb_total) sk_load_row(a_next[i], w + (int64_t)nrow * ldw, kb0 + i, j, K);
-            else a_next[i][0] = a_next[i][1] = a_next[i][2] = a_next[i][3] = make_uint4(0, 0, 0, 0);
-        }
-    }
-    int buf = 0;
-    for (int tile = tile_lo; tile < tile_hi; ++tile) {
-        uint4 a[KPW][4];
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int i = 0; i < KPW; ++i) ring[b][i][0] = ring[b][i][1] = ring[b][i][2] = ring[b][i][3] = make_uint4(0, 0, 0, 0);
+    auto issue = [&](uint4 (&dst)[KPW][4], int tile) {
+        const int nrow = (tile * SK_ROWS + r < N) ? tile * SK_ROWS + r : N - 1;
 #pragma unroll
         for (int i = 0; i < KPW; ++i)
-#pragma unroll
-            for (int c = 0; c < 4; ++c) a[i][c] = a_next[i][c];
-        if (tile + 1 < tile_hi) {
-            const int nrow = ((tile + 1) * SK_ROWS + r < N) ? (tile + 1) * SK_ROWS + r : N - 1;
-#pragma unroll
-            for (int i = 0; i < KPW; ++i)
-                if (kb0 + i < kb_total) sk_load_row(a_next[i], w + (int64_t)nrow * ldw, kb0 + i, j, K);
-        }
+            if (kb0 + i < kb_total) sk_load_row(dst[i], w + (int64_t)nrow * ldw, kb0 + i, j, K);
+    };
+    int buf = 0;
+    auto process = [&](uint4 (&a)[KPW][4], int tile) {
         f32x4_t acc[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -200,6 +193,18 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
             }
         }
         buf ^= 1;
+    };
+#pragma unroll
+    for (int b = 0; b < NB - 1; ++b)
+        if (tile_lo + b < tile_hi) issue(ring[b], tile_lo + b);
+    for (int tile = tile_lo; tile < tile_hi; tile += NB) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            if (tile + b >= tile_hi) break;
+            // the buffer that was worked on last takes the tile NB - 1 ahead
+            if (tile + b + NB - 1 < tile_hi) issue(ring[(b + NB - 1) % NB], tile + b + NB - 1);
+            process(ring[b], tile + b);
+        }
     }
 }
 
@@ -274,8 +279,14 @@ static void sk_launch(int kpw, dim3 grid, hipStream_t stream, void* out, int mod
                       const zi_bf16* w, const zi_bf16* bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
                       int tpw, int vec_out) {
 #define ZI_SK(KPW)                                                                                                  \
-    gemm_skinny_kernel<MT, KPW><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, \
-                                                                         ldw, ldo, tpw, vec_out)
+    do {                                                                                                            \
+        if (MT == 1 && KPW <= 3 && tpw >= 3 && SK_DEEP_RING)                                                                     \
+            gemm_skinny_kernel<MT, KPW, (MT == 1 && KPW <= 3) ? 3 : 2><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(     \
+                out, mode, out_f32, x, w, bias, M, N, K, ldx, ldw, ldo, tpw, vec_out);                              \
+        else                                                                                                        \
+            gemm_skinny_kernel<MT, KPW, 2><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, \
+                                                                                   K, ldx, ldw, ldo, tpw, vec_out); \
+    } while (0)
     switch (kpw) {
         case 1: ZI_SK(1); break;
         case 2: ZI_SK(2); break;
