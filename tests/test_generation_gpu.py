@@ -237,3 +237,32 @@ def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype):
     ref = plain.forward(tiny["cfg"], tiny["weights"], toks["d"][:fed["d"]])
     tol = 2e-4 if dtype == "float32" else 0.06 * float(ref.abs().max())
     assert float((last[0].cpu() - ref[fed["d"] - 1]).abs().max()) < tol
+
+
+def test_decode_graphs_with_the_library_product(tiny):
+    """More than 16 decoding requests: the matrix products go to the library, inside the captured
+    graph.  Every replay is checked against eager launches, with eager prompt steps between them."""
+    from zedinfer_amd.engine import StepEntry
+    V = tiny["cfg"]["vocab_size"]
+    fast = engine(tiny, "bfloat16", max_batch_requests=24, num_kv_blocks=128).engine
+    slow = engine(tiny, "bfloat16", max_batch_requests=24, num_kv_blocks=128).engine
+    slow.use_graphs = False
+    names = [f"r{i}" for i in range(20)]
+    toks = {r: traces.random_tokens(V, 40, seed=80 + i) for i, r in enumerate(names)}
+    seqs = {(e, r): e.open(r) for e in (fast, slow) for r in names}
+    fed = {r: 0 for r in names}
+
+    def both(plan):
+        outs = []
+        for eng in (fast, slow):
+            outs.append(eng.step([StepEntry(seqs[(eng, r)], toks[r][fed[r]:fed[r] + n], [n - 1]) for r, n in plan]))
+        for r, n in plan:
+            fed[r] += n
+        assert torch.equal(outs[0], outs[1]), (plan[0], len(plan))
+
+    both([(r, 5 + i % 4) for i, r in enumerate(names)])
+    for step in range(12):
+        both([(r, 1) for r in names])
+        if step % 4 == 1:
+            both([(names[0], 3), (names[1], 1)])      # an eager mixed step between the replays
+    assert fast.graph_replays >= 8

@@ -242,15 +242,20 @@ def test_linear_skinny_row_does_not_depend_on_batch(ops):
     """The decode-time product cuts k by the weight's shape alone: a row's result is bit-identical
     whether 1, 8 or 64 rows ride along."""
     x, w = rnd(64, 1536, dtype=torch.bfloat16, seed=1), rnd(2048, 1536, dtype=torch.bfloat16, scale=0.05, seed=2)
+    # up to 16 rows run on one kernel, 17 to 64 on another: within each a row does not depend on the others
     full = ops.linear(x, w, out_dtype=torch.float32)
-    for m in (1, 8, 17):
-        part = ops.linear(x[:m].contiguous(), w, out_dtype=torch.float32)
-        assert torch.equal(full[:m], part)
-    # with bfloat16 output up to 16 rows run on the same kernel (more rows go to the library product)
+    for m in (17, 40):
+        assert torch.equal(full[:m], ops.linear(x[:m].contiguous(), w, out_dtype=torch.float32))
+    few = ops.linear(x[:16].contiguous(), w, out_dtype=torch.float32)
+    for m in (1, 8):
+        assert torch.equal(few[:m], ops.linear(x[:m].contiguous(), w, out_dtype=torch.float32))
+    torch.testing.assert_close(few, full[:16], atol=1e-3, rtol=1e-3)
     assert torch.equal(ops.linear(x[:16].contiguous(), w)[:3], ops.linear(x[:3].contiguous(), w))
-    assert torch.equal(ops.linear(x[:3].contiguous(), w), full[:3].to(torch.bfloat16))
+    assert torch.equal(ops.linear(x, w)[:20], ops.linear(x[:20].contiguous(), w))
+    assert torch.equal(ops.linear(x[:3].contiguous(), w), few[:3].to(torch.bfloat16))
     x2, w2 = rnd(64, 8960, dtype=torch.bfloat16, seed=3), rnd(1536, 8960, dtype=torch.bfloat16, scale=0.02, seed=4)
-    assert torch.equal(ops.linear(x2, w2, out_dtype=torch.float32)[5:6], ops.linear(x2[5:6].contiguous(), w2, out_dtype=torch.float32))
+    assert torch.equal(ops.linear(x2[:16].contiguous(), w2, out_dtype=torch.float32)[5:6],
+                       ops.linear(x2[5:6].contiguous(), w2, out_dtype=torch.float32))
 
 
 def test_linear_f32_row_does_not_depend_on_batch(ops):
@@ -452,26 +457,31 @@ def test_attention_prefill_refuses_other_shapes(ops):
 
 # ---- the few-rows product's partial sums and the kernels that consume them ------------------------
 @pytest.mark.parametrize("M,N,K", [(1, 2048, 1536), (8, 1536, 8960), (16, 17920, 1536), (13, 1536, 1536),
-                                   (16, 2048, 1536), (5, 176, 64), (11, 1000, 96), (3, 48, 520), (2, 3584, 18944)])
+                                   (16, 2048, 1536), (5, 176, 64), (11, 1000, 96), (3, 48, 520), (2, 3584, 18944),
+                                   (17, 1536, 1536), (64, 2048, 1536), (33, 1000, 96), (40, 1536, 8960), (64, 17920, 1536),
+                                   (20, 100, 72)])
 def test_linear_sums(ops, M, N, K):
     bf = torch.bfloat16
-    assert not ops.linear_sums_supported(rnd(17, K, dtype=bf), rnd(N, K, dtype=bf))
+    assert not ops.linear_sums_supported(rnd(65, K, dtype=bf), rnd(N, K, dtype=bf))
     x, w = rnd(M, K, dtype=bf, seed=1), rnd(N, K, dtype=bf, scale=0.05, seed=2)
     b = rnd(N, dtype=bf, seed=3)
     sums = ops.linear_sums(x, w)
-    assert sums.shape == (ops.linear_splits(N, K), M, N) and sums.dtype == torch.float32
+    assert sums.shape == (ops.linear_splits(M, N, K), M, N) and sums.dtype == torch.float32
     ref = x.float() @ w.float().t()
     torch.testing.assert_close(sums.sum(0), ref, atol=2e-3, rtol=2e-3)
     # the consumer-side sum is what linear() itself gives, bit for bit
     assert torch.equal(ops.reduce_sums(sums, b), ops.linear(x, w, b))
-    # a row's sums do not depend on the rows that ride along
-    if M > 1:
+    # a row's sums do not depend on the rows that ride along (up to 16 rows, and from 17 rows on)
+    if 1 < M <= 16:
         alone = ops.linear_sums(x[M - 1:M].contiguous(), w)
         assert torch.equal(alone[:, 0], sums[:, M - 1])
+    if M > 17:
+        fewer = ops.linear_sums(x[:17].contiguous(), w)
+        assert torch.equal(fewer[:, 16], sums[:, 16])
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 8960, 1536), (8, 8960, 1536), (14, 176, 64), (16, 256, 96), (2, 208, 80),
-                                   (4, 18944, 3584)])
+                                   (4, 18944, 3584), (64, 8960, 1536), (24, 176, 64), (50, 18944, 3584)])
 def test_linear_swiglu(ops, M, I, K):
     from zedinfer_amd.parts.feed_forward import interleave_rows
     bf = torch.bfloat16
@@ -485,7 +495,7 @@ def test_linear_swiglu(ops, M, I, K):
         out = ops.linear_swiglu(x, w)
         torch.testing.assert_close(out.float(), ref, atol=2e-2, rtol=2e-2)
     else:
-        assert ops.linear_splits(2 * I, K) > 1
+        assert ops.linear_splits(M, 2 * I, K) > 1
     # the same through partial sums and the SwiGLU kernel, and through the interleaved 2-D form
     sums = ops.linear_sums(x, w)
     out2 = ops.swiglu(sums, interleave=8, out_dtype=bf)

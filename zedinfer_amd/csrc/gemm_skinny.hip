@@ -261,16 +261,23 @@ extern "C" int zi_gemm_skinny_supported(int M, int N, int K, int64_t ldx, int64_
     return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
 
-// Splits of k for a weight matrix [N, K]: the leading dimension of the partial sums.
-extern "C" int zi_gemm_skinny_splits(int N, int K) {
+// The kernel for 17..64 rows (gemm_mid.hip): its cut and its launch.
+void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split);
+int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const zi_bf16* w, const zi_bf16* bias, int M,
+                       int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int vec_out, hipStream_t stream);
+
+// Splits of k for M rows against a weight matrix [N, K]: the leading dimension of the partial sums.  A
+// function of N, K and of whether M is at most 16 (the two kernels cut differently).
+extern "C" int zi_gemm_skinny_splits(int M, int N, int K) {
     int kpw, s, tpw;
-    skinny_plan(N, K, &kpw, &s, &tpw);
+    if (M > 16) zi_gemm_mid_plan(N, K, &s, &tpw);
+    else skinny_plan(N, K, &kpw, &s, &tpw);
     return s;
 }
 
 // Floats of workspace for the split partials (0 when the product is not split).
 extern "C" int64_t zi_gemm_skinny_workspace(int M, int N, int K) {
-    const int s = zi_gemm_skinny_splits(N, K);
+    const int s = zi_gemm_skinny_splits(M, N, K);
     return s > 1 ? (int64_t)s * M * N : 0;
 }
 
@@ -309,11 +316,11 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
     ZI_REQUIRE(mode >= 0 && mode <= 2, "gemm_skinny: unknown mode %d", mode);
     ZI_REQUIRE(ldx >= K && ldw >= K, "gemm_skinny: leading dimension too small");
     ZI_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny: x and w must be 16-byte aligned");
-    int kpw, splits, tpw;
-    skinny_plan(N, K, &kpw, &splits, &tpw);
-    const int tiles = (N + SK_ROWS - 1) / SK_ROWS;
+    int kpw = 1, splits, tpw;
     const int mt = (M + 15) / 16;
-    if (mt > 1) tpw = 1;   // more than 16 rows of x do not stay in registers
+    if (mt > 1) zi_gemm_mid_plan(N, K, &splits, &tpw);    // more than 16 rows: the kernel that stages x in LDS
+    else skinny_plan(N, K, &kpw, &splits, &tpw);
+    const int tiles = (N + SK_ROWS - 1) / SK_ROWS;
     const dim3 grid((tiles + tpw - 1) / tpw, splits);
     void* dst = out;
     int kmode = mode;
@@ -341,16 +348,14 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
     else if (kmode == SK_MODE_SWIGLU) vec_out = ldo % 4 == 0 && ((uintptr_t)dst % 8) == 0;
     else vec_out = ldo % 4 == 0 && ((uintptr_t)dst % (out_dt == ZI_F32 ? 16 : 8)) == 0;
     const int of32 = out_dt == ZI_F32;
-#define ZI_SKM(MT)                                                                                                  \
-    sk_launch<MT>(kpw, grid, stream, dst, kmode, of32, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo, tpw, \
-                  vec_out)
-    switch (mt) {
-        case 1: ZI_SKM(1); break;
-        case 2: ZI_SKM(2); break;
-        case 3: ZI_SKM(3); break;
-        default: ZI_SKM(4); break;
+    if (mt > 1) {
+        const int rc = zi_gemm_mid_launch(dst, of32, kmode, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo,
+                                          vec_out, stream);
+        if (rc) return rc;
+    } else {
+        sk_launch<1>(kpw, grid, stream, dst, kmode, of32, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo, tpw,
+                     vec_out);
     }
-#undef ZI_SKM
     if (mode == SK_MODE_PLAIN && splits > 1) {
         const int64_t total = (int64_t)M * N;
         gemm_skinny_reduce_kernel<<<(int)((total + 255) / 256), 256, 0, stream>>>(out, of32, workspace,

@@ -504,20 +504,21 @@ def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
     return _skinny_ok(x, weight, x.shape[1], x.stride(0), weight.stride(0))
 
 
-def linear_splits(N: int, K: int) -> int:
-    """Partial sums the few-rows product with a weight matrix [N, K] leaves (a function of N and K alone)."""
-    return int(_lib.load().zi_gemm_skinny_splits(int(N), int(K)))
+def linear_splits(M: int, N: int, K: int) -> int:
+    """Partial sums the few-rows product of M rows with a weight matrix [N, K] leaves: a function of N, K
+    and of whether M is at most 16 (two kernels, two cuts)."""
+    return int(_lib.load().zi_gemm_skinny_splits(int(M), int(N), int(K)))
 
 
 def linear_sums(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x[M,K] . weight[N,K]^T for M <= FEW_ROWS as float32 partial sums [S, M, N], S =
-    ``linear_splits(N, K)``, without bias: the consumer adds them in rising order."""
+    ``linear_splits(M, N, K)``, without bias: the consumer adds them in rising order."""
     _gpu("linear_sums", x, weight, out)
     if not linear_sums_supported(x, weight):
         raise ValueError(f"linear_sums: needs bfloat16 x and weight, at most {FEW_ROWS} rows, 16-byte aligned rows")
     M, K = x.shape
     N = weight.shape[0]
-    S = linear_splits(N, K)
+    S = linear_splits(M, N, K)
     if out is None:
         out = torch.empty((S, M, N), dtype=torch.float32, device=x.device)
     if tuple(out.shape) != (S, M, N) or out.dtype != torch.float32 or not out.is_contiguous():
@@ -529,7 +530,7 @@ def linear_sums(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tenso
 
 def linear_swiglu_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
     return (linear_sums_supported(x, weight) and weight.shape[0] % 16 == 0
-            and linear_splits(weight.shape[0], weight.shape[1]) == 1)
+            and linear_splits(x.shape[0], weight.shape[0], weight.shape[1]) == 1)
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -568,8 +569,8 @@ def reduce_sums(sums: torch.Tensor, bias: Optional[torch.Tensor] = None, out: Op
     return out
 
 
-SKINNY_MAX_ROWS = 64   # rows the few-rows kernel takes in one launch
-FEW_ROWS = 16          # up to here it beats the library product (x stays in registers over the weight tiles)
+SKINNY_MAX_ROWS = 64   # rows the few-rows kernels take in one launch
+FEW_ROWS = 64          # up to here they beat the library product: the weights stream once, x stays on the chip
 _WORKSPACES = {}
 
 

@@ -63,7 +63,7 @@ class SwiGLU(FeedForward):
         if self.interleave and ops.linear_swiglu_supported(x, self.gate_up):
             ops.linear_swiglu(x, self.gate_up, out=act)
         elif self.interleave and ops.linear_sums_supported(x, self.gate_up):
-            S = ops.linear_splits(2 * I, self.hidden)
+            S = ops.linear_splits(n, 2 * I, self.hidden)
             sums = ops.linear_sums(x, self.gate_up, out=self.rt.buffer("ffn_gate_up_sums", (S, n, 2 * I), torch.float32))
             ops.swiglu(sums, out=act, interleave=self.interleave)
         else:
@@ -78,7 +78,7 @@ class SwiGLU(FeedForward):
             else:
                 ops.swiglu(gu[:, :I], gu[:, I:], out=act)
         if ops.linear_sums_supported(act, self.down):
-            S = ops.linear_splits(self.hidden, I)
+            S = ops.linear_splits(n, self.hidden, I)
             return ops.linear_sums(act, self.down, out=self.rt.buffer("ffn_out_sums", (S, n, self.hidden), torch.float32))
         out = self.rt.buffer("ffn_out", (n, self.hidden))
         return ops.linear(act, self.down, out=out)

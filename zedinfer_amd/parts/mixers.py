@@ -100,7 +100,7 @@ class Attention(Mixer):
         view = batch.groups[memory.group]
         if self.qkv is not None and ops.linear_sums_supported(x, self.qkv):
             # few rows: the projection leaves float32 partial sums; the rotary kernel adds them and the bias
-            S = ops.linear_splits(self.qkv.shape[0], self.hidden)
+            S = ops.linear_splits(n, self.qkv.shape[0], self.hidden)
             sums = self.rt.buffer("attn_qkv_sums", (S, n, self.qd + 2 * self.kvd), torch.float32)
             ops.linear_sums(x, self.qkv, out=sums)
             q = self.rt.buffer("attn_q", (n, self.qd))
@@ -118,7 +118,7 @@ class Attention(Mixer):
         att = self.rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
         if ops.linear_sums_supported(att, self.o):
-            S = ops.linear_splits(self.hidden, self.qd)
+            S = ops.linear_splits(n, self.hidden, self.qd)
             return ops.linear_sums(att, self.o, out=self.rt.buffer("attn_proj_sums", (S, n, self.hidden), torch.float32))
         out = self.rt.buffer("attn_proj", (n, self.hidden))
         return ops.linear(att, self.o, out=out)
