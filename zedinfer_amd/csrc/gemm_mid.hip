@@ -6,7 +6,8 @@
 // wavefronts, each wavefront reads its own 16 weight rows straight from memory into matrix-core operands
 // (v_mfma_f32_16x16x32_bf16, float32 accumulation) and keeps the sums of its 16 x M outputs in registers,
 // so nothing is added across wavefronts.  The next block's weights and x travel while the current one is
-// worked on.  The k dimension is cut over gridDim.y workgroups when N alone gives too few of them; those
+// worked on (a ring of register buffers; loads are issued without branches so that they stay in
+// flight).  The k dimension is cut over gridDim.y workgroups when N alone gives too few of them; those
 // leave float32 partial sums [split][M][N] that the consumer adds in rising order.  The cut depends on N
 // and K only.  Epilogues as in the few-rows kernel: plain (bias), partial sums, SwiGLU over gate/up rows
 // interleaved in blocks of 8.
@@ -20,6 +21,7 @@ typedef __attribute__((ext_vector_type(4))) float gm_f32x4_t;
 #define GM_KB 128
 #define GM_XS (GM_KB + 8)   // LDS row stride of the x slice, in elements
 #define GM_TARGET_WGS 384
+#define GM_RING 3           // k-blocks of weights in flight per wavefront
 
 #define GM_MODE_PLAIN 0
 #define GM_MODE_PARTIAL 1
@@ -44,24 +46,32 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     const int kb_hi = (kb_lo + kb_per_split < kb_total) ? kb_lo + kb_per_split : kb_total;
     const int n0 = blockIdx.x * GM_ROWS + wave * 16;
     const int nrow = (n0 + r < N) ? n0 + r : N - 1;
-    const zi_bf16* wrow = w + (int64_t)nrow * ldw + j * 8;
+    const zi_bf16* wrow_base = w + (int64_t)nrow * ldw;
 
     // what this thread stages of a block's x slice: MT pieces of 16 bytes (row srow + 16 * t, piece spc)
     const int srow = tid / 16, spc = tid % 16;
-    uint4 a_cur[4], a_next[4], xr[MT];
-    auto fetch = [&](uint4 (&a)[4], int kb) {
+    // the weights of GM_RING k-blocks are in flight at once (a ring of register buffers); the x slice of
+    // the next block is fetched while this one is worked on
+    uint4 ring[GM_RING][4], xring[GM_RING][MT];
+    // Loads are issued without branches (addresses are clamped into the matrix, what lies outside is
+    // zeroed afterwards): only then does the compiler let several blocks' loads stay in flight.
+    const int xm_last = M - 1;
+    auto fetch = [&](uint4 (&a)[4], uint4 (&xr)[MT], int kb) {
         const int k0 = kb * GM_KB;
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-            a[c] = (k0 + c * 32 + j * 8 < K) ? *reinterpret_cast<const uint4*>(wrow + k0 + c * 32) : make_uint4(0, 0, 0, 0);
+        for (int c = 0; c < 4; ++c) {
+            const int k = k0 + c * 32 + j * 8;
+            const uint4 v = *reinterpret_cast<const uint4*>(wrow_base + (k < K ? k : K - 8));
+            a[c] = k < K ? v : make_uint4(0, 0, 0, 0);
+        }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
-            const int m = t * 16 + srow;
-            xr[t] = (m < M && k0 + spc * 8 < K) ? *reinterpret_cast<const uint4*>(x + (int64_t)m * ldx + k0 + spc * 8)
-                                                : make_uint4(0, 0, 0, 0);
+            const int m = t * 16 + srow, k = k0 + spc * 8;
+            const uint4 v = *reinterpret_cast<const uint4*>(x + (int64_t)(m < M ? m : xm_last) * ldx + (k < K ? k : K - 8));
+            xr[t] = (m < M && k < K) ? v : make_uint4(0, 0, 0, 0);
         }
     };
-    auto stash = [&](int b) {
+    auto stash = [&](const uint4 (&xr)[MT], int b) {
 #pragma unroll
         for (int t = 0; t < MT; ++t) *reinterpret_cast<uint4*>(&xs[b][(t * 16 + srow) * GM_XS + spc * 8]) = xr[t];
     };
@@ -69,30 +79,41 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    fetch(a_cur, kb_lo);
-    stash(0);
+    // blocks kb_lo .. kb_lo + GM_RING - 2 are requested up front; block kb's x goes to LDS one iteration
+    // before it is used, GM_RING - 2 iterations after it was requested
+    const int kb_last = kb_hi - 1;    // requests past the last block fetch it again: no branch around a load
+#pragma unroll
+    for (int b = 0; b < GM_RING - 1; ++b) fetch(ring[b], xring[b], kb_lo + b < kb_hi ? kb_lo + b : kb_last);
+    stash(xring[0], 0);
     __syncthreads();
     int cur = 0;
-    for (int kb = kb_lo; kb < kb_hi; ++kb, cur ^= 1) {
-        const bool has_next = kb + 1 < kb_hi;
-        if (has_next) fetch(a_next, kb + 1);
+    for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += GM_RING) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            gm_pack a;
-            a.u = a_cur[c];
+        for (int b = 0; b < GM_RING; ++b) {
+            const int kb = kb0 + b;
+            if (kb >= kb_hi) break;
+            fetch(ring[(b + GM_RING - 1) % GM_RING], xring[(b + GM_RING - 1) % GM_RING],
+                  kb + GM_RING - 1 < kb_hi ? kb + GM_RING - 1 : kb_last);
+            // all of the block's x operands are read from LDS before the first product: the reads' latency
+            // is paid once, not once per product
+            gm_pack bb[4][MT];
 #pragma unroll
-            for (int t = 0; t < MT; ++t) {
-                gm_pack b;
-                b.u = *reinterpret_cast<const uint4*>(&xs[cur][(t * 16 + r) * GM_XS + c * 32 + j * 8]);
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, acc[t], 0, 0, 0);
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    bb[c][t].u = *reinterpret_cast<const uint4*>(&xs[cur][(t * 16 + r) * GM_XS + c * 32 + j * 8]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                gm_pack a;
+                a.u = ring[b][c];
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, bb[c][t].b, acc[t], 0, 0, 0);
             }
+            if (kb + 1 < kb_hi) stash(xring[(b + 1) % GM_RING], cur ^ 1);
+            __syncthreads();
+            cur ^= 1;
         }
-        if (has_next) {
-            stash(cur ^ 1);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) a_cur[c] = a_next[c];
-        }
-        __syncthreads();
     }
     // C[n = n0 + j*4 + e][m = t*16 + r]
 #pragma unroll
@@ -162,7 +183,7 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
 void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split) {
     const int groups = (N + GM_ROWS - 1) / GM_ROWS;
     const int kb_total = (K + GM_KB - 1) / GM_KB;
-    int s = (GM_TARGET_WGS + groups - 1) / groups;
+    int s = (GM_TARGET_WGS + groups / 2) / groups;    // to the nearest: 280 groups are enough by themselves
     if (s > 16) s = 16;
     if (s > kb_total / 2) s = kb_total / 2;
     if (s < 1) s = 1;
