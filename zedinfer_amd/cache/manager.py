@@ -70,6 +70,7 @@ class SequenceCache:
         self.held: List[int] = [0] * num_groups
         self.promised: List[int] = [0] * num_groups
         self.closed = False
+        self.version = 0          # grows whenever a block table of the sequence changes
 
 
 class CacheManager:
@@ -168,6 +169,7 @@ class CacheManager:
                     g.pool.give_back(table[i])
                     table[i] = -1
                     seq.held[gi] -= 1
+                    seq.version += 1
 
     def ensure(self, seq: SequenceCache, new_len: int) -> None:
         """Make sure pages exist for every position below ``new_len`` that a token at or after
@@ -199,6 +201,7 @@ class CacheManager:
                         grown[gi] += 1
                     table[i] = g.pool.take()
                     seq.held[gi] += 1
+                    seq.version += 1
                     taken.append((gi, i))
         except OutOfPages:
             for gi, i in taken:
@@ -210,6 +213,7 @@ class CacheManager:
                 seq.promised[gi] -= n
             for gi, n in enumerate(old_lens):
                 del seq.pages[gi][n:]
+            seq.version += 1
             raise
 
     def commit(self, seq: SequenceCache, new_len: int) -> None:
@@ -229,6 +233,7 @@ class CacheManager:
                     g.pool.give_back(p)
             seq.pages[gi] = []
             seq.held[gi] = 0
+            seq.version += 1
             g.pool.uncommit(seq.promised[gi])
             seq.promised[gi] = 0
         self.slots.give_back(seq.slot)

@@ -71,6 +71,7 @@ class DeviceBatch:
     host_len: Optional[np.ndarray] = None
     host_past: Optional[np.ndarray] = None
     host_slot: Optional[np.ndarray] = None
+    host_image: Optional[np.ndarray] = None      # all index arrays as they were copied to the device
 
 
 class StagingRing:
@@ -192,6 +193,7 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     for p in pieces:
         hv[off:off + p.size] = p
         off += p.size
+    image = hv[:sum(sizes)].copy()
     if static is not None:
         if static.numel() < total or static.dtype != torch.int32:
             raise ValueError("the static batch buffer is too small")
@@ -214,4 +216,77 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
                        long_idx=views[9] if 0 < n_long < N else None, num_short=n_short, num_long=n_long,
                        max_short_keys=max_short, max_long_keys=max_long, tile_entry=views[10], tile_off=views[11],
                        num_tiles=len(tiles), host_start=starts,
-                       host_len=lens_a, host_past=past, host_slot=slot)
+                       host_len=lens_a, host_past=past, host_slot=slot, host_image=image)
+
+
+class DecodeImage:
+    """The host image of a decode step's index arrays (every entry one token), kept from step to step.
+
+    While the same sequences go on decoding, only the token ids, the positions and the cache slots
+    change, and a block table row when its sequence took or gave back a page: ``refresh`` rewrites
+    just those in place instead of packing everything anew.  The layout is the one
+    ``build_device_batch`` makes for the same entries and table widths."""
+
+    def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, device: torch.device,
+                 staging: StagingRing, widths: Sequence[int], static: torch.Tensor):
+        self.cache, self.vocab_size, self.staging, self.static = cache, vocab_size, staging, static
+        self.widths = tuple(int(w) for w in widths)
+        self.batch = build_device_batch(entries, cache, vocab_size, device, staging, widths, static)
+        E, R = len(entries), self.batch.num_logit_rows
+        self.seqs = [e.seq for e in entries]
+        self.wants = tuple(len(e.want) for e in entries)
+        self.versions = [e.seq.version for e in entries]
+        sizes = [E, E, E, R, E, E, E, E, E, 0, 0, 0]
+        for w in self.widths:
+            sizes += [E, E * w]
+        self.total = sum(sizes)
+        self.offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        self.image = np.empty(max(self.total, 1), dtype=np.int32)
+        self.image[:self.total] = self.batch.host_image
+        self.page_sizes = [g.page_size for g in cache.groups]
+        self.rows = np.arange(E)
+
+    def piece(self, i: int) -> np.ndarray:
+        return self.image[self.offsets[i]:self.offsets[i + 1]]
+
+    def matches(self, entries: Sequence[StepEntry]) -> bool:
+        if len(entries) != len(self.seqs):
+            return False
+        for e, s, w in zip(entries, self.seqs, self.wants):
+            if e.seq is not s or len(e.tokens) != 1 or len(e.want) != w or (w and e.want[0] != 0):
+                return False
+        return True
+
+    def refresh(self, entries: Sequence[StepEntry]) -> DeviceBatch:
+        """The image for this step (``matches(entries)`` holds), copied to the device buffer."""
+        E = len(entries)
+        toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=E)
+        if toks.min() < 0 or toks.max() >= self.vocab_size:
+            bad = toks[(toks < 0) | (toks >= self.vocab_size)][0]
+            raise ValueError(f"token id {int(bad)} is outside the vocabulary of {self.vocab_size}")
+        pos = np.fromiter((s.length for s in self.seqs), dtype=np.int32, count=E)
+        self.piece(0)[:] = toks
+        self.piece(1)[:] = pos
+        self.piece(6)[:] = pos
+        for g, w in enumerate(self.widths):
+            table = self.piece(13 + 2 * g).reshape(E, w)
+            for i, s in enumerate(self.seqs):
+                if s.version != self.versions[i]:
+                    pg = s.pages[g]
+                    if len(pg) > w:
+                        raise ValueError(f"block tables of group {g} need {len(pg)} columns, {w} given")
+                    table[i, :len(pg)] = pg
+                    table[i, len(pg):] = -1
+            ps = self.page_sizes[g]
+            pages = table[self.rows, pos // ps]
+            if (pages < 0).any():
+                raise RuntimeError("a decoded token's position has no page")
+            self.piece(12 + 2 * g)[:] = pages * ps + pos % ps
+        for i, s in enumerate(self.seqs):
+            self.versions[i] = s.version
+        host = self.staging.acquire(self.total)
+        host.numpy()[:] = self.image[:self.total]
+        self.static[:self.total].copy_(host, non_blocking=True)
+        self.staging.copied()
+        self.batch.host_past = pos
+        return self.batch

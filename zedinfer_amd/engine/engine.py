@@ -22,7 +22,7 @@ from ..config import ModelConfig, ModelForwardConfig, SchedulerConfig, load_conf
 from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
 from ..weights import load_weights, random_weights
-from .batch import DeviceBatch, StagingRing, StepEntry, build_device_batch
+from .batch import DecodeImage, DeviceBatch, StagingRing, StepEntry, build_device_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            "f32": torch.float32}
@@ -172,7 +172,11 @@ class Engine:
             size = 8 * E + 2 * R + sum(E * (w + 1) for w in widths) + 64
             dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
             self._graphs[key] = dg
-        batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer)
+        if dg.image is not None and dg.image.matches(entries):
+            batch = dg.image.refresh(entries)      # the same sequences go on: only what changed is rewritten
+        else:
+            dg.image = DecodeImage(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer)
+            batch = dg.image.batch
         batch.max_short_keys = keys_bucket
         if dg.graph is not None:
             dg.graph.replay()
@@ -198,6 +202,7 @@ class _DecodeGraph:
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
         self.warm = False
+        self.image: Optional[DecodeImage] = None
 
 
 def _pow2_at_least(n: int, floor: int = 1) -> int:
