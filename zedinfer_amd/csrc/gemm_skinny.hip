@@ -1,5 +1,6 @@
-// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for few rows of x (M <= 64): the decode-time
-// matrix product, bound by the one pass over the weights.
+// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for few rows of x: the decode-time matrix product,
+// bound by the one pass over the weights.  Up to 16 rows run on the kernel in this file, 17 to 64
+// on the one in gemm_mid.hip; this file holds the entry point of both.
 //
 // bfloat16 x and w, float32 accumulation on the matrix cores
 // (v_mfma_f32_16x16x32_bf16).  A workgroup of four wavefronts owns tiles of 16 weight
@@ -35,7 +36,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 #define SK_RESIDENT_WGS 480   // workgroups that are surely resident at once (256 compute units, two each)
 #define SK_ENOUGH_WGS 256
 #define SK_MAX_TPW 32
-#define SK_DEEP_RING 0    // three tiles in flight per workgroup measured slower than two (14.3 -> 16.1 us for 17920 x 1536)
 
 #define SK_MODE_PLAIN 0
 #define SK_MODE_PARTIAL 1
@@ -47,22 +47,33 @@ __device__ __forceinline__ bf16x8_t as_bf16x8(const uint4& v) {
     return c.b;
 }
 
-// The four 16-byte pieces of row `row` this lane owns in k-block `kb` (zeros past K; K % 8 == 0): piece c
-// holds k = kb*128 + c*32 + j*8 .. +8, so that one load instruction reads 64 contiguous bytes of each
-// of the wavefront's 16 rows.
+// The four 16-byte pieces of row `row` this lane owns in k-block `kb`: piece c holds
+// k = kb*128 + c*32 + j*8 .. +8, so that one load instruction reads 64 contiguous bytes of each of the
+// wavefront's 16 rows.  Pieces past K are read from the row's last piece instead (K % 8 == 0): no branch
+// goes around a load, so that the compiler lets the loads of several tiles stay in flight.  What such
+// pieces hold does not matter for the weights (x is zero there); `sk_load_row_masked` zeroes them for x.
 __device__ __forceinline__ void sk_load_row(uint4 (&dst)[4], const zi_bf16* row, int kb, int j, int K) {
     const int k0 = kb * SK_KB + j * 8;
 #pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int k = k0 + c * 32;
+        dst[c] = *reinterpret_cast<const uint4*>(row + (k < K ? k : K - 8));
+    }
+}
+__device__ __forceinline__ void sk_load_row_masked(uint4 (&dst)[4], const zi_bf16* row, int kb, int j, int K, bool live) {
+    sk_load_row(dst, row, kb, j, K);
+    const int k0 = kb * SK_KB + j * 8;
+#pragma unroll
     for (int c = 0; c < 4; ++c)
-        dst[c] = (k0 + c * 32 < K) ? *reinterpret_cast<const uint4*>(row + k0 + c * 32) : make_uint4(0, 0, 0, 0);
+        if (!live || k0 + c * 32 >= K) dst[c] = make_uint4(0, 0, 0, 0);
 }
 
-template <int MT, int KPW, int NB>
+template <int KPW>
 __global__ void __launch_bounds__(SK_WAVES* ZI_WAVE)
 gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* x, const zi_bf16* __restrict__ w,
                    const zi_bf16* __restrict__ bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
                    int tiles_per_wg, int vec_out) {
-    constexpr bool XRES = (MT == 1);   // the slice of x stays in registers over the workgroup's tiles
+    constexpr int MT = 1;              // up to 16 rows of x: one matrix-core tile
     __shared__ f32x4_t red[2][SK_WAVES][MT][ZI_WAVE];
     const int lane = threadIdx.x & (ZI_WAVE - 1), wave = threadIdx.x / ZI_WAVE;
     const int r = lane & 15, j = lane >> 4;
@@ -79,25 +90,20 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
         const int m = t * 16 + r;
         xrow[t] = x + (int64_t)(m < M ? m : M - 1) * ldx;
     }
-    uint4 xr[XRES ? KPW : 1][4];
-    if (XRES) {
+    // The slice of x stays in registers over the workgroup's tiles.  It is zero past K and for k-blocks past
+    // the last one (a wavefront that has fewer than KPW blocks reads the last block again and multiplies
+    // it by zero).
+    const int kb_last = kb_total - 1;
+    uint4 xr[KPW][4];
 #pragma unroll
-        for (int i = 0; i < KPW; ++i) {
-            if (kb0 + i < kb_total) sk_load_row(xr[i], xrow[0], kb0 + i, j, K);
-            else xr[i][0] = xr[i][1] = xr[i][2] = xr[i][3] = make_uint4(0, 0, 0, 0);
-        }
-    }
-    // the weight rows of up to NB tiles are in flight at once: a ring of register buffers
-    uint4 ring[NB][KPW][4];
-#pragma unroll
-    for (int b = 0; b < NB; ++b)
-#pragma unroll
-        for (int i = 0; i < KPW; ++i) ring[b][i][0] = ring[b][i][1] = ring[b][i][2] = ring[b][i][3] = make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < KPW; ++i)
+        sk_load_row_masked(xr[i], xrow[0], kb0 + i < kb_total ? kb0 + i : kb_last, j, K, kb0 + i < kb_total);
+    uint4 ring[2][KPW][4];
     auto issue = [&](uint4 (&dst)[KPW][4], int tile) {
         const int nrow = (tile * SK_ROWS + r < N) ? tile * SK_ROWS + r : N - 1;
 #pragma unroll
         for (int i = 0; i < KPW; ++i)
-            if (kb0 + i < kb_total) sk_load_row(dst[i], w + (int64_t)nrow * ldw, kb0 + i, j, K);
+            sk_load_row(dst[i], w + (int64_t)nrow * ldw, kb0 + i < kb_total ? kb0 + i : kb_last, j, K);
     };
     int buf = 0;
     auto process = [&](uint4 (&a)[KPW][4], int tile) {
@@ -105,23 +111,10 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < KPW; ++i) {
-            if (kb0 + i >= kb_total) break;
-            if (XRES) {
+        for (int i = 0; i < KPW; ++i)
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[i][c]), as_bf16x8(xr[i][c]), acc[0], 0, 0, 0);
-            } else {
-                uint4 b[MT][4];
-#pragma unroll
-                for (int t = 0; t < MT; ++t) sk_load_row(b[t], xrow[t], kb0 + i, j, K);
-#pragma unroll
-                for (int c = 0; c < 4; ++c)
-#pragma unroll
-                    for (int t = 0; t < MT; ++t)
-                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[i][c]), as_bf16x8(b[t][c]), acc[t], 0, 0, 0);
-            }
-        }
+            for (int c = 0; c < 4; ++c)
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[i][c]), as_bf16x8(xr[i][c]), acc[0], 0, 0, 0);
 #pragma unroll
         for (int t = 0; t < MT; ++t) red[buf][wave][t][lane] = acc[t];
         __syncthreads();
@@ -194,17 +187,23 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
         }
         buf ^= 1;
     };
-#pragma unroll
-    for (int b = 0; b < NB - 1; ++b)
-        if (tile_lo + b < tile_hi) issue(ring[b], tile_lo + b);
-    for (int tile = tile_lo; tile < tile_hi; tile += NB) {
-#pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            if (tile + b >= tile_hi) break;
-            // the buffer that was worked on last takes the tile NB - 1 ahead
-            if (tile + b + NB - 1 < tile_hi) issue(ring[(b + NB - 1) % NB], tile + b + NB - 1);
-            process(ring[b], tile + b);
-        }
+    // Two buffers take turns: while one tile is worked on the next one's rows travel.  Every load sits in
+    // straight-line code (the last tile is peeled off instead of guarding its prefetch), which is what lets
+    // the compiler wait for the older loads only.
+    issue(ring[0], tile_lo);
+    int tile = tile_lo;
+    for (; tile + 2 < tile_hi; tile += 2) {
+        issue(ring[1], tile + 1);
+        process(ring[0], tile);
+        issue(ring[0], tile + 2);
+        process(ring[1], tile + 1);
+    }
+    if (tile + 1 < tile_hi) {
+        issue(ring[1], tile + 1);
+        process(ring[0], tile);
+        process(ring[1], tile + 1);
+    } else {
+        process(ring[0], tile);
     }
 }
 
@@ -281,19 +280,12 @@ extern "C" int64_t zi_gemm_skinny_workspace(int M, int N, int K) {
     return s > 1 ? (int64_t)s * M * N : 0;
 }
 
-template <int MT>
 static void sk_launch(int kpw, dim3 grid, hipStream_t stream, void* out, int mode, int out_f32, const zi_bf16* x,
                       const zi_bf16* w, const zi_bf16* bias, int M, int N, int K, int64_t ldx, int64_t ldw, int64_t ldo,
                       int tpw, int vec_out) {
 #define ZI_SK(KPW)                                                                                                  \
-    do {                                                                                                            \
-        if (MT == 1 && KPW <= 3 && tpw >= 3 && SK_DEEP_RING)                                                                     \
-            gemm_skinny_kernel<MT, KPW, (MT == 1 && KPW <= 3) ? 3 : 2><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(     \
-                out, mode, out_f32, x, w, bias, M, N, K, ldx, ldw, ldo, tpw, vec_out);                              \
-        else                                                                                                        \
-            gemm_skinny_kernel<MT, KPW, 2><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, \
-                                                                                   K, ldx, ldw, ldo, tpw, vec_out); \
-    } while (0)
+    gemm_skinny_kernel<KPW><<<grid, SK_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, ldw, \
+                                                                     ldo, tpw, vec_out)
     switch (kpw) {
         case 1: ZI_SK(1); break;
         case 2: ZI_SK(2); break;
@@ -353,7 +345,7 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
                                           vec_out, stream);
         if (rc) return rc;
     } else {
-        sk_launch<1>(kpw, grid, stream, dst, kmode, of32, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo, tpw,
+        sk_launch(kpw, grid, stream, dst, kmode, of32, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo, tpw,
                      vec_out);
     }
     if (mode == SK_MODE_PLAIN && splits > 1) {
