@@ -44,6 +44,13 @@ union pf_pack {
     uint16_t h[8];
 };
 
+// v where bit 0 of `keep` is set, else zeros (by value: a select between two register arrays' elements
+// would be made through memory)
+__device__ __forceinline__ uint4 pf_keep(uint4 v, int keep) {
+    const unsigned mask = 0u - (unsigned)(keep & 1);
+    return make_uint4(v.x & mask, v.y & mask, v.z & mask, v.w & mask);
+}
+
 template <int D>
 __global__ void __launch_bounds__(PF_WAVES* ZI_WAVE)
 attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* __restrict__ q, int64_t ldq,
@@ -132,32 +139,51 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     }
     const int ps_mask = ps - 1;
 
-    // global -> registers: the block of keys [kb, kb + 64)
+    // global -> registers: the block of keys [kb, kb + 128).  Straight-line code: every table lookup
+    // is issued, then every load of keys and values, from addresses clamped into the sequence and the
+    // pool; what a thread must not use is zeroed when it goes to LDS.  With a branch around a load the
+    // compiler waits for it on the spot, and the block would not travel during the products.
+    int kvalid = 0, vvalid = 0;
+    const int kmax8 = kmax & ~7, pi_last = max_pages - 1;
     auto fetch = [&](int kb) {
-        const bool inside = kb + PF_BS - 1 <= kmax;    // every key of the block exists (all blocks but the last)
+        int kpage[KPASS], vpage[VPASS], kkey[KPASS], vkey[VPASS];
+        kvalid = 0;
+        vvalid = 0;
 #pragma unroll
         for (int pass = 0; pass < KPASS; ++pass) {
-            const int key = kb + k_kk[pass];
-            kreg[pass] = make_uint4(0, 0, 0, 0);
-            if (k_kk[pass] >= 0 && (inside || key <= kmax) && (D % 32 == 0 || k_c[pass] * 8 < D)) {
-                const int pi = key >> ps_shift;
-                const int page = pi < max_pages ? bt[pi] : -1;
-                if ((unsigned)page < (unsigned)num_pages)
-                    kreg[pass] = *reinterpret_cast<const uint4*>(
-                        kcache + ((((int64_t)page * nkv + g) << ps_shift) + (key & ps_mask)) * D + k_c[pass] * 8);
-            }
+            const int key = kb + (k_kk[pass] >= 0 ? k_kk[pass] : 0);
+            const bool ok = k_kk[pass] >= 0 && key <= kmax && (D % 32 == 0 || k_c[pass] * 8 < D);
+            kkey[pass] = key <= kmax ? key : kmax;
+            const int pi = kkey[pass] >> ps_shift;
+            kpage[pass] = bt[pi < pi_last ? pi : pi_last];
+            kvalid |= (int)ok << pass;
         }
 #pragma unroll
         for (int pass = 0; pass < VPASS; ++pass) {
-            vreg[pass] = make_uint4(0, 0, 0, 0);
             const int key0 = kb + v_col[pass];
-            if (v_dim[pass] >= 0 && (inside || key0 <= kmax)) {
-                const int pi = key0 >> ps_shift;
-                const int page = pi < max_pages ? bt[pi] : -1;
-                if ((unsigned)page < (unsigned)num_pages)
-                    vreg[pass] = *reinterpret_cast<const uint4*>(
-                        vcache + ((((int64_t)page * nkv + g) * D + v_dim[pass]) << ps_shift) + (key0 & ps_mask));
-            }
+            const bool ok = v_dim[pass] >= 0 && key0 <= kmax;
+            vkey[pass] = key0 <= kmax ? key0 : kmax8;
+            const int pi = vkey[pass] >> ps_shift;
+            vpage[pass] = bt[pi < pi_last ? pi : pi_last];
+            vvalid |= (int)ok << pass;
+        }
+#pragma unroll
+        for (int pass = 0; pass < KPASS; ++pass) {
+            const bool held = (unsigned)kpage[pass] < (unsigned)num_pages;   // a window may have freed the page
+            const int page = held ? kpage[pass] : 0;
+            const int c = (D % 32 == 0 || k_c[pass] * 8 < D) ? k_c[pass] : 0;
+            kreg[pass] = *reinterpret_cast<const uint4*>(
+                kcache + ((((int64_t)page * nkv + g) << ps_shift) + (kkey[pass] & ps_mask)) * D + c * 8);
+            if (!held) kvalid &= ~(1 << pass);
+        }
+#pragma unroll
+        for (int pass = 0; pass < VPASS; ++pass) {
+            const bool held = (unsigned)vpage[pass] < (unsigned)num_pages;
+            const int page = held ? vpage[pass] : 0;
+            const int dim = v_dim[pass] >= 0 ? v_dim[pass] : 0;
+            vreg[pass] = *reinterpret_cast<const uint4*>(
+                vcache + ((((int64_t)page * nkv + g) * D + dim) << ps_shift) + (vkey[pass] & ps_mask));
+            if (!held) vvalid &= ~(1 << pass);
         }
     };
     // registers -> LDS buffer `b`: key kb + kk goes to row rho(kk) of the key tile; values go in
@@ -167,18 +193,19 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         uint16_t* vl = v_lds + b * (D * VS);
 #pragma unroll
         for (int pass = 0; pass < KPASS; ++pass)
-            if (k_kk[pass] >= 0) *reinterpret_cast<uint4*>(&kl[k_dst[pass]]) = kreg[pass];
-        if (kb + PF_BS - 1 <= kmax) {     // all blocks but the last: nothing to mask
+            if (k_kk[pass] >= 0) *reinterpret_cast<uint4*>(&kl[k_dst[pass]]) = pf_keep(kreg[pass], kvalid >> pass);
+        if (kb + PF_BS - 1 <= kmax) {     // all blocks but the last: no key past the end
 #pragma unroll
             for (int pass = 0; pass < VPASS; ++pass)
-                if (v_dim[pass] >= 0) *reinterpret_cast<uint4*>(&vl[v_dim[pass] * VS + v_col[pass]]) = vreg[pass];
+                if (v_dim[pass] >= 0)
+                    *reinterpret_cast<uint4*>(&vl[v_dim[pass] * VS + v_col[pass]]) = pf_keep(vreg[pass], vvalid >> pass);
         } else {
 #pragma unroll
             for (int pass = 0; pass < VPASS; ++pass) {
                 if (v_dim[pass] < 0) continue;
                 const int key0 = kb + v_col[pass];
                 pf_pack val;
-                val.u = vreg[pass];
+                val.u = pf_keep(vreg[pass], vvalid >> pass);
 #pragma unroll
                 for (int x = 0; x < 8; ++x)
                     if (key0 + x > kmax) val.h[x] = 0;    // slots past the last key may hold anything
@@ -190,12 +217,8 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     fetch(kb_begin);
     stash(kb_begin, 0);
     __syncthreads();
-    int cur = 0;
-    for (int kb0 = kb_begin; kb0 <= kmax; kb0 += PF_BS, cur ^= 1) {
-        // the next block travels from the cache into registers while this one is worked on; it goes
-        // into the other LDS buffer, which everyone has finished reading at the barrier before
-        const bool has_next = kb0 + PF_BS <= kmax;
-        if (has_next) fetch(kb0 + PF_BS);
+    // one block of keys from LDS buffer `cur` into this wavefront's running softmax and output
+    auto work = [&](int kb0, int cur) {
         const int kb = kb0 + kh * PF_BN;      // this wavefront's 64 keys of the block
         const uint16_t* kl = k_lds + cur * (PF_BS * KS) + kh * (PF_BN * KS);
         const uint16_t* vl = v_lds + cur * (D * VS) + kh * PF_BN;
@@ -275,9 +298,19 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                 o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[b].b, o[dd], 0, 0, 0);
             }
         }
-        if (has_next) stash(kb0 + PF_BS, cur ^ 1);
+    };
+    // The next block travels from the cache into registers while this one is worked on; it goes into
+    // the other LDS buffer, which everyone has finished reading at the barrier before.  The last block
+    // stands outside the loop, so that no branch surrounds the loop's loads.
+    int cur = 0, kb0 = kb_begin;
+    for (; kb0 + PF_BS <= kmax; kb0 += PF_BS, cur ^= 1) {
+        fetch(kb0 + PF_BS);
+        work(kb0, cur);
+        stash(kb0 + PF_BS, cur ^ 1);
         __syncthreads();
     }
+    work(kb0, cur);
+    __syncthreads();
     float l = lsum;
     l += __shfl_xor(l, 16, ZI_WAVE);
     l += __shfl_xor(l, 32, ZI_WAVE);
