@@ -94,6 +94,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     const int quarter = sp.len / DEC_WAVES;
     const int k_begin = sp.lo_al + chunk * sp.len + wave * quarter;
     const int k_end = (k_begin + quarter < p + 1) ? k_begin + quarter : p + 1;   // one past the wavefront's last key
+    const int p8 = p & ~7, pi_last = max_pages - 1;
 
     // the group's queries as the B operand: lane (r, j) holds head r, dims dk*32 + j*8 ..
     dec_bf16x8_t qop[DK];
@@ -112,43 +113,67 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     const float scale_log2 = scale * 1.4426950408889634f;
 
     for (int base = k_begin; base < k_end; base += DEC_BLOCK) {
-        // ---- all loads of the block first: keys (4 tiles x DK) and values (DT x 2)
+        // ---- all loads of the block first, in straight-line code: the six table lookups, then keys
+        // (4 tiles x DK) and values (DT x 2) from addresses clamped into the sequence and the pool.  What
+        // must not count is masked afterwards; with a branch around a load the compiler would wait for it
+        // on the spot, one tile after the other.
         dec_pack kop[4][DK], vop[DT][2];
+        int kpage[4], kslot[4], vpage[2], vslot[2];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
             const int key = base + (tt / 2) * 32 + (r / 4) * 8 + (tt % 2) * 4 + (r % 4);
-            const zi_bf16* kr = nullptr;
-            if (key < k_end && key >= sp.lo) {
-                const int pi = ps_shift >= 0 ? key >> ps_shift : key / ps;
-                const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages) kr = kcache + (((int64_t)page * nkv + kvh) * ps + (key - pi * ps)) * D + j * 8;
-            }
-#pragma unroll
-            for (int dk = 0; dk < DK; ++dk) {
-                kop[tt][dk].u = make_uint4(0, 0, 0, 0);
-                if (kr && dk * 32 + j * 8 < D) kop[tt][dk].u = *reinterpret_cast<const uint4*>(kr + dk * 32);
-            }
+            const int kc = key < p ? key : p;
+            int pi = ps_shift >= 0 ? kc >> ps_shift : kc / ps;
+            kslot[tt] = kc - pi * ps;
+            kpage[tt] = bt[pi < pi_last ? pi : pi_last];
         }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             const int key0 = base + b * 32 + j * 8;
-            const zi_bf16* vr = nullptr;
-            if (key0 < k_end && key0 + 8 > sp.lo) {
-                const int pi = ps_shift >= 0 ? key0 >> ps_shift : key0 / ps;
-                const int page = pi < max_pages ? bt[pi] : -1;
-                if (page >= 0 && page < num_pages) vr = vcache + (((int64_t)page * nkv + kvh) * D + r) * ps + (key0 - pi * ps);
+            const int kc = key0 < p8 ? key0 : p8;
+            int pi = ps_shift >= 0 ? kc >> ps_shift : kc / ps;
+            vslot[b] = kc - pi * ps;
+            vpage[b] = bt[pi < pi_last ? pi : pi_last];
+        }
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+            const int page = (unsigned)kpage[tt] < (unsigned)num_pages ? kpage[tt] : 0;   // a window may have freed it
+            const zi_bf16* kr = kcache + (((int64_t)page * nkv + kvh) * ps + kslot[tt]) * D;
+#pragma unroll
+            for (int dk = 0; dk < DK; ++dk)
+                kop[tt][dk].u = *reinterpret_cast<const uint4*>(kr + ((D % 32 == 0 || dk * 32 + j * 8 < D) ? dk * 32 + j * 8 : 0));
+        }
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            const int page = (unsigned)vpage[b] < (unsigned)num_pages ? vpage[b] : 0;
+            const zi_bf16* vr = vcache + (((int64_t)page * nkv + kvh) * D + r) * ps + vslot[b];
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) vop[dd][b].u = *reinterpret_cast<const uint4*>(vr + (int64_t)dd * 16 * ps);
+        }
+        if (D % 32 != 0) {   // the padding of the last k-step must be zero: the query is, but 0 * NaN is not
+            const unsigned keep = (DK - 1) * 32 + j * 8 < D ? ~0u : 0u;
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt) {
+                uint4& u = kop[tt][DK - 1].u;
+                u.x &= keep; u.y &= keep; u.z &= keep; u.w &= keep;
             }
-            const bool edge = key0 < sp.lo || key0 + 8 > k_end;
+        }
+        // Keys outside [lo, p] get the score -inf below, whatever was loaded for them.  Their values
+        // must be zero, since 0 * NaN is NaN: slots outside the range may hold anything.
+        if (base < sp.lo || base + DEC_BLOCK > k_end) {
 #pragma unroll
-            for (int dd = 0; dd < DT; ++dd) {
-                vop[dd][b].u = make_uint4(0, 0, 0, 0);
-                if (vr) {
-                    vop[dd][b].u = *reinterpret_cast<const uint4*>(vr + (int64_t)dd * 16 * ps);
-                    if (edge) {   // slots outside [lo, p] may hold anything: keep them out of the sum
+            for (int b = 0; b < 2; ++b) {
+                const int key0 = base + b * 32 + j * 8;
+                unsigned keep[4];
 #pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (key0 + e < sp.lo || key0 + e >= k_end) vop[dd][b].h[e] = 0;
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    const int ka = key0 + 2 * e, kb2 = ka + 1;
+                    keep[e] = ((ka >= sp.lo && ka < k_end) ? 0xffffu : 0u) | ((kb2 >= sp.lo && kb2 < k_end) ? 0xffff0000u : 0u);
+                }
+#pragma unroll
+                for (int dd = 0; dd < DT; ++dd) {
+                    uint4& u = vop[dd][b].u;
+                    u.x &= keep[0]; u.y &= keep[1]; u.z &= keep[2]; u.w &= keep[3];
                 }
             }
         }

@@ -93,78 +93,59 @@ extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, i
 // [0, nh*d) of a row are q, the next nkv*d are k, the last nkv*d are v; split s of row t starts at
 // part + s * split_stride + t * ldp.  The splits are added in rising order, the bias is added, and
 // the row is rotated from float32: q goes to q_out (rounded once), k and v into the cache.
-template <typename T, typename TB>
-__global__ void rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __restrict__ part,
-                                           int splits, int64_t split_stride, int64_t ldp,
-                                           const TB* __restrict__ bias, const int32_t* __restrict__ pos,
-                                           const int32_t* __restrict__ slots, const float* __restrict__ inv_freq,
-                                           T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int d,
-                                           int rot, int page_size, int write_kv, int64_t cache_slots, int vec4) {
-    extern __shared__ __attribute__((aligned(16))) float sh[];  // cos[rot/2], sin[rot/2], then the summed row
+// One wavefront per (token, head): blockIdx.y < nh is a query head, the others are key heads, which
+// bring their value head along.  A lane owns the pairs (j, j + rot/2) it rotates and computes their
+// angle itself, so nothing is shared and nothing waits at a barrier.  SP is the number of splits
+// rounded up to a power of two: that many loads are issued at once per value.
+template <typename T, typename TB, int SP>
+__global__ void __launch_bounds__(ZI_WAVE)
+rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __restrict__ part, int splits,
+                           int64_t split_stride, int64_t ldp, const TB* __restrict__ bias,
+                           const int32_t* __restrict__ pos, const int32_t* __restrict__ slots,
+                           const float* __restrict__ inv_freq, T* __restrict__ kcache, T* __restrict__ vcache, int nh,
+                           int nkv, int d, int rot, int page_size, int64_t cache_slots) {
     const int64_t t = blockIdx.x;
+    const int hs = blockIdx.y, lane = threadIdx.x;
     const int half = rot / 2;
     const int qd = nh * d, kvd = nkv * d;
-    const int width = qd + (write_kv ? 2 * kvd : 0);
-    float* cs = sh;
-    float* row = sh + ((rot + 3) & ~3);
+    const bool is_q = hs < nh;
+    const int g = hs - nh;
+    const int col0 = is_q ? hs * d : qd + g * d;
     const float p = (float)pos[t];
-    for (int i = threadIdx.x; i < half; i += blockDim.x) {
-        float s, c;
-        sincosf(p * inv_freq[i], &s, &c);
-        cs[i] = c;
-        cs[half + i] = s;
-    }
     const float* pr = part + t * ldp;
-    if (vec4) {
-        // every split's load is issued before the first is used (host: splits <= 16, 16-byte alignment)
-        for (int i = threadIdx.x * 4; i < width; i += blockDim.x * 4) {
-            float4 d[16];
+    auto value = [&](int col) {
+        float v[SP];
 #pragma unroll
-            for (int s = 0; s < 16; ++s)
-                d[s] = (s < splits) ? *reinterpret_cast<const float4*>(pr + (int64_t)s * split_stride + i)
-                                    : make_float4(0.f, 0.f, 0.f, 0.f);
-            float4 v = d[0];
+        for (int s = 0; s < SP; ++s) v[s] = pr[(int64_t)(s < splits ? s : 0) * split_stride + col];
+        float acc = v[0];
 #pragma unroll
-            for (int s = 1; s < 16; ++s) { v.x += d[s].x; v.y += d[s].y; v.z += d[s].z; v.w += d[s].w; }
-            if (bias) {
-                v.x += zi_load(bias + i); v.y += zi_load(bias + i + 1); v.z += zi_load(bias + i + 2);
-                v.w += zi_load(bias + i + 3);
-            }
-            *reinterpret_cast<float4*>(row + i) = v;
-        }
+        for (int s = 1; s < SP; ++s) acc += s < splits ? v[s] : 0.f;
+        if (bias) acc += zi_load(bias + col);
+        return acc;
+    };
+    T* dst;
+    int64_t vbase = 0;
+    bool store_v = false;
+    if (is_q) {
+        dst = q_out + t * ldq + (int64_t)hs * d;
     } else {
-        for (int i = threadIdx.x; i < width; i += blockDim.x) {
-            float v = pr[i];
-            for (int s = 1; s < splits; ++s) v += pr[s * split_stride + i];
-            if (bias) v += zi_load(bias + i);
-            row[i] = v;
-        }
+        const int slot = slots[t];
+        if (slot < 0 || slot >= cache_slots) return;  // the host checks the range; never write outside the pool
+        const int64_t page = slot / page_size, off = slot % page_size;
+        dst = kcache + ((page * nkv + g) * page_size + off) * d;
+        vbase = (page * nkv + g) * d * page_size + off;
+        store_v = true;
     }
-    __syncthreads();
-    T* qr = q_out + t * ldq;
-    for (int i = threadIdx.x; i < qd; i += blockDim.x) {
-        const int h = i / d, j = i % d;
-        const float* base = row + h * d;
-        float v;
-        if (j < half) v = base[j] * cs[j] - base[j + half] * cs[half + j];
-        else if (j < rot) v = base[j] * cs[j - half] + base[j - half] * cs[j];
-        else v = base[j];
-        zi_store(qr + i, v);
+    for (int j = lane; j < half; j += ZI_WAVE) {
+        const float a = value(col0 + j), b = value(col0 + j + half);
+        float sn, cs;
+        sincosf(p * inv_freq[j], &sn, &cs);
+        zi_store(dst + j, a * cs - b * sn);
+        zi_store(dst + j + half, b * cs + a * sn);
     }
-    if (!write_kv) return;
-    const int slot = slots[t];
-    if (slot < 0 || slot >= cache_slots) return;  // the host checks the range; never write outside the pool
-    const int64_t page = slot / page_size, off = slot % page_size;
-    for (int i = threadIdx.x; i < kvd; i += blockDim.x) {
-        const int h = i / d, j = i % d;
-        const float* base = row + qd + h * d;
-        float kv;
-        if (j < half) kv = base[j] * cs[j] - base[j + half] * cs[half + j];
-        else if (j < rot) kv = base[j] * cs[j - half] + base[j - half] * cs[j];
-        else kv = base[j];
-        zi_store(kcache + ((page * nkv + h) * page_size + off) * d + j, kv);
-        zi_store(vcache + ((page * nkv + h) * d + j) * page_size + off, row[qd + kvd + i]);
-    }
+    for (int j = rot + lane; j < d; j += ZI_WAVE) zi_store(dst + j, value(col0 + j));
+    if (store_v)
+        for (int j = lane; j < d; j += ZI_WAVE) zi_store(vcache + vbase + (int64_t)j * page_size, value(qd + kvd + g * d + j));
 }
 
 extern "C" int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const float* part, int splits,
@@ -186,16 +167,23 @@ extern "C" int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const fl
                    page_size);
         ZI_REQUIRE(kcache && vcache && slots, "rope_kv_store_split: null cache pointer");
     }
-    const size_t lds = (size_t)(((rot + 3) & ~3) + width + 4) * sizeof(float);
-    const int vec4 = width % 4 == 0 && ldp % 4 == 0 && split_stride % 4 == 0 && ((uintptr_t)part % 16) == 0 && splits <= 16;
-    ZI_REQUIRE(lds <= 60 * 1024, "rope_kv_store_split: a row of %lld values does not fit in LDS", (long long)width);
+    ZI_REQUIRE(splits <= 16, "rope_kv_store_split: at most 16 splits (%d)", splits);
+    ZI_REQUIRE(nh + nkv <= 65535, "rope_kv_store_split: too many heads");
     if (n == 0) return 0;
     if (!bias) bias_dt = ZI_F32;
+    const dim3 grid(n, nh + (write_kv ? nkv : 0));
+#define ZI_RKS(SP)                                                                                                  \
+    rope_kv_store_split_kernel<T, TB, SP><<<grid, ZI_WAVE, 0, stream>>>(                                            \
+        (T*)q_out, ldq, part, splits, split_stride, ldp, (const TB*)bias, pos, slots, inv_freq, (T*)kcache, (T*)vcache, \
+        nh, nkv, d, rot, page_size, cache_slots)
     ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(bias_dt, TB, {
-        rope_kv_store_split_kernel<T, TB><<<n, 256, lds, stream>>>(
-            (T*)q_out, ldq, part, splits, split_stride, ldp, (const TB*)bias, pos, slots, inv_freq, (T*)kcache,
-            (T*)vcache, nh, nkv, d, rot, page_size, write_kv, cache_slots, vec4);
+        if (splits <= 1) ZI_RKS(1);
+        else if (splits <= 2) ZI_RKS(2);
+        else if (splits <= 4) ZI_RKS(4);
+        else if (splits <= 8) ZI_RKS(8);
+        else ZI_RKS(16);
     }));
+#undef ZI_RKS
     return zi_check_launch("rope_kv_store_split");
 }
 
