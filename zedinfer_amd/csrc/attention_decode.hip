@@ -60,7 +60,7 @@ __host__ __device__ __forceinline__ DecSplit dec_split(int p, int window) {
 }
 
 template <int D>
-__global__ void __launch_bounds__(DEC_WAVES* ZI_WAVE)
+__global__ void __launch_bounds__(DEC_WAVES* ZI_WAVE, 2)
 attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restrict__ part_o,
                         float* __restrict__ part_ml, const zi_bf16* __restrict__ q, int64_t ldq,
                         const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,

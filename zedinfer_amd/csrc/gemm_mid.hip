@@ -3,41 +3,52 @@
 //
 // A workgroup of four wavefronts owns 64 weight rows (16 a wavefront) and a range of k.  It walks its
 // k-blocks of 128: the block's slice of x (up to 64 rows x 128 values) is staged in LDS once for the four
-// wavefronts, each wavefront reads its own 16 weight rows straight from memory into matrix-core operands
-// (v_mfma_f32_16x16x32_bf16, float32 accumulation) and keeps the sums of its 16 x M outputs in registers,
-// so nothing is added across wavefronts.  The next block's weights and x travel while the current one is
-// worked on (a ring of register buffers; loads are issued without branches so that they stay in
-// flight).  The k dimension is cut over gridDim.y workgroups when N alone gives too few of them; those
+// wavefronts, each wavefront reads its own 16 weight rows from memory as whole cache lines, turns them
+// into matrix-core operands through a piece of LDS of its own (v_mfma_f32_16x16x32_bf16, float32
+// accumulation) and keeps the sums of its 16 x M outputs in registers, so nothing is added across
+// wavefronts.  The next two blocks' weights and x travel while the current one is worked on (a ring of
+// three register buffers; loads are issued without branches so that they stay in flight).  The k dimension is cut over gridDim.y workgroups when N alone gives too few of them; those
 // leave float32 partial sums [split][M][N] that the consumer adds in rising order.  The cut depends on N
 // and K only.  Epilogues as in the few-rows kernel: plain (bias), partial sums, SwiGLU over gate/up rows
 // interleaved in blocks of 8.
 #include "zi_common.h"
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 gm_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float gm_f32x4_t;
+// 16 bytes as a native vector: copies of the struct uint4 are memcpys to the compiler, and an array of
+// them that is only copied stays in memory instead of registers
+typedef __attribute__((ext_vector_type(4))) unsigned gm_u32x4_t;
 
 #define GM_WAVES 4
 #define GM_ROWS 64          // weight rows per workgroup
 #define GM_KB 128
 #define GM_XS (GM_KB + 8)   // LDS row stride of the x slice, in elements
 #define GM_TARGET_WGS 384
-#define GM_RING 3           // k-blocks of weights in flight per wavefront
 
 #define GM_MODE_PLAIN 0
 #define GM_MODE_PARTIAL 1
 #define GM_MODE_SWIGLU 2
 
 union gm_pack {
-    uint4 u;
+    gm_u32x4_t u;
     gm_bf16x8_t b;
 };
 
-template <int MT>
+// v where `keep` holds, else zeros, by arithmetic: after a select the compiler may move the load that
+// made v under a branch, and wait for it there.
+__device__ __forceinline__ gm_u32x4_t gm_keep(gm_u32x4_t v, bool keep) {
+    const unsigned mask = 0u - (unsigned)keep;
+    return v & mask;
+}
+
+template <int MT, int GM_RING>
 __global__ void __launch_bounds__(GM_WAVES* ZI_WAVE)
 gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __restrict__ x,
                 const zi_bf16* __restrict__ w, const zi_bf16* __restrict__ bias, int M, int N, int K, int64_t ldx,
                 int64_t ldw, int64_t ldo, int kb_per_split, int vec_out) {
     __shared__ __attribute__((aligned(16))) uint16_t xs[2][MT * 16 * GM_XS];
+    __shared__ __attribute__((aligned(16))) uint16_t wt[GM_WAVES][16 * GM_XS];   // a wavefront's weight tile
     const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
     const int r = lane & 15, j = lane >> 4;
     const int split = blockIdx.y;
@@ -45,74 +56,112 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     const int kb_lo = split * kb_per_split;
     const int kb_hi = (kb_lo + kb_per_split < kb_total) ? kb_lo + kb_per_split : kb_total;
     const int n0 = blockIdx.x * GM_ROWS + wave * 16;
-    const int nrow = (n0 + r < N) ? n0 + r : N - 1;
-    const zi_bf16* wrow_base = w + (int64_t)nrow * ldw;
+    // Weights are read as whole cache lines: a load instruction takes 4 rows x 256 bytes (lane l: row
+    // l / 16 of the four, 16-byte piece l % 16), four instructions a tile of 16 rows x 128 values.
+    // Loads in the matrix-core operand layout (16 rows x 64 bytes an instruction) were measured a fifth
+    // slower.  The tile is turned into that layout through a piece of LDS that the wavefront owns.
+    const int wq = lane & 15;
+    const zi_bf16* wrow[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int n = n0 + c * 4 + j;
+        wrow[c] = w + (int64_t)(n < N ? n : N - 1) * ldw;
+    }
+    uint16_t* wt_put = &wt[wave][j * GM_XS + wq * 8];        // + c * 4 rows
+    const uint16_t* wt_get = &wt[wave][r * GM_XS + j * 8];   // + c * 32 values
 
     // what this thread stages of a block's x slice: MT pieces of 16 bytes (row srow + 16 * t, piece spc)
     const int srow = tid / 16, spc = tid % 16;
     // the weights of GM_RING k-blocks are in flight at once (a ring of register buffers); the x slice of
     // the next block is fetched while this one is worked on
-    uint4 ring[GM_RING][4], xring[GM_RING][MT];
-    // Loads are issued without branches (addresses are clamped into the matrix, what lies outside is
-    // zeroed afterwards): only then does the compiler let several blocks' loads stay in flight.
+    gm_u32x4_t ring[GM_RING][4], xring[GM_RING][MT];
+    // Loads are issued without branches and their results are not touched before the products need
+    // them: only then does the compiler let several blocks' loads stay in flight.  Addresses are
+    // clamped into the matrices.  Rows of x past M repeat the last row and give outputs that nobody
+    // stores; columns past K would count the last eight twice, so the weights are zeroed there, when
+    // they are used.  A block's x is requested before its weights: loads return in order, and x, which
+    // comes from the cache and is wanted a step earlier, must not queue behind weights from memory.
     const int xm_last = M - 1;
-    auto fetch = [&](uint4 (&a)[4], uint4 (&xr)[MT], int kb) {
+    auto fetch = [&](const int slot, int kb) __attribute__((always_inline)) {
         const int k0 = kb * GM_KB;
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            const int k = k0 + c * 32 + j * 8;
-            const uint4 v = *reinterpret_cast<const uint4*>(wrow_base + (k < K ? k : K - 8));
-            a[c] = k < K ? v : make_uint4(0, 0, 0, 0);
-        }
 #pragma unroll
         for (int t = 0; t < MT; ++t) {
             const int m = t * 16 + srow, k = k0 + spc * 8;
-            const uint4 v = *reinterpret_cast<const uint4*>(x + (int64_t)(m < M ? m : xm_last) * ldx + (k < K ? k : K - 8));
-            xr[t] = (m < M && k < K) ? v : make_uint4(0, 0, 0, 0);
+            xring[slot][t] = *reinterpret_cast<const gm_u32x4_t*>(x + (int64_t)(m < M ? m : xm_last) * ldx + (k < K ? k : K - 8));
         }
-    };
-    auto stash = [&](const uint4 (&xr)[MT], int b) {
+        const int k = k0 + wq * 8;
 #pragma unroll
-        for (int t = 0; t < MT; ++t) *reinterpret_cast<uint4*>(&xs[b][(t * 16 + srow) * GM_XS + spc * 8]) = xr[t];
+        for (int c = 0; c < 4; ++c) ring[slot][c] = *reinterpret_cast<const gm_u32x4_t*>(wrow[c] + (k < K ? k : K - 8));
+    };
+    auto stash = [&](const int slot, int b) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < MT; ++t) *reinterpret_cast<gm_u32x4_t*>(&xs[b][(t * 16 + srow) * GM_XS + spc * 8]) = xring[slot][t];
     };
     gm_f32x4_t acc[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) acc[t] = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    // blocks kb_lo .. kb_lo + GM_RING - 2 are requested up front; block kb's x goes to LDS one iteration
-    // before it is used, GM_RING - 2 iterations after it was requested
-    const int kb_last = kb_hi - 1;    // requests past the last block fetch it again: no branch around a load
-#pragma unroll
-    for (int b = 0; b < GM_RING - 1; ++b) fetch(ring[b], xring[b], kb_lo + b < kb_hi ? kb_lo + b : kb_last);
-    stash(xring[0], 0);
-    __syncthreads();
+    // Blocks kb_lo .. kb_lo + GM_RING - 2 are requested up front; block kb's x goes to LDS one step
+    // before it is used, GM_RING - 2 steps after it was requested.  Block kb lives in ring slot
+    // (kb - kb_lo) % GM_RING.  The compiler counts how many loads may stay in flight at each use only
+    // in straight-line code; behind a branch that may or may not have issued loads it waits for all of
+    // them.  So the walk is cut into pieces without such branches: a steady loop of GM_RING steps that
+    // all request a block, and one of GM_RING straight-line endings, chosen by how many blocks are
+    // left to request.
     int cur = 0;
-    for (int kb0 = kb_lo; kb0 < kb_hi; kb0 += GM_RING) {
+    auto step = [&](const int slot, int kb, const bool request) __attribute__((always_inline)) {
+        if (request) fetch((slot + GM_RING - 1) % GM_RING, kb + GM_RING - 1);
+        // all of the block's x operands are read from LDS before the first product: the reads' latency
+        // is paid once, not once per product
+        // the weight tile goes through the wavefront's LDS piece (zeros past K: the last block only);
+        // LDS serves a wavefront's instructions in order, so no barrier stands between put and get
 #pragma unroll
-        for (int b = 0; b < GM_RING; ++b) {
-            const int kb = kb0 + b;
-            if (kb >= kb_hi) break;
-            fetch(ring[(b + GM_RING - 1) % GM_RING], xring[(b + GM_RING - 1) % GM_RING],
-                  kb + GM_RING - 1 < kb_hi ? kb + GM_RING - 1 : kb_last);
-            // all of the block's x operands are read from LDS before the first product: the reads' latency
-            // is paid once, not once per product
-            gm_pack bb[4][MT];
+        for (int c = 0; c < 4; ++c)
+            *reinterpret_cast<gm_u32x4_t*>(wt_put + c * 4 * GM_XS) = gm_keep(ring[slot][c], kb * GM_KB + wq * 8 < K);
+        gm_pack bb[4][MT], a[4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c)
+        for (int c = 0; c < 4; ++c)
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    bb[c][t].u = *reinterpret_cast<const uint4*>(&xs[cur][(t * 16 + r) * GM_XS + c * 32 + j * 8]);
+            for (int t = 0; t < MT; ++t)
+                bb[c][t].u = *reinterpret_cast<const gm_u32x4_t*>(&xs[cur][(t * 16 + r) * GM_XS + c * 32 + j * 8]);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                gm_pack a;
-                a.u = ring[b][c];
+        for (int c = 0; c < 4; ++c) a[c].u = *reinterpret_cast<const gm_u32x4_t*>(wt_get + c * 32);
 #pragma unroll
-                for (int t = 0; t < MT; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, bb[c][t].b, acc[t], 0, 0, 0);
-            }
-            if (kb + 1 < kb_hi) stash(xring[(b + 1) % GM_RING], cur ^ 1);
-            __syncthreads();
-            cur ^= 1;
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[c].b, bb[c][t].b, acc[t], 0, 0, 0);
+        stash((slot + 1) % GM_RING, cur ^ 1);    // after the last block: something nobody reads
+        __syncthreads();
+        cur ^= 1;
+    };
+    // the ending for `left` blocks still to request: left + GM_RING - 1 blocks to work on
+    auto ending = [&](auto left_c, int kb0) __attribute__((always_inline)) {
+        constexpr int LEFT = decltype(left_c)::value;
+#pragma unroll
+        for (int i = 0; i < LEFT + GM_RING - 1; ++i) step(i % GM_RING, kb0 + i, i < LEFT);
+    };
+#pragma unroll
+    for (int b = 0; b < GM_RING - 1; ++b) fetch(b, kb_lo + b < kb_hi ? kb_lo + b : kb_hi - 1);
+    stash(0, 0);
+    __syncthreads();
+    int kb0 = kb_lo;
+    for (; kb0 + 2 * GM_RING - 1 <= kb_hi; kb0 += GM_RING) {
+#pragma unroll
+        for (int b = 0; b < GM_RING; ++b) step(b, kb0 + b, true);
+    }
+    const int left = kb_hi - kb0 - (GM_RING - 1);    // < 0: fewer blocks than the ring requests up front
+    if (left < 0) {
+#pragma unroll
+        for (int b = 0; b < GM_RING - 1; ++b)
+            if (kb0 + b < kb_hi) step(b, kb0 + b, false);
+    } else {
+        static_assert(GM_RING >= 2 && GM_RING <= 4, "one ending per residue");
+        switch (left) {
+            case 0: ending(std::integral_constant<int, 0>{}, kb0); break;
+            case 1: ending(std::integral_constant<int, 1>{}, kb0); break;
+            case 2: if (GM_RING > 2) ending(std::integral_constant<int, 2>{}, kb0); break;
+            default: if (GM_RING > 3) ending(std::integral_constant<int, 3>{}, kb0); break;
         }
     }
     // C[n = n0 + j*4 + e][m = t*16 + r]
@@ -199,9 +248,9 @@ int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const
     zi_gemm_mid_plan(N, K, &splits, &per);
     const dim3 grid((N + GM_ROWS - 1) / GM_ROWS, splits);
     const int mt = (M + 15) / 16;
-#define ZI_GM(MT)                                                                                                  \
-    gemm_mid_kernel<MT><<<grid, GM_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, ldw, \
-                                                                 ldo, per, vec_out)
+#define ZI_GM(MT)                                                                                            \
+    gemm_mid_kernel<MT, 3><<<grid, GM_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, \
+                                                                    ldw, ldo, per, vec_out)
     switch (mt) {
         case 1: ZI_GM(1); break;
         case 2: ZI_GM(2); break;
