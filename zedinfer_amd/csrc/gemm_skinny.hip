@@ -22,8 +22,8 @@
 //
 // Operand layout.  For one MFMA the A operand is a 16 x 32 tile of w (lane l: row l%16, the eight
 // consecutive k starting at 8 * (l/16)) and the B operand the matching 32 x 16 tile of x^T (lane l: row
-// l%16 of x, the same eight k).  A k-block of 128 is four such MFMAs; each of a wavefront's load
-// instructions reads 64 contiguous bytes of each of its 16 rows.
+// l%16 of x, the same eight k).  A k-block of 128 is four such MFMAs.  x is loaded in that layout; the
+// weights are loaded as whole cache lines and rearranged through LDS.
 #include "zi_common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -31,6 +31,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
 #define SK_ROWS 16
 #define SK_KB 128
+#define SK_WS (SK_KB + 8)   // LDS row stride of a weight tile, in elements
 #define SK_WAVES 4
 #define SK_MAX_KPW 4
 #define SK_RESIDENT_WGS 480   // workgroups that are surely resident at once (256 compute units, two each)
@@ -41,31 +42,26 @@ typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 #define SK_MODE_PARTIAL 1
 #define SK_MODE_SWIGLU 2
 
-__device__ __forceinline__ bf16x8_t as_bf16x8(const uint4& v) {
-    union { uint4 u; bf16x8_t b; } c;
+// 16 bytes as a native vector (copies of the struct uint4 are memcpys to the compiler, and an array of
+// them that is only copied may stay in memory instead of registers)
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4_t;
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t& v) {
+    union { u32x4_t u; bf16x8_t b; } c;
     c.u = v;
     return c.b;
 }
 
-// The four 16-byte pieces of row `row` this lane owns in k-block `kb`: piece c holds
-// k = kb*128 + c*32 + j*8 .. +8, so that one load instruction reads 64 contiguous bytes of each of the
-// wavefront's 16 rows.  Pieces past K are read from the row's last piece instead (K % 8 == 0): no branch
-// goes around a load, so that the compiler lets the loads of several tiles stay in flight.  What such
-// pieces hold does not matter for the weights (x is zero there); `sk_load_row_masked` zeroes them for x.
-__device__ __forceinline__ void sk_load_row(uint4 (&dst)[4], const zi_bf16* row, int kb, int j, int K) {
+// The four 16-byte pieces of x row `row` this lane owns in k-block `kb`, in the matrix-core operand layout:
+// piece c holds k = kb*128 + c*32 + j*8 .. +8.  Pieces past K, and all pieces when `live` is false, are zero.
+__device__ __forceinline__ void sk_load_x(u32x4_t (&dst)[4], const zi_bf16* row, int kb, int j, int K, bool live) {
     const int k0 = kb * SK_KB + j * 8;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const int k = k0 + c * 32;
-        dst[c] = *reinterpret_cast<const uint4*>(row + (k < K ? k : K - 8));
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(row + (k < K ? k : K - 8));
+        dst[c] = (live && k < K) ? v : u32x4_t{0u, 0u, 0u, 0u};
     }
-}
-__device__ __forceinline__ void sk_load_row_masked(uint4 (&dst)[4], const zi_bf16* row, int kb, int j, int K, bool live) {
-    sk_load_row(dst, row, kb, j, K);
-    const int k0 = kb * SK_KB + j * 8;
-#pragma unroll
-    for (int c = 0; c < 4; ++c)
-        if (!live || k0 + c * 32 >= K) dst[c] = make_uint4(0, 0, 0, 0);
 }
 
 template <int KPW>
@@ -75,6 +71,7 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
                    int tiles_per_wg, int vec_out) {
     constexpr int MT = 1;              // up to 16 rows of x: one matrix-core tile
     __shared__ f32x4_t red[2][SK_WAVES][MT][ZI_WAVE];
+    __shared__ __attribute__((aligned(16))) uint16_t wt[SK_WAVES][SK_ROWS * SK_WS];   // a wavefront's weight tile
     const int lane = threadIdx.x & (ZI_WAVE - 1), wave = threadIdx.x / ZI_WAVE;
     const int r = lane & 15, j = lane >> 4;
     const int split = blockIdx.y;
@@ -94,27 +91,53 @@ gemm_skinny_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16*
     // the last one (a wavefront that has fewer than KPW blocks reads the last block again and multiplies
     // it by zero).
     const int kb_last = kb_total - 1;
-    uint4 xr[KPW][4];
+    u32x4_t xr[KPW][4];
 #pragma unroll
     for (int i = 0; i < KPW; ++i)
-        sk_load_row_masked(xr[i], xrow[0], kb0 + i < kb_total ? kb0 + i : kb_last, j, K, kb0 + i < kb_total);
-    uint4 ring[2][KPW][4];
-    auto issue = [&](uint4 (&dst)[KPW][4], int tile) {
-        const int nrow = (tile * SK_ROWS + r < N) ? tile * SK_ROWS + r : N - 1;
+        sk_load_x(xr[i], xrow[0], kb0 + i < kb_total ? kb0 + i : kb_last, j, K, kb0 + i < kb_total);
+    // Weights are read as whole cache lines: a load instruction takes 4 rows x 256 bytes (lane l: row
+    // l / 16 of the four, 16-byte piece l % 16), four instructions a tile of 16 rows x one k-block.  Loads
+    // in the operand layout (16 rows x 64 bytes an instruction) were measured a fifth slower.  A tile is
+    // turned into operands through a piece of LDS that the wavefront owns.  No branch goes around a load
+    // (pieces past K are read from the row's last piece instead, K % 8 == 0; x is zero there), so that the
+    // compiler lets the loads of two tiles stay in flight.
+    const int wq = lane & 15;
+    int wk[KPW];
 #pragma unroll
-        for (int i = 0; i < KPW; ++i)
-            sk_load_row(dst[i], w + (int64_t)nrow * ldw, kb0 + i < kb_total ? kb0 + i : kb_last, j, K);
+    for (int i = 0; i < KPW; ++i) {
+        const int k = (kb0 + i < kb_total ? kb0 + i : kb_last) * SK_KB + wq * 8;
+        wk[i] = k < K ? k : K - 8;
+    }
+    uint16_t* wt_put = &wt[wave][j * SK_WS + wq * 8];        // + c * 4 rows
+    const uint16_t* wt_get = &wt[wave][r * SK_WS + j * 8];   // + c * 32 values
+    u32x4_t ring[2][KPW][4];
+    auto issue = [&](u32x4_t (&dst)[KPW][4], int tile) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int n = tile * SK_ROWS + c * 4 + j;
+            const zi_bf16* row = w + (int64_t)(n < N ? n : N - 1) * ldw;
+#pragma unroll
+            for (int i = 0; i < KPW; ++i) dst[i][c] = *reinterpret_cast<const u32x4_t*>(row + wk[i]);
+        }
     };
     int buf = 0;
-    auto process = [&](uint4 (&a)[KPW][4], int tile) {
+    auto process = [&](u32x4_t (&a)[KPW][4], int tile) {
         f32x4_t acc[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < KPW; ++i)
+        for (int i = 0; i < KPW; ++i) {
+            // LDS serves a wavefront's instructions in order: no barrier between put and get, and the
+            // next block's put cannot overtake this block's get
+            u32x4_t b[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) *reinterpret_cast<u32x4_t*>(wt_put + c * 4 * SK_WS) = a[i][c];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) b[c] = *reinterpret_cast<const u32x4_t*>(wt_get + c * 32);
 #pragma unroll
             for (int c = 0; c < 4; ++c)
-                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[i][c]), as_bf16x8(xr[i][c]), acc[0], 0, 0, 0);
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(b[c]), as_bf16x8(xr[i][c]), acc[0], 0, 0, 0);
+        }
 #pragma unroll
         for (int t = 0; t < MT; ++t) red[buf][wave][t][lane] = acc[t];
         __syncthreads();
