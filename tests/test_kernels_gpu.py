@@ -325,6 +325,81 @@ def test_attention_decode(ops, nh, nkv, d, ps, T, window):
     torch.testing.assert_close(out.float(), plain_out.float(), atol=1e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps,lens,window,S,bias_dtype,rot", [
+    (12, 2, 128, 16, [2100, 1, 64, 65, 257, 300, 1024, 17], 0, 2, torch.bfloat16, 128),
+    (3, 1, 64, 8, [200, 5, 9], 0, 1, None, 64),
+    (8, 2, 48, 8, [33, 700, 256], 0, 3, torch.float32, 32),
+    (4, 2, 128, 16, [500, 120, 99], 100, 5, torch.bfloat16, 128),
+    (6, 3, 80, 32, [150, 64], 0, 2, torch.bfloat16, 0),
+    (12, 2, 128, 16, [17000, 300], 0, 2, torch.bfloat16, 128)])
+def test_attention_decode_fused(ops, nh, nkv, d, ps, lens, window, S, bias_dtype, rot):
+    """One kernel for rotation, cache store and attention of decoded tokens gives what the rotary kernel
+    followed by the decode kernel gives: same output, same new keys and values in the cache.  The slot
+    of the new token holds NaN before, and the sequences differ in length (the new key sits in every
+    place of a block)."""
+    dtype = torch.bfloat16
+    B, width, theta = len(lens), (nh + 2 * nkv) * d, 1e4
+    assert ops.attention_decode_fused_supported(dtype, nh, nkv, d, ps, rot, S, width, B)
+    pages_per = [(L + ps - 1) // ps for L in lens]
+    total_pages = sum(pages_per) + 2
+    g = torch.Generator().manual_seed(5)
+    perm = torch.randperm(total_pages, generator=g).tolist()
+    kc = torch.full((total_pages, nkv, ps, d), float("nan"), dtype=dtype, device="cuda")
+    vc = torch.full((total_pages, nkv, d, ps), float("nan"), dtype=dtype, device="cuda")
+    bt = torch.full((B, max(pages_per)), -1, dtype=torch.int32)
+    slots = torch.empty(B, dtype=torch.int32)
+    for b, L in enumerate(lens):
+        mine = [perm.pop() for _ in range(pages_per[b])]
+        bt[b, :len(mine)] = torch.tensor(mine, dtype=torch.int32)
+        k, v = rnd(L - 1, nkv, d, dtype=dtype, seed=10 + b), rnd(L - 1, nkv, d, dtype=dtype, seed=20 + b)
+        for t in range(L - 1):       # the last position is the new token's: its slot stays NaN
+            kc[mine[t // ps], :, t % ps] = k[t]
+            vc[mine[t // ps], :, :, t % ps] = v[t]
+        slots[b] = mine[(L - 1) // ps] * ps + (L - 1) % ps
+    bt, slots = bt.cuda(), slots.cuda()
+    pos = torch.tensor([L - 1 for L in lens], dtype=torch.int32, device="cuda")
+    seq = torch.arange(B, dtype=torch.int32, device="cuda")
+    sums = rnd(S, B, width, seed=1)
+    bias = rnd(width, seed=2).to(bias_dtype) if bias_dtype is not None else None
+    inv_freq = ops.rope_inv_freq(rot, theta, "cuda") if rot else None
+    scale, T = 1 / math.sqrt(d), max(lens)
+    # the two kernels
+    kc1, vc1 = kc.clone(), vc.clone()
+    q = torch.empty(B, nh * d, dtype=dtype, device="cuda")
+    ops.rope_kv_store_sums(sums, bias, q, pos, slots, inv_freq, kc1, vc1, nh, nkv, d)
+    ref = ops.attention_decode(q, kc1, vc1, seq, pos, bt, nh, nkv, d, scale, T, window)
+    # the one kernel
+    kc2, vc2 = kc.clone(), vc.clone()
+    table = ops.rope_table(pos, inv_freq) if rot else None
+    out = ops.attention_decode_fused(sums, bias, table, slots, kc2, vc2, seq, pos, bt, nh, nkv, d, scale, T, window)
+    assert not torch.isnan(out).any()
+    torch.testing.assert_close(out.float(), ref.float(), atol=4e-3, rtol=1e-2)
+    for b in range(B):
+        pg, o = int(slots[b]) // ps, int(slots[b]) % ps
+        torch.testing.assert_close(kc2[pg, :, o].float(), kc1[pg, :, o].float(), atol=1e-3, rtol=8e-3)
+        assert torch.equal(vc2[pg, :, :, o], vc1[pg, :, :, o])
+    # nothing else in the cache was touched
+    same_k = (kc2 == kc1) | (torch.isnan(kc2) & torch.isnan(kc1))
+    same_v = (vc2 == vc1) | (torch.isnan(vc2) & torch.isnan(vc1))
+    for b in range(B):
+        pg, o = int(slots[b]) // ps, int(slots[b]) % ps
+        same_k[pg, :, o] = True
+    assert bool(same_k.all()) and bool(same_v.all())
+    # a layer that reads another layer's cache: queries only, the cache is left alone
+    kc3, vc3 = kc1.clone(), vc1.clone()
+    out3 = ops.attention_decode_fused(sums, bias, table, None, kc3, vc3, seq, pos, bt, nh, nkv, d, scale, T, window,
+                                      write_kv=False)
+    torch.testing.assert_close(out3.float(), ref.float(), atol=4e-3, rtol=1e-2)
+    assert bool(((kc3 == kc1) | (torch.isnan(kc3) & torch.isnan(kc1))).all())
+    assert bool(((vc3 == vc1) | (torch.isnan(vc3) & torch.isnan(vc1))).all())
+
+
+def test_attention_decode_fused_refuses_other_layouts(ops):
+    assert not ops.attention_decode_fused_supported(torch.bfloat16, 12, 2, 128, 16, 24, 2, 2048, 8)    # rot % 16
+    assert not ops.attention_decode_fused_supported(torch.bfloat16, 12, 2, 128, 16, 128, 2, 2050, 8)   # stride % 4
+    assert not ops.attention_decode_fused_supported(torch.float32, 12, 2, 128, 16, 128, 2, 2048, 8)
+
+
 def test_attention_decode_ignores_stale_slots(ops):
     """Slots of a page beyond the token's position may hold anything, NaN included."""
     nh, nkv, d, ps, T = 4, 2, 128, 16, 37

@@ -59,20 +59,40 @@ __host__ __device__ __forceinline__ DecSplit dec_split(int p, int window) {
     return s;
 }
 
-template <int D>
+// The projections of the step's tokens as they leave the matrix product, for the kernel variant that
+// rotates and stores them itself (FUSED): row t of `sums` holds the query heads, then the key heads, then
+// the value heads, as `splits` float32 partial sums that are added in rising order, then the bias.
+// The first `rot` dims of every query and key head turn by the angles of `table` ([token][rot/2][cos,
+// sin]); the token's new key and value go to slot slots[t] of the cache.
+struct DecProjection {
+    const float* sums;
+    int splits;
+    int64_t split_stride, ldp;
+    const void* bias;      // null: none
+    int bias_f32;
+    const float* table;    // null when rot == 0
+    int rot;
+    const int32_t* slots;
+    int64_t cache_slots;
+    int write_kv;
+};
+
+template <int D, bool FUSED>
 __global__ void __launch_bounds__(DEC_WAVES* ZI_WAVE, 2)
 attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restrict__ part_o,
                         float* __restrict__ part_ml, const zi_bf16* __restrict__ q, int64_t ldq,
-                        const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,
+                        const zi_bf16* kcache, const zi_bf16* vcache,
                         const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
                         int max_pages, int num_pages, int nh, int nkv, int G, int ps, int window, float scale,
-                        int max_chunks) {
+                        int max_chunks, DecProjection pj) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DT = D / 16;          // output tiles of 16 dims
     __shared__ float sm[DEC_WAVES][16], sl[DEC_WAVES][16];
     __shared__ dec_f32x4_t so[DEC_WAVES][DT][ZI_WAVE];
+    __shared__ uint4 sk[DK][4];        // FUSED: the token's own key, in pieces (k-step, j)
+    __shared__ uint16_t sv[D];         // and its value
 
     const int x = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
     const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
@@ -96,15 +116,155 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     const int k_end = (k_begin + quarter < p + 1) ? k_begin + quarter : p + 1;   // one past the wavefront's last key
     const int p8 = p & ~7, pi_last = max_pages - 1;
 
-    // the group's queries as the B operand: lane (r, j) holds head r, dims dk*32 + j*8 ..
-    dec_bf16x8_t qop[DK];
+    // FUSED: eight consecutive columns of the token's projection row (splits added in rising order, then
+    // the bias), and the same after the rotation of head column `hc`, dims dim0 .. dim0 + 7.  Four
+    // splits' loads are issued at a time (the split index is clamped, what is past the count adds zero).
+    const int half = pj.rot / 2;
+    auto value8 = [&](int col, float (&v)[8]) {
+        const float* p0 = pj.sums + (int64_t)t * pj.ldp + col;
 #pragma unroll
-    for (int dk = 0; dk < DK; ++dk) {
+        for (int e = 0; e < 8; ++e) v[e] = 0.f;
+        auto four = [&](int s0) {
+            float4 a[4], b[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const float* ps2 = p0 + (int64_t)(s0 + u < pj.splits ? s0 + u : s0) * pj.split_stride;
+                a[u] = *reinterpret_cast<const float4*>(ps2);
+                b[u] = *reinterpret_cast<const float4*>(ps2 + 4);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const float keep = s0 + u < pj.splits ? 1.f : 0.f;     // x * 1 is exact; sums are finite
+                v[0] += a[u].x * keep; v[1] += a[u].y * keep; v[2] += a[u].z * keep; v[3] += a[u].w * keep;
+                v[4] += b[u].x * keep; v[5] += b[u].y * keep; v[6] += b[u].z * keep; v[7] += b[u].w * keep;
+            }
+        };
+        four(0);      // straight-line: the loads of several calls travel together
+        for (int s0 = 4; s0 < pj.splits; s0 += 4) four(s0);
+        if (pj.bias) {
+            if (pj.bias_f32) {
+                const float4 a = *reinterpret_cast<const float4*>((const float*)pj.bias + col);
+                const float4 b = *reinterpret_cast<const float4*>((const float*)pj.bias + col + 4);
+                v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w; v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+            } else {
+                dec_pack w;
+                w.u = *reinterpret_cast<const uint4*>((const zi_bf16*)pj.bias + col);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += __uint_as_float((uint32_t)w.h[e] << 16);
+            }
+        }
+    };
+    // one column of the row, the same sum
+    auto value1 = [&](int col) {
+        const float* p0 = pj.sums + (int64_t)t * pj.ldp + col;
+        float v = 0.f;
+        auto four = [&](int s0) {
+            float a[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) a[u] = p0[(int64_t)(s0 + u < pj.splits ? s0 + u : s0) * pj.split_stride];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v += a[u] * (s0 + u < pj.splits ? 1.f : 0.f);
+        };
+        four(0);
+        for (int s0 = 4; s0 < pj.splits; s0 += 4) four(s0);
+        if (pj.bias) v += pj.bias_f32 ? ((const float*)pj.bias)[col] : zi_load((const zi_bf16*)pj.bias + col);
+        return v;
+    };
+    auto rotated8 = [&](int hc, int dim0) {
+        float a[8];
+        value8(hc + dim0, a);
+        if (dim0 < pj.rot) {     // rot / 2 is a multiple of 8 (host): the eight dims lie on one side
+            const bool first = dim0 < half;
+            float b[8];
+            value8(hc + (first ? dim0 + half : dim0 - half), b);
+            const float4* cs = reinterpret_cast<const float4*>(pj.table + ((int64_t)t * half + (first ? dim0 : dim0 - half)) * 2);
+#pragma unroll
+            for (int e2 = 0; e2 < 4; ++e2) {
+                const float4 w = cs[e2];     // cos, sin of two pairs
+                a[2 * e2] = first ? a[2 * e2] * w.x - b[2 * e2] * w.y : a[2 * e2] * w.x + b[2 * e2] * w.y;
+                a[2 * e2 + 1] = first ? a[2 * e2 + 1] * w.z - b[2 * e2 + 1] * w.w : a[2 * e2 + 1] * w.z + b[2 * e2 + 1] * w.w;
+            }
+        }
         dec_pack w;
-        w.u = make_uint4(0, 0, 0, 0);
-        if (r < G && dk * 32 + j * 8 < D)
-            w.u = *reinterpret_cast<const uint4*>(q + (int64_t)t * ldq + (int64_t)(kvh * G + r) * D + dk * 32 + j * 8);
-        qop[dk] = w.b;
+        w.u.x = zi_pack_bf16x2(a[0], a[1]); w.u.y = zi_pack_bf16x2(a[2], a[3]);
+        w.u.z = zi_pack_bf16x2(a[4], a[5]); w.u.w = zi_pack_bf16x2(a[6], a[7]);
+        return w;
+    };
+    // The group's queries as the B operand: lane (r, j) holds head r, dims dk*32 + j*8 ...  FUSED: every
+    // wavefront wants the same operand, so each makes the pieces of one k-step and they trade through
+    // LDS.  In the workgroup of the last chunk, which holds position p, they make the token's own key
+    // (a row of lanes that has no query head, or a second pass) and value the same way.  The wavefront
+    // that owns position p stores them to the cache and puts them into its operands; nobody else reads
+    // that slot in this kernel.
+    const bool last_chunk = FUSED && pj.write_kv && chunk == sp.count - 1;
+    const bool owner = last_chunk && p >= k_begin && p < k_begin + quarter;
+    // where position p sits in the operands of its block: score tile tt_p, row r_p; value operand b_p,
+    // lanes j_p, element e_p
+    const int kk_p = (p - k_begin) % DEC_BLOCK;
+    const int tt_p = (kk_p / 32) * 2 + (kk_p % 8) / 4, r_p = ((kk_p % 32) / 8) * 4 + kk_p % 4;
+    const int b_p = kk_p / 32, j_p = (kk_p % 32) / 8, e_p = kk_p % 8;
+    uint4 knew[DK];
+    uint32_t vnew[DT / 2 + 1];
+    dec_bf16x8_t qop[DK];
+    if (FUSED) {
+        uint4* sq = reinterpret_cast<uint4*>(&so[0][0][0]);      // [DK][64]; the merge uses `so` much later
+        const int key_row = G < 16 ? G : 0;      // the lanes that make the key's pieces
+        for (int dk = wave; dk < DK; dk += DEC_WAVES) {
+            const bool piece = dk * 32 + j * 8 < D;
+            const bool for_key = last_chunk && G < 16 && r == key_row;
+            dec_pack w;
+            w.u = make_uint4(0, 0, 0, 0);
+            if ((r < G || for_key) && piece) w = rotated8(for_key ? (nh + kvh) * D : (kvh * G + r) * D, dk * 32 + j * 8);
+            if (for_key) {
+                sk[dk][j] = w.u;
+                w.u = make_uint4(0, 0, 0, 0);
+            }
+            sq[dk * ZI_WAVE + lane] = w.u;
+            if (last_chunk && G == 16 && r == key_row) {
+                dec_pack w2;
+                w2.u = make_uint4(0, 0, 0, 0);
+                if (piece) w2 = rotated8((nh + kvh) * D, dk * 32 + j * 8);
+                sk[dk][j] = w2.u;
+            }
+        }
+        if (last_chunk)
+            for (int dim = threadIdx.x; dim < D; dim += DEC_WAVES * ZI_WAVE)
+                sv[dim] = zi_float_to_bf16(value1((nh + nkv + kvh) * D + dim));
+        __syncthreads();
+#pragma unroll
+        for (int dk = 0; dk < DK; ++dk) {
+            dec_pack w;
+            w.u = sq[dk * ZI_WAVE + lane];
+            qop[dk] = w.b;
+        }
+        if (owner) {
+            const int slot = pj.slots[t];
+            const bool inside = slot >= 0 && slot < pj.cache_slots;   // the host checks the range; never write outside the pool
+            const int64_t page = inside ? slot / ps : 0, off = inside ? slot % ps : 0;
+#pragma unroll
+            for (int dk = 0; dk < DK; ++dk) {
+                knew[dk] = sk[dk][j];
+                if (inside && r == r_p && dk * 32 + j * 8 < D)
+                    *reinterpret_cast<uint4*>(const_cast<zi_bf16*>(kcache) + ((page * nkv + kvh) * ps + off) * D + dk * 32 + j * 8) = knew[dk];
+            }
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) {
+                const int dim = dd * 16 + r;
+                const uint32_t hv = sv[dim];
+                if (inside && j == j_p)
+                    const_cast<zi_bf16*>(vcache)[((page * nkv + kvh) * D + dim) * ps + off].bits = (uint16_t)hv;
+                vnew[dd / 2] = (dd & 1) ? (vnew[dd / 2] | (hv << 16)) : hv;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int dk = 0; dk < DK; ++dk) {
+            dec_pack w;
+            w.u = make_uint4(0, 0, 0, 0);
+            if (r < G && dk * 32 + j * 8 < D)
+                w.u = *reinterpret_cast<const uint4*>(q + (int64_t)t * ldq + (int64_t)(kvh * G + r) * D + dk * 32 + j * 8);
+            qop[dk] = w.b;
+        }
     }
     dec_f32x4_t o[DT];
 #pragma unroll
@@ -174,6 +334,31 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                 for (int dd = 0; dd < DT; ++dd) {
                     uint4& u = vop[dd][b].u;
                     u.x &= keep[0]; u.y &= keep[1]; u.z &= keep[2]; u.w &= keep[3];
+                }
+            }
+        }
+        if (FUSED && owner && p < base + DEC_BLOCK) {     // the last block (p >= base: k_end = p + 1)
+            if (r == r_p) {
+#pragma unroll
+                for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                    for (int dk = 0; dk < DK; ++dk)
+                        if (tt == tt_p) kop[tt][dk].u = knew[dk];
+            }
+            if (j == j_p) {
+                const uint32_t keep = (e_p & 1) ? 0x0000ffffu : 0xffff0000u;
+#pragma unroll
+                for (int dd = 0; dd < DT; ++dd) {
+                    const uint32_t hv = (vnew[dd / 2] >> (16 * (dd & 1))) & 0xffffu, put = (e_p & 1) ? hv << 16 : hv;
+#pragma unroll
+                    for (int b = 0; b < 2; ++b) {
+                        if (b != b_p) continue;
+                        uint4& u = vop[dd][b].u;
+                        if (e_p / 2 == 0) u.x = (u.x & keep) | put;
+                        if (e_p / 2 == 1) u.y = (u.y & keep) | put;
+                        if (e_p / 2 == 2) u.z = (u.z & keep) | put;
+                        if (e_p / 2 == 3) u.w = (u.w & keep) | put;
+                    }
                 }
             }
         }
@@ -333,37 +518,43 @@ extern "C" int zi_attention_decode_supported(int dt, int nh, int nkv, int d, int
     return d >= 16 && d <= 128 && d % 16 == 0 && G <= 16 && page_size > 0 && page_size % 8 == 0;
 }
 
-extern "C" int zi_attention_decode(void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo,
-                                   const void* kcache, const void* vcache, const int32_t* tok_index,
-                                   const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
-                                   int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
-                                   float scale, int max_chunks, float* workspace, int64_t workspace_floats,
-                                   hipStream_t stream) {
+// Checks and launches shared by the two entry points; `pj` is null for queries that come rotated in q.
+static int dec_launch(const char* who, void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo,
+                      const void* kcache, const void* vcache, const int32_t* tok_index, const int32_t* tok_seq,
+                      const int32_t* tok_pos, const int32_t* block_tables, int max_pages, int num_pages, int nh, int nkv,
+                      int d, int page_size, int window, float scale, int max_chunks, float* workspace,
+                      int64_t workspace_floats, const DecProjection* pj, hipStream_t stream) {
     ZI_REQUIRE(zi_attention_decode_supported(dt, nh, nkv, d, page_size),
-               "attention_decode: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, group <= 16, "
-               "page size %% 8 == 0): dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
-    ZI_REQUIRE(n_idx >= 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_decode: bad sizes");
-    ZI_REQUIRE(max_chunks >= 1 && max_chunks <= DEC_MAXC, "attention_decode: max_chunks %d outside 1..%d", max_chunks,
-               DEC_MAXC);
-    ZI_REQUIRE(ldq >= (int64_t)nh * d && ldo >= (int64_t)nh * d && ldq % 8 == 0 && ldo % 4 == 0,
-               "attention_decode: bad row stride");
-    ZI_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 && ((uintptr_t)kcache % 16) == 0 &&
+               "%s: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, group <= 16, "
+               "page size %% 8 == 0): dtype %d heads %d kv_heads %d head_dim %d page %d", who, dt, nh, nkv, d, page_size);
+    ZI_REQUIRE(n_idx >= 0 && max_pages > 0 && num_pages > 0 && window >= 0, "%s: bad sizes", who);
+    ZI_REQUIRE(max_chunks >= 1 && max_chunks <= DEC_MAXC, "%s: max_chunks %d outside 1..%d", who, max_chunks, DEC_MAXC);
+    ZI_REQUIRE(ldo >= (int64_t)nh * d && ldo % 4 == 0 && (pj || (ldq >= (int64_t)nh * d && ldq % 8 == 0)),
+               "%s: bad row stride", who);
+    ZI_REQUIRE((pj || ((uintptr_t)q % 16) == 0) && ((uintptr_t)out % 8) == 0 && ((uintptr_t)kcache % 16) == 0 &&
                    ((uintptr_t)vcache % 16) == 0,
-               "attention_decode: q, out and the caches must be aligned to 16 bytes");
-    ZI_REQUIRE(nkv <= 65535 && nh <= 65535, "attention_decode: too many heads");
+               "%s: q, out and the caches must be aligned to 16 bytes", who);
+    ZI_REQUIRE(nkv <= 65535 && nh <= 65535, "%s: too many heads", who);
     if (n_idx == 0) return 0;
     ZI_REQUIRE(max_chunks == 1 || (workspace && workspace_floats >= zi_attention_decode_workspace(n_idx, nh, d) &&
                                    ((uintptr_t)workspace % 16) == 0),
-               "attention_decode: workspace of %lld floats is too small or not aligned", (long long)workspace_floats);
+               "%s: workspace of %lld floats is too small or not aligned", who, (long long)workspace_floats);
     float* po = workspace;
     float* pml = workspace ? workspace + (int64_t)n_idx * nh * DEC_MAXC * d : nullptr;
     const dim3 grid(n_idx, nkv, max_chunks);
     const int G = nh / nkv;
+    const DecProjection none = {};
 #define ZI_DEC(DD)                                                                                                   \
-    attention_decode_kernel<DD><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                            \
-        (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,         \
-        tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,       \
-        max_chunks)
+    if (pj)                                                                                                          \
+        attention_decode_kernel<DD, true><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
+            (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
+            tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
+            max_chunks, *pj);                                                                                        \
+    else                                                                                                             \
+        attention_decode_kernel<DD, false><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
+            (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
+            tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
+            max_chunks, none)
     switch (d) {
         case 16: ZI_DEC(16); break;
         case 32: ZI_DEC(32); break;
@@ -378,5 +569,59 @@ extern "C" int zi_attention_decode(void* out, const void* q, int dt, int n_idx, 
     if (max_chunks > 1)
         attention_decode_merge_kernel<<<dim3(n_idx, nh), ZI_WAVE, 0, stream>>>((zi_bf16*)out, ldo, po, pml, tok_index,
                                                                               tok_pos, nh, d, window, max_chunks);
-    return zi_check_launch("attention_decode");
+    return zi_check_launch(who);
+}
+
+extern "C" int zi_attention_decode(void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo,
+                                   const void* kcache, const void* vcache, const int32_t* tok_index,
+                                   const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
+                                   int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
+                                   float scale, int max_chunks, float* workspace, int64_t workspace_floats,
+                                   hipStream_t stream) {
+    return dec_launch("attention_decode", out, q, dt, n_idx, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos,
+                      block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks, workspace,
+                      workspace_floats, nullptr, stream);
+}
+
+// 1 when the fused entry point takes this projection layout, else 0 (then: rotate and store first, and
+// call zi_attention_decode).
+extern "C" int zi_attention_decode_fused_supported(int dt, int nh, int nkv, int d, int page_size, int rot, int splits,
+                                                   int64_t split_stride, int64_t ldp) {
+    if (!zi_attention_decode_supported(dt, nh, nkv, d, page_size)) return 0;
+    if (rot < 0 || rot > d || rot % 16) return 0;      // rot / 2 a multiple of 8: eight dims on one side
+    if (splits < 1 || ldp % 4 || (splits > 1 && split_stride % 4)) return 0;
+    return ldp >= (int64_t)(nh + 2 * nkv) * d;
+}
+
+// The same attention for tokens whose projections arrive as float32 partial sums (see DecProjection):
+// the kernel adds and rotates them itself and writes each token's new key and value to the cache, when
+// `write_kv`.  Every token must be the only one of its sequence in the call: a token's keys must not be
+// written by another token of the same call.  `table` holds cos and sin per (token, pair), from
+// zi_rope_table; `dt` is the type of the caches and of out; `bias` is bfloat16 or float32 (bias_dt).
+extern "C" int zi_attention_decode_fused(void* out, int dt, int n_idx, int64_t ldo, const float* sums, int splits,
+                                         int64_t split_stride, int64_t ldp, const void* bias, int bias_dt,
+                                         const float* table, int rot, const int32_t* slots, int64_t cache_slots,
+                                         int write_kv, void* kcache, void* vcache, const int32_t* tok_index,
+                                         const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
+                                         int max_pages, int num_pages, int nh, int nkv, int d, int page_size,
+                                         int window, float scale, int max_chunks, float* workspace,
+                                         int64_t workspace_floats, hipStream_t stream) {
+    ZI_REQUIRE(zi_attention_decode_fused_supported(dt, nh, nkv, d, page_size, rot, splits, split_stride, ldp),
+               "attention_decode_fused: unsupported projection layout (rotary dims %d a multiple of 16 within head_dim %d, "
+               "row and split strides multiples of 4: %lld, %lld)", rot, d, (long long)ldp, (long long)split_stride);
+    ZI_REQUIRE(sums && ((uintptr_t)sums % 16) == 0, "attention_decode_fused: sums must be aligned to 16 bytes");
+    ZI_REQUIRE(rot == 0 || (table && ((uintptr_t)table % 16) == 0), "attention_decode_fused: no angle table, or not aligned");
+    ZI_REQUIRE(((uintptr_t)bias % 16) == 0, "attention_decode_fused: bias must be aligned to 16 bytes");
+    ZI_REQUIRE(!bias || bias_dt == ZI_BF16 || bias_dt == ZI_F32, "attention_decode_fused: bias must be bfloat16 or float32");
+    if (write_kv)
+        ZI_REQUIRE(slots && cache_slots > 0 && cache_slots % page_size == 0,
+                   "attention_decode_fused: cache of %lld slots is not a whole number of pages of %d",
+                   (long long)cache_slots, page_size);
+    DecProjection pj;
+    pj.sums = sums; pj.splits = splits; pj.split_stride = split_stride; pj.ldp = ldp;
+    pj.bias = bias; pj.bias_f32 = bias_dt == ZI_F32;
+    pj.table = table; pj.rot = rot; pj.slots = slots; pj.cache_slots = cache_slots; pj.write_kv = write_kv;
+    return dec_launch("attention_decode_fused", out, nullptr, dt, n_idx, 0, ldo, kcache, vcache, tok_index, tok_seq,
+                      tok_pos, block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks,
+                      workspace, workspace_floats, &pj, stream);
 }

@@ -231,3 +231,27 @@ extern "C" int zi_rope(void* out, const void* in, int dt, int n, int64_t ld_in, 
     });
     return zi_check_launch("rope");
 }
+
+// cos and sin of every (token, pair) angle: out[t][k] = (cos, sin)(pos[t] * inv_freq[k]), float32.  The
+// angles of a step do not depend on the layer; kernels that take this table skip their own sincosf.
+__global__ void rope_table_kernel(float* __restrict__ out, const int32_t* __restrict__ pos,
+                                  const float* __restrict__ inv_freq, int64_t total, int half) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int64_t t = i / half;
+    const int k = (int)(i % half);
+    float s, c;
+    sincosf((float)pos[t] * inv_freq[k], &s, &c);
+    out[2 * i] = c;
+    out[2 * i + 1] = s;
+}
+
+extern "C" int zi_rope_table(float* out, const int32_t* pos, const float* inv_freq, int n, int half,
+                             hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && half >= 0, "rope_table: bad sizes");
+    ZI_REQUIRE(half == 0 || (out && pos && inv_freq), "rope_table: null pointer");
+    const int64_t total = (int64_t)n * half;
+    if (total == 0) return 0;
+    rope_table_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(out, pos, inv_freq, total, half);
+    return zi_check_launch("rope_table");
+}

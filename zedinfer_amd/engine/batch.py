@@ -72,6 +72,12 @@ class DeviceBatch:
     host_past: Optional[np.ndarray] = None
     host_slot: Optional[np.ndarray] = None
     host_image: Optional[np.ndarray] = None      # all index arrays as they were copied to the device
+    # every entry brings exactly one token (a pure decode step): no token's keys are written by
+    # another token of the step, so a mixer may store and attend in one kernel
+    single_tokens: bool = False
+    # what parts compute once per step and share over the layers (for instance the rotation angles),
+    # by a key of their own
+    shared: dict = field(default_factory=dict)
 
 
 class StagingRing:
@@ -216,7 +222,8 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
                        long_idx=views[9] if 0 < n_long < N else None, num_short=n_short, num_long=n_long,
                        max_short_keys=max_short, max_long_keys=max_long, tile_entry=views[10], tile_off=views[11],
                        num_tiles=len(tiles), host_start=starts,
-                       host_len=lens_a, host_past=past, host_slot=slot, host_image=image)
+                       host_len=lens_a, host_past=past, host_slot=slot, host_image=image,
+                       single_tokens=bool((lens_a == 1).all()))
 
 
 class DecodeImage:

@@ -394,6 +394,91 @@ def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
     return out
 
 
+def rope_table(pos: torch.Tensor, inv_freq: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """cos and sin of pos[t] * inv_freq[k] as float32 [n, rotary_dim/2, 2]: the angles of one step, which
+    every layer with the same frequencies shares."""
+    _gpu("rope_table", pos, inv_freq, out)
+    n, half = pos.numel(), inv_freq.numel()
+    _i32(pos, "rope_table positions", n)
+    if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous():
+        raise ValueError("rope_table: inv_freq must be contiguous float32")
+    if out is None:
+        out = torch.empty((n, half, 2), dtype=torch.float32, device=pos.device)
+    if tuple(out.shape) != (n, half, 2) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError(f"rope_table: out must be a contiguous float32 [{n}, {half}, 2] tensor")
+    _lib.call("zi_rope_table", _p(out), _p(pos), _p(inv_freq), n, half, _stream())
+    return out
+
+
+def attention_decode_fused_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, page_size: int, rotary_dim: int,
+                                     splits: int, width: int, rows: int) -> bool:
+    """Whether ``attention_decode_fused`` takes partial sums [splits, rows, width] with this rotation."""
+    if dtype not in _CODES:
+        return False
+    return bool(_lib.load().zi_attention_decode_fused_supported(_CODES[dtype], nh, nkv, d, page_size, rotary_dim,
+                                                                splits, rows * width, width))
+
+
+def attention_decode_fused(sums: torch.Tensor, bias: Optional[torch.Tensor], table: Optional[torch.Tensor],
+                           slots: Optional[torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
+                           tok_seq: torch.Tensor, tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int,
+                           d: int, scale: float, max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
+                           workspace: Optional[torch.Tensor] = None, write_kv: bool = True) -> torch.Tensor:
+    """Rotation, cache store and attention of single decoded tokens in one kernel.
+
+    ``sums`` [S, n, nh*d + 2*nkv*d] float32 are the partial sums of the fused q/k/v projection of the
+    step's n tokens; splits are added in rising order, then ``bias``.  The first ``2 * table.shape[1]``
+    dims of every query and key head turn by the angles of ``table`` ([n, pairs, 2] from ``rope_table``;
+    None: no rotation).  With ``write_kv`` each token's new key and value go to slot ``slots[t]`` of the
+    cache.  Every token must be the only one of its sequence in the call.  Same shapes as
+    ``attention_decode``; the result is what rope_kv_store_sums followed by attention_decode gives."""
+    _gpu("attention_decode_fused", sums, bias, table, slots, kcache, vcache, tok_seq, tok_pos, block_tables, out,
+         workspace)
+    if sums.dim() != 3 or sums.dtype != torch.float32 or not sums.is_contiguous():
+        raise ValueError("attention_decode_fused: sums must be a contiguous float32 [S, n, width] tensor")
+    S, n, width = sums.shape
+    need_w = (nh + 2 * nkv) * d
+    if width < need_w:
+        raise ValueError(f"attention_decode_fused: rows of {width} values, {need_w} needed")
+    if nkv <= 0 or nh % nkv:
+        raise ValueError(f"attention_decode_fused: {nh} query heads are not a multiple of {nkv} key/value heads")
+    if bias is not None and (bias.dim() != 1 or bias.numel() < need_w or not bias.is_contiguous()):
+        raise ValueError(f"attention_decode_fused: bias must hold {need_w} values")
+    pages, ps = _check_cache(kcache, vcache, nkv, d, kcache.dtype, "attention_decode_fused")
+    _i32(tok_seq, "attention_decode_fused tok_seq", n)
+    _i32(tok_pos, "attention_decode_fused tok_pos", n)
+    if write_kv:
+        _i32(slots, "attention_decode_fused slots", n)
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+        raise ValueError("attention_decode_fused: block_tables must be a contiguous int32 [seqs, max_pages] tensor")
+    rot = 0
+    if table is not None:
+        if table.dim() != 3 or table.shape[0] != n or table.shape[2] != 2 or table.dtype != torch.float32 \
+                or not table.is_contiguous():
+            raise ValueError(f"attention_decode_fused: table must be a contiguous float32 [{n}, pairs, 2] tensor")
+        rot = 2 * table.shape[1]
+    if out is None:
+        out = torch.empty((n, nh * d), dtype=kcache.dtype, device=sums.device)
+    ldo, wo = _rows(out, "attention_decode_fused out")
+    if tuple(out.shape) != (n, nh * d) or out.dtype != kcache.dtype:
+        raise ValueError("attention_decode_fused: out has the wrong shape or dtype")
+    if window > 0:
+        max_keys = min(max_keys, window)
+    max_chunks = int(_lib.load().zi_attention_decode_chunks(int(max_keys)))
+    need = attention_decode_workspace(n, nh, d)
+    if max_chunks > 1:
+        if workspace is None:
+            workspace = torch.empty((need,), dtype=torch.float32, device=sums.device)
+        if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
+            raise ValueError(f"attention_decode_fused: workspace must be a contiguous float32 buffer of {need} entries")
+    _lib.call("zi_attention_decode_fused", _p(out), _code(out, "attention_decode_fused"), n, ldo, _p(sums), S,
+              n * width, width, _p(bias), _code(bias, "attention_decode_fused bias") if bias is not None else F32,
+              _p(table), rot, _p(slots), pages * ps, int(write_kv), _p(kcache), _p(vcache), _p(None), _p(tok_seq),
+              _p(tok_pos), _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale),
+              max_chunks, _p(workspace), workspace.numel() if workspace is not None else 0, _stream())
+    return out
+
+
 PREFILL_TILE = 64     # queries one workgroup of the prompt kernel takes
 
 

@@ -180,7 +180,16 @@ class PositionEncoding(Part):
     [n, nkv*d] at ``slots`` of ``memory``'s cache (nothing is stored when ``memory.writes`` is
     False).  ``rotate_and_store_sums`` does the same from the float32 partial sums [S, n,
     nh*d + 2*nkv*d] of a fused q/k/v projection plus its bias, and writes q to ``q_out``; the
-    default adds the sums up and calls ``rotate_and_store``."""
+    default adds the sums up and calls ``rotate_and_store``.
+
+    ``step_table(batch)`` lets a mixer fold the encoding into a kernel of its own: an encoding that
+    is a rotation of pairs (k, k + R/2) of the first R dims of every head returns the step's angles
+    as a float32 tensor [n, R/2, 2] of (cos, sin), computed once per step and kept in
+    ``batch.shared``; an encoding that does nothing returns the string "none"; every other encoding
+    returns None (the default), and the mixer calls ``rotate_and_store*``."""
+
+    def step_table(self, batch):
+        return None
 
     def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
         raise NotImplementedError

@@ -27,6 +27,10 @@ class Attention(Mixer):
     scale (default 1/sqrt(head_dim)), position (a PartSpec of a position encoding)."""
 
     graph_safe = True
+    # Every workgroup of the fused kernel adds and rotates its token's query again (one per chunk of
+    # 256 keys), which costs more than the separate rotary kernel once many tokens decode together:
+    # measured faster at 1 and 8 tokens, slower at 64.
+    FUSED_DECODE_MAX_TOKENS = 16
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -103,6 +107,9 @@ class Attention(Mixer):
             S = ops.linear_splits(n, self.qkv.shape[0], self.hidden)
             sums = self.rt.buffer("attn_qkv_sums", (S, n, self.qd + 2 * self.kvd), torch.float32)
             ops.linear_sums(x, self.qkv, out=sums)
+            att = self.rt.buffer("attn_out", (n, self.qd))
+            if self.attend_from_sums(sums, att, batch, view, memory):
+                return self.project(att, n)
             q = self.rt.buffer("attn_q", (n, self.qd))
             self.position.rotate_and_store_sums(sums, self.bias, q, batch.positions, view.slots, memory, self.nh,
                                                 self.nkv, self.d)
@@ -117,8 +124,32 @@ class Attention(Mixer):
             self.position.rotate_and_store(q, k, v, batch.positions, view.slots, memory, self.nh, self.nkv, self.d)
         att = self.rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
+        return self.project(att, n)
+
+    def project(self, att: torch.Tensor, n: int) -> torch.Tensor:
         if ops.linear_sums_supported(att, self.o):
             S = ops.linear_splits(n, self.hidden, self.qd)
             return ops.linear_sums(att, self.o, out=self.rt.buffer("attn_proj_sums", (S, n, self.hidden), torch.float32))
         out = self.rt.buffer("attn_proj", (n, self.hidden))
         return ops.linear(att, self.o, out=out)
+
+    def attend_from_sums(self, sums, att, batch, view, memory: LayerMemory) -> bool:
+        """A pure decode step (one token a sequence): rotation, cache store and attention in one kernel,
+        when the position encoding is a rotation it can hand over as a table of angles (or nothing) and
+        the kernel takes the shape.  False: nothing was done."""
+        if not batch.single_tokens or batch.num_tokens > self.FUSED_DECODE_MAX_TOKENS:
+            return False
+        table = self.position.step_table(batch)
+        if table is None:
+            return False
+        rot = 0 if isinstance(table, str) else 2 * table.shape[1]
+        S, n, width = sums.shape
+        ps = memory.k.shape[2]
+        if not ops.attention_decode_fused_supported(memory.k.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
+            return False
+        ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
+        ops.attention_decode_fused(sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None,
+                                   memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh,
+                                   self.nkv, self.d, self.scale, batch.max_short_keys, self.window, out=att,
+                                   workspace=ws, write_kv=memory.writes)
+        return True

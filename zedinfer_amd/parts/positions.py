@@ -27,6 +27,15 @@ class RopeNeox(PositionEncoding):
             raise ValueError(f"rope_neox: rotary_dim {self.rotary_dim} must be even and within head_dim {self.head_dim}")
         self.inv_freq = ops.rope_inv_freq(self.rotary_dim, self.theta, rt.device)
 
+    def step_table(self, batch):
+        key = ("rope_neox", self.rotary_dim, self.theta)
+        table = batch.shared.get(key)
+        if table is None:
+            out = self.rt.buffer(f"rope_table_{self.rotary_dim}_{self.theta!r}",
+                                 (batch.num_tokens, self.rotary_dim // 2, 2), torch.float32)
+            table = batch.shared[key] = ops.rope_table(batch.positions, self.inv_freq, out=out)
+        return table
+
     def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
         if memory.writes:
             ops.rope_kv_store(q, k, v, positions, slots, self.inv_freq, memory.k, memory.v, nh, nkv, d)
@@ -44,6 +53,9 @@ class RopeNeox(PositionEncoding):
 @register_position_encoding("none")
 class NoPosition(PositionEncoding):
     """No encoding: keys and values are stored as they are."""
+
+    def step_table(self, batch):
+        return "none"
 
     def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
         if memory.writes:
