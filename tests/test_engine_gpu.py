@@ -1,6 +1,8 @@
 """The engine against the plain implementation: each request alone and whole; most of it in one
 step and the last 32 tokens one by one; portions of changing size; and mixed batches with so few
-pages that they are used again.  In float32 and in bfloat16, on three tiny configurations."""
+pages that they are used again.  In float32 and in bfloat16, on three tiny configurations; bfloat16
+both with the float32 checkpoint (weights stored in 32 bits stay so) and with a bfloat16 checkpoint
+("bfloat16w"), which is what the serving kernels for bfloat16 weights take."""
 import os
 
 import pytest
@@ -27,19 +29,31 @@ def tiny(request, tmp_path_factory):
     cfg, w = plain.load_folder(folder)
     reqs = {f"r{i}": traces.random_tokens(cfg["vocab_size"], n, seed=100 + i) for i, n in enumerate(LENGTHS[name])}
     ref = {rid: plain.forward(cfg, w, toks) for rid, toks in reqs.items()}
-    return dict(name=name, folder=folder, cfg=cfg, weights=w, requests=reqs, reference=ref)
+    folder16 = tiny_configs.write_tiny(str(tmp_path_factory.mktemp(f"tiny{name}bf16")), name, dtype=torch.bfloat16)
+    _, w16 = plain.load_folder(folder16)
+    ref16 = {rid: plain.forward(cfg, w16, toks) for rid, toks in reqs.items()}
+    return dict(name=name, folder=folder, cfg=cfg, weights=w, requests=reqs, reference=ref,
+                folder16=folder16, reference16=ref16)
+
+
+def variant(tiny, dtype):
+    """(model folder, engine dtype, reference logits) of a dtype parameter."""
+    if dtype == "bfloat16w":
+        return tiny["folder16"], "bfloat16", tiny["reference16"]
+    return tiny["folder"], dtype, tiny["reference"]
 
 
 def make_engine(tiny, dtype, pages):
     from zedinfer_amd.config import SchedulerConfig
     from zedinfer_amd.engine import Engine
     ps = tiny_configs.PAGE_SIZES[tiny["name"]]
-    return Engine.from_folder(tiny["folder"], dtype,
+    folder, engine_dtype, _ = variant(tiny, dtype)
+    return Engine.from_folder(folder, engine_dtype,
                               SchedulerConfig(num_kv_blocks=pages, kv_block_size=ps, max_batch_requests=4))
 
 
 def check(tiny, dtype, steps, outputs):
-    worst, mean, scale, rows, where = traces.compare(steps, outputs, tiny["reference"], tiny["requests"])
+    worst, mean, scale, rows, where = traces.compare(steps, outputs, variant(tiny, dtype)[2], tiny["requests"])
     print(f"[{tiny['name']} {dtype}] rows={rows} worst={worst:.3e} mean={mean:.3e} scale={scale:.3e} at {where}")
     assert rows > 0
     if dtype == "float32":
@@ -49,7 +63,7 @@ def check(tiny, dtype, steps, outputs):
         assert mean <= BF16_REL_MEAN * scale
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w"])
 @pytest.mark.parametrize("shape", ["whole", "last32", "portions", "mixed"])
 def test_engine_matches_plain(tiny, dtype, shape):
     steps = {"whole": traces.whole, "last32": traces.last_decoded, "portions": traces.portions,
@@ -64,9 +78,10 @@ def test_engine_matches_plain(tiny, dtype, shape):
     check(tiny, dtype, steps, out)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w"])
 def test_replay_tool(tiny, dtype, tmp_path):
     """The same mixed trace through bin/trace_run as a child process."""
     steps = traces.mixed(tiny["requests"], seed=3)
-    out = traces.run_tool(tiny["folder"], dtype, steps, str(tmp_path / "out"), traces.max_live_tokens(steps))
+    folder, engine_dtype, _ = variant(tiny, dtype)
+    out = traces.run_tool(folder, engine_dtype, steps, str(tmp_path / "out"), traces.max_live_tokens(steps))
     check(tiny, dtype, steps, out)

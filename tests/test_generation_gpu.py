@@ -239,6 +239,53 @@ def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype):
     assert float((last[0].cpu() - ref[fed["d"] - 1]).abs().max()) < tol
 
 
+def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatch, tmp_path):
+    """Pure decode steps of few tokens rotate, store and attend in one kernel.  With that path switched
+    off the same steps give the same logits (the caches hold the same keys and values, so later steps
+    agree too), across page edges and with sequences of different lengths."""
+    from zedinfer_amd.engine import StepEntry
+    from zedinfer_amd.parts.mixers import Attention
+    V = tiny["cfg"]["vocab_size"]
+    # a bfloat16 checkpoint: weights stored in 32 bits would stay so and take the plain kernels
+    folder16 = tiny_configs.write_tiny(str(tmp_path / "bf16"), tiny["name"], dtype=torch.bfloat16)
+    tiny16 = dict(tiny, folder=folder16, weights=plain.load_folder(folder16)[1])
+    one, two = engine(tiny16, "bfloat16").engine, engine(tiny16, "bfloat16").engine
+    for eng in (one, two):
+        eng.use_graphs = False
+    toks = {r: traces.random_tokens(V, 120, seed=70 + i) for i, r in enumerate("abc")}
+    fed = {r: 0 for r in toks}
+    seqs = {(e, r): e.open(r) for e in (one, two) for r in toks}
+    calls = {"fused": 0}
+    from zedinfer_amd import ops
+    real = ops.attention_decode_fused
+
+    def counted(*a, **k):
+        calls["fused"] += 1
+        return real(*a, **k)
+    monkeypatch.setattr(ops, "attention_decode_fused", counted)
+
+    def both(plan):
+        outs = []
+        for eng in (one, two):
+            monkeypatch.setattr(Attention, "FUSED_DECODE_MAX_TOKENS", 16 if eng is one else 0)
+            outs.append(eng.step([StepEntry(seqs[(eng, r)], toks[r][fed[r]:fed[r] + n], [n - 1]) for r, n in plan]))
+        for r, n in plan:
+            fed[r] += n
+        scale = float(outs[1].abs().max())
+        assert float((outs[0] - outs[1]).abs().max()) <= 0.02 * scale, plan
+        return outs
+
+    both([("a", 37), ("b", 5), ("c", 1)])
+    before = calls["fused"]
+    for _ in range(40):
+        both([("a", 1), ("b", 1), ("c", 1)])
+    layers = tiny["cfg"]["num_hidden_layers"]
+    assert calls["fused"] - before == 40 * layers       # only the first engine, every layer
+    last = both([("b", 1)])[0]
+    ref = plain.forward(tiny["cfg"], tiny16["weights"], toks["b"][:fed["b"]])
+    assert float((last[0].cpu() - ref[fed["b"] - 1]).abs().max()) < 0.06 * float(ref.abs().max())
+
+
 def test_decode_graphs_with_the_library_product(tiny):
     """More than 16 decoding requests: the matrix products go to the library, inside the captured
     graph.  Every replay is checked against eager launches, with eager prompt steps between them."""
