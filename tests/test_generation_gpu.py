@@ -189,13 +189,18 @@ def test_command_lines(tiny, tmp_path):
     assert r.returncode == 0 and "Throughput" in r.stdout and "18 tokens generated" in r.stdout, r.stderr + r.stdout
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w"])
+def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype, tmp_path):
     """Steps of single decoded tokens are captured as graphs and replayed.  Every replay is checked
     against an engine that launches eagerly, with eager prompt portions, closes and new requests
-    (reused pages, other batch sizes) between the replays."""
+    (reused pages, other batch sizes) between the replays.  "bfloat16w": a bfloat16 checkpoint, whose
+    decode steps take the few-rows products and the one-kernel attention with its per-step table."""
     from zedinfer_amd.engine import StepEntry
     V = tiny["cfg"]["vocab_size"]
+    if dtype == "bfloat16w":
+        folder16 = tiny_configs.write_tiny(str(tmp_path / "bf16"), tiny["name"], dtype=torch.bfloat16)
+        tiny = dict(tiny, folder=folder16, weights=plain.load_folder(folder16)[1])
+        dtype = "bfloat16"
     fast, slow = engine(tiny, dtype).engine, engine(tiny, dtype).engine
     assert fast.use_graphs
     slow.use_graphs = False

@@ -108,6 +108,9 @@ class DecoderModel:
     def run(self, batch, memories: Sequence[LayerMemory]) -> Optional[torch.Tensor]:
         """Run the tokens of ``batch`` through the schedule; float32 logits [wanted, vocab]
         at ``batch.logit_rows``, or None when no row is wanted."""
+        shared = getattr(batch, "shared", None)
+        if shared is not None:
+            shared.clear()      # what parts share holds for one run: a batch object may serve several steps
         resid = self.embedding.forward(batch.token_ids)
         delta = None
         for st, mem in zip(self.fc.schedule, memories):
