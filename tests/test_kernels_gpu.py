@@ -400,6 +400,30 @@ def test_attention_decode_fused_refuses_other_layouts(ops):
     assert not ops.attention_decode_fused_supported(torch.float32, 12, 2, 128, 16, 128, 2, 2048, 8)
 
 
+@pytest.mark.parametrize("far", [37, 255, 256, 511, 690])
+def test_attention_decode_far_key_stands_out(ops, far):
+    """One key among hundreds is made to dominate one head (at a chunk's edges too): its value must come
+    through the split-keys kernel and the merge of its chunks; a window that ends just after it hides
+    it, one key wider shows it again."""
+    nh, nkv, d, ps, T = 8, 2, 64, 16, 700
+    dtype = torch.bfloat16
+    k, v = rnd(T, nkv, d, dtype=dtype, seed=1) * 0.1, rnd(T, nkv, d, dtype=dtype, seed=2)
+    q = rnd(1, nh, d, dtype=dtype, seed=3)
+    head, g = 5, 5 // (nh // nkv)
+    k[far, g] = (q[0, head].float() * 60.0 / q[0, head].float().norm() ** 2 * math.sqrt(d)).to(dtype)
+    kc, vc, table = make_paged(k, v, ps, 64)
+    pos = torch.tensor([T - 1], dtype=torch.int32, device="cuda")
+    seq = torch.zeros(1, dtype=torch.int32, device="cuda")
+    bt = table[None].contiguous()
+    scale = 1 / math.sqrt(d)
+    out = ops.attention_decode(q.view(1, nh * d), kc, vc, seq, pos, bt, nh, nkv, d, scale, T)
+    torch.testing.assert_close(out.view(nh, d)[head].float(), v[far, g].float(), atol=2e-2, rtol=2e-2)
+    hidden = ops.attention_decode(q.view(1, nh * d), kc, vc, seq, pos, bt, nh, nkv, d, scale, T, T - 1 - far)
+    assert float((hidden.view(nh, d)[head].float() - v[far, g].float()).abs().max()) > 0.1
+    shown = ops.attention_decode(q.view(1, nh * d), kc, vc, seq, pos, bt, nh, nkv, d, scale, T, T - far)
+    torch.testing.assert_close(shown.view(nh, d)[head].float(), v[far, g].float(), atol=2e-2, rtol=2e-2)
+
+
 def test_attention_decode_ignores_stale_slots(ops):
     """Slots of a page beyond the token's position may hold anything, NaN included."""
     nh, nkv, d, ps, T = 4, 2, 128, 16, 37
