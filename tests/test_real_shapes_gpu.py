@@ -1,6 +1,9 @@
-"""Two layers of the Qwen2.5-1.5B and 7B layer shapes (real widths, head counts and groups; a smaller
+"""Two layers of the Qwen2.5-1.5B, 7B and 32B layer shapes (real widths, head counts and groups; a smaller
 vocabulary and two layers so that the plain implementation stays affordable on the CPU) against the plain
-implementation: a prompt in portions, then decoded tokens, alone and beside a second request."""
+implementation: a prompt in portions, then decoded tokens, alone and beside a second request.  In float32,
+in bfloat16 with the float32 checkpoint (weights stored in 32 bits stay so) and in bfloat16 with a bfloat16
+checkpoint ("bfloat16w"): the serving kernels (few-rows products and their cuts along k, partial sums, the
+one-kernel decode attention, prompt attention, the library product) at the shapes they serve."""
 import pytest
 import torch
 
@@ -14,6 +17,8 @@ SHAPES = {
                  head_dim=128, tie_word_embeddings=True),
     "7B": dict(hidden_size=3584, intermediate_size=18944, num_attention_heads=28, num_key_value_heads=4,
                head_dim=128, tie_word_embeddings=False),
+    "32B": dict(hidden_size=5120, intermediate_size=27648, num_attention_heads=40, num_key_value_heads=8,
+                head_dim=128, tie_word_embeddings=False),
 }
 
 
@@ -33,15 +38,24 @@ def model(request, tmp_path_factory):
     pcfg, w = plain.load_folder(folder)
     reqs = {"p": traces.random_tokens(4099, 330, seed=1), "q": traces.random_tokens(4099, 97, seed=2)}
     ref = {rid: plain.forward(pcfg, w, toks) for rid, toks in reqs.items()}
-    return dict(folder=folder, requests=reqs, reference=ref)
+    del w
+    folder16 = str(tmp_path_factory.mktemp("real16" + request.param))
+    write_model_folder(folder16, cfg, expected_weights(qwen2_forward_config(cfg)), seed=7, dtype=torch.bfloat16,
+                       noisy_norms=True)
+    _, w16 = plain.load_folder(folder16)
+    ref16 = {rid: plain.forward(pcfg, w16, toks) for rid, toks in reqs.items()}
+    return dict(folder=folder, requests=reqs, reference=ref, folder16=folder16, reference16=ref16)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w"])
 def test_real_layer_shapes_match_plain(model, dtype):
     from zedinfer_amd.config import SchedulerConfig
     from zedinfer_amd.engine import Engine
-    engine = Engine.from_folder(model["folder"], dtype, SchedulerConfig(num_kv_blocks=40, kv_block_size=16,
-                                                                        max_batch_requests=4))
+    folder, reference = model["folder"], model["reference"]
+    if dtype == "bfloat16w":
+        folder, reference, dtype = model["folder16"], model["reference16"], "bfloat16"
+    engine = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=40, kv_block_size=16,
+                                                               max_batch_requests=4))
     reqs = model["requests"]
     p, q = reqs["p"], reqs["q"]
     want = lambda n: list(range(n))   # noqa: E731
@@ -63,7 +77,7 @@ def test_real_layer_shapes_match_plain(model, dtype):
                       "end": ["p"] if fp == len(p) - 1 else []})
         fp += 1
     out = traces.run_in_process(engine, steps)
-    worst, mean, scale, rows, where = traces.compare(steps, out, model["reference"], reqs)
+    worst, mean, scale, rows, where = traces.compare(steps, out, reference, reqs)
     print(f"[{dtype}] rows={rows} worst={worst:.3e} mean={mean:.3e} scale={scale:.3e} at {where}")
     assert rows == len(p) + len(q)
     if dtype == "float32":
