@@ -32,7 +32,7 @@ def engine(tiny, dtype="float32", **kw):
 
 
 def test_greedy_generation_matches_plain(tiny):
-    """BASELINE's tiny workloads: prompts 5/17/33 (A) and 1/31/64/100 (B), 16 greedy tokens each."""
+    """The tiny workloads: prompts of 5/17/33 tokens (A) and 1/31/64/100 (B), 16 greedy tokens each."""
     from zedinfer_amd import GenerationConfig
     lens = [5, 17, 33] if tiny["name"] == "A" else [1, 31, 64, 100]
     V = tiny["cfg"]["vocab_size"]

@@ -56,7 +56,9 @@ def _p(t: Optional[torch.Tensor]) -> c_void_p:
 
 
 def _stream() -> c_void_p:
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the raw handle of torch's current stream on the current device; torch.cuda.current_stream() builds
+    # a Python object and resolves the device each time, which costs more than a whole launch
+    return c_void_p(torch._C._cuda_getCurrentRawStream(torch._C._cuda_getDevice()))
 
 
 def _i32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
