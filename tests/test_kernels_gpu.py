@@ -480,6 +480,10 @@ def prefill_tiles(entries, tile=64):
     (28, 4, 128, 64, 64, [(0, 130), (130, 200)]),
     (2, 1, 112, 128, 0, [(17, 129)]),
     (14, 2, 64, 16, 150, [(0, 1000)]),
+    (4, 2, 128, 16, 0, [(0, 2100), (2100, 130)]),        # tiles that see more than 2,048 keys are cut and merged
+    (2, 1, 64, 16, 0, [(4000, 200), (2047, 3), (2040, 70)]),   # cuts at absolute multiples of 2,048, inside a tile too
+    (3, 1, 32, 8, 300, [(1900, 400)]),                   # a window across a cut
+    (2, 2, 128, 32, 2500, [(3000, 1500)]),               # a window wider than a cut
 ])
 def test_attention_prefill(ops, nh, nkv, d, ps, window, portions):
     """The matrix-core prompt kernel against the float32 reference: portions at several pasts, two
@@ -520,6 +524,25 @@ def test_attention_prefill(ops, nh, nkv, d, ps, window, portions):
                               dev([e[2] for e in entries]), bt, nh, nkv, d, scale, window, out=out2)
         n0 = entries[0][1]
         assert bool((out2[:n0] == 7.0).all()) and torch.equal(out2[n0:], out[n0:])
+
+
+def test_attention_prefill_bound_too_low_shows(ops):
+    """The host sizes the launch from an upper bound of the keys a query sees; a bound that is too low
+    must not write outside the workspace, and leaves NaN where it did not suffice."""
+    nh, nkv, d, ps, T = 2, 1, 64, 16, 2300
+    dtype = torch.bfloat16
+    k, v = rnd(T, nkv, d, dtype=dtype, seed=1), rnd(T, nkv, d, dtype=dtype, seed=2)
+    kc, vc, table = make_paged(k, v, ps, T // ps + 2)
+    q = rnd(T, nh, d, dtype=dtype, seed=3)
+    te, to = prefill_tiles([(0, T, 0)])
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    args = (q.view(T, nh * d), kc, vc, te, to, dev([0]), dev([T]), dev([0]), table[None].contiguous(), nh, nkv, d, 0.125)
+    good = ops.attention_prefill(*args, max_keys=T)
+    assert not torch.isnan(good).any()
+    low = ops.attention_prefill(*args, max_keys=2048)
+    assert not torch.isnan(low[:2048]).any() and torch.equal(low[:2048], good[:2048])
+    assert bool(torch.isnan(low[2048:]).all())
+    assert ops.attention_prefill_workspace(T, nh, d, 2048) == 0 and ops.attention_prefill_workspace(T, nh, d, 2049) > 0
 
 
 def test_attention_prefill_far_key_stands_out(ops):

@@ -13,6 +13,11 @@
 // the dot product (reference formulas:
 // src/backend/ops/self_attention/cpu/paged_attention_cpu.cpp:106-162).
 //
+// A tile that sees more than 2,048 keys is cut along the keys, at absolute multiples of 2,048, over several
+// workgroups (gridDim.y), so that a portion of a long prompt, which has few tiles but a long walk each,
+// still fills the chip; those workgroups leave (maximum, sum, unnormalised output) per query and a second
+// kernel merges them in rising order of the keys.  The cut depends on the query's position alone.
+//
 // Operand layout.  Scores are computed transposed: the A operand is a 16-key tile of
 // K, the B operand the 16 queries, so a lane ends up with the scores of ONE query
 // (lane % 16) and four keys per tile.  Keys are placed in LDS rows in a permuted
@@ -37,6 +42,8 @@ typedef __attribute__((ext_vector_type(4))) float pf_f32x4_t;
 #define PF_BM 64                 // queries per workgroup
 #define PF_BN 64                 // keys per wavefront and block
 #define PF_BS (PF_BN * PF_KH)    // keys per block
+#define PF_CHUNK 2048            // keys one workgroup walks at most: a tile with more is cut over several
+#define PF_MAXC 64               // most such cuts of one tile
 
 union pf_pack {
     uint4 u;
@@ -58,7 +65,8 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                          const int32_t* __restrict__ tile_entry, const int32_t* __restrict__ tile_off,
                          const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                          const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
-                         int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale) {
+                         int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale,
+                         float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DP = DK * 32;         // head_dim padded to a multiple of 32
@@ -81,7 +89,12 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     const int pos0 = past + off;            // position of the tile's first query
     const int kmax = pos0 + count - 1;      // last key any query of the tile sees
     const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-    const int kb_begin = (lo_tile / PF_BS) * PF_BS;
+    const int kb_first = (lo_tile / PF_BS) * PF_BS;
+    // this workgroup's cut of the tile's keys: [kb_begin, khi], inside chunk c of absolute multiples of PF_CHUNK
+    const int c0 = kb_first / PF_CHUNK, nc = kmax / PF_CHUNK - c0 + 1, c = c0 + blockIdx.y;
+    if (c * PF_CHUNK > kmax) return;
+    const int kb_begin = (c * PF_CHUNK > kb_first) ? c * PF_CHUNK : kb_first;
+    const int khi = ((c + 1) * PF_CHUNK - 1 < kmax) ? (c + 1) * PF_CHUNK - 1 : kmax;
 
     // this wavefront's queries (sub-tile qs) and its share of every block's keys (kh)
     const int qs = wave % 4, kh = wave / 4;
@@ -303,7 +316,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     // the other LDS buffer, which everyone has finished reading at the barrier before.  The last block
     // stands outside the loop, so that no branch surrounds the loop's loads.
     int cur = 0, kb0 = kb_begin;
-    for (; kb0 + PF_BS <= kmax; kb0 += PF_BS, cur ^= 1) {
+    for (; kb0 + PF_BS <= khi; kb0 += PF_BS, cur ^= 1) {
         fetch(kb0 + PF_BS);
         work(kb0, cur);
         stash(kb0 + PF_BS, cur ^ 1);
@@ -347,6 +360,25 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         }
     }
     if (!qvalid) return;
+    if (nc > 1) {
+        // one of several cuts of this tile's keys: leave (maximum, sum, unnormalised output) for the merge.
+        // A launch sized for fewer cuts than the tile has must not write outside the workspace: the
+        // query's output is made NaN instead, so that it shows.
+        if (nc > max_chunks) {
+            if (blockIdx.y == 0)
+                for (int dd = 0; dd < DT; ++dd)
+                    for (int x = 0; x < 4; ++x) zi_store(out + (int64_t)(start + off + row) * ldo + (int64_t)h * D + dd * 16 + j * 4 + x, NAN);
+            return;
+        }
+        const int64_t slot = ((int64_t)(start + off + row) * nh + h) * max_chunks + blockIdx.y;
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = o[dd];
+        if (j == 0) {
+            part_ml[slot * 2] = m;
+            part_ml[slot * 2 + 1] = l;
+        }
+        return;
+    }
     const float inv = 1.f / l;
     zi_bf16* orow = out + (int64_t)(start + off + row) * ldo + (int64_t)h * D;
 #pragma unroll
@@ -356,6 +388,56 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         w.y = zi_pack_bf16x2(o[dd][2] * inv, o[dd][3] * inv);
         *reinterpret_cast<uint2*>(orow + dd * 16 + j * 4) = w;
     }
+}
+
+// Merge the cuts of one (query, head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c, in rising order
+// of the keys.  One wavefront per (query row of a tile, head); tiles with one cut were written directly.
+__global__ void __launch_bounds__(ZI_WAVE)
+attention_prefill_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const float* __restrict__ part_o,
+                               const float* __restrict__ part_ml, const int32_t* __restrict__ tile_entry,
+                               const int32_t* __restrict__ tile_off, const int32_t* __restrict__ entry_start,
+                               const int32_t* __restrict__ entry_len, const int32_t* __restrict__ entry_past, int nh,
+                               int D, int window, int max_chunks) {
+    const int tile = blockIdx.x / PF_BM, qi = blockIdx.x % PF_BM, h = blockIdx.y, lane = threadIdx.x;
+    const int e = tile_entry[tile], off = tile_off[tile];
+    const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
+    const int count = (len - off < PF_BM) ? len - off : PF_BM;
+    if (qi >= count) return;
+    const int pos0 = past + off, kmax = pos0 + count - 1;
+    const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int c0 = ((lo_tile / PF_BS) * PF_BS) / PF_CHUNK, nc = kmax / PF_CHUNK - c0 + 1;
+    if (nc == 1 || nc > max_chunks) return;
+    const int64_t row = start + off + qi;
+    const int64_t slot0 = (row * nh + h) * max_chunks;
+    // cut c's (m, l) sit in lane c; a cut none of whose keys this query sees left m = -inf, l = 0
+    const float mc = lane < nc ? part_ml[(slot0 + lane) * 2] : -INFINITY;
+    const float lc = lane < nc ? part_ml[(slot0 + lane) * 2 + 1] : 0.f;
+    const float M = zi_wave_max(mc);
+    const float wc = (mc == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(mc - M);
+    float L = 0.f, acc[2] = {0.f, 0.f};
+    for (int c = 0; c < nc; ++c) {
+        const float w = __shfl(wc, c, ZI_WAVE);
+        L += w * __shfl(lc, c, ZI_WAVE);
+#pragma unroll
+        for (int v = 0; v < 2; ++v)
+            if (lane + v * ZI_WAVE < D) acc[v] += w * part_o[(slot0 + c) * D + lane + v * ZI_WAVE];
+    }
+    const float inv = 1.f / L;
+#pragma unroll
+    for (int v = 0; v < 2; ++v)
+        if (lane + v * ZI_WAVE < D) zi_store(out + row * ldo + (int64_t)h * D + lane + v * ZI_WAVE, acc[v] * inv);
+}
+
+// Floats of workspace a launch over `rows` query rows needs when tiles are cut into up to `max_chunks`.
+extern "C" int64_t zi_attention_prefill_workspace(int rows, int nh, int d, int max_chunks) {
+    return max_chunks > 1 ? (int64_t)rows * nh * max_chunks * (d + 2) : 0;
+}
+
+// Cuts the launch must cover when no query sees more than `keys` keys (position + 1; with a window: the
+// window plus one tile and one block, at most).
+extern "C" int zi_attention_prefill_chunks(int keys) {
+    if (keys < 1) keys = 1;
+    return (keys + PF_CHUNK - 1) / PF_CHUNK;
 }
 
 // 1 when the shape is this kernel's, else 0.
@@ -375,27 +457,35 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
                                     const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
                                     const int32_t* entry_past, const int32_t* block_tables, int max_pages,
                                     int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
+                                    int rows, int max_chunks, float* workspace, int64_t workspace_floats,
                                     hipStream_t stream) {
     ZI_REQUIRE(zi_attention_prefill_supported(dt, nh, nkv, d, page_size),
                "attention_prefill: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, page size a power "
                "of two from 8): dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
-    ZI_REQUIRE(num_tiles >= 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_prefill: bad sizes");
+    ZI_REQUIRE(num_tiles >= 0 && max_pages > 0 && num_pages > 0 && window >= 0 && rows >= 0, "attention_prefill: bad sizes");
     ZI_REQUIRE(ldq >= (int64_t)nh * d && ldo >= (int64_t)nh * d && ldq % 8 == 0 && ldo % 4 == 0,
                "attention_prefill: bad row stride");
     ZI_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 8) == 0 && ((uintptr_t)kcache % 16) == 0 &&
                    ((uintptr_t)vcache % 16) == 0,
                "attention_prefill: q, out and the caches must be aligned to 16 bytes");
     ZI_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
+    ZI_REQUIRE(max_chunks >= 1 && max_chunks <= PF_MAXC, "attention_prefill: max_chunks %d outside 1..%d (contexts up to %d keys)",
+               max_chunks, PF_MAXC, PF_MAXC * PF_CHUNK);
+    ZI_REQUIRE(max_chunks == 1 || (workspace && ((uintptr_t)workspace % 16) == 0 &&
+                                   workspace_floats >= zi_attention_prefill_workspace(rows, nh, d, max_chunks)),
+               "attention_prefill: workspace of %lld floats is too small or not aligned", (long long)workspace_floats);
     if (num_tiles == 0) return 0;
-    ZI_REQUIRE((int64_t)num_tiles * nh < (1ll << 31), "attention_prefill: too many tiles");
-    const dim3 grid(num_tiles * nh);
+    ZI_REQUIRE((int64_t)num_tiles * nh < (1ll << 31) && (int64_t)num_tiles * PF_BM < (1ll << 31), "attention_prefill: too many tiles");
+    const dim3 grid(num_tiles * nh, max_chunks);
     int ps_shift = 0;
     while ((1 << ps_shift) < page_size) ++ps_shift;
+    float* po = workspace;
+    float* pml = workspace ? workspace + (int64_t)rows * nh * max_chunks * d : nullptr;
 #define ZI_PF(DD)                                                                                              \
     attention_prefill_kernel<DD><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                                     \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
-        window, scale)
+        window, scale, po, pml, max_chunks)
     switch (d) {
         case 16: ZI_PF(16); break;
         case 32: ZI_PF(32); break;
@@ -407,5 +497,8 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
         default: ZI_PF(128); break;
     }
 #undef ZI_PF
+    if (max_chunks > 1)
+        attention_prefill_merge_kernel<<<dim3(num_tiles * PF_BM, nh), ZI_WAVE, 0, stream>>>(
+            (zi_bf16*)out, ldo, po, pml, tile_entry, tile_off, entry_start, entry_len, entry_past, nh, d, window, max_chunks);
     return zi_check_launch("attention_prefill");
 }

@@ -33,7 +33,8 @@ _PROTOTYPES = {
     "zi_attention_decode_fused_supported": [I, I, I, I, I, I, I, L, L],
     "zi_rope_table": [P, P, P, I, I, P],
     "zi_attention_decode_chunks": [I],
-    "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
+    "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, P],
+    "zi_attention_prefill_chunks": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],
     "zi_attention_prefill_tile": [],
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
@@ -81,6 +82,8 @@ def load() -> ctypes.CDLL:
             fn.restype = c_int
         lib.zi_gemm_skinny_workspace.argtypes = [I, I, I]
         lib.zi_gemm_skinny_workspace.restype = c_int64
+        lib.zi_attention_prefill_workspace.argtypes = [I, I, I, I]
+        lib.zi_attention_prefill_workspace.restype = c_int64
         lib.zi_argmax_workspace.argtypes = [I, I]
         lib.zi_argmax_workspace.restype = c_int64
         _lib, _lib_path = lib, path

@@ -490,17 +490,35 @@ def attention_prefill_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, p
     return bool(_lib.load().zi_attention_prefill_supported(_CODES[dtype], nh, nkv, d, page_size))
 
 
+def attention_prefill_workspace(rows: int, nh: int, d: int, max_keys: int, window: int = 0) -> int:
+    """float32 entries of workspace ``attention_prefill`` needs for ``rows`` query rows of which none sees
+    more than ``max_keys`` keys (0: none)."""
+    lib = _lib.load()
+    return int(lib.zi_attention_prefill_workspace(int(rows), nh, d, _prefill_chunks(max_keys, window)))
+
+
+def _prefill_chunks(max_keys: int, window: int) -> int:
+    if window > 0:      # a windowed tile's keys span at most the window, a tile and a block
+        max_keys = min(max_keys, window + PREFILL_TILE + 128) + 2047
+    return int(_lib.load().zi_attention_prefill_chunks(int(max_keys)))
+
+
 def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tile_entry: torch.Tensor,
                       tile_off: torch.Tensor, entry_start: torch.Tensor, entry_len: torch.Tensor,
                       entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
-                      window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      window: int = 0, out: Optional[torch.Tensor] = None, max_keys: int = 0,
+                      workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
     of 16 up to 128, page size a power of two from 8).
 
     Entry e brings ``entry_len[e]`` tokens, rows ``entry_start[e]...`` of q, that continue a sequence
     holding ``entry_past[e]`` tokens whose block table is row e of ``block_tables``.  Tile i covers the
     queries [tile_off[i], tile_off[i] + PREFILL_TILE) of entry ``tile_entry[i]``; rows of ``out`` that no
-    tile covers are left alone."""
+    tile covers are left alone.  ``max_keys`` is an upper bound, known on the host, of the keys any query
+    sees (its position + 1; 0: what the block tables could hold): tiles that see more than 2,048 keys are
+    cut over several workgroups and merged, which needs ``workspace`` (``attention_prefill_workspace``
+    entries of float32; allocated here when not given).  A bound that is too low leaves NaN in the rows
+    concerned."""
     _gpu("attention_prefill", q, kcache, vcache, tile_entry, tile_off, entry_start, entry_len, entry_past,
          block_tables, out)
     ldq, wq = _rows(q, "attention_prefill q")
@@ -526,9 +544,19 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
     ldo, wo = _rows(out, "attention_prefill out")
     if tuple(out.shape) != (n, nh * d) or out.dtype != q.dtype:
         raise ValueError("attention_prefill: out has the wrong shape or dtype")
+    if max_keys <= 0:
+        max_keys = block_tables.shape[1] * ps      # no bound given: what the block tables could hold
+    max_chunks = _prefill_chunks(int(max_keys), int(window))
+    need = int(_lib.load().zi_attention_prefill_workspace(n, nh, d, max_chunks))
+    if need:
+        if workspace is None:
+            workspace = torch.empty((need,), dtype=torch.float32, device=q.device)
+        if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
+            raise ValueError(f"attention_prefill: workspace must be a contiguous float32 buffer of {need} entries")
     _lib.call("zi_attention_prefill", _p(out), _p(q), _code(q, "attention_prefill"), num_tiles, ldq, ldo, _p(kcache),
               _p(vcache), _p(tile_entry), _p(tile_off), _p(entry_start), _p(entry_len), _p(entry_past),
-              _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), _stream())
+              _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), n,
+              max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, _stream())
     return out
 
 

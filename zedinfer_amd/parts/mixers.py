@@ -90,9 +90,12 @@ class Attention(Mixer):
             ops.attention(q, *args, self.window, out=att)
         elif n_long > 0:
             if ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
+                need = ops.attention_prefill_workspace(q.shape[0], self.nh, self.d, batch.max_long_keys, self.window)
+                ws = self.rt.buffer("attn_prompt_split", (need,), torch.float32) if need else None
                 ops.attention_prefill(q, memory.k, memory.v, batch.tile_entry, batch.tile_off, batch.entry_start,
                                       batch.entry_len, batch.entry_past, view.block_tables, self.nh, self.nkv,
-                                      self.d, self.scale, self.window, out=att)
+                                      self.d, self.scale, self.window, out=att, max_keys=batch.max_long_keys,
+                                      workspace=ws)
             else:
                 ops.attention(q, *args, self.window, out=att, tok_index=batch.long_idx)
 
