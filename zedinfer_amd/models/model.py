@@ -13,7 +13,7 @@ import torch
 
 from .. import ops
 from ..config.forward_config import LayerSpec, ModelForwardConfig, PartSpec
-from ..parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, KVCacheRequest, LayerMemory,
+from ..parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, KVCacheRequest, LayerMemory, Part,
                      Runtime, StateRequest)
 from ..weights.loader import WeightSpec
 
@@ -64,6 +64,7 @@ class DecoderModel:
         self.rt = rt
         self.embedding = _build(EMBEDDINGS, fc.embedding, weights, rt)
         self.blocks = []
+        self.parts = []         # every part that was built, blocks included
         for layer in fc.layers:
             block_cls = BLOCKS.get(layer.block)
             missing = [n for n in block_cls.norm_names if n not in layer.norms]
@@ -73,8 +74,12 @@ class DecoderModel:
             mixer = _build(MIXERS, layer.mixer, weights, rt)
             ffn = _build(FEED_FORWARDS, layer.feed_forward, weights, rt)
             self.blocks.append(block_cls(norms, mixer, ffn, rt))
+            # a mixer's position encoding is a part of its own
+            self.parts += [self.blocks[-1], mixer, ffn, *norms.values()]
+            self.parts += [p for p in vars(mixer).values() if isinstance(p, Part)]
         self.final_norm = _build(NORMS, fc.final_norm, weights, rt)
         self.lm_head = _build(HEADS, fc.lm_head, weights, rt)
+        self.parts += [self.embedding, self.final_norm, self.lm_head]
         self.vocab_size = fc.vocab_size
         self.hidden_size = fc.hidden_size
 
@@ -101,8 +106,8 @@ class DecoderModel:
         return out
 
     def graph_safe(self) -> bool:
-        """Whether a step's launches can be captured and replayed: every mixer says so."""
-        return all(getattr(b.mixer, "graph_safe", False) for b in self.blocks)
+        """Whether a step's launches can be captured and replayed: every part says so."""
+        return all(getattr(p, "graph_safe", False) for p in self.parts)
 
     # ---- one step -------------------------------------------------------------
     def run(self, batch, memories: Sequence[LayerMemory]) -> Optional[torch.Tensor]:

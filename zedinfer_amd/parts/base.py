@@ -117,6 +117,11 @@ class Part:
     """Base of all parts."""
 
     kind: str = ""
+    # A part whose forward only launches kernels that read device arrays (no copies to the host, no
+    # launches whose number or size depends on the arrays' contents, no allocations after its first
+    # calls) may set this.  When every part of a model does, steps of decoded tokens are captured as
+    # graphs and replayed; a part that leaves the default keeps the whole model on eager launches.
+    graph_safe: bool = False
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -137,11 +142,6 @@ class Mixer(Part):
     the few-rows matrix product leaves when it is cut along k).  ``batch`` is the step's
     device-side description (``engine.batch.DeviceBatch``); ``memory`` is this run's
     ``LayerMemory``."""
-
-    # A mixer whose forward only launches kernels that read the batch's device arrays (no copies to
-    # the host, no launches that depend on the arrays' contents) may set this: steps of decoded
-    # tokens are then captured as graphs and replayed.
-    graph_safe: bool = False
 
     def cache_request(self) -> Optional[KVCacheRequest]:
         return None

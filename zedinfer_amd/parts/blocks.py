@@ -14,6 +14,8 @@ class PreNormBlock(Block):
     (reference: src/frontend/models/transformer_forward.cpp:63-149).  The residual stream is
     float32 and every add into it happens inside the norm that follows it."""
 
+    graph_safe = True
+
     norm_names = ("input", "post_mixer")
 
     def __init__(self, norms, mixer, feed_forward, rt: Runtime):

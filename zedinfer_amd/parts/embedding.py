@@ -16,6 +16,8 @@ class TokenEmbedding(Part):
     """h[i,:] = table[ids[i],:], unscaled, widened into the float32 residual stream
     (reference: src/frontend/models/transformer_forward.cpp:54-60).  params: vocab_size, hidden_size."""
 
+    graph_safe = True
+
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
         return {"weight": WeightSpec((int(spec.params["vocab_size"]), int(spec.params["hidden_size"])))}
@@ -36,6 +38,8 @@ class LinearHead(Part):
     ``tied_to`` in the spec's weights the checkpoint may leave the tensor out and the embedding
     table stands in (reference: src/frontend/models/base.cpp:410-416).
     params: vocab_size, hidden_size, tied_to (tensor name or None)."""
+
+    graph_safe = True
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:

@@ -36,6 +36,8 @@ class SwiGLU(FeedForward):
     blocks of 8, so that the few-rows product can apply the activation in its epilogue.
     params: hidden_size, intermediate_size."""
 
+    graph_safe = True
+
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
         H, I = int(spec.params["hidden_size"]), int(spec.params["intermediate_size"])

@@ -17,6 +17,8 @@ class RMSNorm(Norm):
     (reference: src/backend/ops/rms_norm/cpu/rms_norm_cpu.cpp:14-29).
     params: dim, eps, add_one (default False)."""
 
+    graph_safe = True
+
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
         return {"weight": WeightSpec((int(spec.params["dim"]),))}

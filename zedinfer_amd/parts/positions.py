@@ -18,6 +18,8 @@ class RopeNeox(PositionEncoding):
     the reference rotates the whole head, no scaling: rope_nvidia.cu:50).
     params: head_dim, theta, rotary_dim (default head_dim)."""
 
+    graph_safe = True
+
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         super().__init__(spec, weights, rt)
         self.head_dim = int(spec.params["head_dim"])
@@ -53,6 +55,8 @@ class RopeNeox(PositionEncoding):
 @register_position_encoding("none")
 class NoPosition(PositionEncoding):
     """No encoding: keys and values are stored as they are."""
+
+    graph_safe = True
 
     def step_table(self, batch):
         return "none"
