@@ -88,7 +88,7 @@ def measure_decode(engine_factory, batch, steps, warmup, vocab):
     assert ctx1 - ctx0 == batch * steps
     for r in reqs:
         r.cancelled = True
-    loop.step()
+    loop.run_loop()
     return batch * steps / dt, dt / steps * 1000.0, (ctx0 + ctx1) / 2.0
 
 

@@ -103,6 +103,76 @@ def test_stop_token_ends_generation(tiny):
     assert res.finish_reason == "stop" and res.output_ids == free[:first + 1]
 
 
+def test_steps_queued_ahead_give_the_same_tokens(tiny):
+    """Decode steps that are queued before the step before them has finished (their tokens are read on
+    the device) against a loop that waits for every step: requests of different lengths, greedy and
+    sampled, one that ends on a stop token while a step ahead already computes for it, one that arrives
+    while the others decode, and prompts that enter in portions.  Every request gets the same tokens and
+    the same reason to end, and no page is lost."""
+    from zedinfer_amd import GenerationConfig, InferenceEngine, InferenceRequest, SchedulerConfig
+    from zedinfer_amd.engine import ServingLoop
+    V = tiny["cfg"]["vocab_size"]
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    prompts = [traces.random_tokens(V, n, seed=40 + i) for i, n in enumerate([9, 31, 50, 3, 20])]
+
+    def configs():
+        return [GenerationConfig(max_new_tokens=30, ignore_eos=True),
+                GenerationConfig(max_new_tokens=30),                                    # ends on the stop token
+                GenerationConfig(max_new_tokens=17, temperature=0.8, top_k=20, seed=5, ignore_eos=True),
+                GenerationConfig(max_new_tokens=2, ignore_eos=True),
+                GenerationConfig(max_new_tokens=25, temperature=0.6, top_p=0.9, seed=6, ignore_eos=True)]
+
+    def run(look_ahead, stops):
+        ie = InferenceEngine.create(tiny["folder"], "float32", SchedulerConfig(
+            num_kv_blocks=64, kv_block_size=ps, max_batch_requests=4, max_prefill_tokens=24, max_batch_tokens=32))
+        loop = ServingLoop(ie.engine, stops, look_ahead=look_ahead)
+        cf = configs()
+        reqs = [loop.submit_async(InferenceRequest(p, c)) for p, c in zip(prompts[:4], cf[:4])]
+        for _ in range(9):
+            loop.step()
+        reqs.append(loop.submit_async(InferenceRequest(prompts[4], cf[4])))     # arrives while the others decode
+        loop.run_loop()
+        assert all(r.done and not r.error for r in reqs)
+        ie.engine.cache.check()
+        assert not ie.engine.cache.live
+        return [(r.result.output_ids, r.result.finish_reason) for r in reqs], loop.steps_ahead
+
+    free, _ = run(False, [])
+    stop = free[1][0][11]           # a token the second request makes on its way
+    want, none_ahead = run(False, [stop])
+    got, ahead = run(True, [stop])
+    assert none_ahead == 0 and ahead > 10
+    assert want[1][1] == "stop" and len(want[1][0]) <= 12
+    assert got == want
+
+
+def test_steps_queued_ahead_with_the_serving_kernels(tiny, tmp_path):
+    """A bfloat16 checkpoint, greedy, steps queued ahead and replayed as graphs: every token a request
+    gets is the best, or within rounding of the best, at its place in the plain run of its sequence."""
+    from zedinfer_amd import GenerationConfig, InferenceEngine, InferenceRequest, SchedulerConfig
+    V = tiny["cfg"]["vocab_size"]
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    folder = tiny_configs.write_tiny(str(tmp_path), tiny["name"], dtype=torch.bfloat16)
+    cfg, w = plain.load_folder(folder)
+    prompts = [traces.random_tokens(V, n, seed=50 + i) for i, n in enumerate([9, 31, 3])]
+    ie = InferenceEngine.create(folder, "bfloat16", SchedulerConfig(num_kv_blocks=64, kv_block_size=ps,
+                                                                    max_batch_requests=4))
+    loop = ie.serving_loop()
+    reqs = [loop.submit_async(InferenceRequest(p, GenerationConfig(max_new_tokens=n, ignore_eos=True)))
+            for p, n in zip(prompts, (24, 17, 30))]
+    loop.run_loop()
+    assert loop.steps_ahead > 10 and ie.engine.graph_replays > 10
+    for p, r in zip(prompts, reqs):
+        out = r.result.output_ids
+        assert len(out) == r.config.max_new_tokens
+        ref = plain.forward(cfg, w, p + out[:-1])
+        for i, t in enumerate(out):
+            row = ref[len(p) - 1 + i]
+            assert float(row.max() - row[t]) <= 0.03 * float(row.abs().max()), (i, t, int(row.argmax()))
+    ie.engine.cache.check()
+    assert not ie.engine.cache.live
+
+
 def test_out_of_pages_fails_the_request_not_the_engine(tiny):
     from zedinfer_amd import GenerationConfig
     ie = engine(tiny, num_kv_blocks=4)

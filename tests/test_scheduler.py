@@ -185,3 +185,113 @@ def test_sampling_options_are_validated():
             s.submit(req(2, **bad))
     with pytest.raises(ValueError, match="stream_callback"):
         s.submit(req(2, stream=True))
+
+
+# ---- the batch after the one that runs ------------------------------------------------------
+
+def commit(cache, batch):
+    """What the engine does when it queues a step: the new tokens get their places."""
+    for e in batch.entries():
+        cache.ensure(e.seq, e.seq.length + len(e.tokens))
+        cache.commit(e.seq, e.seq.length + len(e.tokens))
+
+
+def test_batch_ahead_is_known_when_only_the_tokens_are_open():
+    s, c = make()
+    a, b = req(5, max_new=6), req(3, max_new=6)
+    s.submit(a)
+    s.submit(b)
+    first = s.schedule()            # both prompts, whole
+    commit(c, first)
+    ahead = s.schedule_ahead(first)
+    assert ahead is not None and ahead.decode_requests == [a, b] and ahead.tokens_on_device
+    assert [list(e.want) for e in ahead.entries()] == [[0], [0]] and all(len(e.tokens) == 1 for e in ahead.entries())
+    commit(c, ahead)
+    s.process_results(first, [7, 8])
+    assert a.output_ids == [7] and b.output_ids == [8]
+    s.process_results(ahead, [9, 10])
+    assert a.output_ids == [7, 9] and b.output_ids == [8, 10] and a.generated_count == 2
+    # what the ordinary schedule makes next is the same kind of batch, with the tokens on the host
+    nxt = s.schedule()
+    assert nxt.decode_requests == [a, b] and [e.tokens for e in nxt.entries()] == [[9], [10]]
+    c.check()
+
+
+def test_no_batch_ahead_when_the_results_could_change_it():
+    # the last token of a request: it ends with this step's result
+    s, c = make()
+    a = req(4, max_new=2)
+    s.submit(a)
+    first = s.schedule()
+    commit(c, first)
+    assert s.schedule_ahead(first) is not None          # 1 of 2 after this step
+    s.process_results(first, [7])
+    second = s.schedule()
+    commit(c, second)
+    assert s.schedule_ahead(second) is None             # 2 of 2 after this step
+    # a cancelled request, and one whose sampling reads its history
+    for kw, cancel in ((dict(), True), (dict(repetition_penalty=1.3, temperature=0.8), False)):
+        s, c = make()
+        a = req(4, max_new=8, **kw)
+        s.submit(a)
+        first = s.schedule()
+        commit(c, first)
+        a.cancelled = cancel
+        assert s.schedule_ahead(first) is None
+    # a prompt that is only partly in
+    s, c = make(max_batch_tokens=8, max_prefill_tokens=8)
+    a, b = req(3, max_new=8), req(12, max_new=8)
+    s.submit(a)
+    s.submit(b)
+    first = s.schedule()            # a whole, 5 tokens of b
+    assert first.prefill_chunk_sizes == [3, 5]
+    commit(c, first)
+    assert s.schedule_ahead(first) is None
+    # a waiting prompt that could be admitted now
+    s, c = make()
+    a = req(3, max_new=8)
+    s.submit(a)
+    first = s.schedule()
+    commit(c, first)
+    s.submit(req(3, max_new=8))
+    assert s.schedule_ahead(first) is None
+    # no page for the next token
+    s, c = make(pages=2, page_size=4, generation_reserve=1)
+    a = req(8, max_new=8)
+    s.submit(a)
+    first = s.schedule()
+    commit(c, first)
+    assert s.schedule_ahead(first) is None
+    c.check()
+
+
+def test_batch_ahead_while_the_head_of_the_queue_cannot_enter():
+    s, c = make(max_batch_requests=1)
+    a, b = req(3, max_new=8), req(3, max_new=8)
+    s.submit(a)
+    s.submit(b)
+    first = s.schedule()
+    assert first.prefill_requests == [a]
+    commit(c, first)
+    ahead = s.schedule_ahead(first)
+    assert ahead is not None and ahead.decode_requests == [a]
+
+
+def test_token_computed_for_a_request_that_ended_is_dropped():
+    s, c = make()
+    a, b = req(5, max_new=6), req(3, max_new=6)
+    s.submit(a)
+    s.submit(b)
+    first = s.schedule()
+    commit(c, first)
+    ahead = s.schedule_ahead(first)
+    commit(c, ahead)
+    free_before = c.groups[0].pool.num_free
+    s.process_results(first, [99, 8])                   # a ends on the stop token
+    assert a.done and a.finish_reason == "stop" and a.result.output_ids == [99]
+    assert c.groups[0].pool.num_free > free_before      # its pages are back while the step ahead still runs
+    s.process_results(ahead, [5, 10])
+    assert a.result.output_ids == [99] and b.output_ids == [8, 10]
+    c.check()
+    nxt = s.schedule()
+    assert nxt.decode_requests == [b]

@@ -134,18 +134,31 @@ class Engine:
         self.cache.close(seq)
 
     # ---- the step ------------------------------------------------------------------
-    def step(self, entries: Sequence[StepEntry], copy: bool = True) -> Optional[torch.Tensor]:
+    def step(self, entries: Sequence[StepEntry], copy: bool = True,
+             token_source: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted, vocab] in the order of the entries and
         of each entry's ``want`` (None when nothing is wanted).  With ``copy`` False the result is
         a view of a workspace that the next step overwrites.  Raises OutOfPages, with no
-        request's length changed, when the pool cannot hold the new tokens."""
+        request's length changed, when the pool cannot hold the new tokens.
+
+        ``token_source``: an int32 device tensor [entries].  Every entry then brings one token whose
+        value is read from there on the device (``tokens`` holds a placeholder), so that a step can be
+        queued before the host has seen what the step before it sampled."""
+        single = all(len(e.tokens) == 1 for e in entries)
+        if token_source is not None:
+            if not single:
+                raise ValueError("tokens can come from the device only when every entry brings one token")
+            if (token_source.dtype != torch.int32 or token_source.device != self.device
+                    or token_source.shape != (len(entries),)):
+                raise ValueError(f"token_source must be an int32 tensor [{len(entries)}] on {self.device}")
         for e in entries:
             self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
-        if (self.use_graphs and 0 < len(entries) <= self.graph_max_entries
-                and all(len(e.tokens) == 1 for e in entries)):
-            logits = self._graph_step(entries)
+        if self.use_graphs and 0 < len(entries) <= self.graph_max_entries and single:
+            logits = self._graph_step(entries, token_source)
         else:
             batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging)
+            if token_source is not None:
+                batch.token_ids.copy_(token_source, non_blocking=True)
             logits = self.model.run(batch, self.memories)
         for e in entries:
             self.cache.commit(e.seq, e.seq.length + len(e.tokens))
@@ -153,7 +166,8 @@ class Engine:
         return logits.clone() if (copy and logits is not None) else logits
 
     # ---- decode steps as graphs ------------------------------------------------------
-    def _graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _graph_step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None
+                    ) -> Optional[torch.Tensor]:
         """A step in which every entry brings one token.  Its launches depend on the number of entries
         and wanted rows, on the width of the block tables and on the size of the attention launch
         only: the first step of a kind runs eagerly and is captured, later ones replay the graph
@@ -177,6 +191,8 @@ class Engine:
         else:
             dg.image = DecodeImage(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer)
             batch = dg.image.batch
+        if token_source is not None:
+            batch.token_ids.copy_(token_source, non_blocking=True)
         batch.max_short_keys = keys_bucket
         if dg.graph is not None:
             dg.graph.replay()

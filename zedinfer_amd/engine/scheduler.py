@@ -55,11 +55,15 @@ class ScheduledBatch:
         r = self.prefill_requests[i]
         return self.prefill_chunk_starts[i] + self.prefill_chunk_sizes[i] >= len(r.input_ids)
 
+    # a batch that was scheduled before the tokens of the step before it were known: its decode
+    # tokens are read on the device from what that step sampled, in the order of decode_requests
+    tokens_on_device: bool = False
+
     def entries(self) -> List[StepEntry]:
         """Decode rows first, then the prompt portions; logits are wanted for each decode token and
         for the last token of a portion that completes its prompt
         (reference: src/zedinfer/batch_context.cpp:21-85)."""
-        out = [StepEntry(r.seq, [r.last_token], [0]) for r in self.decode_requests]
+        out = [StepEntry(r.seq, [0 if self.tokens_on_device else r.last_token], [0]) for r in self.decode_requests]
         for i, r in enumerate(self.prefill_requests):
             s, n = self.prefill_chunk_starts[i], self.prefill_chunk_sizes[i]
             out.append(StepEntry(r.seq, r.input_ids[s:s + n], [n - 1] if self.completes_prompt(i) else []))
@@ -193,6 +197,39 @@ class Scheduler:
                     break
         return batch
 
+    def schedule_ahead(self, batch: ScheduledBatch) -> Optional[ScheduledBatch]:
+        """The batch after ``batch``, made while ``batch`` still runs, or None when it cannot be known
+        yet.  It can when the results of ``batch`` will change nothing but the tokens: the requests it
+        samples for are all that run, none of them reaches its length with this token, is cancelled or
+        needs its history for sampling, and ``schedule()`` would not admit a prompt now.  A request that
+        ends on a stop token in ``batch`` has one token too many computed; ``process_results`` drops it.
+        A waiting prompt that only a request's end makes room for enters one step later than it
+        would without looking ahead."""
+        with self._lock:
+            sampled = batch.sampled_requests()
+            if not sampled or len(sampled) != len(self.active) or any(a is not b for a, b in zip(self.active, sampled)):
+                return None
+            if len(sampled) > self.config.max_batch_tokens:
+                return None
+            if self.waiting:
+                head = self.waiting[0]
+                if head.seq is not None:
+                    return None         # a prompt is partly in: its next portion belongs to the next step
+                if len(self.active) < self.config.max_batch_requests and self.cache.can_open(self._reserve(head)):
+                    return None
+            for r in sampled:
+                made = (r.generated_count if r.phase == RequestPhase.DECODE else 0) + 1
+                if r.done or r.cancelled or made >= r.config.max_new_tokens:
+                    return None
+                if r.sampler.params.repetition_penalty != 1.0:
+                    return None
+            try:
+                for r in sampled:
+                    self.cache.ensure(r.seq, r.seq.length + 1)
+            except OutOfPages:
+                return None             # the ordinary step decides who fails
+            return ScheduledBatch(decode_requests=list(sampled), tokens_on_device=True)
+
     # ---- after the step ------------------------------------------------------------------
     def process_results(self, batch: ScheduledBatch, tokens: Sequence[int]) -> None:
         """``tokens``: one sampled token per request of ``batch.sampled_requests()``, in that order.
@@ -202,6 +239,8 @@ class Scheduler:
             raise ValueError(f"{len(tokens)} tokens for {len(sampled)} sampled requests")
         with self._lock:
             for req, tok in zip(sampled, tokens):
+                if req.done:
+                    continue            # it ended while this step, scheduled ahead, was running
                 tok = int(tok)
                 first = req.phase != RequestPhase.DECODE
                 req.phase = RequestPhase.DECODE

@@ -8,23 +8,50 @@ include/zedinfer/engine.hpp:96-166, src/zedinfer/engine.cpp:338-522).
 """
 from __future__ import annotations
 
+import os
 import time
 from typing import Iterable, List, Optional, Sequence
 
 import torch
 
 from ..config import SchedulerConfig
+from ..ops.staging import StagingRing
 from ..sampling.sampler import Sampler
 from .engine import Engine
 from .request import GenerationConfig, GenerationResult, InferenceRequest, RequestPhase
 from .scheduler import ScheduledBatch, Scheduler
 
 
+class _Flight:
+    """A step that has been queued on the device: its batch, where its tokens will arrive on the host,
+    and the event after which they are there."""
+
+    def __init__(self, batch: ScheduledBatch, tokens_dev: Optional[torch.Tensor], tokens_host: Optional[torch.Tensor],
+                 done: torch.cuda.Event, t0: float):
+        self.batch, self.tokens_dev, self.tokens_host, self.done, self.t0 = batch, tokens_dev, tokens_host, done, t0
+
+    def wait(self) -> List[int]:
+        self.done.synchronize()
+        return self.tokens_host.tolist() if self.tokens_host is not None else []
+
+
 class ServingLoop:
-    def __init__(self, engine: Engine, stop_token_ids: Iterable[int] = ()):
+    """``look_ahead``: while a decode step runs, the next one is queued behind it with its tokens read
+    on the device from what the running step samples, so the device does not wait for the host between
+    steps.  The tokens a request gets are the same either way (``Scheduler.schedule_ahead`` says when the
+    next batch is known early).  The reference's loop waits for every step's tokens before it schedules
+    the next (src/zedinfer/serving_loop.cpp:330-408)."""
+
+    def __init__(self, engine: Engine, stop_token_ids: Iterable[int] = (), look_ahead: Optional[bool] = None):
         self.engine = engine
         self.scheduler = Scheduler(engine.sched, engine.cache, stop_token_ids)
         self.sampler = Sampler(engine.device, engine.vocab_size)
+        self.look_ahead = os.environ.get("ZEDINFER_DISABLE_LOOKAHEAD", "0") in ("", "0") if look_ahead is None \
+            else bool(look_ahead)
+        self.steps_ahead = 0            # steps that were queued before the one before them had finished
+        self._flight: Optional[_Flight] = None
+        self._token_ring = StagingRing(engine.device)
+        self._last_results = 0.0
         self._running = False
 
     def submit_async(self, request: InferenceRequest) -> InferenceRequest:
@@ -38,24 +65,52 @@ class ServingLoop:
     def active_count(self) -> int:
         return self.scheduler.active_count()
 
-    def step(self) -> bool:
-        """One scheduled batch through the model.  Returns False when there was nothing to run."""
-        batch = self.scheduler.schedule()
-        if batch.empty():
-            return False
+    def _launch(self, batch: ScheduledBatch, token_source: Optional[torch.Tensor]) -> Optional[_Flight]:
+        """Queue the batch's step, its sampling and the copy of the tokens to the host; nothing is waited
+        for.  A step that raises fails its batch, not the loop."""
         t0 = time.perf_counter()
         try:
-            logits = self.engine.step(batch.entries(), copy=False)
+            logits = self.engine.step(batch.entries(), copy=False, token_source=token_source)
             sampled = batch.sampled_requests()
-            tokens: List[int] = []
+            tokens_dev = tokens_host = None
             if sampled:
-                tokens = self.sampler.sample(logits, [r.sampler for r in sampled], [r.output_ids for r in sampled])
-            else:
-                torch.cuda.synchronize(self.engine.device)
-        except Exception as e:  # noqa: BLE001  (a failed step fails its batch, not the loop)
+                tokens_dev = self.sampler.launch(logits, [r.sampler for r in sampled], [r.output_ids for r in sampled])
+                tokens_host = self._token_ring.acquire(len(sampled))
+                tokens_host.copy_(tokens_dev, non_blocking=True)
+                self._token_ring.copied()
+            done = torch.cuda.Event()
+            done.record()
+        except Exception as e:  # noqa: BLE001
             self.scheduler.fail_batch(batch, f"step failed: {type(e).__name__}: {e}")
+            return None
+        return _Flight(batch, tokens_dev, tokens_host, done, t0)
+
+    def step(self) -> bool:
+        """One scheduled batch through the model, to the point where its tokens have reached their
+        requests.  Returns False when there was nothing to run."""
+        flight, self._flight = self._flight, None
+        if flight is None:
+            batch = self.scheduler.schedule()
+            if batch.empty():
+                return False
+            flight = self._launch(batch, None)
+            if flight is None:
+                return True
+        batch = flight.batch
+        if self.look_ahead and flight.tokens_dev is not None:
+            ahead = self.scheduler.schedule_ahead(batch)
+            if ahead is not None:
+                self._flight = self._launch(ahead, flight.tokens_dev)
+                self.steps_ahead += self._flight is not None
+        try:
+            tokens = flight.wait()
+        except Exception as e:  # noqa: BLE001
+            self.scheduler.fail_batch(batch, f"step failed: {type(e).__name__}: {e}")
+            self._flight = None
             return True
-        ms = (time.perf_counter() - t0) * 1000.0
+        now = time.perf_counter()
+        ms = (now - max(flight.t0, self._last_results)) * 1000.0
+        self._last_results = now
         # time is split like the reference's: a step's time goes to prefill for prompt portions and is
         # shared evenly among the decoding requests (reference: serving_loop.cpp:287-305)
         n_dec, n_pre = len(batch.decode_requests), len(batch.prefill_requests)
@@ -64,6 +119,8 @@ class ServingLoop:
         for r in batch.decode_requests:
             r.stats.decode_time_ms += ms / n_dec if not n_pre else ms * 0.5 / n_dec
         self.scheduler.process_results(batch, tokens)
+        if self._flight is not None and all(r.done for r in self._flight.batch.decode_requests):
+            self._flight = None         # everything the step ahead computes for has ended
         return True
 
     def run_loop(self) -> None:

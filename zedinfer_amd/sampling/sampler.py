@@ -18,6 +18,7 @@ import numpy as np
 import torch
 
 from .. import ops
+from ..ops.staging import StagingRing
 
 
 @dataclass
@@ -65,20 +66,30 @@ class Sampler:
     def __init__(self, device: torch.device, vocab_size: int):
         self.device = device
         self.vocab_size = vocab_size
+        self.staging = StagingRing(device)
 
     def sample(self, logits: torch.Tensor, samplers: Sequence[RequestSampler],
                histories: Optional[Sequence[Sequence[int]]] = None) -> List[int]:
         """``samplers[i]`` and ``histories[i]`` (the tokens generated so far) belong to row i."""
+        return self.launch(logits, samplers, histories).tolist()
+
+    def launch(self, logits: torch.Tensor, samplers: Sequence[RequestSampler],
+               histories: Optional[Sequence[Sequence[int]]] = None) -> torch.Tensor:
+        """As ``sample``, but the tokens stay on the device (int32 [rows]) and nothing is waited for."""
         R = logits.shape[0]
         if R != len(samplers):
             raise ValueError(f"{R} rows of logits for {len(samplers)} requests")
         if all(s.params.greedy and s.params.repetition_penalty == 1.0 for s in samplers):
-            return ops.argmax(logits).tolist()
-        temp = np.array([0.0 if s.params.greedy else s.params.temperature for s in samplers], dtype=np.float32)
-        top_k = np.array([s.params.top_k for s in samplers], dtype=np.int32)
-        top_p = np.array([s.params.top_p for s in samplers], dtype=np.float32)
-        pen = np.array([s.params.repetition_penalty for s in samplers], dtype=np.float32)
-        u = np.array([0.0 if s.params.greedy else s.draw() for s in samplers], dtype=np.float32)
+            return ops.argmax(logits)
+        # the per-row parameters travel in one pinned buffer, so that nothing here waits for the device
+        par = self.staging.acquire(5 * R)
+        pv = par.numpy().reshape(5, R)
+        pv[0].view(np.float32)[:] = [0.0 if s.params.greedy else s.params.temperature for s in samplers]
+        pv[1][:] = [s.params.top_k for s in samplers]
+        pv[2].view(np.float32)[:] = [s.params.top_p for s in samplers]
+        pen = pv[3].view(np.float32)
+        pen[:] = [s.params.repetition_penalty for s in samplers]
+        pv[4].view(np.float32)[:] = [0.0 if s.params.greedy else s.draw() for s in samplers]
         recent = recent_len = None
         if histories is not None and any(p != 1.0 for p in pen):
             width = max(1, max(len(h) if pen[i] != 1.0 else 0 for i, h in enumerate(histories)))
@@ -90,6 +101,7 @@ class Sampler:
                     rl[i] = len(h)
             recent = torch.from_numpy(rc).to(self.device)
             recent_len = torch.from_numpy(rl).to(self.device)
-        dev = lambda a: torch.from_numpy(a).to(self.device)  # noqa: E731
-        out = ops.sample(logits, dev(temp), dev(top_k), dev(top_p), dev(pen), dev(u), recent, recent_len)
-        return out.tolist()
+        d = par.to(self.device, non_blocking=True).view(5, R)
+        self.staging.copied()
+        return ops.sample(logits, d[0].view(torch.float32), d[1], d[2].view(torch.float32), d[3].view(torch.float32),
+                          d[4].view(torch.float32), recent, recent_len)
