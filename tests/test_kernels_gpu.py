@@ -325,18 +325,9 @@ def test_attention_decode(ops, nh, nkv, d, ps, T, window):
     torch.testing.assert_close(out.float(), plain_out.float(), atol=1e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize("nh,nkv,d,ps,lens,window,S,bias_dtype,rot", [
-    (12, 2, 128, 16, [2100, 1, 64, 65, 257, 300, 1024, 17], 0, 2, torch.bfloat16, 128),
-    (3, 1, 64, 8, [200, 5, 9], 0, 1, None, 64),
-    (8, 2, 48, 8, [33, 700, 256], 0, 3, torch.float32, 32),
-    (4, 2, 128, 16, [500, 120, 99], 100, 5, torch.bfloat16, 128),
-    (6, 3, 80, 32, [150, 64], 0, 2, torch.bfloat16, 0),
-    (12, 2, 128, 16, [17000, 300], 0, 2, torch.bfloat16, 128)])
-def test_attention_decode_fused(ops, nh, nkv, d, ps, lens, window, S, bias_dtype, rot):
-    """One kernel for rotation, cache store and attention of decoded tokens gives what the rotary kernel
-    followed by the decode kernel gives: same output, same new keys and values in the cache.  The slot
-    of the new token holds NaN before, and the sequences differ in length (the new key sits in every
-    place of a block)."""
+def fused_decode_case(ops, nh, nkv, d, ps, lens, S, bias_dtype, rot):
+    """Sequences of the given lengths in a shuffled paged cache whose last position (the new token's)
+    and unused slots hold NaN, and the partial sums of the new tokens' projections."""
     dtype = torch.bfloat16
     B, width, theta = len(lens), (nh + 2 * nkv) * d, 1e4
     assert ops.attention_decode_fused_supported(dtype, nh, nkv, d, ps, rot, S, width, B)
@@ -362,6 +353,27 @@ def test_attention_decode_fused(ops, nh, nkv, d, ps, lens, window, S, bias_dtype
     sums = rnd(S, B, width, seed=1)
     bias = rnd(width, seed=2).to(bias_dtype) if bias_dtype is not None else None
     inv_freq = ops.rope_inv_freq(rot, theta, "cuda") if rot else None
+    return kc, vc, bt, slots, pos, seq, sums, bias, inv_freq
+
+
+FUSED_DECODE_CASES = [
+    (12, 2, 128, 16, [2100, 1, 64, 65, 257, 300, 1024, 17], 0, 2, torch.bfloat16, 128),
+    (3, 1, 64, 8, [200, 5, 9], 0, 1, None, 64),
+    (8, 2, 48, 8, [33, 700, 256], 0, 3, torch.float32, 32),
+    (4, 2, 128, 16, [500, 120, 99], 100, 5, torch.bfloat16, 128),
+    (6, 3, 80, 32, [150, 64], 0, 2, torch.bfloat16, 0),
+    (12, 2, 128, 16, [17000, 300], 0, 2, torch.bfloat16, 128)]
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps,lens,window,S,bias_dtype,rot", FUSED_DECODE_CASES)
+def test_attention_decode_fused(ops, nh, nkv, d, ps, lens, window, S, bias_dtype, rot):
+    """One kernel for rotation, cache store and attention of decoded tokens gives what the rotary kernel
+    followed by the decode kernel gives: same output, same new keys and values in the cache.  The slot
+    of the new token holds NaN before, and the sequences differ in length (the new key sits in every
+    place of a block)."""
+    B = len(lens)
+    kc, vc, bt, slots, pos, seq, sums, bias, inv_freq = fused_decode_case(ops, nh, nkv, d, ps, lens, S, bias_dtype, rot)
+    dtype = torch.bfloat16
     scale, T = 1 / math.sqrt(d), max(lens)
     # the two kernels
     kc1, vc1 = kc.clone(), vc.clone()
@@ -392,6 +404,63 @@ def test_attention_decode_fused(ops, nh, nkv, d, ps, lens, window, S, bias_dtype
     torch.testing.assert_close(out3.float(), ref.float(), atol=4e-3, rtol=1e-2)
     assert bool(((kc3 == kc1) | (torch.isnan(kc3) & torch.isnan(kc1))).all())
     assert bool(((vc3 == vc1) | (torch.isnan(vc3) & torch.isnan(vc1))).all())
+
+
+@pytest.mark.parametrize("nh,nkv,d,ps,lens,window,S,bias_dtype,rot", FUSED_DECODE_CASES + [
+    (40, 8, 128, 16, [300, 70, 1], 0, 2, torch.bfloat16, 128),            # groups of three heads a partial sum
+    (2, 1, 16, 8, [9, 300, 40, 41, 42, 43, 44, 45, 46, 47, 48, 49, 50, 51, 52, 53], 0, 1, None, 16)])  # 16 tokens
+def test_attention_decode_project(ops, nh, nkv, d, ps, lens, window, S, bias_dtype, rot):
+    """The output projection read straight from the unmerged chunks against the merged attention times
+    the weight: the merge is the merge kernel's (its bfloat16 result is the operand), so only the order
+    of the float32 sums differs.  Widths that are no multiple of 64 or of 4."""
+    B = len(lens)
+    kc, vc, bt, slots, pos, seq, sums, bias, inv_freq = fused_decode_case(ops, nh, nkv, d, ps, lens, S, bias_dtype, rot)
+    scale, T = 1 / math.sqrt(d), max(lens)
+    table = ops.rope_table(pos, inv_freq) if rot else None
+    kc1, vc1 = kc.clone(), vc.clone()
+    att = ops.attention_decode_fused(sums, bias, table, slots, kc1, vc1, seq, pos, bt, nh, nkv, d, scale, T, window)
+    kc2, vc2 = kc.clone(), vc.clone()
+    ws = torch.full((ops.attention_decode_workspace(B, nh, d),), float("nan"), device="cuda")
+    got_ws = ops.attention_decode_fused(sums, bias, table, slots, kc2, vc2, seq, pos, bt, nh, nkv, d, scale, T, window,
+                                        workspace=ws, leave_chunks=True)
+    assert got_ws is ws
+    assert bool(((kc2 == kc1) | (torch.isnan(kc2) & torch.isnan(kc1))).all())
+    for N in (1536, 200, 70):
+        w = (rnd(N, nh * d, seed=7) / math.sqrt(nh * d)).to(torch.bfloat16)
+        assert ops.attention_decode_project_supported(w, B, nh, d)
+        want = att.float() @ w.float().T
+        parts = torch.full((ops.attention_decode_project_splits(nh), B, N), float("nan"), device="cuda")
+        out = ops.attention_decode_project(ws, w, pos, nh, d, T, window, out=parts)
+        assert out is parts and not torch.isnan(parts).any()
+        torch.testing.assert_close(parts.sum(0), want, atol=2e-4 * max(1.0, float(want.abs().max())), rtol=1e-4)
+        # a partial sum is the product over its heads alone
+        hg = -(-nh // parts.shape[0])
+        first = att.float()[:, :hg * d] @ w.float()[:, :hg * d].T
+        torch.testing.assert_close(parts[0], first, atol=2e-4 * max(1.0, float(first.abs().max())), rtol=1e-4)
+
+
+def test_attention_decode_project_shows_a_bound_too_low(ops):
+    """Chunks the launch did not cover: the token's whole row is NaN, the other tokens' rows are right."""
+    nh, nkv, d, ps, lens = 4, 2, 64, 16, [700, 100]
+    kc, vc, bt, slots, pos, seq, sums, bias, inv_freq = fused_decode_case(ops, nh, nkv, d, ps, lens, 2, None, 64)
+    scale = 1 / math.sqrt(d)
+    table = ops.rope_table(pos, inv_freq)
+    w = (rnd(96, nh * d, seed=7) / 16).to(torch.bfloat16)
+    att = ops.attention_decode_fused(sums, bias, table, slots, kc.clone(), vc.clone(), seq, pos, bt, nh, nkv, d, scale, 700)
+    ws = ops.attention_decode_fused(sums, bias, table, slots, kc.clone(), vc.clone(), seq, pos, bt, nh, nkv, d, scale, 200,
+                                    leave_chunks=True)
+    parts = ops.attention_decode_project(ws, w, pos, nh, d, 200)
+    assert bool(torch.isnan(parts[:, 0]).all())
+    torch.testing.assert_close(parts.sum(0)[1], att.float()[1] @ w.float().T, atol=2e-4, rtol=1e-4)
+
+
+def test_attention_decode_project_refuses_other_shapes(ops):
+    w = torch.zeros(64, 12 * 128, dtype=torch.bfloat16, device="cuda")
+    assert ops.attention_decode_project_supported(w, 16, 12, 128)
+    assert not ops.attention_decode_project_supported(w, 17, 12, 128)            # more tokens than a tile's columns
+    assert not ops.attention_decode_project_supported(w.float(), 8, 12, 128)
+    assert not ops.attention_decode_project_supported(w, 8, 6, 128)              # not this weight's columns
+    assert not ops.attention_decode_project_supported(w[:, :1532], 8, 12, 128)
 
 
 def test_attention_decode_fused_refuses_other_layouts(ops):

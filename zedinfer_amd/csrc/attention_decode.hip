@@ -85,7 +85,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                         const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
                         int max_pages, int num_pages, int nh, int nkv, int G, int ps, int window, float scale,
-                        int max_chunks, DecProjection pj) {
+                        int max_chunks, int leave_parts, DecProjection pj) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DT = D / 16;          // output tiles of 16 dims
@@ -103,7 +103,8 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     if (sp.count > max_chunks) {
         // The host sized the launch (and the workspace) for fewer keys than this token sees.  Nothing
         // may be written to the workspace then; the token's output is made NaN so that it shows.
-        if (chunk == 0)
+        // (With leave_parts the kernel that reads the chunks sees the same count and does that.)
+        if (chunk == 0 && !leave_parts)
             for (int i = tid; i < G * D; i += DEC_WAVES * ZI_WAVE)
                 zi_store(out + (int64_t)t * ldo + (int64_t)kvh * G * D + i, NAN);
         return;
@@ -433,7 +434,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         a[w] = (sm[w][r] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(sm[w][r] - M);
         L += a[w] * sl[w][r];
     }
-    const bool final = sp.count == 1;
+    const bool final = sp.count == 1 && !leave_parts;
     const float inv = final ? 1.f / L : 1.f;
     const int64_t slot = ((int64_t)x * nh + kvh * G + r) * DEC_MAXC + chunk;
     for (int dd = wave; dd < DT; dd += DEC_WAVES) {
@@ -497,6 +498,138 @@ attention_decode_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const floa
         if (lane + v * ZI_WAVE < D) zi_store(out + (int64_t)t * ldo + (int64_t)h * D + lane + v * ZI_WAVE, acc[v] * inv);
 }
 
+// The output projection straight from the chunks: sums[s][t][:] = W[:, heads of split s] . merged
+// attention of token t for those heads, as float32 partial sums over groups of `hg` heads that the
+// next kernel adds in rising order.  One workgroup per (64 rows of W, group of heads): thread (token,
+// eight dims) merges the token's chunks for a head as the merge kernel does (maximum first, then the
+// weighted sums in rising order; the result is rounded to bfloat16 as if it had been stored), the
+// four wavefronts multiply 16 rows each on the matrix cores with the up to 16 tokens as columns.
+// The attention kernel must have left every token's chunks in the workspace (leave_parts).  A token
+// that sees more chunks than the launch covered gets NaN.
+#define DPJ_ROWS 64
+template <int D>
+__global__ void __launch_bounds__(256)
+attention_decode_project_kernel(float* __restrict__ sums, const float* __restrict__ part_o,
+                                const float* __restrict__ part_ml, const int32_t* __restrict__ tok_pos, int n, int nh,
+                                int window, int max_chunks, const zi_bf16* __restrict__ w, int64_t ldw, int N, int hg) {
+    constexpr int DK = (D + 31) / 32;
+    constexpr int XS = DK * 32 + 8;     // row stride of the merged head in LDS, in elements (16-byte rows, no bank repeat)
+    __shared__ __attribute__((aligned(16))) uint16_t sx[16][XS];
+    const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
+    const int r = lane & 15, j = lane >> 4;
+    const int split = blockIdx.y, h0 = split * hg, h1 = (h0 + hg < nh) ? h0 + hg : nh;
+    const int row = blockIdx.x * DPJ_ROWS + wave * 16 + r;
+    const zi_bf16* wr = w + (int64_t)(row < N ? row : N - 1) * ldw;
+    // the merging thread's token and dims
+    const int mt = tid >> 4, d0 = (tid & 15) * 8;
+    dec_f32x4_t acc = dec_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int h = h0; h < h1; ++h) {
+        // ---- the weights of this head's columns first: they do not wait for the merge
+        dec_pack a[DK];
+#pragma unroll
+        for (int dk = 0; dk < DK; ++dk) {
+            const bool in = dk * 32 + j * 8 < D;
+            a[dk].u = *reinterpret_cast<const uint4*>(wr + (int64_t)h * D + (in ? dk * 32 + j * 8 : 0));
+        }
+        // ---- merge: eight dims of one token.  The sixteen lanes of a token share its chunks' (maximum,
+        // sum): lane q loads those of chunks q, q + 16, ..., and they trade maxima and weights by
+        // shuffles, as the merge kernel's lanes do.  These loads and the first eight chunks' outputs
+        // travel together.
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = 0.f;
+        const int q = tid & 15, mtc = mt < n ? mt : n - 1;
+        const int count = dec_split(tok_pos[mtc], window).count;
+        const int64_t slot0 = ((int64_t)mtc * nh + h) * DEC_MAXC;
+        const float2* ml = reinterpret_cast<const float2*>(part_ml) + slot0;
+        const float* po0 = part_o + slot0 * D + (d0 < D ? d0 : 0);
+        float2 mlq[DEC_MAXC / 16];
+        float4 lo[8], hi[8];
+#pragma unroll
+        for (int u = 0; u < DEC_MAXC / 16; ++u) mlq[u] = ml[q + 16 * u < count ? q + 16 * u : 0];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int cc = c < count ? c : 0;
+            lo[c] = *reinterpret_cast<const float4*>(po0 + (int64_t)cc * D);
+            hi[c] = *reinterpret_cast<const float4*>(po0 + (int64_t)cc * D + 4);
+        }
+        float M = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < DEC_MAXC / 16; ++u) M = fmaxf(M, q + 16 * u < count ? mlq[u].x : -INFINITY);
+#pragma unroll
+        for (int off = 1; off < 16; off *= 2) M = fmaxf(M, __shfl_xor(M, off, ZI_WAVE));
+        // maxima are in base-2 units; a chunk without keys has maximum -inf and weight 0
+        float wq[DEC_MAXC / 16], lq[DEC_MAXC / 16];
+#pragma unroll
+        for (int u = 0; u < DEC_MAXC / 16; ++u) {
+            const bool use = q + 16 * u < count && mlq[u].x != -INFINITY;
+            wq[u] = use ? __builtin_amdgcn_exp2f(mlq[u].x - M) : 0.f;
+            lq[u] = use ? mlq[u].y : 0.f;
+        }
+        float L = 0.f;
+        const int lane0 = lane & ~15;
+#pragma unroll
+        for (int u = 0; u < DEC_MAXC / 16; ++u) {
+            if (u * 16 >= count) break;      // uniform over the token's lanes
+            for (int c0 = u * 16; c0 < u * 16 + 16 && c0 < count; c0 += 8) {
+                if (c0 > 0) {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) {
+                        const int cc = c0 + c < count ? c0 + c : c0;
+                        lo[c] = *reinterpret_cast<const float4*>(po0 + (int64_t)cc * D);
+                        hi[c] = *reinterpret_cast<const float4*>(po0 + (int64_t)cc * D + 4);
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < 8; ++c) {
+                    const int src = lane0 + ((c0 + c) & 15);
+                    const float wc = __shfl(wq[u], src, ZI_WAVE);     // 0 for chunks past the count
+                    L += wc * __shfl(lq[u], src, ZI_WAVE);
+                    v[0] += wc * lo[c].x; v[1] += wc * lo[c].y; v[2] += wc * lo[c].z; v[3] += wc * lo[c].w;
+                    v[4] += wc * hi[c].x; v[5] += wc * hi[c].y; v[6] += wc * hi[c].z; v[7] += wc * hi[c].w;
+                }
+            }
+        }
+        {
+            const float inv = count > max_chunks ? NAN : 1.f / L;      // chunks the launch did not cover: it shows
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] *= inv;
+        }
+#pragma unroll
+        for (int dk = 0; dk < DK; ++dk) {     // the padding of the last k-step is zero on both sides
+            const unsigned keep = dk * 32 + j * 8 < D ? ~0u : 0u;
+            a[dk].u.x &= keep; a[dk].u.y &= keep; a[dk].u.z &= keep; a[dk].u.w &= keep;
+        }
+        if (h > h0) __syncthreads();        // the last head's operands have been read
+        if (d0 < DK * 32) {
+            uint4 u;
+            u.x = zi_pack_bf16x2(v[0], v[1]); u.y = zi_pack_bf16x2(v[2], v[3]);
+            u.z = zi_pack_bf16x2(v[4], v[5]); u.w = zi_pack_bf16x2(v[6], v[7]);
+            if (mt >= n || d0 >= D) u = make_uint4(0, 0, 0, 0);
+            *reinterpret_cast<uint4*>(&sx[mt][d0]) = u;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int dk = 0; dk < DK; ++dk) {
+            dec_pack b;
+            b.u = *reinterpret_cast<const uint4*>(&sx[r][dk * 32 + j * 8]);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[dk].b, b.b, acc, 0, 0, 0);
+        }
+    }
+    // lane (r, j) holds rows 4j .. 4j+3 of its wavefront's tile for token r
+    if (r < n) {
+        const int row0 = blockIdx.x * DPJ_ROWS + wave * 16 + j * 4;
+        float* dst = sums + ((int64_t)split * n + r) * N + row0;
+        if ((N & 3) == 0 && row0 + 3 < N) {
+            *reinterpret_cast<dec_f32x4_t*>(dst) = acc;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (row0 + e < N) dst[e] = acc[e];
+        }
+    }
+}
+
 // Floats of workspace the split kernel needs for n tokens.
 extern "C" int64_t zi_attention_decode_workspace(int n, int nh, int d) {
     return (int64_t)n * nh * DEC_MAXC * (d + 2);
@@ -529,14 +662,16 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
                "page size %% 8 == 0): dtype %d heads %d kv_heads %d head_dim %d page %d", who, dt, nh, nkv, d, page_size);
     ZI_REQUIRE(n_idx >= 0 && max_pages > 0 && num_pages > 0 && window >= 0, "%s: bad sizes", who);
     ZI_REQUIRE(max_chunks >= 1 && max_chunks <= DEC_MAXC, "%s: max_chunks %d outside 1..%d", who, max_chunks, DEC_MAXC);
-    ZI_REQUIRE(ldo >= (int64_t)nh * d && ldo % 4 == 0 && (pj || (ldq >= (int64_t)nh * d && ldq % 8 == 0)),
+    const int leave_parts = out == nullptr;     // the chunks stay in the workspace for zi_attention_decode_project
+    ZI_REQUIRE((leave_parts || (ldo >= (int64_t)nh * d && ldo % 4 == 0)) && (pj || (ldq >= (int64_t)nh * d && ldq % 8 == 0)),
                "%s: bad row stride", who);
     ZI_REQUIRE((pj || ((uintptr_t)q % 16) == 0) && ((uintptr_t)out % 8) == 0 && ((uintptr_t)kcache % 16) == 0 &&
                    ((uintptr_t)vcache % 16) == 0,
                "%s: q, out and the caches must be aligned to 16 bytes", who);
     ZI_REQUIRE(nkv <= 65535 && nh <= 65535, "%s: too many heads", who);
     if (n_idx == 0) return 0;
-    ZI_REQUIRE(max_chunks == 1 || (workspace && workspace_floats >= zi_attention_decode_workspace(n_idx, nh, d) &&
+    ZI_REQUIRE((max_chunks == 1 && !leave_parts) ||
+                   (workspace && workspace_floats >= zi_attention_decode_workspace(n_idx, nh, d) &&
                                    ((uintptr_t)workspace % 16) == 0),
                "%s: workspace of %lld floats is too small or not aligned", who, (long long)workspace_floats);
     float* po = workspace;
@@ -549,12 +684,12 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
         attention_decode_kernel<DD, true><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
-            max_chunks, *pj);                                                                                        \
+            max_chunks, leave_parts, *pj);                                                                                      \
     else                                                                                                             \
         attention_decode_kernel<DD, false><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
-            max_chunks, none)
+            max_chunks, leave_parts, none)
     switch (d) {
         case 16: ZI_DEC(16); break;
         case 32: ZI_DEC(32); break;
@@ -566,7 +701,7 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
         default: ZI_DEC(128); break;
     }
 #undef ZI_DEC
-    if (max_chunks > 1)
+    if (max_chunks > 1 && !leave_parts)
         attention_decode_merge_kernel<<<dim3(n_idx, nh), ZI_WAVE, 0, stream>>>((zi_bf16*)out, ldo, po, pml, tok_index,
                                                                               tok_pos, nh, d, window, max_chunks);
     return zi_check_launch(who);
@@ -624,4 +759,53 @@ extern "C" int zi_attention_decode_fused(void* out, int dt, int n_idx, int64_t l
     return dec_launch("attention_decode_fused", out, nullptr, dt, n_idx, 0, ldo, kcache, vcache, tok_index, tok_seq,
                       tok_pos, block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks,
                       workspace, workspace_floats, &pj, stream);
+}
+
+// Heads whose merged attention one workgroup of the projection multiplies (one partial sum for each
+// such group): as few as keep the partial sums at 16 or fewer.
+extern "C" int zi_attention_decode_project_heads(int nh) { return nh <= 16 ? 1 : (nh + 15) / 16; }
+
+// 1 when zi_attention_decode_project takes the shape, else 0 (then: merge into `out` and multiply).
+extern "C" int zi_attention_decode_project_supported(int dt, int n, int nh, int d, int64_t ldw) {
+    return dt == ZI_BF16 && n >= 1 && n <= 16 && nh >= 1 && d >= 16 && d <= 128 && d % 16 == 0 && ldw % 8 == 0 &&
+           ldw >= (int64_t)nh * d;
+}
+
+// The output projection of n <= 16 decoded tokens read from the chunks that zi_attention_decode(_fused)
+// left in `workspace` when it was called with out == nullptr for the same n, nh, d, tok_pos, window and
+// max_chunks (and without tok_index): sums[s][t][:] = W[:, columns of the heads of group s] . attention
+// of token t, float32, s < ceil(nh / zi_attention_decode_project_heads(nh)), rows of `sums` N long.
+// W is [N, nh * d] bfloat16 with row stride ldw.
+extern "C" int zi_attention_decode_project(float* sums, const float* workspace, int64_t workspace_floats, int n,
+                                           const int32_t* tok_pos, int window, int max_chunks, const void* w, int dt,
+                                           int64_t ldw, int N, int nh, int d, hipStream_t stream) {
+    ZI_REQUIRE(zi_attention_decode_project_supported(dt, n, nh, d, ldw),
+               "attention_decode_project: unsupported shape (bfloat16, 1..16 tokens, head_dim a multiple of 16 up to "
+               "128, row stride a multiple of 8): dtype %d tokens %d heads %d head_dim %d stride %lld", dt, n, nh, d,
+               (long long)ldw);
+    ZI_REQUIRE(N >= 1 && window >= 0 && max_chunks >= 1 && max_chunks <= DEC_MAXC, "attention_decode_project: bad sizes");
+    ZI_REQUIRE(sums && tok_pos && w && ((uintptr_t)sums % 16) == 0 && ((uintptr_t)w % 16) == 0,
+               "attention_decode_project: sums and weights must be aligned to 16 bytes");
+    ZI_REQUIRE(workspace && workspace_floats >= zi_attention_decode_workspace(n, nh, d) && ((uintptr_t)workspace % 16) == 0,
+               "attention_decode_project: workspace of %lld floats is too small or not aligned", (long long)workspace_floats);
+    const float* po = workspace;
+    const float* pml = workspace + (int64_t)n * nh * DEC_MAXC * d;
+    const int hg = zi_attention_decode_project_heads(nh);
+    const dim3 grid((N + DPJ_ROWS - 1) / DPJ_ROWS, (nh + hg - 1) / hg);
+    ZI_REQUIRE(grid.y <= 65535, "attention_decode_project: too many heads");
+#define ZI_DPJ(DD)                                                                                                    \
+    attention_decode_project_kernel<DD><<<grid, 256, 0, stream>>>(sums, po, pml, tok_pos, n, nh, window, max_chunks,   \
+                                                                  (const zi_bf16*)w, ldw, N, hg)
+    switch (d) {
+        case 16: ZI_DPJ(16); break;
+        case 32: ZI_DPJ(32); break;
+        case 48: ZI_DPJ(48); break;
+        case 64: ZI_DPJ(64); break;
+        case 80: ZI_DPJ(80); break;
+        case 96: ZI_DPJ(96); break;
+        case 112: ZI_DPJ(112); break;
+        default: ZI_DPJ(128); break;
+    }
+#undef ZI_DPJ
+    return zi_check_launch("attention_decode_project");
 }

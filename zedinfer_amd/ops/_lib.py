@@ -31,6 +31,9 @@ _PROTOTYPES = {
     "zi_attention_decode_fused": [P, I, I, L, P, I, L, L, P, I, P, I, P, L, I, P, P, P, P, P, P, I, I, I, I, I, I, I, F,
                                   I, P, L, P],
     "zi_attention_decode_fused_supported": [I, I, I, I, I, I, I, L, L],
+    "zi_attention_decode_project": [P, P, L, I, P, I, I, P, I, L, I, I, I, P],
+    "zi_attention_decode_project_supported": [I, I, I, I, L],
+    "zi_attention_decode_project_heads": [I],
     "zi_rope_table": [P, P, P, I, I, P],
     "zi_attention_decode_chunks": [I],
     "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, P],

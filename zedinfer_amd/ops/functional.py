@@ -425,7 +425,8 @@ def attention_decode_fused(sums: torch.Tensor, bias: Optional[torch.Tensor], tab
                            slots: Optional[torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
                            tok_seq: torch.Tensor, tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int,
                            d: int, scale: float, max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
-                           workspace: Optional[torch.Tensor] = None, write_kv: bool = True) -> torch.Tensor:
+                           workspace: Optional[torch.Tensor] = None, write_kv: bool = True,
+                           leave_chunks: bool = False) -> torch.Tensor:
     """Rotation, cache store and attention of single decoded tokens in one kernel.
 
     ``sums`` [S, n, nh*d + 2*nkv*d] float32 are the partial sums of the fused q/k/v projection of the
@@ -433,7 +434,9 @@ def attention_decode_fused(sums: torch.Tensor, bias: Optional[torch.Tensor], tab
     dims of every query and key head turn by the angles of ``table`` ([n, pairs, 2] from ``rope_table``;
     None: no rotation).  With ``write_kv`` each token's new key and value go to slot ``slots[t]`` of the
     cache.  Every token must be the only one of its sequence in the call.  Same shapes as
-    ``attention_decode``; the result is what rope_kv_store_sums followed by attention_decode gives."""
+    ``attention_decode``; the result is what rope_kv_store_sums followed by attention_decode gives.
+    With ``leave_chunks`` the chunks of the keys are not merged: they stay in ``workspace`` (which is
+    returned) for ``attention_decode_project``, and ``out`` is not written."""
     _gpu("attention_decode_fused", sums, bias, table, slots, kcache, vcache, tok_seq, tok_pos, block_tables, out,
          workspace)
     if sums.dim() != 3 or sums.dtype != torch.float32 or not sums.is_contiguous():
@@ -459,25 +462,70 @@ def attention_decode_fused(sums: torch.Tensor, bias: Optional[torch.Tensor], tab
                 or not table.is_contiguous():
             raise ValueError(f"attention_decode_fused: table must be a contiguous float32 [{n}, pairs, 2] tensor")
         rot = 2 * table.shape[1]
-    if out is None:
-        out = torch.empty((n, nh * d), dtype=kcache.dtype, device=sums.device)
-    ldo, wo = _rows(out, "attention_decode_fused out")
-    if tuple(out.shape) != (n, nh * d) or out.dtype != kcache.dtype:
-        raise ValueError("attention_decode_fused: out has the wrong shape or dtype")
+    ldo = 0
+    if leave_chunks:
+        out = None
+    else:
+        if out is None:
+            out = torch.empty((n, nh * d), dtype=kcache.dtype, device=sums.device)
+        ldo, wo = _rows(out, "attention_decode_fused out")
+        if tuple(out.shape) != (n, nh * d) or out.dtype != kcache.dtype:
+            raise ValueError("attention_decode_fused: out has the wrong shape or dtype")
     if window > 0:
         max_keys = min(max_keys, window)
     max_chunks = int(_lib.load().zi_attention_decode_chunks(int(max_keys)))
     need = attention_decode_workspace(n, nh, d)
-    if max_chunks > 1:
+    if max_chunks > 1 or leave_chunks:
         if workspace is None:
             workspace = torch.empty((need,), dtype=torch.float32, device=sums.device)
         if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
             raise ValueError(f"attention_decode_fused: workspace must be a contiguous float32 buffer of {need} entries")
-    _lib.call("zi_attention_decode_fused", _p(out), _code(out, "attention_decode_fused"), n, ldo, _p(sums), S,
+    _lib.call("zi_attention_decode_fused", _p(out), _code(kcache, "attention_decode_fused"), n, ldo, _p(sums), S,
               n * width, width, _p(bias), _code(bias, "attention_decode_fused bias") if bias is not None else F32,
               _p(table), rot, _p(slots), pages * ps, int(write_kv), _p(kcache), _p(vcache), _p(None), _p(tok_seq),
               _p(tok_pos), _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale),
               max_chunks, _p(workspace), workspace.numel() if workspace is not None else 0, _stream())
+    return workspace if leave_chunks else out
+
+
+def attention_decode_project_supported(weight: torch.Tensor, n: int, nh: int, d: int) -> bool:
+    """Whether ``attention_decode_project`` multiplies ``weight`` [N, nh*d] with n tokens' chunks."""
+    if weight.dtype not in _CODES or weight.dim() != 2 or weight.stride(1) != 1 or weight.shape[1] != nh * d:
+        return False
+    return bool(_lib.load().zi_attention_decode_project_supported(_CODES[weight.dtype], n, nh, d, weight.stride(0)))
+
+
+def attention_decode_project_splits(nh: int) -> int:
+    """Partial sums ``attention_decode_project`` leaves: one for each group of heads."""
+    hg = int(_lib.load().zi_attention_decode_project_heads(nh))
+    return -(-nh // hg)
+
+
+def attention_decode_project(workspace: torch.Tensor, weight: torch.Tensor, tok_pos: torch.Tensor, nh: int, d: int,
+                             max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The output projection of decoded tokens straight from the chunks that ``attention_decode_fused(...,
+    leave_chunks=True)`` left in ``workspace`` (same tokens, heads, ``max_keys`` and ``window``): float32
+    partial sums [splits, n, N] over groups of heads, to be added in rising order.  ``weight`` is [N, nh*d]."""
+    _gpu("attention_decode_project", workspace, weight, tok_pos, out)
+    n = tok_pos.numel()
+    _i32(tok_pos, "attention_decode_project tok_pos", n)
+    if not attention_decode_project_supported(weight, n, nh, d):
+        raise ValueError(f"attention_decode_project: unsupported shape: {n} tokens, {nh} heads of {d}, weight "
+                         f"{tuple(weight.shape)} {weight.dtype}")
+    N = weight.shape[0]
+    S = attention_decode_project_splits(nh)
+    if out is None:
+        out = torch.empty((S, n, N), dtype=torch.float32, device=weight.device)
+    if tuple(out.shape) != (S, n, N) or out.dtype != torch.float32 or not out.is_contiguous():
+        raise ValueError(f"attention_decode_project: out must be a contiguous float32 [{S}, {n}, {N}] tensor")
+    need = attention_decode_workspace(n, nh, d)
+    if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
+        raise ValueError(f"attention_decode_project: workspace must be a contiguous float32 buffer of {need} entries")
+    if window > 0:
+        max_keys = min(max_keys, window)
+    max_chunks = int(_lib.load().zi_attention_decode_chunks(int(max_keys)))
+    _lib.call("zi_attention_decode_project", _p(out), _p(workspace), workspace.numel(), n, _p(tok_pos), int(window),
+              max_chunks, _p(weight), _code(weight, "attention_decode_project"), weight.stride(0), N, nh, d, _stream())
     return out
 
 

@@ -31,6 +31,9 @@ class Attention(Mixer):
     # 256 keys), which costs more than the separate rotary kernel once many tokens decode together:
     # measured faster at 1 and 8 tokens, slower at 64.
     FUSED_DECODE_MAX_TOKENS = 16
+    # The one-kernel decode path leaves its chunks unmerged and the output projection merges them as it
+    # loads its operand: one launch less a layer.
+    PROJECT_FROM_CHUNKS = True
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -110,9 +113,9 @@ class Attention(Mixer):
             S = ops.linear_splits(n, self.qkv.shape[0], self.hidden)
             sums = self.rt.buffer("attn_qkv_sums", (S, n, self.qd + 2 * self.kvd), torch.float32)
             ops.linear_sums(x, self.qkv, out=sums)
-            att = self.rt.buffer("attn_out", (n, self.qd))
-            if self.attend_from_sums(sums, att, batch, view, memory):
-                return self.project(att, n)
+            out = self.decode_from_sums(sums, batch, view, memory)
+            if out is not None:
+                return out
             q = self.rt.buffer("attn_q", (n, self.qd))
             self.position.rotate_and_store_sums(sums, self.bias, q, batch.positions, view.slots, memory, self.nh,
                                                 self.nkv, self.d)
@@ -136,23 +139,31 @@ class Attention(Mixer):
         out = self.rt.buffer("attn_proj", (n, self.hidden))
         return ops.linear(att, self.o, out=out)
 
-    def attend_from_sums(self, sums, att, batch, view, memory: LayerMemory) -> bool:
+    def decode_from_sums(self, sums, batch, view, memory: LayerMemory) -> Optional[torch.Tensor]:
         """A pure decode step (one token a sequence): rotation, cache store and attention in one kernel,
         when the position encoding is a rotation it can hand over as a table of angles (or nothing) and
-        the kernel takes the shape.  False: nothing was done."""
+        the kernel takes the shape; then the output projection, read straight from the attention's
+        chunks over the keys where that kernel takes the shape.  None: nothing was done."""
         if not batch.single_tokens or batch.num_tokens > self.FUSED_DECODE_MAX_TOKENS:
-            return False
+            return None
         table = self.position.step_table(batch)
         if table is None:
-            return False
+            return None
         rot = 0 if isinstance(table, str) else 2 * table.shape[1]
         S, n, width = sums.shape
         ps = memory.k.shape[2]
         if not ops.attention_decode_fused_supported(memory.k.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
-            return False
+            return None
         ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
-        ops.attention_decode_fused(sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None,
-                                   memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh,
-                                   self.nkv, self.d, self.scale, batch.max_short_keys, self.window, out=att,
-                                   workspace=ws, write_kv=memory.writes)
-        return True
+        args = (sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None, memory.k, memory.v,
+                batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale,
+                batch.max_short_keys, self.window)
+        if self.PROJECT_FROM_CHUNKS and ops.attention_decode_project_supported(self.o, n, self.nh, self.d):
+            ops.attention_decode_fused(*args, workspace=ws, write_kv=memory.writes, leave_chunks=True)
+            out = self.rt.buffer("attn_proj_heads", (ops.attention_decode_project_splits(self.nh), n, self.hidden),
+                                 torch.float32)
+            return ops.attention_decode_project(ws, self.o, batch.positions, self.nh, self.d, batch.max_short_keys,
+                                                self.window, out=out)
+        att = self.rt.buffer("attn_out", (n, self.qd))
+        ops.attention_decode_fused(*args, out=att, workspace=ws, write_kv=memory.writes)
+        return self.project(att, n)
