@@ -386,6 +386,12 @@ def test_attention_decode_fused(ops, nh, nkv, d, ps, lens, window, S, bias_dtype
     out = ops.attention_decode_fused(sums, bias, table, slots, kc2, vc2, seq, pos, bt, nh, nkv, d, scale, T, window)
     assert not torch.isnan(out).any()
     torch.testing.assert_close(out.float(), ref.float(), atol=4e-3, rtol=1e-2)
+    # token t is of sequence t: the same without the list of sequences
+    kc4, vc4 = kc.clone(), vc.clone()
+    out4 = ops.attention_decode_fused(sums, bias, table, slots, kc4, vc4, None, pos, bt, nh, nkv, d, scale, T, window)
+    assert torch.equal(out4, out)
+    assert bool(((kc4 == kc2) | (torch.isnan(kc4) & torch.isnan(kc2))).all())
+    assert bool(((vc4 == vc2) | (torch.isnan(vc4) & torch.isnan(vc2))).all())
     for b in range(B):
         pg, o = int(slots[b]) // ps, int(slots[b]) % ps
         torch.testing.assert_close(kc2[pg, :, o].float(), kc1[pg, :, o].float(), atol=1e-3, rtol=8e-3)

@@ -110,7 +110,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         return;
     }
     if (chunk >= sp.count) return;
-    const int32_t* bt = block_tables + (int64_t)tok_seq[t] * max_pages;
+    const int32_t* bt = block_tables + (int64_t)(tok_seq ? tok_seq[t] : t) * max_pages;   // no list: token t is of sequence t
     const int ps_shift = (ps & (ps - 1)) == 0 ? __ffs(ps) - 1 : -1;   // no division for the usual page sizes
     const int quarter = sp.len / DEC_WAVES;
     const int k_begin = sp.lo_al + chunk * sp.len + wave * quarter;
@@ -733,6 +733,9 @@ extern "C" int zi_attention_decode_fused_supported(int dt, int nh, int nkv, int 
 // `write_kv`.  Every token must be the only one of its sequence in the call: a token's keys must not be
 // written by another token of the same call.  `table` holds cos and sin per (token, pair), from
 // zi_rope_table; `dt` is the type of the caches and of out; `bias` is bfloat16 or float32 (bias_dt).
+// `tok_seq` may be null (here and in zi_attention_decode): token t is then of sequence t, row t of
+// block_tables.  With out == nullptr the chunks stay unmerged in the workspace for
+// zi_attention_decode_project.
 extern "C" int zi_attention_decode_fused(void* out, int dt, int n_idx, int64_t ldo, const float* sums, int splits,
                                          int64_t split_stride, int64_t ldp, const void* bias, int bias_dt,
                                          const float* table, int rot, const int32_t* slots, int64_t cache_slots,

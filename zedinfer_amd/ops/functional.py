@@ -423,7 +423,7 @@ def attention_decode_fused_supported(dtype: torch.dtype, nh: int, nkv: int, d: i
 
 def attention_decode_fused(sums: torch.Tensor, bias: Optional[torch.Tensor], table: Optional[torch.Tensor],
                            slots: Optional[torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
-                           tok_seq: torch.Tensor, tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int,
+                           tok_seq: Optional[torch.Tensor], tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int,
                            d: int, scale: float, max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
                            workspace: Optional[torch.Tensor] = None, write_kv: bool = True,
                            leave_chunks: bool = False) -> torch.Tensor:
@@ -433,8 +433,9 @@ def attention_decode_fused(sums: torch.Tensor, bias: Optional[torch.Tensor], tab
     step's n tokens; splits are added in rising order, then ``bias``.  The first ``2 * table.shape[1]``
     dims of every query and key head turn by the angles of ``table`` ([n, pairs, 2] from ``rope_table``;
     None: no rotation).  With ``write_kv`` each token's new key and value go to slot ``slots[t]`` of the
-    cache.  Every token must be the only one of its sequence in the call.  Same shapes as
-    ``attention_decode``; the result is what rope_kv_store_sums followed by attention_decode gives.
+    cache.  Every token must be the only one of its sequence in the call; ``tok_seq`` None means that
+    token t is of sequence t (row t of ``block_tables``), which saves the kernel a dependent load.  Same shapes
+    as ``attention_decode``; the result is what rope_kv_store_sums followed by attention_decode gives.
     With ``leave_chunks`` the chunks of the keys are not merged: they stay in ``workspace`` (which is
     returned) for ``attention_decode_project``, and ``out`` is not written."""
     _gpu("attention_decode_fused", sums, bias, table, slots, kcache, vcache, tok_seq, tok_pos, block_tables, out,
@@ -450,12 +451,15 @@ def attention_decode_fused(sums: torch.Tensor, bias: Optional[torch.Tensor], tab
     if bias is not None and (bias.dim() != 1 or bias.numel() < need_w or not bias.is_contiguous()):
         raise ValueError(f"attention_decode_fused: bias must hold {need_w} values")
     pages, ps = _check_cache(kcache, vcache, nkv, d, kcache.dtype, "attention_decode_fused")
-    _i32(tok_seq, "attention_decode_fused tok_seq", n)
+    if tok_seq is not None:
+        _i32(tok_seq, "attention_decode_fused tok_seq", n)
     _i32(tok_pos, "attention_decode_fused tok_pos", n)
     if write_kv:
         _i32(slots, "attention_decode_fused slots", n)
     if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
         raise ValueError("attention_decode_fused: block_tables must be a contiguous int32 [seqs, max_pages] tensor")
+    if tok_seq is None and block_tables.shape[0] < n:
+        raise ValueError(f"attention_decode_fused: {n} tokens without tok_seq need {n} rows of block_tables")
     rot = 0
     if table is not None:
         if table.dim() != 3 or table.shape[0] != n or table.shape[2] != 2 or table.dtype != torch.float32 \

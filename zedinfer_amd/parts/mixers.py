@@ -155,8 +155,9 @@ class Attention(Mixer):
         if not ops.attention_decode_fused_supported(memory.k.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
             return None
         ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
+        # every entry brings one token: token t is of entry t
         args = (sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None, memory.k, memory.v,
-                batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale,
+                None, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale,
                 batch.max_short_keys, self.window)
         if self.PROJECT_FROM_CHUNKS and ops.attention_decode_project_supported(self.o, n, self.nh, self.d):
             ops.attention_decode_fused(*args, workspace=ws, write_kv=memory.writes, leave_chunks=True)
