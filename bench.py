@@ -26,6 +26,14 @@ SHAPE = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", hidden_size
              vocab_size=151936, max_position_embeddings=32768, num_hidden_layers=28, num_attention_heads=12,
              num_key_value_heads=2, head_dim=128, rope_theta=1000000.0, rms_norm_eps=1e-6,
              tie_word_embeddings=True, use_sliding_window=False, torch_dtype="bfloat16")
+# Other shapes of the same architecture, for measurements beside the headline (--shape)
+SHAPES = {
+    "1.5B": {},
+    "7B": dict(hidden_size=3584, intermediate_size=18944, vocab_size=152064, num_hidden_layers=28,
+               num_attention_heads=28, num_key_value_heads=4, tie_word_embeddings=False),
+    "32B": dict(hidden_size=5120, intermediate_size=27648, vocab_size=152064, num_hidden_layers=64,
+                num_attention_heads=40, num_key_value_heads=8, tie_word_embeddings=False),
+}
 FULL_LAYERS = 28
 PROMPT = 2048
 CONTEXT = 4096
@@ -45,6 +53,7 @@ def decode_bytes(c, layers, batch, ctx_tokens_total, el):
     H = c["hidden_size"]
     qd, kvd = c["num_attention_heads"] * c["head_dim"], c["num_key_value_heads"] * c["head_dim"]
     per_layer = matmul_params_per_layer(c) + (qd + 2 * kvd) + 2 * H
+    # the output head is read once; an untied input table is only gathered from
     weights = (layers * per_layer + c["vocab_size"] * H + H) * el
     kv = ctx_tokens_total * 2 * layers * kvd * el
     return weights + kv
@@ -119,6 +128,7 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--shape", default="1.5B", choices=sorted(SHAPES), help="layer sizes of Qwen2.5-<shape>")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
@@ -131,7 +141,11 @@ def main():
     from zedinfer_amd.config import Qwen2Config, SchedulerConfig
     from zedinfer_amd.engine import Engine
 
-    shape = dict(SHAPE, num_hidden_layers=args.layers)
+    full_layers = SHAPES[args.shape].get("num_hidden_layers", FULL_LAYERS)
+    if args.layers == FULL_LAYERS and args.shape != "1.5B":
+        args.layers = full_layers
+    shape = dict(SHAPE, **SHAPES[args.shape])
+    shape["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(shape)
     el = 2 if args.dtype == "bf16" else 4
     weights_cache = {}
@@ -160,15 +174,15 @@ def main():
     need = decode_bytes(shape, args.layers, args.batch, ctx_mid, el)
     achieved = need / (ms_step / 1000.0) / 1e9
     out = {
-        "metric": "decode tok/s at batch 8, 2,048-token prompts (Qwen2.5-1.5B shape)",
+        "metric": f"decode tok/s at batch {args.batch}, 2,048-token prompts (Qwen2.5-{args.shape} shape)",
         "value": round(tps, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: seeded random weights, seeded uniform-random token ids",
-        "config": {"model": "Qwen2.5-1.5B shape", "global_batch": args.batch, "seq_len": PROMPT,
-                   "context_len": CONTEXT, "parallelism": "single GPU", "num_layers": FULL_LAYERS,
+        "config": {"model": f"Qwen2.5-{args.shape} shape", "global_batch": args.batch, "seq_len": PROMPT,
+                   "context_len": CONTEXT, "parallelism": "single GPU", "num_layers": full_layers,
                    "layers_run": args.layers, "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
-                   "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": True,
+                   "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": bool(shape["tie_word_embeddings"]),
                    "kv_page_tokens": 16, "sampling": "greedy"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},

@@ -32,8 +32,10 @@ class Attention(Mixer):
     # measured faster at 1 and 8 tokens, slower at 64.
     FUSED_DECODE_MAX_TOKENS = 16
     # The one-kernel decode path leaves its chunks unmerged and the output projection merges them as it
-    # loads its operand: one launch less a layer.
-    PROJECT_FROM_CHUNKS = True
+    # loads its operand: one launch less a layer.  That kernel does not stream a large weight as well as
+    # the plain product does (measured: 6.9 against 4.4 + 3.7 us with 4.7 MB of weight, 31.7 against
+    # about 16 us with 52 MB), so it is taken for small output weights only.
+    PROJECT_FROM_CHUNKS_MAX_BYTES = 8 << 20
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -159,7 +161,8 @@ class Attention(Mixer):
         args = (sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None, memory.k, memory.v,
                 None, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale,
                 batch.max_short_keys, self.window)
-        if self.PROJECT_FROM_CHUNKS and ops.attention_decode_project_supported(self.o, n, self.nh, self.d):
+        if (self.o.numel() * self.o.element_size() <= self.PROJECT_FROM_CHUNKS_MAX_BYTES
+                and ops.attention_decode_project_supported(self.o, n, self.nh, self.d)):
             ops.attention_decode_fused(*args, workspace=ws, write_kv=memory.writes, leave_chunks=True)
             out = self.rt.buffer("attn_proj_heads", (ops.attention_decode_project_splits(self.nh), n, self.hidden),
                                  torch.float32)
