@@ -295,3 +295,21 @@ def test_token_computed_for_a_request_that_ended_is_dropped():
     c.check()
     nxt = s.schedule()
     assert nxt.decode_requests == [b]
+
+
+def test_token_computed_ahead_for_a_cancelled_request_is_dropped():
+    s, c = make()
+    a, b = req(5, max_new=6), req(3, max_new=6)
+    s.submit(a)
+    s.submit(b)
+    first = s.schedule()
+    commit(c, first)
+    ahead = s.schedule_ahead(first)
+    commit(c, ahead)
+    s.process_results(first, [7, 8])
+    a.cancelled = True                                  # for instance from its stream callback
+    s.process_results(ahead, [9, 10])
+    assert a.output_ids == [7] and b.output_ids == [8, 10]
+    nxt = s.schedule()                                  # the ordinary schedule ends it
+    assert a.done and a.finish_reason == "stop" and a.result.output_ids == [7] and nxt.decode_requests == [b]
+    c.check()

@@ -239,8 +239,8 @@ class Scheduler:
             raise ValueError(f"{len(tokens)} tokens for {len(sampled)} sampled requests")
         with self._lock:
             for req, tok in zip(sampled, tokens):
-                if req.done:
-                    continue            # it ended while this step, scheduled ahead, was running
+                if req.done or (batch.tokens_on_device and req.cancelled):
+                    continue            # it ended, or was cancelled, while this step, scheduled ahead, was running
                 tok = int(tok)
                 first = req.phase != RequestPhase.DECODE
                 req.phase = RequestPhase.DECODE
