@@ -2,6 +2,8 @@
 """The headline benchmark: decode tokens a second of the Qwen2.5-1.5B shape on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py --shape 7B --mix 64                    (continuous batching of 64 requests)
+    python bench.py --shape 32B --prompt-len 8192 --prefill-len 16384 --steps 32 --warmup 8
 
 A step is one decode step of the serving loop (schedule, model, sampling) with ``batch`` running
 requests that each hold a 2,048-token prompt.  Prints ONE JSON line.  Besides the decode speed it
@@ -69,15 +71,16 @@ def rand_ids(rng, n, vocab):
     return [rng.randrange(100, vocab - 100) for _ in range(n)]
 
 
-def measure_decode(engine_factory, batch, steps, warmup, vocab):
-    """tokens a second and ms a step of `steps` decode steps with `batch` running requests."""
+def measure_decode(engine_factory, batch, steps, warmup, vocab, prompt_len=PROMPT):
+    """tokens a second and ms a step of `steps` decode steps with `batch` running requests that each
+    hold a prompt of `prompt_len` tokens."""
     import torch
     from zedinfer_amd import GenerationConfig, InferenceRequest
     from zedinfer_amd.engine import InferenceEngine
     ie = InferenceEngine(engine_factory())
     loop = ie.serving_loop()
     rng = random.Random(1234 + batch)
-    reqs = [loop.submit_async(InferenceRequest(rand_ids(rng, PROMPT, vocab),
+    reqs = [loop.submit_async(InferenceRequest(rand_ids(rng, prompt_len, vocab),
                                                GenerationConfig(max_new_tokens=warmup + steps + 2 * batch + 8,
                                                                 ignore_eos=True)))
             for _ in range(batch)]
@@ -101,7 +104,32 @@ def measure_decode(engine_factory, batch, steps, warmup, vocab):
     return batch * steps / dt, dt / steps * 1000.0, (ctx0 + ctx1) / 2.0
 
 
-def measure_prefill(engine_factory, vocab, rounds=3):
+def measure_mix(engine_factory, requests, vocab, new_tokens=256, lo=128, hi=4096):
+    """Continuous batching: `requests` prompts of lengths uniform in [lo, hi], all queued at once,
+    `new_tokens` greedy tokens each; generated tokens a second over the whole run, prompt tokens a
+    second, and the wall time (reference: examples/batch_bench.cpp:168-171)."""
+    import torch
+    from zedinfer_amd import GenerationConfig, InferenceRequest
+    from zedinfer_amd.engine import InferenceEngine
+    ie = InferenceEngine(engine_factory())
+    loop = ie.serving_loop()
+    rng = random.Random(4321)
+    warm = loop.submit_async(InferenceRequest(rand_ids(rng, hi, vocab), GenerationConfig(max_new_tokens=8, ignore_eos=True)))
+    loop.run_loop()
+    assert not warm.error, warm.error
+    lens = [rng.randint(lo, hi) for _ in range(requests)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    reqs = [loop.submit_async(InferenceRequest(rand_ids(rng, n, vocab),
+                                               GenerationConfig(max_new_tokens=new_tokens, ignore_eos=True))) for n in lens]
+    loop.run_loop()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert all(not r.error and len(r.output_ids) == new_tokens for r in reqs), [r.error for r in reqs if r.error][:1]
+    return requests * new_tokens / dt, sum(lens) / dt, dt, sum(lens)
+
+
+def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT):
     import torch
     from zedinfer_amd import ops
     from zedinfer_amd.engine import StepEntry
@@ -109,11 +137,11 @@ def measure_prefill(engine_factory, vocab, rounds=3):
     rng = random.Random(77)
     times = []
     for i in range(rounds + 1):
-        seq = eng.open(("prefill", i), PROMPT)
-        ids = rand_ids(rng, PROMPT, vocab)
+        seq = eng.open(("prefill", i), tokens)
+        ids = rand_ids(rng, tokens, vocab)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        logits = eng.step([StepEntry(seq, ids, [PROMPT - 1])], copy=False)
+        logits = eng.step([StepEntry(seq, ids, [tokens - 1])], copy=False)
         ops.argmax(logits).tolist()
         times.append(time.perf_counter() - t0)
         eng.close(seq)
@@ -129,6 +157,11 @@ def main():
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the model has (reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--shape", default="1.5B", choices=sorted(SHAPES), help="layer sizes of Qwen2.5-<shape>")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT, help="tokens every decoding request holds at the start")
+    ap.add_argument("--prefill-len", type=int, default=PROMPT, help="tokens of the timed prefill")
+    ap.add_argument("--mix", type=int, default=0, metavar="R",
+                    help="instead: continuous batching of R requests, prompts uniform in [128, 4096], 256 greedy "
+                         "tokens each, prompts cut at 2,048 tokens a step")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
@@ -150,11 +183,14 @@ def main():
     el = 2 if args.dtype == "bf16" else 4
     weights_cache = {}
 
-    def factory(batch):
+    def factory(batch, prompt=args.prompt_len):
         def make():
-            pages = batch * (CONTEXT // 16) + 16
+            context = max(CONTEXT, 2 * prompt)
+            # pages for what the requests will hold, not for the whole context: 64 long requests must fit
+            tokens = min(context, prompt + args.warmup + args.steps + 2 * batch + 64)
+            pages = batch * (-(-tokens // 16)) + 16
             sched = SchedulerConfig(num_kv_blocks=pages, kv_block_size=16, max_batch_requests=max(batch, 1),
-                                    max_batch_tokens=PROMPT + batch, max_prefill_tokens=PROMPT, max_seq_len=CONTEXT)
+                                    max_batch_tokens=prompt + batch, max_prefill_tokens=prompt, max_seq_len=context)
             if "w" not in weights_cache:
                 e = Engine.from_config(cfg, "Qwen2ForCausalLM", args.dtype, seed=0, sched=sched)
                 weights_cache["w"] = e
@@ -164,22 +200,35 @@ def main():
         return make
 
     V = cfg.vocab_size
+    PF = args.prefill_len
+    if args.mix:
+        def mix_engine():
+            sched = SchedulerConfig(num_kv_blocks=args.mix * (-(-(4096 + 256 + 64) // 16)) + 16, kv_block_size=16,
+                                    max_batch_requests=args.mix, max_batch_tokens=2048 + args.mix,
+                                    max_prefill_tokens=2048, max_seq_len=8192)
+            return Engine.from_config(cfg, "Qwen2ForCausalLM", args.dtype, seed=0, sched=sched)
+        gen, pre, secs, ptoks = measure_mix(mix_engine, args.mix, V)
+        print(json.dumps({"metric": f"continuous batching, generated tok/s (Qwen2.5-{args.shape} shape)",
+                          "value": round(gen, 1), "unit": "tok/s", "requests": args.mix, "prompt_tokens": ptoks,
+                          "new_tokens_each": 256, "seconds": round(secs, 3), "prompt_tok_s": round(pre, 1),
+                          "dtype": args.dtype, "layers_run": args.layers, "num_layers": full_layers}))
+        return 0
     if args.prefill_only:
-        pms = measure_prefill(factory(1), V)
-        fl = prefill_flops(shape, args.layers, PROMPT)
-        print(json.dumps({"prefill": {"value": round(PROMPT / pms * 1000.0, 1), "tokens": PROMPT, "ms": round(pms, 3),
+        pms = measure_prefill(factory(1, PF), V, tokens=PF)
+        fl = prefill_flops(shape, args.layers, PF)
+        print(json.dumps({"prefill": {"value": round(PF / pms * 1000.0, 1), "tokens": PF, "ms": round(pms, 3),
                                       "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}}))
         return 0
-    tps, ms_step, ctx_mid = measure_decode(factory(args.batch), args.batch, args.steps, args.warmup, V)
+    tps, ms_step, ctx_mid = measure_decode(factory(args.batch), args.batch, args.steps, args.warmup, V, args.prompt_len)
     need = decode_bytes(shape, args.layers, args.batch, ctx_mid, el)
     achieved = need / (ms_step / 1000.0) / 1e9
     out = {
-        "metric": f"decode tok/s at batch {args.batch}, 2,048-token prompts (Qwen2.5-{args.shape} shape)",
+        "metric": f"decode tok/s at batch {args.batch}, {args.prompt_len:,}-token prompts (Qwen2.5-{args.shape} shape)",
         "value": round(tps, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: seeded random weights, seeded uniform-random token ids",
-        "config": {"model": f"Qwen2.5-{args.shape} shape", "global_batch": args.batch, "seq_len": PROMPT,
-                   "context_len": CONTEXT, "parallelism": "single GPU", "num_layers": full_layers,
+        "config": {"model": f"Qwen2.5-{args.shape} shape", "global_batch": args.batch, "seq_len": args.prompt_len,
+                   "context_len": max(CONTEXT, 2 * args.prompt_len), "parallelism": "single GPU", "num_layers": full_layers,
                    "layers_run": args.layers, "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
                    "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": bool(shape["tie_word_embeddings"]),
@@ -189,14 +238,14 @@ def main():
     }
     if not args.no_points:
         torch.cuda.empty_cache()
-        pms = measure_prefill(factory(1), V)
-        fl = prefill_flops(shape, args.layers, PROMPT)
-        out["prefill"] = {"value": round(PROMPT / pms * 1000.0, 1), "tokens": PROMPT, "ms": round(pms, 3),
+        pms = measure_prefill(factory(1, PF), V, tokens=PF)
+        fl = prefill_flops(shape, args.layers, PF)
+        out["prefill"] = {"value": round(PF / pms * 1000.0, 1), "tokens": PF, "ms": round(pms, 3),
                           "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}
         points = {}
         for b, st in ((1, min(args.steps, 64)), (64, min(args.steps, 32))):
             torch.cuda.empty_cache()
-            t, _, _ = measure_decode(factory(b), b, st, min(args.warmup, 8), V)
+            t, _, _ = measure_decode(factory(b), b, st, min(args.warmup, 8), V, args.prompt_len)
             points[f"decode_b{b}"] = round(t, 2)
         out["points"] = points
     print(json.dumps(out))
