@@ -240,6 +240,35 @@ def test_sampling_in_the_engine_is_seeded_per_request(tiny):
     assert greedy == plain.greedy_generate(tiny["cfg"], tiny["weights"], prompts[3], 10)
 
 
+def test_generation_config_of_the_model_folder_is_the_default(tiny, tmp_path, monkeypatch):
+    """do_sample in the folder's generation_config.json: a request that sets no sampling option samples
+    with the file's values, one that asks for argmax is greedy, ZEDINFER_FORCE_ARGMAX makes all greedy
+    (reference: src/zedinfer/engine.cpp:49-126, scheduler.cpp:576-600)."""
+    import json
+    import shutil
+    from zedinfer_amd import GenerationConfig, InferenceEngine, SchedulerConfig
+    monkeypatch.delenv("ZEDINFER_FORCE_ARGMAX", raising=False)
+    folder = str(tmp_path / "model")
+    shutil.copytree(tiny["folder"], folder)
+    with open(os.path.join(folder, "generation_config.json"), "w") as f:
+        json.dump(dict(do_sample=True, temperature=0.8, top_k=30, seed=9), f)
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    sc = lambda: SchedulerConfig(num_kv_blocks=64, kv_block_size=ps, max_batch_requests=4)  # noqa: E731
+    prompt = traces.random_tokens(tiny["cfg"]["vocab_size"], 21, seed=8)
+    greedy = plain.greedy_generate(tiny["cfg"], tiny["weights"], prompt, 12)
+    ie = InferenceEngine.create(folder, "float32", sc())
+    assert ie.default_sampling.temperature == 0.8 and not ie.default_sampling.greedy
+    got = ie.generate_tokens(prompt, GenerationConfig(max_new_tokens=12, ignore_eos=True)).output_ids
+    own = engine(tiny).generate_tokens(prompt, GenerationConfig(max_new_tokens=12, temperature=0.8, top_k=30, seed=9,
+                                                               ignore_eos=True)).output_ids
+    assert got == own and got != greedy
+    assert ie.generate_tokens(prompt, GenerationConfig(max_new_tokens=12, use_argmax=True, ignore_eos=True)
+                              ).output_ids == greedy
+    monkeypatch.setenv("ZEDINFER_FORCE_ARGMAX", "1")
+    forced = InferenceEngine.create(folder, "float32", sc())
+    assert forced.generate_tokens(prompt, GenerationConfig(max_new_tokens=12, ignore_eos=True)).output_ids == greedy
+
+
 def test_command_lines(tiny, tmp_path):
     env = dict(os.environ, PYTHONPATH=ROOT)
     run = lambda *a: subprocess.run([sys.executable, *a], capture_output=True, text=True, env=env, timeout=300)  # noqa: E731

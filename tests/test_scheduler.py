@@ -313,3 +313,55 @@ def test_token_computed_ahead_for_a_cancelled_request_is_dropped():
     nxt = s.schedule()                                  # the ordinary schedule ends it
     assert a.done and a.finish_reason == "stop" and a.result.output_ids == [7] and nxt.decode_requests == [b]
     c.check()
+
+
+# ---- what a request samples with when it sets nothing -----------------------------------------
+
+def test_default_sampling_from_the_model_folder(tmp_path, monkeypatch):
+    # reference: create_sampler_from_generation_config, src/zedinfer/engine.cpp:49-126
+    import json
+    from zedinfer_amd.sampling import default_sampling
+    monkeypatch.delenv("ZEDINFER_FORCE_ARGMAX", raising=False)
+    monkeypatch.delenv("ZEDINFER_REPETITION_PENALTY", raising=False)
+    folder = str(tmp_path)
+    assert default_sampling(folder).greedy                              # no file
+    path = tmp_path / "generation_config.json"
+    path.write_text(json.dumps(dict(do_sample=False, temperature=0.6)))
+    assert default_sampling(folder).greedy
+    path.write_text(json.dumps(dict(do_sample=True)))
+    p = default_sampling(folder)
+    assert (p.temperature, p.top_k, p.top_p, p.repetition_penalty, p.seed, p.greedy) == (1.0, 0, 1.0, 1.0, 0, False)
+    path.write_text(json.dumps(dict(do_sample=True, temperature=0.6, top_k=20, top_p=0.95, repetition_penalty=1.05, seed=7)))
+    p = default_sampling(folder)
+    assert (p.temperature, p.top_k, p.top_p, p.repetition_penalty, p.seed) == (0.6, 20, 0.95, 1.05, 7)
+    monkeypatch.setenv("ZEDINFER_REPETITION_PENALTY", "1.2")
+    assert default_sampling(folder).repetition_penalty == 1.2
+    monkeypatch.setenv("ZEDINFER_FORCE_ARGMAX", "1")
+    assert default_sampling(folder).greedy
+    monkeypatch.setenv("ZEDINFER_FORCE_ARGMAX", "0")
+    assert not default_sampling(folder).greedy
+    monkeypatch.delenv("ZEDINFER_REPETITION_PENALTY")
+    path.write_text(json.dumps(dict(do_sample=True, top_p=1.5)))        # does not validate
+    assert default_sampling(folder).greedy
+    path.write_text("{ not json")
+    assert default_sampling(folder).greedy
+
+
+def test_requests_without_sampling_options_take_the_default():
+    from zedinfer_amd.sampling import SamplingParams
+    cfg = SchedulerConfig(num_kv_blocks=16, kv_block_size=4)
+    cache = CacheManager({0: KVCacheRequest("full", 1, 16)}, {}, 16, 4, cfg.max_batch_requests, torch.float32, None,
+                         cfg.max_batch_tokens)
+    s = Scheduler(cfg, cache, default_sampling=SamplingParams(temperature=0.6, top_k=20, seed=7))
+    plain_req, own, greedy, seeded = req(3), req(3, temperature=0.9), req(3, use_argmax=True), req(3, seed=11)
+    for r in (plain_req, own, greedy, seeded):
+        s.submit(r)
+    assert (plain_req.sampler.params.temperature, plain_req.sampler.params.top_k, plain_req.sampler.params.seed) == (0.6, 20, 7)
+    assert (own.sampler.params.temperature, own.sampler.params.top_k) == (0.9, 0)
+    assert greedy.sampler.params.greedy
+    assert (seeded.sampler.params.temperature, seeded.sampler.params.seed) == (0.6, 11)
+    # without a default: greedy, as before
+    s2, _ = make()
+    r = req(3)
+    s2.submit(r)
+    assert r.sampler.params.greedy

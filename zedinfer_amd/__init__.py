@@ -14,5 +14,11 @@ from .config import SchedulerConfig
 from .engine import (Engine, GenerationConfig, GenerationResult, InferenceEngine, InferenceRequest, StepEntry)
 from .sampling import SamplingParams
 
+
+def load_model(model_path: str, dtype="bfloat16", scheduler_config=None) -> InferenceEngine:
+    """Model, cache, scheduler and sampler from a model folder (``InferenceEngine.create``)."""
+    return InferenceEngine.create(model_path, dtype, scheduler_config)
+
+
 __all__ = ["Engine", "GenerationConfig", "GenerationResult", "InferenceEngine", "InferenceRequest",
-           "SamplingParams", "SchedulerConfig", "StepEntry", "models"]
+           "SamplingParams", "SchedulerConfig", "StepEntry", "load_model", "models"]

@@ -21,6 +21,7 @@ from ..cache.pages import OutOfPages
 from ..config import ModelConfig, ModelForwardConfig, SchedulerConfig, load_config
 from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
+from ..sampling.sampler import default_sampling
 from ..weights import load_weights, random_weights
 from .batch import DecodeImage, DeviceBatch, StagingRing, StepEntry, build_device_batch
 
@@ -65,6 +66,7 @@ class Engine:
         self.memories = self.cache.memories(fc.schedule)
         self.vocab_size = fc.vocab_size
         self.steps_run = 0
+        self.default_sampling = None      # what requests without sampling options use (None: greedy)
         self.staging = StagingRing(self.device)
         # Steps of single decoded tokens are captured as HIP graphs and replayed, one graph per
         # (entries, wanted rows, block-table widths, attention launch size).
@@ -84,7 +86,9 @@ class Engine:
         fc = arch.forward_config(cfg)
         dt = parse_dtype(dtype)
         weights = load_weights(folder, expected_weights(fc), dt, device)
-        return cls(fc, weights, dt, sched, device)
+        engine = cls(fc, weights, dt, sched, device)
+        engine.default_sampling = default_sampling(folder)
+        return engine
 
     @classmethod
     def from_config(cls, cfg: ModelConfig, arch_name: Optional[str] = None, dtype="bfloat16", seed: int = 0,

@@ -40,7 +40,19 @@ class GenerationConfig:
             raise ValueError("stream_callback required when stream=True")
         self.sampling().validate()
 
-    def sampling(self) -> SamplingParams:
+    def overrides_sampling(self) -> bool:
+        """Whether the request sets a sampling option of its own (the reference's has_sampling_override,
+        generation_types.hpp:56-67); a seed alone is none."""
+        return (self.use_argmax or self.temperature != 0.0 or self.top_k != 0 or self.top_p != 1.0
+                or self.repetition_penalty != 1.0)
+
+    def sampling(self, default: Optional[SamplingParams] = None) -> SamplingParams:
+        """The request's own options, or ``default`` (the engine's: from the model's
+        generation_config.json) when it sets none; its seed, when it has one, holds either way
+        (reference: pick_sampler, src/zedinfer/scheduler.cpp:576-600)."""
+        if default is not None and not self.overrides_sampling():
+            return SamplingParams(default.temperature, default.top_k, default.top_p, default.repetition_penalty,
+                                  self.seed or default.seed, default.use_argmax)
         return SamplingParams(self.temperature, self.top_k, self.top_p, self.repetition_penalty, self.seed,
                               self.use_argmax)
 

@@ -76,10 +76,12 @@ class ScheduledBatch:
 
 
 class Scheduler:
-    def __init__(self, config: SchedulerConfig, cache: CacheManager, stop_token_ids: Iterable[int] = ()):
+    def __init__(self, config: SchedulerConfig, cache: CacheManager, stop_token_ids: Iterable[int] = (),
+                 default_sampling=None):
         config.validate()
         self.config = config
         self.cache = cache
+        self.default_sampling = default_sampling      # for requests that set no sampling option (None: greedy)
         self.stop_token_ids = set(int(t) for t in stop_token_ids)
         self.waiting: Deque[InferenceRequest] = deque()
         self.active: List[InferenceRequest] = []
@@ -103,7 +105,7 @@ class Scheduler:
             req.request_id = self._next_id
             self._next_id += 1
             req.phase = RequestPhase.QUEUED
-            req.sampler = RequestSampler(req.config.sampling())
+            req.sampler = RequestSampler(req.config.sampling(self.default_sampling))
             req.stats.prompt_tokens = len(req.input_ids)
             self.waiting.append(req)
             self._work.notify_all()

@@ -44,7 +44,8 @@ class ServingLoop:
 
     def __init__(self, engine: Engine, stop_token_ids: Iterable[int] = (), look_ahead: Optional[bool] = None):
         self.engine = engine
-        self.scheduler = Scheduler(engine.sched, engine.cache, stop_token_ids)
+        self.scheduler = Scheduler(engine.sched, engine.cache, stop_token_ids,
+                                   getattr(engine, "default_sampling", None))
         self.sampler = Sampler(engine.device, engine.vocab_size)
         self.look_ahead = os.environ.get("ZEDINFER_DISABLE_LOOKAHEAD", "0") in ("", "0") if look_ahead is None \
             else bool(look_ahead)
@@ -160,6 +161,11 @@ class InferenceEngine:
     def create(cls, model_path: str, dtype="bfloat16", scheduler_config: Optional[SchedulerConfig] = None
                ) -> "InferenceEngine":
         return cls(Engine.from_folder(model_path, dtype, scheduler_config))
+
+    @property
+    def default_sampling(self):
+        """What requests without sampling options of their own sample with."""
+        return self.engine.default_sampling
 
     def serving_loop(self) -> ServingLoop:
         return self._loop

@@ -17,6 +17,9 @@ def has_gpu() -> bool:
     return torch.cuda.is_available()
 
 
+has_cuda = has_gpu      # the reference module's name for it (python/zedinfer_ops.cpp:316-355)
+
+
 def device_synchronize() -> None:
     torch.cuda.synchronize()
 

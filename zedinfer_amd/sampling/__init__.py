@@ -1,3 +1,3 @@
-from .sampler import RequestSampler, Sampler, SamplingParams
+from .sampler import RequestSampler, Sampler, SamplingParams, default_sampling
 
 __all__ = ["RequestSampler", "Sampler", "SamplingParams"]

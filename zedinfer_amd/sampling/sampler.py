@@ -10,6 +10,8 @@ src/zedinfer/scheduler.cpp:584-600).
 """
 from __future__ import annotations
 
+import json
+import os
 import random
 from dataclasses import dataclass
 from typing import List, Optional, Sequence
@@ -45,6 +47,45 @@ class SamplingParams:
             raise ValueError("repetition_penalty must be positive")
         if not self.use_argmax and self.temperature < 0.0:
             raise ValueError("temperature must be non-negative (0 means greedy)")
+
+
+def default_sampling(model_path: Optional[str]) -> SamplingParams:
+    """What a request samples with when it sets no sampling option of its own: the model folder's
+    generation_config.json when it says ``do_sample`` (temperature default 1, top_k 0, top_p 1,
+    repetition_penalty 1, seed 0), else greedy; also greedy when the file is missing, unreadable or its
+    values do not validate.  ``ZEDINFER_FORCE_ARGMAX`` (set, not "0") forces greedy,
+    ``ZEDINFER_REPETITION_PENALTY`` overrides the file's penalty
+    (reference: src/zedinfer/engine.cpp:49-126)."""
+    greedy = SamplingParams(use_argmax=True)
+    force = os.environ.get("ZEDINFER_FORCE_ARGMAX", "")
+    if force not in ("", "0"):
+        return greedy
+    if not model_path:
+        return greedy
+    path = os.path.join(model_path, "generation_config.json")
+    if not os.path.isfile(path):
+        return greedy
+    try:
+        with open(path) as f:
+            j = json.load(f)
+        if not bool(j.get("do_sample", False)):
+            return greedy
+        p = SamplingParams(temperature=float(j.get("temperature", 1.0)), top_k=int(j.get("top_k", 0)),
+                           top_p=float(j.get("top_p", 1.0)), repetition_penalty=float(j.get("repetition_penalty", 1.0)),
+                           seed=int(j.get("seed", 0)))
+        env = os.environ.get("ZEDINFER_REPETITION_PENALTY", "")
+        if env:
+            try:
+                p.repetition_penalty = float(env)
+            except ValueError:
+                pass
+        # the reference's check: a temperature of 0 is not a valid sampler here, it falls back to greedy
+        if not (p.temperature > 0.0):
+            return greedy
+        p.validate()
+        return p
+    except (OSError, ValueError, TypeError):
+        return greedy
 
 
 class RequestSampler:
