@@ -599,6 +599,17 @@ def test_attention_prefill(ops, nh, nkv, d, ps, window, portions):
                               dev([e[2] for e in entries]), bt, nh, nkv, d, scale, window, out=out2)
         n0 = entries[0][1]
         assert bool((out2[:n0] == 7.0).all()) and torch.equal(out2[n0:], out[n0:])
+    # head sizes 64 and 128 have a second kernel (keys and values straight into LDS): the same bits
+    if d in (64, 128):
+        before = ops.attention_prefill_variant(0)
+        try:
+            out3 = torch.full((n_tok, nh * d), 7.0, dtype=dtype, device="cuda")
+            ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, te, to, dev([e[0] for e in entries]),
+                                  dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale,
+                                  window, out=out3)
+        finally:
+            ops.attention_prefill_variant(before)
+        assert before == 1 and torch.equal(out3, out)
 
 
 def test_attention_prefill_bound_too_low_shows(ops):

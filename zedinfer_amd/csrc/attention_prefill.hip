@@ -390,6 +390,310 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// The same attention for head sizes 64 and 128 with keys and values loaded straight into LDS
+// (global_load_lds_dwordx4): no registers, no address arithmetic and no LDS stores are spent on staging.
+// One load instruction of a wavefront fills 1 KB of LDS, lane l the 16 bytes at l * 16; which 16 bytes of
+// the cache a lane asks for is free, so the tiles keep the order the matrix cores want (keys permuted as
+// above, values transposed) and their rows are not padded but rotated: the 16-byte piece c of row r sits
+// at place (c + r) mod pieces-per-row, which spreads a quarter-wave's reads over the banks as the padding
+// did.  Two buffers, each a pair of LDS arrays of its own, used in turn by an unrolled loop: the loads
+// of the next block are issued right after the barrier that makes this block visible, so the compiler's
+// wait before a barrier (it waits for every load into LDS there) never waits for a block that is still
+// needed later.  Values of keys past the last key and of pages that a window has given back are loaded
+// from 16 zero bytes instead (0 * NaN would be NaN); the one piece that straddles the last key is
+// cleaned in LDS.  Keys need no such care: their scores are masked.
+__device__ __attribute__((aligned(16))) const unsigned pf_zero16[4] = {0u, 0u, 0u, 0u};
+
+template <int D>
+__global__ void __launch_bounds__(PF_WAVES* ZI_WAVE)
+attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* __restrict__ q, int64_t ldq,
+                             const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,
+                             const int32_t* __restrict__ tile_entry, const int32_t* __restrict__ tile_off,
+                             const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
+                             const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
+                             int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale,
+                             float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
+    static_assert(D == 64 || D == 128, "this variant takes head sizes 64 and 128");
+    constexpr int DK = D / 32, DT = D / 16;
+    constexpr int KC = D / 8;                        // 16-byte pieces of a key row
+    constexpr int VC = PF_BS / 8;                    // and of a row of the transposed value tile: 16
+    constexpr int KCH = PF_BS * KC, VCH = D * VC;    // pieces of the two tiles
+    constexpr int THREADS = PF_WAVES * ZI_WAVE;
+    constexpr int KI = KCH / THREADS, VI = VCH / THREADS;   // load instructions a wavefront issues per tile
+    __shared__ __attribute__((aligned(16))) uint4 k_a[KCH];
+    __shared__ __attribute__((aligned(16))) uint4 k_b[KCH];
+    __shared__ __attribute__((aligned(16))) uint4 v_a[VCH];
+    __shared__ __attribute__((aligned(16))) uint4 v_b[VCH];
+    __shared__ int32_t bt_lds[PF_CHUNK / 8 + 8];     // the pages of this workgroup's keys (page size >= 8)
+
+    const int tile = blockIdx.x / nh, h = blockIdx.x % nh;
+    const int g = h / (nh / nkv);
+    const int e = tile_entry[tile], off = tile_off[tile];
+    const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
+    const int count = (len - off < PF_BM) ? len - off : PF_BM;
+    const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
+    const int r = lane & 15, j = lane >> 4;
+    const int32_t* bt = block_tables + (int64_t)e * max_pages;
+    const int pos0 = past + off;
+    const int kmax = pos0 + count - 1;
+    const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
+    const int kb_first = (lo_tile / PF_BS) * PF_BS;
+    const int c0 = kb_first / PF_CHUNK, nc = kmax / PF_CHUNK - c0 + 1, c = c0 + blockIdx.y;
+    if (c * PF_CHUNK > kmax) return;
+    const int kb_begin = (c * PF_CHUNK > kb_first) ? c * PF_CHUNK : kb_first;
+    const int khi = ((c + 1) * PF_CHUNK - 1 < kmax) ? (c + 1) * PF_CHUNK - 1 : kmax;
+
+    const int qs = wave % 4, kh = wave / 4;
+    const int row = qs * 16 + r;
+    const bool wave_active = qs * 16 < count;
+    const bool qvalid = row < count;
+    const int qrow = qvalid ? row : count - 1;
+    const int qpos = pos0 + qrow;
+    const int wave_first = pos0 + ((qs * 16 < count) ? qs * 16 : count - 1);
+    const int wave_last = pos0 + ((qs * 16 + 15 < count) ? qs * 16 + 15 : count - 1);
+    const float scale_log2 = scale * 1.4426950408889634f;
+    const int wave_lo = (window > 0 && pos0 + qs * 16 - window + 1 > 0) ? pos0 + qs * 16 - window + 1 : 0;
+    pf_bf16x8_t qop[DK];
+    {
+        const zi_bf16* qr = q + (int64_t)(start + off + qrow) * ldq + (int64_t)h * D + j * 8;
+#pragma unroll
+        for (int dk = 0; dk < DK; ++dk) {
+            pf_pack p;
+            p.u = *reinterpret_cast<const uint4*>(qr + dk * 32);
+            qop[dk] = p.b;
+        }
+    }
+    pf_f32x4_t o[DT];
+#pragma unroll
+    for (int dd = 0; dd < DT; ++dd) o[dd] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, lsum = 0.f;
+
+    // the block table's entries for keys [kb_begin, khi], once
+    const int ps = 1 << ps_shift, ps_mask = ps - 1;
+    const int pi_last = max_pages - 1, pi_first = kb_begin >> ps_shift;
+    if (tid <= (khi >> ps_shift) - pi_first) bt_lds[tid] = bt[pi_first + tid < pi_last ? pi_first + tid : pi_last];
+    // What a lane loads does not change from block to block: for its KI pieces of the key tile the key
+    // (as an offset into the block) and the piece of its row, for its VI pieces of the value tile the
+    // dim and the eight keys.  Place L of a tile is row L / pieces-per-row; the piece there is rotated.
+    int k_key[KI], k_piece[KI], v_dim[VI], v_key[VI];
+#pragma unroll
+    for (int i = 0; i < KI; ++i) {
+        const int L = (wave * KI + i) * ZI_WAVE + lane;
+        const int rho = L / KC;
+        const int t = (rho % PF_BN) / 16, rr = rho % 16;
+        k_key[i] = (rho / PF_BN) * PF_BN + (t / 2) * 32 + (rr / 4) * 8 + (t % 2) * 4 + rr % 4;
+        k_piece[i] = (L % KC - rho) & (KC - 1);
+    }
+#pragma unroll
+    for (int i = 0; i < VI; ++i) {
+        const int L = (wave * VI + i) * ZI_WAVE + lane;
+        v_dim[i] = L / VC;
+        v_key[i] = ((L % VC - v_dim[i]) & (VC - 1)) * 8;
+    }
+    const zi_bf16* kbase = kcache + (int64_t)g * ps * D;
+    const zi_bf16* vbase = vcache + (int64_t)g * D * ps;
+    const int64_t page_stride = (int64_t)nkv * ps * D;
+    const int khi8 = khi & ~7;
+    __syncthreads();      // the table is in LDS
+
+    auto issue = [&](int kb, uint4* kl, uint4* vl) {
+#pragma unroll
+        for (int i = 0; i < KI; ++i) {
+            const int key = kb + k_key[i];
+            const int kc = key <= khi ? key : khi;
+            const int pg = bt_lds[(kc >> ps_shift) - pi_first];
+            const int page = (unsigned)pg < (unsigned)num_pages ? pg : 0;     // not held: a window has passed it
+            const zi_bf16* src = kbase + page * page_stride + (int64_t)(kc & ps_mask) * D + k_piece[i] * 8;
+            __builtin_amdgcn_global_load_lds(src, kl + (wave * KI + i) * ZI_WAVE, 16, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < VI; ++i) {
+            const int key0 = kb + v_key[i];
+            const int kc = key0 <= khi ? key0 : khi8;
+            const int pg = bt_lds[(kc >> ps_shift) - pi_first];
+            const bool ok = key0 <= kmax && (unsigned)pg < (unsigned)num_pages;
+            const zi_bf16* src = ok ? vbase + pg * page_stride + ((int64_t)v_dim[i] << ps_shift) + (kc & ps_mask)
+                                    : reinterpret_cast<const zi_bf16*>(pf_zero16);
+            __builtin_amdgcn_global_load_lds(src, vl + (wave * VI + i) * ZI_WAVE, 16, 0, 0);
+        }
+    };
+    // The piece of every value row that holds the last key and keys past it: what lies past is cleared
+    // (those slots of the page may hold anything).  Only in the block that holds the last key.
+    auto clean = [&](int kb, uint4* vl) {
+        if (kb + PF_BS - 1 > kmax && ((kmax + 1) & 7) != 0) {
+            if (tid < D) {
+                const int piece = (kmax - kb) / 8, keep = (kmax + 1) & 7;
+                pf_pack val;
+                uint4* at = vl + tid * VC + ((piece + tid) & (VC - 1));
+                val.u = *at;
+#pragma unroll
+                for (int x = 0; x < 8; ++x)
+                    if (x >= keep) val.h[x] = 0;
+                *at = val.u;
+            }
+            __syncthreads();
+        }
+    };
+    auto work = [&](int kb0, const uint4* kl, const uint4* vl) {
+        const int kb = kb0 + kh * PF_BN;      // this wavefront's 64 keys of the block
+        if (wave_active && kb <= wave_last && kb + PF_BN > wave_lo) {
+        pf_f32x4_t s[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            s[t] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const int rho = kh * PF_BN + t * 16 + r;
+#pragma unroll
+            for (int dk = 0; dk < DK; ++dk) {
+                pf_pack a;
+                a.u = kl[rho * KC + ((dk * 4 + j + rho) & (KC - 1))];
+                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, qop[dk], s[t], 0, 0, 0);
+            }
+        }
+        const bool whole = kb + PF_BN - 1 <= wave_first && (window <= 0 || kb > wave_last - window);
+        float mx = -INFINITY;
+        if (whole) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    s[t][x] *= scale_log2;
+                    mx = fmaxf(mx, s[t][x]);
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
+                    const bool vis = key <= qpos && (window <= 0 || key > qpos - window);
+                    const float v = vis ? s[t][x] * scale_log2 : -INFINITY;
+                    s[t][x] = v;
+                    mx = fmaxf(mx, v);
+                }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float corr = __builtin_amdgcn_exp2f(m - m_use);
+        m = m_new;
+        float psum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                s[t][x] = __builtin_amdgcn_exp2f(s[t][x] - m_use);
+                psum += s[t][x];
+            }
+        pf_pack pb[2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+            pb[b].u.x = zi_pack_bf16x2(s[2 * b][0], s[2 * b][1]);
+            pb[b].u.y = zi_pack_bf16x2(s[2 * b][2], s[2 * b][3]);
+            pb[b].u.z = zi_pack_bf16x2(s[2 * b + 1][0], s[2 * b + 1][1]);
+            pb[b].u.w = zi_pack_bf16x2(s[2 * b + 1][2], s[2 * b + 1][3]);
+        }
+        lsum = lsum * corr + psum;
+        if (__any(corr != 1.f)) {
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) {
+                o[dd][0] *= corr; o[dd][1] *= corr; o[dd][2] *= corr; o[dd][3] *= corr;
+            }
+        }
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd) {
+            const int dim = dd * 16 + r;
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                pf_pack a;
+                a.u = vl[dim * VC + ((kh * 8 + b * 4 + j + dim) & (VC - 1))];
+                o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[b].b, o[dd], 0, 0, 0);
+            }
+        }
+        }
+    };
+    // Two blocks a turn, buffer a then b.  At each barrier the block about to be worked on has arrived
+    // (the compiler waits for all loads into LDS before a barrier) and everyone has finished with the
+    // other buffer, so the block after it is requested into that one at once.
+    issue(kb_begin, k_a, v_a);
+    int kb0 = kb_begin;
+    while (true) {
+        __syncthreads();
+        if (kb0 + PF_BS <= khi) issue(kb0 + PF_BS, k_b, v_b);
+        clean(kb0, v_a);
+        work(kb0, k_a, v_a);
+        if (kb0 + PF_BS > khi) break;
+        kb0 += PF_BS;
+        __syncthreads();
+        if (kb0 + PF_BS <= khi) issue(kb0 + PF_BS, k_a, v_a);
+        clean(kb0, v_b);
+        work(kb0, k_b, v_b);
+        if (kb0 + PF_BS > khi) break;
+        kb0 += PF_BS;
+    }
+    __syncthreads();
+    float l = lsum;
+    l += __shfl_xor(l, 16, ZI_WAVE);
+    l += __shfl_xor(l, 32, ZI_WAVE);
+    {
+        // the two wavefronts of a query sub-tile merge their (maximum, sum, output) through LDS; nobody reads
+        // the tiles any more
+        float* mo = reinterpret_cast<float*>(k_a);                   // [qs][DT][64][4]: as large as a key tile
+        float* ml = reinterpret_cast<float*>(v_a);                   // [qs][64][2]
+        static_assert(sizeof(float) * 4 * DT * ZI_WAVE * 4 <= sizeof(uint4) * KCH, "the key tile holds the merge");
+        if (kh > 0) {
+            float* dst = mo + qs * (DT * ZI_WAVE * 4);
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(dst + (dd * ZI_WAVE + lane) * 4) = o[dd];
+            ml[(qs * ZI_WAVE + lane) * 2] = m;
+            ml[(qs * ZI_WAVE + lane) * 2 + 1] = l;
+        }
+        __syncthreads();
+        if (kh > 0) return;
+        const float* src = mo + qs * (DT * ZI_WAVE * 4);
+        const float m2 = ml[(qs * ZI_WAVE + lane) * 2];
+        const float l2 = ml[(qs * ZI_WAVE + lane) * 2 + 1];
+        const float mm = fmaxf(m, m2);
+        const float mu = (mm == -INFINITY) ? 0.f : mm;
+        const float a1 = __builtin_amdgcn_exp2f(m - mu), a2 = __builtin_amdgcn_exp2f(m2 - mu);
+        l = l * a1 + l2 * a2;
+        m = mm;
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd) {
+            const pf_f32x4_t v = *reinterpret_cast<const pf_f32x4_t*>(src + (dd * ZI_WAVE + lane) * 4);
+            o[dd][0] = o[dd][0] * a1 + v[0] * a2; o[dd][1] = o[dd][1] * a1 + v[1] * a2;
+            o[dd][2] = o[dd][2] * a1 + v[2] * a2; o[dd][3] = o[dd][3] * a1 + v[3] * a2;
+        }
+    }
+    if (!qvalid) return;
+    if (nc > 1) {
+        if (nc > max_chunks) {
+            if (blockIdx.y == 0)
+                for (int dd = 0; dd < DT; ++dd)
+                    for (int x = 0; x < 4; ++x) zi_store(out + (int64_t)(start + off + row) * ldo + (int64_t)h * D + dd * 16 + j * 4 + x, NAN);
+            return;
+        }
+        const int64_t slot = ((int64_t)(start + off + row) * nh + h) * max_chunks + blockIdx.y;
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = o[dd];
+        if (j == 0) {
+            part_ml[slot * 2] = m;
+            part_ml[slot * 2 + 1] = l;
+        }
+        return;
+    }
+    const float inv = 1.f / l;
+    zi_bf16* orow = out + (int64_t)(start + off + row) * ldo + (int64_t)h * D;
+#pragma unroll
+    for (int dd = 0; dd < DT; ++dd) {
+        uint2 w;
+        w.x = zi_pack_bf16x2(o[dd][0] * inv, o[dd][1] * inv);
+        w.y = zi_pack_bf16x2(o[dd][2] * inv, o[dd][3] * inv);
+        *reinterpret_cast<uint2*>(orow + dd * 16 + j * 4) = w;
+    }
+}
+
 // Merge the cuts of one (query, head): out = sum_c 2^(m_c - M) o_c / sum_c 2^(m_c - M) l_c, in rising order
 // of the keys.  One wavefront per (query row of a tile, head); tiles with one cut were written directly.
 __global__ void __launch_bounds__(ZI_WAVE)
@@ -452,6 +756,15 @@ extern "C" int zi_attention_prefill_tile() { return PF_BM; }
 // Tile i covers the queries [tile_off[i], tile_off[i] + 64) of entry tile_entry[i] (fewer at the
 // entry's end); entry e brings entry_len[e] tokens that start at row entry_start[e] of q and at
 // position entry_past[e] of its sequence, whose block table is row e of block_tables.
+// Which kernel head sizes 64 and 128 take: 1 (the default) loads keys and values straight into LDS, 0 stages
+// them through registers like the other head sizes.  For measurements and tests.
+static int pf_variant = 1;
+extern "C" int zi_attention_prefill_variant(int variant) {
+    const int before = pf_variant;
+    if (variant == 0 || variant == 1) pf_variant = variant;
+    return before;
+}
+
 extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
                                     const void* kcache, const void* vcache, const int32_t* tile_entry,
                                     const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
@@ -486,6 +799,14 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
         window, scale, po, pml, max_chunks)
+#define ZI_PF_DMA(DD)                                                                                          \
+    attention_prefill_dma_kernel<DD><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                                 \
+        (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
+        tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
+        window, scale, po, pml, max_chunks)
+    if (pf_variant == 1 && d == 128) ZI_PF_DMA(128);
+    else if (pf_variant == 1 && d == 64) ZI_PF_DMA(64);
+    else
     switch (d) {
         case 16: ZI_PF(16); break;
         case 32: ZI_PF(32); break;
@@ -497,6 +818,7 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
         default: ZI_PF(128); break;
     }
 #undef ZI_PF
+#undef ZI_PF_DMA
     if (max_chunks > 1)
         attention_prefill_merge_kernel<<<dim3(num_tiles * PF_BM, nh), ZI_WAVE, 0, stream>>>(
             (zi_bf16*)out, ldo, po, pml, tile_entry, tile_off, entry_start, entry_len, entry_past, nh, d, window, max_chunks);

@@ -38,6 +38,7 @@ _PROTOTYPES = {
     "zi_attention_decode_chunks": [I],
     "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, P],
     "zi_attention_prefill_chunks": [I],
+    "zi_attention_prefill_variant": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],
     "zi_attention_prefill_tile": [],
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],

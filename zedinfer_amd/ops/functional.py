@@ -536,6 +536,13 @@ def attention_decode_project(workspace: torch.Tensor, weight: torch.Tensor, tok_
     return out
 
 
+def attention_prefill_variant(variant: int = -1) -> int:
+    """Which prompt-attention kernel head sizes 64 and 128 take: 1 (the default) loads keys and values
+    straight into LDS, 0 stages them through registers like the other head sizes; both give the same
+    bits.  Returns the variant in force before; -1 only asks."""
+    return int(_lib.load().zi_attention_prefill_variant(int(variant)))
+
+
 PREFILL_TILE = 64     # queries one workgroup of the prompt kernel takes
 
 
