@@ -88,8 +88,11 @@ def test_rms_norm(ops, dtype, n, H, eps):
 
 
 @pytest.mark.parametrize("dtype", DT)
-def test_add_rms_norm(ops, dtype):
-    n, H, eps = 6, 200, 1e-6
+@pytest.mark.parametrize("n,H", [(6, 200), (64, 1536), (201, 72), (130, 5120), (77, 3584), (66, 8192), (65, 34)])
+def test_add_rms_norm(ops, dtype, n, H):
+    """Few rows (a workgroup a row) and many (a wavefront a row), widths of every number of 1 KB runs,
+    and one that is no multiple of four (the plain kernel)."""
+    eps = 1e-6
     resid = rnd(n, H, seed=3)
     delta = rnd(n, H, dtype=dtype, seed=4)
     w = rnd(H, dtype=dtype, seed=5)

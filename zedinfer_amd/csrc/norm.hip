@@ -119,6 +119,51 @@ __global__ void add_rmsnorm_vec_kernel(TO* __restrict__ out, float* __restrict__
     }
 }
 
+// Many rows (prompt portions), one addend: a wavefront per row, four rows a workgroup.  A lane owns NV
+// groups of four consecutive values, 256 values apart, so every load instruction of the wavefront reads
+// 1 KB of the row; all loads are issued before the first use, the sum of squares is taken within the
+// wavefront (no barrier), and the row is read once.  H <= 1024 * NV, H % 4 == 0.
+template <typename TD, typename TW, typename TO, int NV>
+__global__ void __launch_bounds__(4 * ZI_WAVE)
+add_rmsnorm_rows_kernel(TO* __restrict__ out, float* __restrict__ resid, const TD* __restrict__ delta,
+                        const TW* __restrict__ w, int n, int H, float eps, float w_offset) {
+    const int lane = threadIdx.x & (ZI_WAVE - 1), wave = threadIdx.x / ZI_WAVE;
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= n) return;
+    float* rr = resid + row * H;
+    const TD* dr = delta + row * H;
+    float4 v[NV], d[NV], wv[NV];
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+        const int j = (c * ZI_WAVE + lane) * 4, jc = j < H ? j : 0;     // past the row: its start again, unused
+        v[c] = zi_load4(rr + jc);
+        d[c] = zi_load4(dr + jc);
+        wv[c] = zi_load4(w + jc);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+        const int j = (c * ZI_WAVE + lane) * 4;
+        v[c].x += d[c].x; v[c].y += d[c].y; v[c].z += d[c].z; v[c].w += d[c].w;
+        if (j < H) {
+            zi_store4(rr + j, v[c]);
+            ss += v[c].x * v[c].x + v[c].y * v[c].y + v[c].z * v[c].z + v[c].w * v[c].w;
+        }
+    }
+    ss = zi_wave_sum(ss);
+    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
+    TO* orow = out + row * H;
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+        const int j = (c * ZI_WAVE + lane) * 4;
+        if (j < H)
+            zi_store4(orow + j, make_float4((wv[c].x + w_offset) * v[c].x * rstd, (wv[c].y + w_offset) * v[c].y * rstd,
+                                            (wv[c].z + w_offset) * v[c].z * rstd, (wv[c].w + w_offset) * v[c].w * rstd));
+    }
+}
+
+#define NORM_MANY_ROWS 64     // from this many rows on, a wavefront per row
+
 extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* delta, int delta_dt, int splits,
                               int64_t split_stride, const void* w, int w_dt, int n, int hidden, float eps, int add_one,
                               hipStream_t stream) {
@@ -129,6 +174,26 @@ extern "C" int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* d
     if (n == 0) return 0;
     const bool aligned = ((uintptr_t)out % 16) == 0 && ((uintptr_t)resid % 16) == 0 && ((uintptr_t)delta % 16) == 0 &&
                          ((uintptr_t)w % 16) == 0 && split_stride % 4 == 0;
+    if (n >= NORM_MANY_ROWS && splits == 1 && hidden % 4 == 0 && hidden <= 8192 && aligned) {
+        const int nv = (hidden + 4 * ZI_WAVE - 1) / (4 * ZI_WAVE);
+        const int wgs = (n + 3) / 4;
+#define ZI_NORM_ROWS(NV)                                                                                            \
+    add_rmsnorm_rows_kernel<TD, TW, TO, NV><<<wgs, 4 * ZI_WAVE, 0, stream>>>(                                       \
+        (TO*)out, resid, (const TD*)delta, (const TW*)w, n, hidden, eps, add_one ? 1.f : 0.f)
+        ZI_DISPATCH_DTYPE(delta_dt, TD, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
+            if (nv <= 2) ZI_NORM_ROWS(2);
+            else if (nv <= 4) ZI_NORM_ROWS(4);
+            else if (nv <= 6) ZI_NORM_ROWS(6);
+            else if (nv <= 8) ZI_NORM_ROWS(8);
+            else if (nv <= 12) ZI_NORM_ROWS(12);
+            else if (nv <= 16) ZI_NORM_ROWS(16);
+            else if (nv <= 20) ZI_NORM_ROWS(20);
+            else if (nv <= 24) ZI_NORM_ROWS(24);
+            else ZI_NORM_ROWS(32);
+        })));
+#undef ZI_NORM_ROWS
+        return zi_check_launch("add_rmsnorm");
+    }
     if (hidden % 4 == 0 && hidden <= 8192 && splits <= 16 && aligned) {
         const int vecs = hidden / 4;
         const int it = vecs > 1024 ? 2 : 1;
