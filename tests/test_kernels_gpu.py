@@ -220,6 +220,48 @@ def test_rope_kv_store(ops, dtype):
     assert int((kc != 0).any(-1).any(1).sum()) == n
 
 
+@pytest.mark.parametrize("nh,nkv,d,rot,ps", [(12, 2, 128, 128, 16), (6, 2, 48, 32, 8), (3, 1, 64, 0, 32), (5, 5, 80, 80, 8)])
+@pytest.mark.parametrize("layout", ["runs", "shifted", "scattered"])
+def test_rope_kv_store_many_tokens(ops, nh, nkv, d, rot, ps, layout):
+    """From 64 tokens on bfloat16 takes the kernel that moves 16-byte pieces: against the kernel for few
+    tokens, eight tokens at a time (the same arithmetic; a product may be fused differently, hence one
+    rounding step), with slots in runs from multiples of eight (a value run is one store), runs that start
+    elsewhere, slots scattered, a tail of fewer than eight tokens, and slots out of range that are skipped."""
+    dtype = torch.bfloat16
+    n, pages, theta = 203, 40, 5e4
+    qkv = rnd(n, (nh + 2 * nkv) * d + 8, dtype=dtype)[:, 8:]             # rows that do not start the buffer
+    q, k, v = qkv[:, :nh * d], qkv[:, nh * d:(nh + nkv) * d], qkv[:, (nh + nkv) * d:]
+    pos = torch.arange(1000, 1000 + n, dtype=torch.int32, device="cuda")
+    if layout == "scattered":
+        slots = torch.randperm(pages * ps)[:n].to(torch.int32)
+    else:
+        slots = torch.arange(n, dtype=torch.int32) + (0 if layout == "runs" else 3)
+    slots[17] = -1
+    slots = slots.cuda()
+    inv = ops.rope_inv_freq(rot, theta, "cuda") if rot else None
+
+    def run(step):
+        qq = qkv.clone()
+        kc = torch.full((pages, nkv, ps, d), 3.0, dtype=dtype, device="cuda")
+        vc = torch.full((pages, nkv, d, ps), 3.0, dtype=dtype, device="cuda")
+        for a in range(0, n, step):
+            b = min(n, a + step)
+            ops.rope_kv_store(qq[a:b, :nh * d], qq[a:b, nh * d:(nh + nkv) * d], qq[a:b, (nh + nkv) * d:], pos[a:b],
+                              slots[a:b], inv, kc, vc, nh, nkv, d)
+        return qq[:, :nh * d], kc, vc
+
+    q1, kc1, vc1 = run(n)       # one call: the kernel for many tokens
+    q2, kc2, vc2 = run(8)       # eight tokens a call: the kernel for few
+    torch.testing.assert_close(q1.float(), q2.float(), atol=0.0, rtol=8e-3)
+    torch.testing.assert_close(kc1.float(), kc2.float(), atol=0.0, rtol=8e-3)
+    assert torch.equal(vc1, vc2)
+    assert int((vc1 != 3.0).any(1).any(1).sum()) == n - 1      # every token's slot but the one out of range
+    # queries only
+    q3 = qkv.clone()
+    ops.rope_kv_store(q3[:, :nh * d], None, None, pos, None, inv, None, None, nh, nkv, d)
+    assert torch.equal(q3[:, :nh * d], q1) and torch.equal(q3[:, nh * d:], qkv[:, nh * d:])
+
+
 @pytest.mark.parametrize("xdt,wdt,odt", [(torch.float32,) * 3, (torch.bfloat16,) * 3,
                                           (torch.bfloat16, torch.float32, torch.bfloat16),
                                           (torch.bfloat16, torch.bfloat16, torch.float32)])

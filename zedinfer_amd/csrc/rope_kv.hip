@@ -66,6 +66,125 @@ __global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k,
     }
 }
 
+// The same for many tokens (prompt portions) in bfloat16: a workgroup takes eight consecutive tokens, the
+// angles of their positions go to LDS once, and everything moves in 16-byte pieces: a thread rotates
+// eight dims of a head and their eight partners at a time.  Values are staged in LDS; when the eight
+// tokens' slots are eight consecutive slots of one page that start at a multiple of eight (the usual case
+// inside a prompt), a thread writes the eight tokens' values of one dim as one 16-byte run of the
+// transposed value cache, else value by value.  half = rot / 2 must be a multiple of 8 (or 0).
+#define RKT_TOKENS 8
+__global__ void __launch_bounds__(256)
+rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k, const zi_bf16* __restrict__ v,
+                          int64_t ldq, int64_t ldk, int64_t ldv, const int32_t* __restrict__ pos,
+                          const int32_t* __restrict__ slots, const float* __restrict__ inv_freq,
+                          zi_bf16* __restrict__ kcache, zi_bf16* __restrict__ vcache, int n, int nh, int nkv, int d,
+                          int rot, int page_size, int write_kv, int64_t cache_slots) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char rkt_lds[];
+    const int half = rot / 2, kvd = nkv * d;
+    float* cs = reinterpret_cast<float*>(rkt_lds);                                   // [token][cos[half], sin[half]]
+    uint16_t* vt = reinterpret_cast<uint16_t*>(rkt_lds + (size_t)RKT_TOKENS * rot * sizeof(float));   // [token][kvd]
+    const int t0 = blockIdx.x * RKT_TOKENS, tid = threadIdx.x;
+    const int nt = (n - t0 < RKT_TOKENS) ? n - t0 : RKT_TOKENS;
+    for (int i = tid; i < nt * half; i += 256) {
+        const int tt = i / half, jj = i % half;
+        float sn, c;
+        sincosf((float)pos[t0 + tt] * inv_freq[jj], &sn, &c);
+        cs[tt * rot + jj] = c;
+        cs[tt * rot + half + jj] = sn;
+    }
+    if (write_kv)
+        for (int i = tid; i < nt * (kvd / 8); i += 256) {
+            const int tt = i / (kvd / 8), c8 = i % (kvd / 8);
+            *reinterpret_cast<uint4*>(vt + tt * kvd + c8 * 8) =
+                *reinterpret_cast<const uint4*>(v + (int64_t)(t0 + tt) * ldv + c8 * 8);
+        }
+    __syncthreads();
+    auto unpack = [](uint4 u, float (&f)[8]) {
+        f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
+        f[2] = __uint_as_float(u.y << 16); f[3] = __uint_as_float(u.y & 0xffff0000u);
+        f[4] = __uint_as_float(u.z << 16); f[5] = __uint_as_float(u.z & 0xffff0000u);
+        f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
+    };
+    auto pack = [](const float (&f)[8]) {
+        return make_uint4(zi_pack_bf16x2(f[0], f[1]), zi_pack_bf16x2(f[2], f[3]), zi_pack_bf16x2(f[4], f[5]),
+                          zi_pack_bf16x2(f[6], f[7]));
+    };
+    // queries, in place: (token, head, eight dims of the first half and their partners)
+    const int hp = half / 8;
+    for (int i = tid; i < nt * nh * hp; i += 256) {
+        const int tt = i / (nh * hp), rem = i % (nh * hp), h = rem / hp, j0 = (rem % hp) * 8;
+        zi_bf16* base = q + (int64_t)(t0 + tt) * ldq + (int64_t)h * d + j0;
+        float a[8], b[8], lo[8], hi[8];
+        unpack(*reinterpret_cast<const uint4*>(base), a);
+        unpack(*reinterpret_cast<const uint4*>(base + half), b);
+        const float* c = cs + tt * rot + j0;
+        const float* sn = c + half;
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            lo[x] = a[x] * c[x] - b[x] * sn[x];
+            hi[x] = b[x] * c[x] + a[x] * sn[x];
+        }
+        *reinterpret_cast<uint4*>(base) = pack(lo);
+        *reinterpret_cast<uint4*>(base + half) = pack(hi);
+    }
+    if (!write_kv) return;
+    // keys into the cache: (token, kv head, eight dims)
+    const int dp = d / 8;
+    for (int i = tid; i < nt * nkv * dp; i += 256) {
+        const int tt = i / (nkv * dp), rem = i % (nkv * dp), h = rem / dp, j0 = (rem % dp) * 8;
+        const int slot = slots[t0 + tt];
+        if (slot < 0 || slot >= cache_slots) continue;     // the host checks the range; never write outside the pool
+        const int64_t page = slot / page_size, off = slot % page_size;
+        const zi_bf16* kr = k + (int64_t)(t0 + tt) * ldk + (int64_t)h * d;
+        float a[8], o8[8];
+        unpack(*reinterpret_cast<const uint4*>(kr + j0), a);
+        if (j0 < rot) {
+            const bool first = j0 < half;
+            const int jj = first ? j0 : j0 - half;
+            float b[8];
+            unpack(*reinterpret_cast<const uint4*>(kr + (first ? j0 + half : jj)), b);
+            const float* c = cs + tt * rot + jj;
+            const float* sn = c + half;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) o8[x] = first ? a[x] * c[x] - b[x] * sn[x] : a[x] * c[x] + b[x] * sn[x];
+        } else {
+#pragma unroll
+            for (int x = 0; x < 8; ++x) o8[x] = a[x];
+        }
+        *reinterpret_cast<uint4*>(kcache + ((page * nkv + h) * page_size + off) * d + j0) = pack(o8);
+    }
+    // values: transposed.  Eight tokens in eight consecutive slots from a multiple of eight: one run per dim.
+    bool run = nt == RKT_TOKENS;
+    const int s0 = slots[t0];
+    if (run) {
+#pragma unroll
+        for (int x = 1; x < RKT_TOKENS; ++x) run = run && slots[t0 + x] == s0 + x;
+        run = run && s0 >= 0 && (s0 & 7) == 0 && s0 + RKT_TOKENS <= cache_slots;
+    }
+    if (run) {
+        const int64_t page = s0 / page_size, off = s0 % page_size;
+        for (int i = tid; i < kvd; i += 256) {
+            const int h = i / d, dim = i % d;
+            uint4 u;
+            u.x = (uint32_t)vt[0 * kvd + i] | ((uint32_t)vt[1 * kvd + i] << 16);
+            u.y = (uint32_t)vt[2 * kvd + i] | ((uint32_t)vt[3 * kvd + i] << 16);
+            u.z = (uint32_t)vt[4 * kvd + i] | ((uint32_t)vt[5 * kvd + i] << 16);
+            u.w = (uint32_t)vt[6 * kvd + i] | ((uint32_t)vt[7 * kvd + i] << 16);
+            *reinterpret_cast<uint4*>(vcache + ((page * nkv + h) * d + dim) * page_size + off) = u;
+        }
+    } else {
+        for (int i = tid; i < nt * kvd; i += 256) {
+            const int tt = i / kvd, col = i % kvd, h = col / d, dim = col % d;
+            const int slot = slots[t0 + tt];
+            if (slot < 0 || slot >= cache_slots) continue;
+            const int64_t page = slot / page_size, off = slot % page_size;
+            vcache[((page * nkv + h) * d + dim) * page_size + off].bits = vt[i];
+        }
+    }
+}
+
+#define ROPE_MANY_TOKENS 64     // from this many tokens on, the tile kernel (bfloat16, 16-byte pieces)
+
 extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, int n, int64_t ldq, int64_t ldk,
                                 int64_t ldv, const int32_t* pos, const int32_t* slots, const float* inv_freq,
                                 void* kcache, void* vcache, int64_t cache_slots, int nh, int nkv, int d, int rot,
@@ -81,6 +200,19 @@ extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, i
     }
     ZI_REQUIRE(rot * sizeof(float) <= 48 * 1024, "rope_kv_store: rotary dims %d too large", rot);
     if (n == 0) return 0;
+    {
+        // the tile kernel: bfloat16, rows and pointers that allow 16-byte pieces, eight rotated dims on one side
+        const bool al = ((uintptr_t)q % 16) == 0 && ldq % 8 == 0 && d % 8 == 0 && (rot / 2) % 8 == 0 &&
+                        (!write_kv || (((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0 && ((uintptr_t)kcache % 16) == 0 &&
+                                       ((uintptr_t)vcache % 16) == 0 && ldk % 8 == 0 && ldv % 8 == 0 && page_size % 8 == 0));
+        const size_t lds = (size_t)RKT_TOKENS * rot * sizeof(float) + (write_kv ? (size_t)RKT_TOKENS * nkv * d * 2 : 0);
+        if (dt == ZI_BF16 && n >= ROPE_MANY_TOKENS && al && lds <= 48 * 1024 && (rot == 0 || inv_freq)) {
+            rope_kv_store_tile_kernel<<<(n + RKT_TOKENS - 1) / RKT_TOKENS, 256, lds, stream>>>(
+                (zi_bf16*)q, (const zi_bf16*)k, (const zi_bf16*)v, ldq, ldk, ldv, pos, slots, inv_freq, (zi_bf16*)kcache,
+                (zi_bf16*)vcache, n, nh, nkv, d, rot, page_size, write_kv, cache_slots);
+            return zi_check_launch("rope_kv_store");
+        }
+    }
     ZI_DISPATCH_DTYPE(dt, T, {
         rope_kv_store_kernel<T><<<n, 256, rot * sizeof(float), stream>>>(
             (T*)q, (const T*)k, (const T*)v, ldq, ldk, ldv, pos, slots, inv_freq, (T*)kcache, (T*)vcache, nh, nkv, d,
