@@ -146,6 +146,21 @@ def test_steps_queued_ahead_give_the_same_tokens(tiny):
     assert got == want
 
 
+def test_steps_queued_ahead_without_graphs(tiny, monkeypatch):
+    """The same with decode steps launched kernel by kernel (no graphs): the tokens of a step queued
+    ahead are copied into the step's batch on the device."""
+    from zedinfer_amd import GenerationConfig
+    monkeypatch.setenv("ZEDINFER_DISABLE_GRAPHS", "1")
+    V = tiny["cfg"]["vocab_size"]
+    prompts = [traces.random_tokens(V, n, seed=60 + i) for i, n in enumerate([9, 31, 3])]
+    ie = engine(tiny)
+    assert not ie.engine.use_graphs
+    results = ie.generate(prompts, GenerationConfig(max_new_tokens=14, ignore_eos=True))
+    assert ie.serving_loop().steps_ahead > 5 and ie.engine.graph_replays == 0
+    for p, r in zip(prompts, results):
+        assert r.output_ids == plain.greedy_generate(tiny["cfg"], tiny["weights"], p, 14)
+
+
 def test_steps_queued_ahead_with_the_serving_kernels(tiny, tmp_path):
     """A bfloat16 checkpoint, greedy, steps queued ahead and replayed as graphs: every token a request
     gets is the best, or within rounding of the best, at its place in the plain run of its sequence."""
