@@ -69,6 +69,20 @@ def test_swiglu(ops, dtype, n, I):
     torch.testing.assert_close(out.float(), ref.to(dtype).float(), **tol(dtype, 1e-6, 1e-2))
 
 
+@pytest.mark.parametrize("n,I", [(64, 64), (136, 200), (8, 8), (2048, 8960), (72, 1000)])
+def test_swiglu_from_the_transposed_product(ops, n, I):
+    """[2I, n] with gate and up rows in blocks of 8 in, [n, I] out: the same bits as the kernel for the
+    product the usual way round."""
+    gu = rnd(n, 2 * I, dtype=torch.bfloat16, scale=3.0)                 # 8 gate columns, their 8 up columns, ...
+    want = ops.swiglu(gu, interleave=8)
+    got = ops.swiglu_t(gu.t().contiguous())
+    assert torch.equal(got, want)
+    x, w = rnd(n, 96, dtype=torch.bfloat16, seed=1), rnd(2 * I, 96, dtype=torch.bfloat16, scale=0.1, seed=2)
+    torch.testing.assert_close(ops.linear_transposed(x, w).float(), ops.linear(x, w).float().t(), atol=2e-2, rtol=2e-2)
+    with pytest.raises(ValueError, match="multiples of 8"):
+        ops.swiglu_t(torch.zeros(32, 12, dtype=torch.bfloat16, device="cuda"))
+
+
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("n,H,eps", [(1, 1536, 1e-6), (7, 100, 1e-5), (3, 5120, 1e-6), (2, 33, 0.1)])
 def test_rms_norm(ops, dtype, n, H, eps):

@@ -114,6 +114,60 @@ swiglu_il8_kernel(zi_bf16* __restrict__ out, const zi_bf16* __restrict__ gu, int
     }
 }
 
+// The same from the transposed product: gut [2I, n] holds, for every block of 8 channels, 8 rows of gate
+// values over the n tokens and then the 8 rows of their up values (the matrix product of the stacked
+// weight with x^T, which the library sometimes makes faster than x with the weight transposed).  Writes
+// out [n, I].  A workgroup takes 64 channels x 64 tokens: a thread reads 16 bytes (8 tokens) of the gate
+// and up rows of two neighbouring channels, the tile turns in LDS (4-byte words of two channels, rows of
+// 33 words), and every token's 64 channels leave as 128 contiguous bytes.  n % 8 == 0, I % 8 == 0.
+__global__ void __launch_bounds__(256)
+swiglu_il8_t_kernel(zi_bf16* __restrict__ out, const zi_bf16* __restrict__ gut, int n, int inter, int64_t ldt) {
+    __shared__ uint32_t tile[64 * 33];
+    const int c0 = blockIdx.x * 64, m0 = blockIdx.y * 64, tid = threadIdx.x;
+    {
+        const int tg = tid % 8, cp = tid / 8;                 // eight tokens, a pair of channels
+        const int c = c0 + 2 * cp, m = m0 + tg * 8;
+        if (c < inter && m < n) {                              // inter and n are multiples of 8: whole pieces
+            const zi_bf16* g = gut + (int64_t)((c / 8) * 16 + c % 8) * ldt + m;
+            const uint4 ga = *reinterpret_cast<const uint4*>(g), gb = *reinterpret_cast<const uint4*>(g + ldt);
+            const uint4 ua = *reinterpret_cast<const uint4*>(g + 8 * ldt), ub = *reinterpret_cast<const uint4*>(g + 9 * ldt);
+            const uint32_t gaw[4] = {ga.x, ga.y, ga.z, ga.w}, gbw[4] = {gb.x, gb.y, gb.z, gb.w};
+            const uint32_t uaw[4] = {ua.x, ua.y, ua.z, ua.w}, ubw[4] = {ub.x, ub.y, ub.z, ub.w};
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int sh = (k & 1) * 16;
+                const float g0 = __uint_as_float((gaw[k / 2] >> sh) << 16), g1 = __uint_as_float((gbw[k / 2] >> sh) << 16);
+                const float u0 = __uint_as_float((uaw[k / 2] >> sh) << 16), u1 = __uint_as_float((ubw[k / 2] >> sh) << 16);
+                tile[(tg * 8 + k) * 33 + cp] = zi_pack_bf16x2(u0 * (g0 / (1.f + expf(-g0))), u1 * (g1 / (1.f + expf(-g1))));
+            }
+        }
+    }
+    __syncthreads();
+    {
+        const int tok = tid / 4, q = tid % 4;                  // a token, 16 of the 64 channels
+        const int m = m0 + tok, c = c0 + q * 16;
+        if (m < n && c < inter) {
+            const uint32_t* src = tile + tok * 33 + q * 8;
+            zi_bf16* dst = out + (int64_t)m * inter + c;
+            *reinterpret_cast<uint4*>(dst) = make_uint4(src[0], src[1], src[2], src[3]);
+            if (c + 8 < inter) *reinterpret_cast<uint4*>(dst + 8) = make_uint4(src[4], src[5], src[6], src[7]);
+        }
+    }
+}
+
+// out [n, inter] from gut [2 * inter, n] (row stride ldt), bfloat16, gate and up rows in blocks of 8.
+extern "C" int zi_swiglu_t(void* out, const void* gut, int dt, int n, int inter, int64_t ldt, hipStream_t stream) {
+    ZI_REQUIRE(dt == ZI_BF16, "swiglu_t: bfloat16 only");
+    ZI_REQUIRE(n >= 0 && inter > 0 && n % 8 == 0 && inter % 8 == 0 && ldt >= n && ldt % 8 == 0,
+               "swiglu_t: tokens %d and channels %d must be multiples of 8 (row stride %lld)", n, inter, (long long)ldt);
+    ZI_REQUIRE(((uintptr_t)out % 16) == 0 && ((uintptr_t)gut % 16) == 0, "swiglu_t: pointers must be aligned to 16 bytes");
+    if (n == 0) return 0;
+    const dim3 grid((inter + 63) / 64, (n + 63) / 64);
+    ZI_REQUIRE(grid.y <= 65535, "swiglu_t: too many tokens");
+    swiglu_il8_t_kernel<<<grid, 256, 0, stream>>>((zi_bf16*)out, (const zi_bf16*)gut, n, inter, ldt);
+    return zi_check_launch("swiglu_t");
+}
+
 extern "C" int zi_swiglu(void* out, int out_dt, const void* gate, const void* up, int dt, int n, int inter,
                          int64_t ld_gate, int64_t ld_up, int interleave, int splits, int64_t split_stride,
                          hipStream_t stream) {

@@ -21,6 +21,7 @@ _PROTOTYPES = {
     "zi_gather_rows": [P, P, I, P, I, I, I, P],
     "zi_add": [P, I, P, I, P, I, L, P],
     "zi_swiglu": [P, I, P, P, I, I, I, L, L, I, I, L, P],
+    "zi_swiglu_t": [P, P, I, I, I, L, P],
     "zi_rmsnorm": [P, I, P, I, P, I, I, I, L, L, F, I, P],
     "zi_add_rmsnorm": [P, I, P, P, I, I, L, P, I, I, I, F, I, P],
     "zi_rope_kv_store": [P, P, P, I, I, L, L, L, P, P, P, P, P, L, I, I, I, I, I, I, P],

@@ -154,6 +154,24 @@ def swiglu(gate: torch.Tensor, up: Optional[torch.Tensor] = None, out: Optional[
     return out
 
 
+def swiglu_t(gate_up_t: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The same from the transposed product: ``gate_up_t`` [2I, n] bfloat16 holds, block of 8 channels by
+    block, 8 rows of gate values and the 8 rows of their up values; returns [n, I].  n and I must be
+    multiples of 8."""
+    _gpu("swiglu_t", gate_up_t, out)
+    ldt, n = _rows(gate_up_t, "swiglu_t input")
+    if gate_up_t.dtype != torch.bfloat16 or gate_up_t.shape[0] % 16 or n % 8:
+        raise ValueError(f"swiglu_t: a bfloat16 [2I, n] tensor with I and n multiples of 8 is needed, got "
+                         f"{tuple(gate_up_t.shape)} {gate_up_t.dtype}")
+    I = gate_up_t.shape[0] // 2
+    if out is None:
+        out = torch.empty((n, I), dtype=torch.bfloat16, device=gate_up_t.device)
+    if tuple(out.shape) != (n, I) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError("swiglu_t: out has the wrong shape or dtype")
+    _lib.call("zi_swiglu_t", _p(out), _p(gate_up_t), BF16, n, I, ldt, _stream())
+    return out
+
+
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None,
              out_dtype: Optional[torch.dtype] = None, add_one: bool = False) -> torch.Tensor:
     """y = (w [+1]) * x * rsqrt(mean(x^2) + eps) over the last dimension of a 2-D x."""
@@ -667,6 +685,23 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     _lib.call("zi_gemm_generic", _p(out), _code(out, "linear out"), _p(x), _code(x, "linear x"), _p(weight),
               _code(weight, "linear weight"), _p(bias), _code(bias, "linear bias") if bias is not None else F32,
               M, N, K, ldx, ldw, ldo, _stream())
+    return out
+
+
+def linear_transposed(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out [N, M] = weight [N, K] . x[M, K]^T: the transposed result of ``linear`` by the library's product
+    with the operands' roles swapped, which it makes faster than ``linear`` at some sizes (bfloat16, many
+    rows, no bias)."""
+    _gpu("linear_transposed", x, weight, out)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.dim() != 2 or weight.dim() != 2 \
+            or x.shape[1] != weight.shape[1] or not x.is_contiguous() or not weight.is_contiguous():
+        raise ValueError("linear_transposed: contiguous bfloat16 x [M, K] and weight [N, K] are needed")
+    M, N = x.shape[0], weight.shape[0]
+    if out is None:
+        out = torch.empty((N, M), dtype=torch.bfloat16, device=x.device)
+    if tuple(out.shape) != (N, M) or out.dtype != torch.bfloat16 or not out.is_contiguous():
+        raise ValueError(f"linear_transposed: out must be a contiguous bfloat16 [{N}, {M}] tensor")
+    torch.mm(weight, x.t(), out=out)
     return out
 
 
