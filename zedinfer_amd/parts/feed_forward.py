@@ -1,6 +1,7 @@
 """Feed-forward parts."""
 from __future__ import annotations
 
+import os
 from typing import Dict
 
 import torch
@@ -42,7 +43,8 @@ class SwiGLU(FeedForward):
     # 31 against 37 at 512, 73 against 67 at 1,024).  Which one is taken for (rows, 2I, H) is measured once,
     # the first time that many rows come: three runs each of product plus activation; the transposed one
     # must win by 5% (two runs of a program then seldom choose differently; their results differ by
-    # rounding only).  The transposed result goes through the activation kernel that turns it back.
+    # rounding only; ZEDINFER_GATE_UP_TRANSPOSED=0 or 1 fixes the choice instead).  The transposed result
+    # goes through the activation kernel that turns it back.
     TRANSPOSED_MIN_ROWS = 128
     _transposed_wins: Dict[tuple, bool] = {}
 
@@ -71,6 +73,9 @@ class SwiGLU(FeedForward):
 
         key = (n, 2 * I, self.hidden)
         wins = SwiGLU._transposed_wins.get(key)
+        forced = os.environ.get("ZEDINFER_GATE_UP_TRANSPOSED", "")      # "0" / "1": no measurement, always that way
+        if wins is None and forced in ("0", "1"):
+            wins = SwiGLU._transposed_wins[key] = forced == "1"
         if wins is None:
             def clock(fn):
                 fn()
