@@ -243,7 +243,7 @@ def main():
         out["prefill"] = {"value": round(PF / pms * 1000.0, 1), "tokens": PF, "ms": round(pms, 3),
                           "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}
         points = {}
-        for b, st in ((1, min(args.steps, 64)), (64, min(args.steps, 32))):
+        for b, st in ((1, min(args.steps, 64)), (64, min(args.steps, 32)), (256, min(args.steps, 16))):
             torch.cuda.empty_cache()
             t, _, _ = measure_decode(factory(b), b, st, min(args.warmup, 8), V, args.prompt_len)
             points[f"decode_b{b}"] = round(t, 2)

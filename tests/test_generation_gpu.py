@@ -405,15 +405,17 @@ def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatc
     assert float((last[0].cpu() - ref[fed["b"] - 1]).abs().max()) < 0.06 * float(ref.abs().max())
 
 
-def test_decode_graphs_with_the_library_product(tiny):
-    """More than 16 decoding requests: the matrix products go to the library, inside the captured
-    graph.  Every replay is checked against eager launches, with eager prompt steps between them."""
+@pytest.mark.parametrize("requests", [20, 70])
+def test_decode_graphs_with_the_library_product(tiny, requests):
+    """More than 16 decoding requests (and more than 64: beyond every few-rows kernel): the matrix
+    products go to the library, inside the captured graph.  Every replay is checked against eager
+    launches, with eager prompt steps between them."""
     from zedinfer_amd.engine import StepEntry
     V = tiny["cfg"]["vocab_size"]
-    fast = engine(tiny, "bfloat16", max_batch_requests=24, num_kv_blocks=128).engine
-    slow = engine(tiny, "bfloat16", max_batch_requests=24, num_kv_blocks=128).engine
+    fast = engine(tiny, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
+    slow = engine(tiny, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
     slow.use_graphs = False
-    names = [f"r{i}" for i in range(20)]
+    names = [f"r{i}" for i in range(requests)]
     toks = {r: traces.random_tokens(V, 40, seed=80 + i) for i, r in enumerate(names)}
     seqs = {(e, r): e.open(r) for e in (fast, slow) for r in names}
     fed = {r: 0 for r in names}
