@@ -405,7 +405,7 @@ def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatc
     assert float((last[0].cpu() - ref[fed["b"] - 1]).abs().max()) < 0.06 * float(ref.abs().max())
 
 
-@pytest.mark.parametrize("requests", [20, 70])
+@pytest.mark.parametrize("requests", [20, 70, 136])
 def test_decode_graphs_with_the_library_product(tiny, requests):
     """More than 16 decoding requests (and more than 64: beyond every few-rows kernel): the matrix
     products go to the library, inside the captured graph.  Every replay is checked against eager

@@ -63,7 +63,7 @@ class SwiGLU(FeedForward):
             ops.linear(x, self.gate_up, out=gu)
             ops.swiglu(gu, out=act, interleave=self.interleave)
 
-        if n < self.TRANSPOSED_MIN_ROWS or n % 8 or not x.is_contiguous() or torch.cuda.is_current_stream_capturing():
+        if n < self.TRANSPOSED_MIN_ROWS or n % 8 or not x.is_contiguous():
             return straight()
         gut = gu.view(-1)[:2 * I * n].view(2 * I, n)      # the same memory
 
@@ -76,6 +76,8 @@ class SwiGLU(FeedForward):
         forced = os.environ.get("ZEDINFER_GATE_UP_TRANSPOSED", "")      # "0" / "1": no measurement, always that way
         if wins is None and forced in ("0", "1"):
             wins = SwiGLU._transposed_wins[key] = forced == "1"
+        if wins is None and torch.cuda.is_current_stream_capturing():
+            return straight()           # nothing can be measured while a graph is recorded
         if wins is None:
             def clock(fn):
                 fn()
