@@ -28,9 +28,14 @@ class Runtime:
         self.device = torch.device(device)
         self.dtype = dtype
         self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self._views: Dict[tuple, torch.Tensor] = {}     # (name, dtype, shape) -> the view handed out last time
 
     def buffer(self, name: str, shape: Tuple[int, ...], dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         dtype = dtype or self.dtype
+        vkey = (name, dtype, tuple(shape))
+        view = self._views.get(vkey)
+        if view is not None:
+            return view                 # steps of a shape seen before ask for the same views again
         n = 1
         for s in shape:
             n *= int(s)
@@ -39,7 +44,11 @@ class Runtime:
         if buf is None or buf.numel() < n:
             buf = torch.empty((max(n, 1),), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-        return buf[:n].view(shape)
+            self._views = {k: v for k, v in self._views.items() if k[:2] != key}    # they point into the old one
+        if len(self._views) >= 4096:
+            self._views.clear()
+        view = self._views[vkey] = buf[:n].view(tuple(shape))
+        return view
 
     def reserve(self, name: str, numel: int, dtype: Optional[torch.dtype] = None) -> None:
         self.buffer(name, (numel,), dtype)
