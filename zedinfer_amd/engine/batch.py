@@ -76,6 +76,8 @@ class DeviceBatch:
     # every entry brings exactly one token (a pure decode step): no token's keys are written by
     # another token of the step, so a mixer may store and attend in one kernel
     single_tokens: bool = False
+    # logits are wanted at every token, in order: nothing needs to be picked
+    all_rows_wanted: bool = False
     # what parts compute once per step and share over the layers (for instance the rotation angles),
     # by a key of their own
     shared: dict = field(default_factory=dict)
@@ -194,7 +196,8 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
                        max_short_keys=max_short, max_long_keys=max_long, tile_entry=views[10], tile_off=views[11],
                        num_tiles=len(tiles), host_start=starts,
                        host_len=lens_a, host_past=past, host_slot=slot, host_image=image,
-                       single_tokens=bool((lens_a == 1).all()))
+                       single_tokens=bool((lens_a == 1).all()),
+                       all_rows_wanted=bool(R == N and (logit_rows == np.arange(N, dtype=np.int32)).all()))
 
 
 class DecodeImage:

@@ -128,6 +128,8 @@ class DecoderModel:
         if delta is not None and delta.dim() == 3:
             # float32 partial sums (few tokens): norm every row, then pick the wanted ones
             x_all = self.final_norm.add_forward(resid, delta)
+            if getattr(batch, "all_rows_wanted", False):
+                return self.lm_head.forward(x_all)
             x = ops.gather_rows(x_all, rows, out=self.rt.buffer("norm_rows", (batch.num_logit_rows, self.hidden_size),
                                                                x_all.dtype))
             return self.lm_head.forward(x)
