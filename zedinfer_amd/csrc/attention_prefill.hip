@@ -395,9 +395,11 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 // (global_load_lds_dwordx4): no registers, no address arithmetic and no LDS stores are spent on staging.
 // One load instruction of a wavefront fills 1 KB of LDS, lane l the 16 bytes at l * 16; which 16 bytes of
 // the cache a lane asks for is free, so the tiles keep the order the matrix cores want (keys permuted as
-// above, values transposed) and their rows are not padded but rotated: the 16-byte piece c of row r sits
-// at place (c + r) mod pieces-per-row, which spreads a quarter-wave's reads over the banks as the padding
-// did.  Two buffers, each a pair of LDS arrays of its own, used in turn by an unrolled loop: the loads
+// above, values transposed) and their rows are not padded but swizzled: the 16-byte piece c of row r sits
+// at place c xor (r mod pieces-per-row) (rows of 128 bytes: c xor (r / 2 mod 8), two rows share the 64
+// banks), which spreads a quarter-wave's reads over the banks without a conflict: 16-byte reads in this
+// order run at the rate of consecutive ones, those of rows padded by 16 bytes or rotated by the row number
+// an eighth slower.  Two buffers, each a pair of LDS arrays of its own, used in turn by an unrolled loop: the loads
 // of the next block are issued right after the barrier that makes this block visible, so the compiler's
 // wait before a barrier (it waits for every load into LDS there) never waits for a block that is still
 // needed later.  Values of keys past the last key and of pages that a window has given back are loaded
@@ -421,6 +423,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     constexpr int KCH = PF_BS * KC, VCH = D * VC;    // pieces of the two tiles
     constexpr int THREADS = PF_WAVES * ZI_WAVE;
     constexpr int KI = KCH / THREADS, VI = VCH / THREADS;   // load instructions a wavefront issues per tile
+    constexpr int KSW = 16 / KC;                     // key rows that share 256 bytes of LDS (and one swizzle)
     __shared__ __attribute__((aligned(16))) uint4 k_a[KCH];
     __shared__ __attribute__((aligned(16))) uint4 k_b[KCH];
     __shared__ __attribute__((aligned(16))) uint4 v_a[VCH];
@@ -475,7 +478,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     if (tid <= (khi >> ps_shift) - pi_first) bt_lds[tid] = bt[pi_first + tid < pi_last ? pi_first + tid : pi_last];
     // What a lane loads does not change from block to block: for its KI pieces of the key tile the key
     // (as an offset into the block) and the piece of its row, for its VI pieces of the value tile the
-    // dim and the eight keys.  Place L of a tile is row L / pieces-per-row; the piece there is rotated.
+    // dim and the eight keys.  Place L of a tile is row L / pieces-per-row; the piece there is swizzled.
     int k_key[KI], k_piece[KI], v_dim[VI], v_key[VI];
 #pragma unroll
     for (int i = 0; i < KI; ++i) {
@@ -483,13 +486,13 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
         const int rho = L / KC;
         const int t = (rho % PF_BN) / 16, rr = rho % 16;
         k_key[i] = (rho / PF_BN) * PF_BN + (t / 2) * 32 + (rr / 4) * 8 + (t % 2) * 4 + rr % 4;
-        k_piece[i] = (L % KC - rho) & (KC - 1);
+        k_piece[i] = (L % KC) ^ ((rho / KSW) & (KC - 1));
     }
 #pragma unroll
     for (int i = 0; i < VI; ++i) {
         const int L = (wave * VI + i) * ZI_WAVE + lane;
         v_dim[i] = L / VC;
-        v_key[i] = ((L % VC - v_dim[i]) & (VC - 1)) * 8;
+        v_key[i] = ((L % VC) ^ (v_dim[i] & (VC - 1))) * 8;
     }
     const zi_bf16* kbase = kcache + (int64_t)g * ps * D;
     const zi_bf16* vbase = vcache + (int64_t)g * D * ps;
@@ -525,7 +528,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             if (tid < D) {
                 const int piece = (kmax - kb) / 8, keep = (kmax + 1) & 7;
                 pf_pack val;
-                uint4* at = vl + tid * VC + ((piece + tid) & (VC - 1));
+                uint4* at = vl + tid * VC + (piece ^ (tid & (VC - 1)));
                 val.u = *at;
 #pragma unroll
                 for (int x = 0; x < 8; ++x)
@@ -546,7 +549,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
 #pragma unroll
             for (int dk = 0; dk < DK; ++dk) {
                 pf_pack a;
-                a.u = kl[rho * KC + ((dk * 4 + j + rho) & (KC - 1))];
+                a.u = kl[rho * KC + ((dk * 4 + j) ^ ((rho / KSW) & (KC - 1)))];
                 s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, qop[dk], s[t], 0, 0, 0);
             }
         }
@@ -607,7 +610,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 pf_pack a;
-                a.u = vl[dim * VC + ((kh * 8 + b * 4 + j + dim) & (VC - 1))];
+                a.u = vl[dim * VC + ((kh * 8 + b * 4 + j) ^ (dim & (VC - 1)))];
                 o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[b].b, o[dd], 0, 0, 0);
             }
         }
