@@ -23,7 +23,7 @@ typedef __attribute__((ext_vector_type(4))) unsigned gm_u32x4_t;
 #define GM_WAVES 4
 #define GM_ROWS 64          // weight rows per workgroup
 #define GM_KB 128
-#define GM_XS (GM_KB + 8)   // LDS row stride of the x slice, in elements
+#define GM_XS GM_KB         // LDS row stride, in elements: rows of 16 pieces of 16 bytes, piece c of row r at place c xor (r mod 16)
 #define GM_TARGET_WGS 384
 
 #define GM_MODE_PLAIN 0
@@ -67,8 +67,8 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
         const int n = n0 + c * 4 + j;
         wrow[c] = w + (int64_t)(n < N ? n : N - 1) * ldw;
     }
-    uint16_t* wt_put = &wt[wave][j * GM_XS + wq * 8];        // + c * 4 rows
-    const uint16_t* wt_get = &wt[wave][r * GM_XS + j * 8];   // + c * 32 values
+    // LDS rows are not padded but swizzled (16-byte reads in operand order then run at the full LDS rate)
+    uint16_t* const wt_w = &wt[wave][0];
 
     // what this thread stages of a block's x slice: MT pieces of 16 bytes (row srow + 16 * t, piece spc)
     const int srow = tid / 16, spc = tid % 16;
@@ -95,7 +95,8 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     };
     auto stash = [&](const int slot, int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < MT; ++t) *reinterpret_cast<gm_u32x4_t*>(&xs[b][(t * 16 + srow) * GM_XS + spc * 8]) = xring[slot][t];
+        for (int t = 0; t < MT; ++t)
+            *reinterpret_cast<gm_u32x4_t*>(&xs[b][(t * 16 + srow) * GM_XS + (spc ^ srow) * 8]) = xring[slot][t];
     };
     gm_f32x4_t acc[MT];
 #pragma unroll
@@ -117,15 +118,16 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
         // LDS serves a wavefront's instructions in order, so no barrier stands between put and get
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-            *reinterpret_cast<gm_u32x4_t*>(wt_put + c * 4 * GM_XS) = gm_keep(ring[slot][c], kb * GM_KB + wq * 8 < K);
+            *reinterpret_cast<gm_u32x4_t*>(wt_w + (c * 4 + j) * GM_XS + (wq ^ (c * 4 + j)) * 8) =
+                gm_keep(ring[slot][c], kb * GM_KB + wq * 8 < K);
         gm_pack bb[4][MT], a[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
             for (int t = 0; t < MT; ++t)
-                bb[c][t].u = *reinterpret_cast<const gm_u32x4_t*>(&xs[cur][(t * 16 + r) * GM_XS + c * 32 + j * 8]);
+                bb[c][t].u = *reinterpret_cast<const gm_u32x4_t*>(&xs[cur][(t * 16 + r) * GM_XS + ((c * 4 + j) ^ r) * 8]);
 #pragma unroll
-        for (int c = 0; c < 4; ++c) a[c].u = *reinterpret_cast<const gm_u32x4_t*>(wt_get + c * 32);
+        for (int c = 0; c < 4; ++c) a[c].u = *reinterpret_cast<const gm_u32x4_t*>(wt_w + r * GM_XS + ((c * 4 + j) ^ r) * 8);
 #pragma unroll
         for (int c = 0; c < 4; ++c)
 #pragma unroll
