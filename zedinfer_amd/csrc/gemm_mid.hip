@@ -81,14 +81,17 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     // stores; columns past K would count the last eight twice, so the weights are zeroed there, when
     // they are used.  A block's x is requested before its weights: loads return in order, and x, which
     // comes from the cache and is wanted a step earlier, must not queue behind weights from memory.
-    const int xm_last = M - 1;
+    const zi_bf16* xrow[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const int m = t * 16 + srow;
+        xrow[t] = x + (int64_t)(m < M ? m : M - 1) * ldx;
+    }
     auto fetch = [&](const int slot, int kb) __attribute__((always_inline)) {
         const int k0 = kb * GM_KB;
+        const int kx = k0 + spc * 8 < K ? k0 + spc * 8 : K - 8;
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-            const int m = t * 16 + srow, k = k0 + spc * 8;
-            xring[slot][t] = *reinterpret_cast<const gm_u32x4_t*>(x + (int64_t)(m < M ? m : xm_last) * ldx + (k < K ? k : K - 8));
-        }
+        for (int t = 0; t < MT; ++t) xring[slot][t] = *reinterpret_cast<const gm_u32x4_t*>(xrow[t] + kx);
         const int k = k0 + wq * 8;
 #pragma unroll
         for (int c = 0; c < 4; ++c) ring[slot][c] = *reinterpret_cast<const gm_u32x4_t*>(wrow[c] + (k < K ? k : K - 8));
