@@ -128,6 +128,9 @@ def batch_bench(argv: Optional[List[str]] = None) -> int:
     p.add_argument("-p", "--prefill-len", type=int, default=128)
     p.add_argument("-d", "--decode-len", "--max-tokens", type=int, default=128, dest="decode_len")
     p.add_argument("-r", "--rounds", type=int, default=1)
+    p.add_argument("--no-warmup", action="store_true",
+                   help="count the first batch too (it records the decode graphs and measures the matrix products' "
+                        "way round once; the reference has no such first-time costs and no warm-up round)")
     args = p.parse_args(argv)
     if args.decode_len <= 0:
         print("--decode-len/--max-tokens must be > 0 for benchmark runs", file=sys.stderr)
@@ -149,7 +152,7 @@ def batch_bench(argv: Optional[List[str]] = None) -> int:
     lo, hi = (100, min(30000, V - 1)) if V > 200 else (0, V - 1)
     total_ms, total_tokens = 0.0, 0
     loop = ie.serving_loop()
-    for r in range(args.rounds):
+    for r in range(0 if args.no_warmup else -1, args.rounds):
         reqs = []
         t0 = time.perf_counter()
         for i in range(args.batch_size):
@@ -163,6 +166,9 @@ def batch_bench(argv: Optional[List[str]] = None) -> int:
         if failed:
             print(f"{len(failed)} request(s) failed: {failed[0].error}", file=sys.stderr)
         n = sum(len(q.output_ids) for q in reqs)
+        if r < 0:
+            print(f"Warm-up (not counted): {args.batch_size} requests, {n} tokens generated, {ms:.2f} ms")
+            continue
         total_ms, total_tokens = total_ms + ms, total_tokens + n
         print(f"Round {r + 1}: {args.batch_size} requests, {n} tokens generated, {ms:.2f} ms")
     avg_ms, avg_tok = total_ms / args.rounds, total_tokens / args.rounds
