@@ -188,6 +188,51 @@ def test_steps_queued_ahead_with_the_serving_kernels(tiny, tmp_path):
     assert not ie.engine.cache.live
 
 
+@pytest.mark.parametrize("seed", [0, 1])
+def test_requests_arriving_and_cancelled_while_the_loop_runs(tiny, seed):
+    """Requests of random lengths arrive while others decode, a pool so small that admission has to
+    wait for pages, some requests cancelled on the way: every request that finishes has the tokens it
+    gets alone, a cancelled one a prefix of them, and every page and slot is back at the end."""
+    import random
+    from zedinfer_amd import GenerationConfig, InferenceRequest
+    rng = random.Random(100 + seed)
+    V = tiny["cfg"]["vocab_size"]
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    ie = engine(tiny, num_kv_blocks=(160 + 16) // ps + 6, max_prefill_tokens=24, max_batch_tokens=40,
+                max_batch_requests=4, generation_reserve=8)
+    loop = ie.serving_loop()
+    todo = []
+    for i in range(18):
+        prompt = traces.random_tokens(V, rng.choice([1, 2, 3, 9, 17, 33, 48, 70]), seed=200 + 50 * seed + i)
+        todo.append((rng.randrange(0, 40), prompt, rng.randrange(1, 15)))
+    todo.sort(key=lambda x: x[0])
+    cancel_at = {3: rng.randrange(5, 30), 8: rng.randrange(10, 45), 12: rng.randrange(20, 60)}
+    reqs, step = [], 0
+    while todo or loop.scheduler.has_work():
+        while todo and todo[0][0] <= step:
+            _, prompt, n = todo.pop(0)
+            reqs.append(loop.submit_async(InferenceRequest(prompt, GenerationConfig(max_new_tokens=n, ignore_eos=True))))
+        for i, at in cancel_at.items():
+            if at == step and i < len(reqs):
+                reqs[i].cancelled = True
+        loop.step()
+        step += 1
+        assert step < 2000
+    assert len(reqs) == 18 and loop.steps_ahead > 0
+    finished = 0
+    for i, q in enumerate(reqs):
+        assert q.done and q.error is None, (i, q.error)
+        want = plain.greedy_generate(tiny["cfg"], tiny["weights"], q.input_ids, q.config.max_new_tokens)
+        if q.cancelled and len(q.output_ids) < len(want):
+            assert q.output_ids == want[:len(q.output_ids)], i
+        else:
+            assert q.output_ids == want, i
+            finished += 1
+    assert finished >= 15
+    ie.engine.cache.check()
+    assert not ie.engine.cache.live
+
+
 def test_out_of_pages_fails_the_request_not_the_engine(tiny):
     from zedinfer_amd import GenerationConfig
     ie = engine(tiny, num_kv_blocks=4)
