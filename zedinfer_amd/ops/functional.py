@@ -645,8 +645,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     """out[M,N] = x[M,K] . weight[N,K]^T + bias[N], accumulated in float32
     (reference: src/backend/ops/linear/op.cpp:57-58).
 
-    bfloat16 inputs with bfloat16 weights and output go to the library matrix product, as
-    the reference sends them to its vendor library (reference:
+    bfloat16 inputs with bfloat16 weights and output (or float32 output and more than 64 rows) go
+    to the library matrix product, as the reference sends them to its vendor library (reference:
     src/backend/ops/linear/nvidia/linear_cublas.cu:134-231); every other pairing, and all of
     the float32 path, runs the plain FMA kernel, which has no reduced-precision mode."""
     _gpu("linear", x, weight, bias, out)
@@ -666,6 +666,11 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         return out
     bf = torch.bfloat16
     all_bf = x.dtype == bf and weight.dtype == bf and (bias is None or bias.dtype == bf)
+    if all_bf and out.dtype == torch.float32 and M > SKINNY_MAX_ROWS and bias is None and out.is_contiguous():
+        # float32 output for many rows (logits of a large decode batch or of every place of a prompt): the
+        # library's product with float32 results, one pass over the weights instead of one per 64 rows
+        torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
+        return out
     if all_bf and (M <= FEW_ROWS or out.dtype == torch.float32) and _skinny_ok(x, weight, K, ldx, ldw):
         # few rows (decoding), or float32 output (logits): the hand-written matrix-core kernel
         lib = _lib.load()
