@@ -237,12 +237,12 @@ def test_rope_kv_store(ops, dtype):
 @pytest.mark.parametrize("nh,nkv,d,rot,ps", [(12, 2, 128, 128, 16), (6, 2, 48, 32, 8), (3, 1, 64, 0, 32), (5, 5, 80, 80, 8)])
 @pytest.mark.parametrize("layout", ["runs", "shifted", "scattered"])
 def test_rope_kv_store_many_tokens(ops, nh, nkv, d, rot, ps, layout):
-    """From 64 tokens on bfloat16 takes the kernel that moves 16-byte pieces: against the kernel for few
+    """From 1,024 tokens on bfloat16 takes the kernel that moves 16-byte pieces: against the kernel for few
     tokens, eight tokens at a time (the same arithmetic; a product may be fused differently, hence one
     rounding step), with slots in runs from multiples of eight (a value run is one store), runs that start
     elsewhere, slots scattered, a tail of fewer than eight tokens, and slots out of range that are skipped."""
     dtype = torch.bfloat16
-    n, pages, theta = 203, 40, 5e4
+    n, pages, theta = 1051, 160, 5e4
     qkv = rnd(n, (nh + 2 * nkv) * d + 8, dtype=dtype)[:, 8:]             # rows that do not start the buffer
     q, k, v = qkv[:, :nh * d], qkv[:, nh * d:(nh + nkv) * d], qkv[:, (nh + nkv) * d:]
     pos = torch.arange(1000, 1000 + n, dtype=torch.int32, device="cuda")

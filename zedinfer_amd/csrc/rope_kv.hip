@@ -183,7 +183,10 @@ rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k
     }
 }
 
-#define ROPE_MANY_TOKENS 64     // from this many tokens on, the tile kernel (bfloat16, 16-byte pieces)
+// From this many tokens on, the tile kernel (bfloat16, 16-byte pieces).  Below, a workgroup a token is
+// faster (256 tokens with scattered slots, a large decode batch: 4.2 against 8.3 us; the two meet at 1,024
+// tokens in one run of slots, and 2,048 take 7.0 against 8.8 us).
+#define ROPE_MANY_TOKENS 1024
 
 extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, int n, int64_t ldq, int64_t ldk,
                                 int64_t ldv, const int32_t* pos, const int32_t* slots, const float* inv_freq,
