@@ -199,7 +199,7 @@ def test_requests_arriving_and_cancelled_while_the_loop_runs(tiny, seed):
     V = tiny["cfg"]["vocab_size"]
     ps = tiny_configs.PAGE_SIZES[tiny["name"]]
     ie = engine(tiny, num_kv_blocks=(160 + 16) // ps + 6, max_prefill_tokens=24, max_batch_tokens=40,
-                max_batch_requests=4, generation_reserve=8)
+                max_batch_requests=4, generation_reserve=16)      # the reserve covers every request's new tokens: admission waits, nothing fails
     loop = ie.serving_loop()
     todo = []
     for i in range(18):
