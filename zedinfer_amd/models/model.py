@@ -133,6 +133,9 @@ class DecoderModel:
             x = ops.gather_rows(x_all, rows, out=self.rt.buffer("norm_rows", (batch.num_logit_rows, self.hidden_size),
                                                                x_all.dtype))
             return self.lm_head.forward(x)
+        if getattr(batch, "all_rows_wanted", False):      # every row, in order: nothing to pick
+            x = self.final_norm.add_forward(resid, delta) if delta is not None else self.final_norm.forward(resid)
+            return self.lm_head.forward(x)
         r = self.rt.buffer("resid_rows", (batch.num_logit_rows, self.hidden_size), torch.float32)
         ops.gather_rows(resid, rows, out=r)
         if delta is not None:
