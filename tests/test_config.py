@@ -93,3 +93,23 @@ def test_scheduler_config_defaults():
     assert s.gpu_memory_utilization == pytest.approx(0.9)
     with pytest.raises(ValueError):
         SchedulerConfig(kv_block_size=0).validate()
+
+
+def test_workspaces_that_are_outgrown_stay_alive():
+    """A graph captured with a workspace goes on using it after a larger step has outgrown it: the old
+    allocation must keep its address and its contents, and views of a shape come back as they were."""
+    import torch
+    from zedinfer_amd.parts import Runtime
+    rt = Runtime("cpu", torch.float32)
+    small = rt.buffer("x", (4,))
+    small.fill_(3.0)
+    assert rt.buffer("x", (4,)) is small and rt.outgrown_bytes() == 0
+    ptr = small.data_ptr()
+    large = rt.buffer("x", (400,))
+    large.fill_(7.0)
+    other = [torch.full((4,), 9.0) for _ in range(64)]      # allocations that could take freed memory
+    assert small.data_ptr() == ptr and bool((small == 3.0).all()) and rt.outgrown_bytes() == 16
+    assert rt.buffer("x", (4,)).data_ptr() == large.data_ptr()    # new steps use the new allocation
+    grown = rt.buffer("x", (401,))
+    assert grown.data_ptr() != large.data_ptr() and rt._buffers[("x", torch.float32)].numel() >= 600
+    del other

@@ -23,7 +23,7 @@ from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
 from ..sampling.sampler import default_sampling
 from ..weights import load_weights, random_weights
-from .batch import DecodeImage, DeviceBatch, StagingRing, StepEntry, build_device_batch
+from .batch import SHORT_ENTRY, DecodeImage, DeviceBatch, StagingRing, StepEntry, build_device_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            "f32": torch.float32}
@@ -76,6 +76,13 @@ class Engine:
         self.graph_limit = 48
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.graph_replays = 0
+        # A step that is one portion of one prompt is padded to the next multiple of PROMPT_GRAPH_STEP
+        # tokens and captured too (launching a step kernel by kernel costs the host about 5 ms, more than
+        # the GPU needs for a short prompt), one graph per (padded tokens, wanted rows, table widths,
+        # attention launch size).  Portions of more tokens are bound by the GPU and run as they are.
+        self.prompt_graph_max_tokens = int(os.environ.get("ZEDINFER_PROMPT_GRAPH_MAX_TOKENS", "1024"))
+        self._prompt_graphs: Dict[tuple, "_DecodeGraph"] = {}
+        self.prompt_graph_replays = 0
 
     # ---- construction ------------------------------------------------------------
     @classmethod
@@ -127,6 +134,7 @@ class Engine:
         other.memories = other.cache.memories(self.fc.schedule)
         other.staging = StagingRing(self.device)
         other._graphs = {}
+        other._prompt_graphs = {}
         other.steps_run = other.graph_replays = 0
         return other
 
@@ -159,6 +167,9 @@ class Engine:
             self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
         if self.use_graphs and 0 < len(entries) <= self.graph_max_entries and single:
             logits = self._graph_step(entries, token_source)
+        elif (self.use_graphs and len(entries) == 1 and token_source is None and len(entries[0].want) <= 1
+              and SHORT_ENTRY < len(entries[0].tokens) <= self.prompt_graph_max_tokens):
+            logits = self._prompt_graph_step(entries)
         else:
             batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging)
             if token_source is not None:
@@ -205,6 +216,47 @@ class Engine:
         logits = self.model.run(batch, self.memories)      # allocates every workspace; its result is this step's
         if dg.warm:
             # the second step of this kind: capture (nothing runs), to be replayed from the third on
+            torch.cuda.synchronize(self.device)
+            first = logits.clone() if logits is not None else None
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                dg.logits = self.model.run(batch, self.memories)
+            dg.graph = g
+            return first
+        dg.warm = True
+        return logits
+
+
+    # ---- one portion of one prompt as a graph -------------------------------------------
+    PROMPT_GRAPH_STEP = 64
+
+    def _prompt_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """A step of one entry of more than SHORT_ENTRY tokens, run as if it brought a multiple of
+        PROMPT_GRAPH_STEP tokens (see ``build_device_batch``): the first step of a kind runs eagerly, the
+        second is captured, later ones replay."""
+        e = entries[0]
+        n = len(e.tokens)
+        padded = -(-n // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
+        R = len(e.want)
+        widths = tuple(_pow2_at_least(len(e.seq.pages[g]), 8) for g in range(len(self.cache.groups)))
+        keys_bucket = _pow2_at_least(e.seq.length + padded, 2048)
+        key = (padded, R, widths, keys_bucket)
+        dg = self._prompt_graphs.get(key)
+        if dg is None:
+            if len(self._prompt_graphs) >= self.graph_limit:
+                self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
+            size = 8 * padded + R + 16 + sum(padded + w for w in widths) + 64
+            dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
+            self._prompt_graphs[key] = dg
+        batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
+                                   pad_to=padded)
+        batch.max_long_keys = keys_bucket
+        if dg.graph is not None:
+            dg.graph.replay()
+            self.prompt_graph_replays += 1
+            return dg.logits
+        logits = self.model.run(batch, self.memories)
+        if dg.warm:
             torch.cuda.synchronize(self.device)
             first = logits.clone() if logits is not None else None
             g = torch.cuda.CUDAGraph()

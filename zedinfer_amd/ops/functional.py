@@ -789,12 +789,17 @@ def reduce_sums(sums: torch.Tensor, bias: Optional[torch.Tensor] = None, out: Op
 SKINNY_MAX_ROWS = 64   # rows the few-rows kernels take in one launch
 FEW_ROWS = 64          # up to here they beat the library product: the weights stream once, x stays on the chip
 _WORKSPACES = {}
+_OUTGROWN_WORKSPACES: list = []
 
 
 def _workspace(device: torch.device, floats: int) -> torch.Tensor:
-    """A float32 scratch buffer per device that only grows (split partial sums live in it)."""
+    """A float32 scratch buffer per device that only grows (split partial sums live in it).  One that is
+    outgrown is kept: a captured graph may still use it."""
     ws = _WORKSPACES.get(device)
     if ws is None or ws.numel() < floats:
+        if ws is not None:
+            _OUTGROWN_WORKSPACES.append(ws)
+            floats = max(floats, 2 * ws.numel())
         ws = torch.empty((max(floats, 1 << 20),), dtype=torch.float32, device=device)
         _WORKSPACES[device] = ws
     return ws

@@ -21,7 +21,11 @@ class Runtime:
 
     ``buffer(name, shape)`` hands out a view into a named allocation that only
     ever grows, so that steady-state steps allocate nothing and buffers keep
-    their addresses (what a captured graph needs).
+    their addresses (what a captured graph needs).  When a larger step outgrows
+    an allocation, the old one is kept, not freed: graphs captured earlier go on
+    reading and writing it, and freed memory would by then belong to someone
+    else.  Allocations grow by at least half, so what is kept stays below twice
+    the largest.
     """
 
     def __init__(self, device: torch.device | str, dtype: torch.dtype):
@@ -29,6 +33,7 @@ class Runtime:
         self.dtype = dtype
         self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
         self._views: Dict[tuple, torch.Tensor] = {}     # (name, dtype, shape) -> the view handed out last time
+        self._outgrown: list = []                       # allocations that captured graphs may still use
 
     def buffer(self, name: str, shape: Tuple[int, ...], dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         dtype = dtype or self.dtype
@@ -42,13 +47,22 @@ class Runtime:
         key = (name, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < n:
-            buf = torch.empty((max(n, 1),), dtype=dtype, device=self.device)
+            if buf is not None:
+                self._outgrown.append(buf)
+                n_alloc = max(n, buf.numel() + buf.numel() // 2)
+            else:
+                n_alloc = max(n, 1)
+            buf = torch.empty((n_alloc,), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self._views = {k: v for k, v in self._views.items() if k[:2] != key}    # they point into the old one
         if len(self._views) >= 4096:
             self._views.clear()
         view = self._views[vkey] = buf[:n].view(tuple(shape))
         return view
+
+    def outgrown_bytes(self) -> int:
+        """Bytes of allocations that were outgrown and are kept for graphs captured before."""
+        return sum(b.numel() * b.element_size() for b in self._outgrown)
 
     def reserve(self, name: str, numel: int, dtype: Optional[torch.dtype] = None) -> None:
         self.buffer(name, (numel,), dtype)
