@@ -407,8 +407,9 @@ def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype, tmp_path):
 def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
     """A step that is one portion of one prompt is padded to a multiple of 64 tokens and, from the third
     step of a shape on, replayed as a graph.  Every step is checked against an engine that launches
-    eagerly and does not pad: portions of different lengths that share a graph, with and without a wanted
-    row, decode steps (graphs of their own) and a mixed step between them, and at the end the caches, which
+    eagerly and does not pad: portions of different lengths that share a graph, alone and beside decoded
+    tokens, with and without a wanted row, decode steps (graphs of their own) and a step of two portions
+    between them, and at the end the caches, which
     the padding must not have touched: decoding on gives the plain implementation's logits."""
     from zedinfer_amd.engine import StepEntry
     V = tiny["cfg"]["vocab_size"]
@@ -416,10 +417,10 @@ def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
         folder16 = tiny_configs.write_tiny(str(tmp_path / "bf16"), tiny["name"], dtype=torch.bfloat16)
         tiny = dict(tiny, folder=folder16, weights=plain.load_folder(folder16)[1])
         dtype = "bfloat16"
-    fast, slow = engine(tiny, dtype, num_kv_blocks=400).engine, engine(tiny, dtype, num_kv_blocks=400).engine
+    fast, slow = engine(tiny, dtype, num_kv_blocks=700).engine, engine(tiny, dtype, num_kv_blocks=700).engine
     assert fast.use_graphs
     slow.use_graphs = False
-    toks = {r: traces.random_tokens(V, 600, seed=80 + i) for i, r in enumerate("abcd")}
+    toks = {r: traces.random_tokens(V, 1200, seed=80 + i) for i, r in enumerate("abcd")}
     fed = {r: 0 for r in toks}
     seqs = {}
     scale = [1.0]
@@ -435,6 +436,7 @@ def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
             outs.append(eng.step(entries))
         for r, n in plan:
             fed[r] += n
+            assert fed[r] <= len(toks[r])
         if outs[1] is None:
             assert outs[0] is None
         else:
@@ -449,10 +451,14 @@ def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
         for r in "abcd":
             both([(r, n)], want)
         both([("a", 1), ("b", 1), ("c", 1)])              # a decode graph between them
-    both([("a", 30), ("d", 1)])                           # a mixed step runs eagerly
+    before = fast.prompt_graph_replays
+    for i in range(8):               # a portion beside decoded tokens: recorded the fourth time, then replayed
+        both([("a", 1), ("d", 40 + 3 * i), ("b", 1)])
+    assert fast.prompt_graph_replays >= before + 4
+    both([("a", 30), ("d", 3)])                           # two portions: launched kernel by kernel
     for r in "bcd":
         both([(r, 77)], True)
-    assert fast.prompt_graph_replays >= 10 and slow.prompt_graph_replays == 0
+    assert fast.prompt_graph_replays >= 14 and slow.prompt_graph_replays == 0
     for _ in range(3):
         last = both([("a", 1), ("b", 1), ("c", 1), ("d", 1)])
     ref = plain.forward(tiny["cfg"], tiny["weights"], toks["d"][:fed["d"]])

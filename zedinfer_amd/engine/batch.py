@@ -89,10 +89,10 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
                        static: Optional[torch.Tensor] = None, pad_to: int = 0) -> DeviceBatch:
     """Check the entries, then pack every index array into one host buffer and copy it over once.
 
-    ``pad_to`` (one entry only): the entry is run as if it brought that many tokens.  The tokens past its
-    own are token 0 at the positions that follow; they have no place in the cache (slot -1: nothing is
-    stored for them) and no token of the entry sees them, so they change nothing but the shapes, which
-    then recur from step to step.
+    ``pad_to``: the one entry that brings more than SHORT_ENTRY tokens is run as if it brought that many.
+    The tokens past its own are token 0 at the positions that follow; they have no place in the cache
+    (slot -1: nothing is stored for them) and no real token sees them, so they change nothing but the
+    shapes, which then recur from step to step.
 
     ``table_widths`` pads each group's block table to a given width; ``static`` is a device buffer
     the arrays are copied into instead of a fresh one (the layout depends only on the number of
@@ -118,9 +118,11 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     E = len(entries)
     real = list(lens)
     if pad_to:
-        if E != 1 or pad_to < lens[0]:
-            raise ValueError("only a single entry can be padded, and only to more tokens than it brings")
-        lens = [int(pad_to)]
+        longs = [i for i, n in enumerate(lens) if n > SHORT_ENTRY]
+        if len(longs) != 1 or pad_to < lens[longs[0]]:
+            raise ValueError("padding needs exactly one entry of more than SHORT_ENTRY tokens, and no fewer tokens than it brings")
+        lens = list(lens)
+        lens[longs[0]] = int(pad_to)
     N = int(sum(lens))
     starts = np.zeros(E, dtype=np.int32)
     starts[1:] = np.cumsum(lens)[:-1]
@@ -128,9 +130,8 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     slot = np.array([e.seq.slot for e in entries], dtype=np.int32)
     lens_a = np.array(lens, dtype=np.int32)
 
-    token_ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
-    if N > token_ids.size:
-        token_ids = np.concatenate([token_ids, np.zeros(N - token_ids.size, dtype=np.int64)])
+    token_ids = np.concatenate([np.concatenate([np.asarray(e.tokens, dtype=np.int64), np.zeros(n - r, dtype=np.int64)])
+                                for e, n, r in zip(entries, lens, real)])
     if token_ids.min() < 0 or token_ids.max() >= vocab_size:
         bad = token_ids[(token_ids < 0) | (token_ids >= vocab_size)][0]
         raise ValueError(f"token id {int(bad)} is outside the vocabulary of {vocab_size}")
@@ -144,8 +145,8 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     group_slots, group_tables, widths = [], [], []
     for g in range(G):
         group_slots.append(np.concatenate(
-            [cache.token_slots(e.seq, g, int(p), n) for e, p, n in zip(entries, past, real)]
-            + [np.full(N - sum(real), -1, dtype=np.int32)]))
+            [np.concatenate([cache.token_slots(e.seq, g, int(p), r), np.full(n - r, -1, dtype=np.int32)])
+             for e, p, n, r in zip(entries, past, lens, real)]))
         width = max(1, max(len(e.seq.pages[g]) for e in entries))
         if table_widths is not None:
             if table_widths[g] < width:

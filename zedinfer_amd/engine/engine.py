@@ -76,10 +76,11 @@ class Engine:
         self.graph_limit = 48
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.graph_replays = 0
-        # A step that is one portion of one prompt is padded to the next multiple of PROMPT_GRAPH_STEP
-        # tokens and captured too (launching a step kernel by kernel costs the host about 5 ms, more than
-        # the GPU needs for a short prompt), one graph per (padded tokens, wanted rows, table widths,
-        # attention launch size).  Portions of more tokens are bound by the GPU and run as they are.
+        # A step that is one portion of one prompt, alone or beside single decoded tokens, has the portion
+        # padded to the next multiple of PROMPT_GRAPH_STEP tokens and is captured too (launching a step
+        # kernel by kernel costs the host about 5 ms, more than the GPU needs for a short prompt), one graph
+        # per (entries, padded tokens, wanted rows, table widths, attention launch sizes).  Portions of
+        # more tokens are bound by the GPU and run as they are.
         self.prompt_graph_max_tokens = int(os.environ.get("ZEDINFER_PROMPT_GRAPH_MAX_TOKENS", "1024"))
         self._prompt_graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.prompt_graph_replays = 0
@@ -167,8 +168,7 @@ class Engine:
             self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
         if self.use_graphs and 0 < len(entries) <= self.graph_max_entries and single:
             logits = self._graph_step(entries, token_source)
-        elif (self.use_graphs and len(entries) == 1 and token_source is None and len(entries[0].want) <= 1
-              and SHORT_ENTRY < len(entries[0].tokens) <= self.prompt_graph_max_tokens):
+        elif self.use_graphs and token_source is None and self._one_portion(entries):
             logits = self._prompt_graph_step(entries)
         else:
             batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging)
@@ -230,33 +230,56 @@ class Engine:
     # ---- one portion of one prompt as a graph -------------------------------------------
     PROMPT_GRAPH_STEP = 64
 
+    def _one_portion(self, entries: Sequence[StepEntry]) -> bool:
+        """One portion of one prompt of a size worth a graph, beside any number of single decoded tokens;
+        at most one row wanted of each."""
+        portions = 0
+        for e in entries:
+            n = len(e.tokens)
+            if n == 1 and len(e.want) <= 1:
+                continue
+            if not (SHORT_ENTRY < n <= self.prompt_graph_max_tokens and len(e.want) <= 1):
+                return False
+            portions += 1
+        return portions == 1 and len(entries) <= self.graph_max_entries
+
     def _prompt_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """A step of one entry of more than SHORT_ENTRY tokens, run as if it brought a multiple of
-        PROMPT_GRAPH_STEP tokens (see ``build_device_batch``): the first step of a kind runs eagerly, the
-        second is captured, later ones replay."""
-        e = entries[0]
-        n = len(e.tokens)
-        padded = -(-n // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
-        R = len(e.want)
-        widths = tuple(_pow2_at_least(len(e.seq.pages[g]), 8) for g in range(len(self.cache.groups)))
-        keys_bucket = _pow2_at_least(e.seq.length + padded, 2048)
-        key = (padded, R, widths, keys_bucket)
+        """A step of one portion of a prompt (more than SHORT_ENTRY tokens) beside single decoded tokens,
+        with the portion run as if it brought a multiple of PROMPT_GRAPH_STEP tokens (see
+        ``build_device_batch``): the first step of a kind runs eagerly, the second is captured, later
+        ones replay."""
+        E = len(entries)
+        portion = next(e for e in entries if len(e.tokens) > 1)
+        padded = -(-len(portion.tokens) // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
+        R = sum(len(e.want) for e in entries)
+        widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
+                       for g in range(len(self.cache.groups)))
+        long_bucket = _pow2_at_least(portion.seq.length + padded, 2048)
+        short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if e is not portion], default=0), 256)
+        key = (E, padded, R, widths, long_bucket, short_bucket)
         dg = self._prompt_graphs.get(key)
         if dg is None:
             if len(self._prompt_graphs) >= self.graph_limit:
                 self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
-            size = 8 * padded + R + 16 + sum(padded + w for w in widths) + 64
+            N = padded + E - 1
+            size = 8 * N + R + 8 * E + sum(N + E * w for w in widths) + 64
             dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
             self._prompt_graphs[key] = dg
         batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
                                    pad_to=padded)
-        batch.max_long_keys = keys_bucket
+        batch.max_long_keys = long_bucket
+        if E > 1:
+            batch.max_short_keys = short_bucket
         if dg.graph is not None:
             dg.graph.replay()
             self.prompt_graph_replays += 1
             return dg.logits
         logits = self.model.run(batch, self.memories)
-        if dg.warm:
+        dg.seen += 1
+        # Recording costs about as much as ten steps: a portion alone is recorded the second time its shape
+        # comes, a shape with decoded tokens beside the portion (their number moves from step to step) only
+        # the fourth time.
+        if dg.seen >= (2 if E == 1 else 4):
             torch.cuda.synchronize(self.device)
             first = logits.clone() if logits is not None else None
             g = torch.cuda.CUDAGraph()
@@ -264,7 +287,6 @@ class Engine:
                 dg.logits = self.model.run(batch, self.memories)
             dg.graph = g
             return first
-        dg.warm = True
         return logits
 
 
@@ -274,6 +296,7 @@ class _DecodeGraph:
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
         self.warm = False
+        self.seen = 0
         self.image: Optional[DecodeImage] = None
 
 
