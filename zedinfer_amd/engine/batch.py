@@ -86,13 +86,17 @@ class DeviceBatch:
 def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
                        device: torch.device, staging: Optional[StagingRing] = None,
                        table_widths: Optional[Sequence[int]] = None,
-                       static: Optional[torch.Tensor] = None, pad_to: int = 0) -> DeviceBatch:
+                       static: Optional[torch.Tensor] = None, pad_to: int = 0, pad_entries: int = 0,
+                       pad_rows: int = 0) -> DeviceBatch:
     """Check the entries, then pack every index array into one host buffer and copy it over once.
 
     ``pad_to``: the one entry that brings more than SHORT_ENTRY tokens is run as if it brought that many.
     The tokens past its own are token 0 at the positions that follow; they have no place in the cache
     (slot -1: nothing is stored for them) and no real token sees them, so they change nothing but the
-    shapes, which then recur from step to step.
+    shapes, which then recur from step to step.  ``pad_entries`` adds that many entries of one token that
+    belong to no request (token 0 at position 0, no slot, an empty block table, state slot 0: only for
+    models without per-request state), ``pad_rows`` that many wanted rows after the real ones (the first
+    token's), to the same end.
 
     ``table_widths`` pads each group's block table to a given width; ``static`` is a device buffer
     the arrays are copied into instead of a fresh one (the layout depends only on the number of
@@ -115,7 +119,8 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
             if not (0 <= w < n):
                 raise ValueError(f"request {e.seq.request_id!r}: wanted place {w} is outside its {n} tokens")
         lens.append(n)
-    E = len(entries)
+    E = len(entries) + int(pad_entries)
+    lens = lens + [1] * int(pad_entries)
     real = list(lens)
     if pad_to:
         longs = [i for i, n in enumerate(lens) if n > SHORT_ENTRY]
@@ -126,18 +131,18 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     N = int(sum(lens))
     starts = np.zeros(E, dtype=np.int32)
     starts[1:] = np.cumsum(lens)[:-1]
-    past = np.array([e.seq.length for e in entries], dtype=np.int32)
-    slot = np.array([e.seq.slot for e in entries], dtype=np.int32)
+    past = np.array([e.seq.length for e in entries] + [0] * int(pad_entries), dtype=np.int32)
+    slot = np.array([e.seq.slot for e in entries] + [0] * int(pad_entries), dtype=np.int32)
     lens_a = np.array(lens, dtype=np.int32)
 
     token_ids = np.concatenate([np.concatenate([np.asarray(e.tokens, dtype=np.int64), np.zeros(n - r, dtype=np.int64)])
-                                for e, n, r in zip(entries, lens, real)])
+                                for e, n, r in zip(entries, lens, real)] + [np.zeros(int(pad_entries), dtype=np.int64)])
     if token_ids.min() < 0 or token_ids.max() >= vocab_size:
         bad = token_ids[(token_ids < 0) | (token_ids >= vocab_size)][0]
         raise ValueError(f"token id {int(bad)} is outside the vocabulary of {vocab_size}")
     positions = np.concatenate([np.arange(p, p + n, dtype=np.int32) for p, n in zip(past, lens)])
     tok_seq = np.repeat(np.arange(E, dtype=np.int32), lens)
-    rows = [starts[i] + w for i, e in enumerate(entries) for w in e.want]
+    rows = [starts[i] + w for i, e in enumerate(entries) for w in e.want] + [0] * int(pad_rows)
     logit_rows = np.asarray(rows, dtype=np.int32)
     R = len(rows)
 
@@ -146,7 +151,7 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     for g in range(G):
         group_slots.append(np.concatenate(
             [np.concatenate([cache.token_slots(e.seq, g, int(p), r), np.full(n - r, -1, dtype=np.int32)])
-             for e, p, n, r in zip(entries, past, lens, real)]))
+             for e, p, n, r in zip(entries, past, lens, real)] + [np.full(int(pad_entries), -1, dtype=np.int32)]))
         width = max(1, max(len(e.seq.pages[g]) for e in entries))
         if table_widths is not None:
             if table_widths[g] < width:

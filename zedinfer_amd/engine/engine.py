@@ -84,6 +84,7 @@ class Engine:
         self.prompt_graph_max_tokens = int(os.environ.get("ZEDINFER_PROMPT_GRAPH_MAX_TOKENS", "1024"))
         self._prompt_graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.prompt_graph_replays = 0
+        self._has_state = bool(self.model.state_requests())
 
     # ---- construction ------------------------------------------------------------
     @classmethod
@@ -248,10 +249,16 @@ class Engine:
         with the portion run as if it brought a multiple of PROMPT_GRAPH_STEP tokens (see
         ``build_device_batch``): the first step of a kind runs eagerly, the second is captured, later
         ones replay."""
-        E = len(entries)
         portion = next(e for e in entries if len(e.tokens) > 1)
         padded = -(-len(portion.tokens) // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
-        R = sum(len(e.want) for e in entries)
+        wanted = sum(len(e.want) for e in entries)
+        E, R, more_entries = len(entries), wanted, 0
+        if E > 1 and not self._has_state:
+            # the number of decoding requests moves from step to step: it is brought to a multiple of 8 with
+            # entries that belong to no request, and the wanted rows to one for each of them and the portion
+            more_entries = -(-(E - 1) // 8) * 8 - (E - 1)
+            E += more_entries
+            R = E
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
         long_bucket = _pow2_at_least(portion.seq.length + padded, 2048)
@@ -266,28 +273,27 @@ class Engine:
             dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
             self._prompt_graphs[key] = dg
         batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
-                                   pad_to=padded)
+                                   pad_to=padded, pad_entries=more_entries, pad_rows=R - wanted)
         batch.max_long_keys = long_bucket
         if E > 1:
             batch.max_short_keys = short_bucket
         if dg.graph is not None:
             dg.graph.replay()
             self.prompt_graph_replays += 1
-            return dg.logits
+            return dg.logits[:wanted] if wanted else None
         logits = self.model.run(batch, self.memories)
         dg.seen += 1
         # Recording costs about as much as ten steps: a portion alone is recorded the second time its shape
-        # comes, a shape with decoded tokens beside the portion (their number moves from step to step) only
-        # the fourth time.
-        if dg.seen >= (2 if E == 1 else 4):
+        # comes, a shape with decoded tokens beside the portion only the third time.
+        if dg.seen >= (2 if E == 1 else 3):
             torch.cuda.synchronize(self.device)
             first = logits.clone() if logits is not None else None
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 dg.logits = self.model.run(batch, self.memories)
             dg.graph = g
-            return first
-        return logits
+            logits = first
+        return logits[:wanted] if (wanted and logits is not None) else None
 
 
 class _DecodeGraph:
