@@ -407,9 +407,9 @@ def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype, tmp_path):
 def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
     """A step that is one portion of one prompt is padded to a multiple of 64 tokens and, from the third
     step of a shape on, replayed as a graph.  Every step is checked against an engine that launches
-    eagerly and does not pad: portions of different lengths that share a graph, alone and beside decoded
-    tokens, with and without a wanted row, decode steps (graphs of their own) and a step of two portions
-    between them, and at the end the caches, which
+    eagerly and does not pad: portions of different lengths that share a graph, alone, two in a step and
+    beside decoded tokens, with and without a wanted row, decode steps (graphs of their own) and a step that
+    takes no graph between them, and at the end the caches, which
     the padding must not have touched: decoding on gives the plain implementation's logits."""
     from zedinfer_amd.engine import StepEntry
     V = tiny["cfg"]["vocab_size"]
@@ -417,10 +417,10 @@ def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
         folder16 = tiny_configs.write_tiny(str(tmp_path / "bf16"), tiny["name"], dtype=torch.bfloat16)
         tiny = dict(tiny, folder=folder16, weights=plain.load_folder(folder16)[1])
         dtype = "bfloat16"
-    fast, slow = engine(tiny, dtype, num_kv_blocks=700).engine, engine(tiny, dtype, num_kv_blocks=700).engine
+    fast, slow = engine(tiny, dtype, num_kv_blocks=1000).engine, engine(tiny, dtype, num_kv_blocks=1000).engine
     assert fast.use_graphs
     slow.use_graphs = False
-    toks = {r: traces.random_tokens(V, 1200, seed=80 + i) for i, r in enumerate("abcd")}
+    toks = {r: traces.random_tokens(V, 1800, seed=80 + i) for i, r in enumerate("abcd")}
     fed = {r: 0 for r in toks}
     seqs = {}
     scale = [1.0]
@@ -455,7 +455,11 @@ def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
     for i in range(8):               # a portion beside decoded tokens: recorded the fourth time, then replayed
         both([("a", 1), ("d", 40 + 3 * i), ("b", 1)])
     assert fast.prompt_graph_replays >= before + 4
-    both([("a", 30), ("d", 3)])                           # two portions: launched kernel by kernel
+    before = fast.prompt_graph_replays
+    for i in range(12):              # two portions and a decoded token: the padded total is what counts
+        both([("a", 6 + i), ("b", 1), ("c", 20 - i)])
+    assert fast.prompt_graph_replays >= before + 3          # (a wider block table on the way starts a new graph)
+    both([("a", 30), ("d", 3)])                           # an entry of three tokens: launched kernel by kernel
     for r in "bcd":
         both([(r, 77)], True)
     assert fast.prompt_graph_replays >= 14 and slow.prompt_graph_replays == 0

@@ -90,8 +90,8 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
                        pad_rows: int = 0) -> DeviceBatch:
     """Check the entries, then pack every index array into one host buffer and copy it over once.
 
-    ``pad_to``: the one entry that brings more than SHORT_ENTRY tokens is run as if it brought that many.
-    The tokens past its own are token 0 at the positions that follow; they have no place in the cache
+    ``pad_to``: every entry that brings more than SHORT_ENTRY tokens is run as if it brought a multiple of
+    that many.  The tokens past its own are token 0 at the positions that follow; they have no place in the cache
     (slot -1: nothing is stored for them) and no real token sees them, so they change nothing but the
     shapes, which then recur from step to step.  ``pad_entries`` adds that many entries of one token that
     belong to no request (token 0 at position 0, no slot, an empty block table, state slot 0: only for
@@ -123,11 +123,7 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     lens = lens + [1] * int(pad_entries)
     real = list(lens)
     if pad_to:
-        longs = [i for i, n in enumerate(lens) if n > SHORT_ENTRY]
-        if len(longs) != 1 or pad_to < lens[longs[0]]:
-            raise ValueError("padding needs exactly one entry of more than SHORT_ENTRY tokens, and no fewer tokens than it brings")
-        lens = list(lens)
-        lens[longs[0]] = int(pad_to)
+        lens = [-(-n // int(pad_to)) * int(pad_to) if n > SHORT_ENTRY else n for n in lens]
     N = int(sum(lens))
     starts = np.zeros(E, dtype=np.int32)
     starts[1:] = np.cumsum(lens)[:-1]

@@ -232,50 +232,51 @@ class Engine:
     PROMPT_GRAPH_STEP = 64
 
     def _one_portion(self, entries: Sequence[StepEntry]) -> bool:
-        """One portion of one prompt of a size worth a graph, beside any number of single decoded tokens;
-        at most one row wanted of each."""
-        portions = 0
+        """Portions of prompts (more than SHORT_ENTRY tokens each) of a size worth a graph together, beside
+        any number of single decoded tokens; at most one row wanted of each."""
+        total = 0
         for e in entries:
             n = len(e.tokens)
-            if n == 1 and len(e.want) <= 1:
-                continue
-            if not (SHORT_ENTRY < n <= self.prompt_graph_max_tokens and len(e.want) <= 1):
+            if len(e.want) > 1 or 1 < n <= SHORT_ENTRY:
                 return False
-            portions += 1
-        return portions == 1 and len(entries) <= self.graph_max_entries
+            if n > 1:
+                total += -(-n // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
+        return 0 < total <= self.prompt_graph_max_tokens and len(entries) <= self.graph_max_entries
 
     def _prompt_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """A step of one portion of a prompt (more than SHORT_ENTRY tokens) beside single decoded tokens,
         with the portion run as if it brought a multiple of PROMPT_GRAPH_STEP tokens (see
         ``build_device_batch``): the first step of a kind runs eagerly, the second is captured, later
         ones replay."""
-        portion = next(e for e in entries if len(e.tokens) > 1)
-        padded = -(-len(portion.tokens) // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
+        step = self.PROMPT_GRAPH_STEP
+        portions = [e for e in entries if len(e.tokens) > 1]
+        padded = sum(-(-len(e.tokens) // step) * step for e in portions)      # tokens of all portions, padded
         wanted = sum(len(e.want) for e in entries)
         E, R, more_entries = len(entries), wanted, 0
         if E > 1 and not self._has_state:
-            # the number of decoding requests moves from step to step: it is brought to a multiple of 8 with
-            # entries that belong to no request, and the wanted rows to one for each of them and the portion
-            more_entries = -(-(E - 1) // 8) * 8 - (E - 1)
+            # the numbers of portions and of decoding requests move from step to step: the entries are brought
+            # to a multiple of 8 with entries that belong to no request, and a row is wanted of every entry
+            more_entries = -(-E // 8) * 8 - E
             E += more_entries
             R = E
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
-        long_bucket = _pow2_at_least(portion.seq.length + padded, 2048)
-        short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if e is not portion], default=0), 256)
-        key = (E, padded, R, widths, long_bucket, short_bucket)
+        long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions), 2048)
+        short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
+        singles = len(entries) - len(portions) + more_entries
+        key = (E, singles, padded, R, widths, long_bucket, short_bucket)
         dg = self._prompt_graphs.get(key)
         if dg is None:
             if len(self._prompt_graphs) >= self.graph_limit:
                 self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
-            N = padded + E - 1
+            N = padded + singles
             size = 8 * N + R + 8 * E + sum(N + E * w for w in widths) + 64
             dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
             self._prompt_graphs[key] = dg
         batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
-                                   pad_to=padded, pad_entries=more_entries, pad_rows=R - wanted)
+                                   pad_to=step, pad_entries=more_entries, pad_rows=R - wanted)
         batch.max_long_keys = long_bucket
-        if E > 1:
+        if singles:
             batch.max_short_keys = short_bucket
         if dg.graph is not None:
             dg.graph.replay()
@@ -285,7 +286,7 @@ class Engine:
         dg.seen += 1
         # Recording costs about as much as ten steps: a portion alone is recorded the second time its shape
         # comes, a shape with decoded tokens beside the portion only the third time.
-        if dg.seen >= (2 if E == 1 else 3):
+        if dg.seen >= (2 if len(entries) == 1 else 3):
             torch.cuda.synchronize(self.device)
             first = logits.clone() if logits is not None else None
             g = torch.cuda.CUDAGraph()
