@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from zedinfer_amd.cache import CacheManager, IdPool, OutOfPages, OutOfSlots, PagePool
-from zedinfer_amd.parts import KVCacheRequest, StateRequest
+from zedinfer_amd.parts import KVCacheRequest
 
 
 def manager(pages=12, page_size=4, requests=4, window=0, max_step_tokens=8):

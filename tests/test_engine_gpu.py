@@ -3,7 +3,6 @@ step and the last 32 tokens one by one; portions of changing size; and mixed bat
 pages that they are used again.  In float32 and in bfloat16, on three tiny configurations; bfloat16
 both with the float32 checkpoint (weights stored in 32 bits stay so) and with a bfloat16 checkpoint
 ("bfloat16w"), which is what the serving kernels for bfloat16 weights take."""
-import os
 
 import pytest
 import torch

@@ -31,7 +31,7 @@ import torch
 
 from ..config.forward_config import ScheduleStep
 from ..parts.base import KVCacheRequest, LayerMemory, StateRequest
-from .pages import IdPool, OutOfPages, OutOfSlots, PagePool
+from .pages import IdPool, OutOfPages, PagePool
 
 
 @dataclass

@@ -10,7 +10,6 @@ this engine does not hold: ``ping`` takes token ids (``--prompt-ids``).
 from __future__ import annotations
 
 import argparse
-import json
 import os
 import random
 import sys

@@ -12,7 +12,7 @@ mixers and feed-forwards.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, Tuple
 
 
 @dataclass(frozen=True)

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import json
 import os
-from dataclasses import dataclass, field, fields, asdict
+from dataclasses import dataclass, asdict
 from typing import Any, Dict, Mapping, Tuple
 
 

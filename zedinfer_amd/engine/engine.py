@@ -10,20 +10,18 @@ block tables before the run and commits the new lengths after it.
 from __future__ import annotations
 
 import os
-from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, Optional, Sequence
 
 import torch
 
 from .. import ops
 from ..cache.manager import CacheManager, SequenceCache
-from ..cache.pages import OutOfPages
 from ..config import ModelConfig, ModelForwardConfig, SchedulerConfig, load_config
 from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
 from ..sampling.sampler import default_sampling
 from ..weights import load_weights, random_weights
-from .batch import SHORT_ENTRY, DecodeImage, DeviceBatch, StagingRing, StepEntry, build_device_batch
+from .batch import SHORT_ENTRY, DecodeImage, StagingRing, StepEntry, build_device_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            "f32": torch.float32}

@@ -18,7 +18,7 @@ from ..config import SchedulerConfig
 from ..ops.staging import StagingRing
 from ..sampling.sampler import Sampler
 from .engine import Engine
-from .request import GenerationConfig, GenerationResult, InferenceRequest, RequestPhase
+from .request import GenerationConfig, GenerationResult, InferenceRequest
 from .scheduler import ScheduledBatch, Scheduler
 
 

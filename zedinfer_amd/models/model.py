@@ -7,12 +7,12 @@ of src/frontend/models/transformer_forward.cpp:63-156).
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, Optional, Sequence
 
 import torch
 
 from .. import ops
-from ..config.forward_config import LayerSpec, ModelForwardConfig, PartSpec
+from ..config.forward_config import ModelForwardConfig, PartSpec
 from ..parts import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, KVCacheRequest, LayerMemory, Part,
                      Runtime, StateRequest)
 from ..weights.loader import WeightSpec

@@ -1,7 +1,7 @@
 """Block arrangements."""
 from __future__ import annotations
 
-from typing import Dict, Optional
+from typing import Optional
 
 import torch
 

@@ -15,7 +15,7 @@ bfloat16.  In the float32 engine everything floating is widened to float32
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Iterable, List, Mapping, Optional, Tuple
+from typing import Dict, List, Mapping, Optional, Tuple
 
 import torch
 
