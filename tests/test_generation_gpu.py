@@ -472,6 +472,36 @@ def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
         eng.cache.check()
 
 
+def test_graphs_that_are_dropped_and_recorded_again(tiny):
+    """With room for two shapes of each kind, steps of four shapes in turn drop recorded graphs and record
+    them again; every step equals the eager engine's."""
+    from zedinfer_amd.engine import StepEntry
+    V = tiny["cfg"]["vocab_size"]
+    fast, slow = engine(tiny, num_kv_blocks=300).engine, engine(tiny, num_kv_blocks=300).engine
+    slow.use_graphs = False
+    fast.graph_limit = fast.prompt_graph_limit = 2
+    toks = {r: traces.random_tokens(V, 900, seed=90 + i) for i, r in enumerate("abc")}
+    fed = {r: 0 for r in toks}
+    seqs = {(eng, r): eng.open(r) for eng in (fast, slow) for r in toks}
+
+    def both(plan):
+        outs = [eng.step([StepEntry(seqs[(eng, r)], toks[r][fed[r]:fed[r] + n], [n - 1]) for r, n in plan])
+                for eng in (fast, slow)]
+        for r, n in plan:
+            fed[r] += n
+        assert float((outs[0] - outs[1]).abs().max()) <= 2e-5 * max(1.0, float(outs[1].abs().max())), plan
+
+    for _ in range(3):
+        for plan in ([("a", 1)], [("a", 1), ("b", 1)], [("a", 1), ("b", 1), ("c", 1)], [("b", 1), ("c", 1)]):
+            for _ in range(3):
+                both(plan)
+        for plan in ([("a", 10)], [("b", 70)], [("a", 1), ("c", 9)], [("c", 70)]):
+            for _ in range(3):
+                both(plan)
+    assert len(fast._graphs) <= 2 and len(fast._prompt_graphs) <= 2
+    assert fast.graph_replays >= 10 and fast.prompt_graph_replays >= 5
+
+
 def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatch, tmp_path):
     """Pure decode steps of few tokens rotate, store and attend in one kernel.  With that path switched
     off the same steps give the same logits (the caches hold the same keys and values, so later steps

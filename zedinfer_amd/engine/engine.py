@@ -80,6 +80,7 @@ class Engine:
         # per (entries, padded tokens, wanted rows, table widths, attention launch sizes).  Portions of
         # more tokens are bound by the GPU and run as they are.
         self.prompt_graph_max_tokens = int(os.environ.get("ZEDINFER_PROMPT_GRAPH_MAX_TOKENS", "1024"))
+        self.prompt_graph_limit = 128    # shapes held; the one used longest ago goes first
         self._prompt_graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.prompt_graph_replays = 0
         self._has_state = bool(self.model.state_requests())
@@ -193,10 +194,12 @@ class Engine:
         max_keys = max(e.seq.length for e in entries) + 1
         keys_bucket = _pow2_at_least(max_keys, 256)
         key = (E, R, widths, keys_bucket)
-        dg = self._graphs.get(key)
-        if dg is None:
+        dg = self._graphs.pop(key, None)
+        if dg is not None:
+            self._graphs[key] = dg              # used last: the last to go
+        else:
             if len(self._graphs) >= self.graph_limit:
-                self._graphs.pop(next(iter(self._graphs)))
+                self._drop_oldest(self._graphs)
             size = 8 * E + 2 * R + sum(E * (w + 1) for w in widths) + 64
             dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
             self._graphs[key] = dg
@@ -225,6 +228,13 @@ class Engine:
         dg.warm = True
         return logits
 
+
+    def _drop_oldest(self, graphs: Dict[tuple, "_DecodeGraph"]) -> None:
+        """Forget the first graph of the dictionary.  One that was recorded may still be running, and with
+        it goes the memory it was recorded with: the device is waited for first (this is rare)."""
+        dg = graphs.pop(next(iter(graphs)))
+        if dg.graph is not None:
+            torch.cuda.synchronize(self.device)
 
     # ---- one portion of one prompt as a graph -------------------------------------------
     PROMPT_GRAPH_STEP = 64
@@ -263,10 +273,12 @@ class Engine:
         short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
         singles = len(entries) - len(portions) + more_entries
         key = (E, singles, padded, R, widths, long_bucket, short_bucket)
-        dg = self._prompt_graphs.get(key)
-        if dg is None:
-            if len(self._prompt_graphs) >= self.graph_limit:
-                self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
+        dg = self._prompt_graphs.pop(key, None)
+        if dg is not None:
+            self._prompt_graphs[key] = dg       # used last: the last to go
+        else:
+            if len(self._prompt_graphs) >= self.prompt_graph_limit:
+                self._drop_oldest(self._prompt_graphs)
             N = padded + singles
             size = 8 * N + R + 8 * E + sum(N + E * w for w in widths) + 64
             dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
