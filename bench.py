@@ -129,14 +129,14 @@ def measure_mix(engine_factory, requests, vocab, new_tokens=256, lo=128, hi=4096
     return requests * new_tokens / dt, sum(lens) / dt, dt, sum(lens)
 
 
-def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT):
+def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT, warm=1):
     import torch
     from zedinfer_amd import ops
     from zedinfer_amd.engine import StepEntry
     eng = engine_factory()
     rng = random.Random(77)
     times = []
-    for i in range(rounds + 1):
+    for i in range(rounds + warm):
         seq = eng.open(("prefill", i), tokens)
         ids = rand_ids(rng, tokens, vocab)
         torch.cuda.synchronize()
@@ -145,7 +145,7 @@ def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT):
         ops.argmax(logits).tolist()
         times.append(time.perf_counter() - t0)
         eng.close(seq)
-    return sum(times[1:]) / rounds * 1000.0
+    return sum(times[warm:]) / rounds * 1000.0
 
 
 def main():
@@ -247,6 +247,11 @@ def main():
             torch.cuda.empty_cache()
             t, _, _ = measure_decode(factory(b), b, st, min(args.warmup, 8), V, args.prompt_len)
             points[f"decode_b{b}"] = round(t, 2)
+        # the reference's own short run (its bench -p 128): a prompt step of this size replays as a graph
+        # from its third time on, so two steps warm up
+        torch.cuda.empty_cache()
+        short = measure_prefill(factory(1, 128), V, tokens=128, warm=2)
+        points["prefill_128"] = round(128 / short * 1000.0, 1)
         out["points"] = points
     print(json.dumps(out))
     return 0
