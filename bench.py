@@ -41,6 +41,7 @@ PROMPT = 2048
 CONTEXT = 4096
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+CHOICES = {}       # decisions the engine made in its warm-up (Engine.warm_up), printed with the result
 
 
 def matmul_params_per_layer(c):
@@ -134,6 +135,9 @@ def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT, warm=1):
     from zedinfer_amd import ops
     from zedinfer_amd.engine import StepEntry
     eng = engine_factory()
+    # which of two equivalent orientations the library's gate/up product takes at this many rows is
+    # measured here, before the clock starts, and reported with the result
+    CHOICES.update({" ".join(str(x) for x in k): v for k, v in eng.warm_up([tokens]).items()})
     rng = random.Random(77)
     times = []
     for i in range(rounds + warm):
@@ -217,7 +221,8 @@ def main():
         pms = measure_prefill(factory(1, PF), V, tokens=PF)
         fl = prefill_flops(shape, args.layers, PF)
         print(json.dumps({"prefill": {"value": round(PF / pms * 1000.0, 1), "tokens": PF, "ms": round(pms, 3),
-                                      "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}}))
+                                      "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)},
+                          "choices": CHOICES}))
         return 0
     tps, ms_step, ctx_mid = measure_decode(factory(args.batch), args.batch, args.steps, args.warmup, V, args.prompt_len)
     need = decode_bytes(shape, args.layers, args.batch, ctx_mid, el)
@@ -253,6 +258,7 @@ def main():
         short = measure_prefill(factory(1, 128), V, tokens=128, warm=2)
         points["prefill_128"] = round(128 / short * 1000.0, 1)
         out["points"] = points
+    out["choices"] = CHOICES
     print(json.dumps(out))
     return 0
 

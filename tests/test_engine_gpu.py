@@ -2,7 +2,13 @@
 step and the last 32 tokens one by one; portions of changing size; and mixed batches with so few
 pages that they are used again.  In float32 and in bfloat16, on three tiny configurations; bfloat16
 both with the float32 checkpoint (weights stored in 32 bits stay so) and with a bfloat16 checkpoint
-("bfloat16w"), which is what the serving kernels for bfloat16 weights take."""
+("bfloat16w"), which is what the serving kernels for bfloat16 weights take.
+
+Every variant runs a second time with "sharp" weights (a trailing "s": matrices of width
+tiny_configs.SHARP_STD instead of 0.02).  With the narrow weights attention is nearly uniform and a
+forward pass without rotation, or without the 1/sqrt(d), stays inside the bfloat16 tolerance; with the
+sharp ones either moves the logits by their whole size while bfloat16 rounding stays below 2 % of it
+(tests/test_tolerances.py holds that on the CPU)."""
 
 import pytest
 import torch
@@ -10,15 +16,12 @@ import torch
 import tiny_configs
 import traces
 from plain import qwen2_plain as plain
+from tolerances import BF16_REL_MEAN, BF16_REL_WORST, F32_TOL
 
 pytestmark = pytest.mark.gpu
 
 LENGTHS = {"A": [5, 17, 33, 100, 70, 64, 90, 41, 128, 77], "B": [1, 31, 64, 100, 47, 90, 120, 66, 35, 80],
            "C": [1, 31, 64, 100, 47, 90, 120, 66, 35, 80]}
-# float32: rounding of a few hundred float32 operations; bfloat16: activations are rounded to 8 bits
-# of mantissa after every op.
-F32_TOL = 2e-4
-BF16_REL_WORST, BF16_REL_MEAN = 0.06, 0.012
 
 
 @pytest.fixture(scope="module", params=["A", "B", "C"])
@@ -31,15 +34,30 @@ def tiny(request, tmp_path_factory):
     folder16 = tiny_configs.write_tiny(str(tmp_path_factory.mktemp(f"tiny{name}bf16")), name, dtype=torch.bfloat16)
     _, w16 = plain.load_folder(folder16)
     ref16 = {rid: plain.forward(cfg, w16, toks) for rid, toks in reqs.items()}
-    return dict(name=name, folder=folder, cfg=cfg, weights=w, requests=reqs, reference=ref,
-                folder16=folder16, reference16=ref16)
+    out = dict(name=name, folder=folder, cfg=cfg, weights=w, requests=reqs, reference=ref,
+               folder16=folder16, reference16=ref16)
+    # the sharp variants: the same sizes and requests, wider weights
+    sharp = tiny_configs.write_tiny(str(tmp_path_factory.mktemp(f"tiny{name}s")), name, std=tiny_configs.SHARP_STD)
+    sharp16 = tiny_configs.write_tiny(str(tmp_path_factory.mktemp(f"tiny{name}sbf16")), name, dtype=torch.bfloat16,
+                                      std=tiny_configs.SHARP_STD)
+    for key, f in (("", sharp), ("16", sharp16)):
+        wf = plain.load_folder(f)[1]
+        out["sharp_folder" + key] = f
+        out["sharp_reference" + key] = {rid: plain.forward(cfg, wf, toks) for rid, toks in reqs.items()}
+    return out
+
+
+DTYPES = ["float32", "bfloat16", "bfloat16w", "float32s", "bfloat16s", "bfloat16ws"]
 
 
 def variant(tiny, dtype):
     """(model folder, engine dtype, reference logits) of a dtype parameter."""
+    pre = ""
+    if dtype.endswith("s"):
+        pre, dtype = "sharp_", dtype[:-1]
     if dtype == "bfloat16w":
-        return tiny["folder16"], "bfloat16", tiny["reference16"]
-    return tiny["folder"], dtype, tiny["reference"]
+        return tiny[pre + "folder16"], "bfloat16", tiny[pre + "reference16"]
+    return tiny[pre + "folder"], dtype, tiny[pre + "reference"]
 
 
 def make_engine(tiny, dtype, pages):
@@ -55,14 +73,14 @@ def check(tiny, dtype, steps, outputs):
     worst, mean, scale, rows, where = traces.compare(steps, outputs, variant(tiny, dtype)[2], tiny["requests"])
     print(f"[{tiny['name']} {dtype}] rows={rows} worst={worst:.3e} mean={mean:.3e} scale={scale:.3e} at {where}")
     assert rows > 0
-    if dtype == "float32":
+    if dtype.startswith("float32"):
         assert worst <= F32_TOL * max(1.0, scale), f"first/worst difference at (step, request, position) {where}"
     else:
         assert worst <= BF16_REL_WORST * scale, f"worst difference at {where}"
         assert mean <= BF16_REL_MEAN * scale
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w"])
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", ["whole", "last32", "portions", "mixed"])
 def test_engine_matches_plain(tiny, dtype, shape):
     steps = {"whole": traces.whole, "last32": traces.last_decoded, "portions": traces.portions,
@@ -77,7 +95,7 @@ def test_engine_matches_plain(tiny, dtype, shape):
     check(tiny, dtype, steps, out)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w", "bfloat16ws"])
 def test_replay_tool(tiny, dtype, tmp_path):
     """The same mixed trace through bin/trace_run as a child process."""
     steps = traces.mixed(tiny["requests"], seed=3)

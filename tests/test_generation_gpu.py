@@ -550,19 +550,39 @@ def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatc
 
 
 @pytest.mark.parametrize("requests", [20, 70, 136])
-def test_decode_graphs_with_the_library_product(tiny, requests):
-    """More than 16 decoding requests (and more than 64: beyond every few-rows kernel): the matrix
-    products go to the library, inside the captured graph.  Every replay is checked against eager
-    launches, with eager prompt steps between them."""
+def test_decode_graphs_with_the_library_product(tiny, requests, monkeypatch, tmp_path):
+    """More than 16 decoding requests on a bfloat16 checkpoint: 17..64 rows take the second few-rows
+    kernel, more than 64 the library's product (also for the float32 logits), inside the captured graph;
+    the rotary launch is its own again and the attention takes every token of the step.  Every replay is
+    checked against eager launches, with eager prompt steps between them, and the last step against the
+    plain implementation; the calls are counted to show which product ran (weights stored in 32 bits
+    would go to the plain product instead, which this test is not about)."""
     from zedinfer_amd.engine import StepEntry
+    from zedinfer_amd.ops import _lib
+    from tolerances import bf16_within
     V = tiny["cfg"]["vocab_size"]
-    fast = engine(tiny, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
-    slow = engine(tiny, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
+    folder16 = tiny_configs.write_tiny(str(tmp_path / "bf16"), tiny["name"], dtype=torch.bfloat16,
+                                       std=tiny_configs.SHARP_STD)
+    tiny16 = dict(tiny, folder=folder16, weights=plain.load_folder(folder16)[1])
+    fast = engine(tiny16, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
+    slow = engine(tiny16, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
     slow.use_graphs = False
     names = [f"r{i}" for i in range(requests)]
     toks = {r: traces.random_tokens(V, 40, seed=80 + i) for i, r in enumerate(names)}
     seqs = {(e, r): e.open(r) for e in (fast, slow) for r in names}
     fed = {r: 0 for r in names}
+    calls = {}
+    real_call, real_mm = _lib.call, torch.mm
+
+    def counted_call(name, *a):
+        calls[name] = calls.get(name, 0) + 1
+        return real_call(name, *a)
+
+    def counted_mm(*a, **k):
+        calls["library"] = calls.get("library", 0) + 1
+        return real_mm(*a, **k)
+    monkeypatch.setattr(_lib, "call", counted_call)
+    monkeypatch.setattr(torch, "mm", counted_mm)
 
     def both(plan):
         outs = []
@@ -571,10 +591,28 @@ def test_decode_graphs_with_the_library_product(tiny, requests):
         for r, n in plan:
             fed[r] += n
         assert torch.equal(outs[0], outs[1]), (plan[0], len(plan))
+        return outs[0]
 
     both([(r, 5 + i % 4) for i, r in enumerate(names)])
+    calls.clear()
     for step in range(12):
-        both([(r, 1) for r in names])
+        last = both([(r, 1) for r in names])
+        if step == 0:
+            first = dict(calls)
         if step % 4 == 1:
             both([(names[0], 3), (names[1], 1)])      # an eager mixed step between the replays
     assert fast.graph_replays >= 8
+    # which kernels a decode step of this many rows took (counted over the step's two engines)
+    assert first.get("zi_gemm_generic", 0) == 0, first
+    assert first.get("zi_attention_decode", 0) > 0 and first.get("zi_attention_decode_fused", 0) == 0, first
+    if requests <= 64:
+        assert first.get("zi_gemm_skinny", 0) > 0 and first.get("library", 0) == 0, first
+    else:
+        assert first.get("library", 0) > 0, first
+    worst = mean = scale = 0.0
+    for i, r in enumerate(names):
+        ref = plain.forward(tiny["cfg"], tiny16["weights"], toks[r][:fed[r]])[-1]
+        d = (last[i].cpu() - ref).abs()
+        worst, mean, scale = max(worst, float(d.max())), mean + float(d.mean()) / requests, max(scale, float(ref.abs().max()))
+    print(f"{requests} requests: worst {worst:.3e} mean {mean:.3e} of scale {scale:.3e}; calls of a step {first}")
+    assert bf16_within(worst, mean, scale)

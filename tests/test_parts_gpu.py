@@ -98,33 +98,36 @@ def test_swiglu_part(dtype, n):
 
 @pytest.mark.parametrize("n,H,I", [(256, 72, 200), (136, 96, 72), (1024, 128, 344)])
 def test_swiglu_part_both_orientations_of_the_product(n, H, I):
-    """Many rows in bfloat16: the part measures once whether the library makes the gate/up product faster
-    transposed; both ways, forced here, give the plain result (and nearly each other's)."""
+    """Many rows in bfloat16: the library may make the gate/up product faster transposed.  Both ways,
+    chosen here through the runtime's recorded choices, give the plain result (and nearly each other's);
+    without a choice the forward pass takes the straight one and measures nothing; ``tune`` measures
+    outside of a step, records its decision, and the forward pass then follows it."""
     from zedinfer_amd.parts import FEED_FORWARDS
-    from zedinfer_amd.parts.feed_forward import SwiGLU
     dtype = torch.bfloat16
     w = {"gate": rnd(I, H, seed=1, scale=0.2), "up": rnd(I, H, seed=2, scale=0.2), "down": rnd(H, I, seed=3, scale=0.2)}
     x = rnd(n, H, seed=4)
+    rt = runtime(dtype)
     part = FEED_FORWARDS.get("swiglu")(spec("swiglu", {"hidden_size": H, "intermediate_size": I}),
-                                       {k: v.to(dtype).cuda() for k, v in w.items()}, runtime(dtype))
+                                       {k: v.to(dtype).cuda() for k, v in w.items()}, rt)
     wf = {k: v.to(dtype).float() for k, v in w.items()}
     xf = x.to(dtype).float()
     ref = plain.linear(plain.swiglu(plain.linear(xf, wf["gate"]), plain.linear(xf, wf["up"])), wf["down"])
-    key = (n, 2 * I, H)
+    key = ("gate_up_transposed", n, 2 * I, H)
     got = {}
-    before = dict(SwiGLU._transposed_wins)
-    try:
-        for wins in (False, True):
-            SwiGLU._transposed_wins[key] = wins
-            got[wins] = as_rows(part.forward(x.to(dtype).cuda())).cpu()
-            assert_close_to_scale(got[wins], ref, dtype)
-        SwiGLU._transposed_wins.pop(key)
-        measured = as_rows(part.forward(x.to(dtype).cuda())).cpu()           # measures, then takes one of the two
-        assert key in SwiGLU._transposed_wins
-        assert torch.equal(measured, got[SwiGLU._transposed_wins[key]])
-    finally:
-        SwiGLU._transposed_wins.clear()
-        SwiGLU._transposed_wins.update(before)
+    assert not rt.choices
+    default = as_rows(part.forward(x.to(dtype).cuda())).cpu()
+    assert not rt.choices                                   # a step decides and measures nothing
+    for wins in (False, True):
+        rt.choices[key] = wins
+        got[wins] = as_rows(part.forward(x.to(dtype).cuda())).cpu()
+        assert_close_to_scale(got[wins], ref, dtype)
+    assert torch.equal(default, got[False])
+    del rt.choices[key]
+    part.tune(n)
+    assert isinstance(rt.choices.get(key), bool)
+    part.tune(n)                                            # decided once
+    measured = as_rows(part.forward(x.to(dtype).cuda())).cpu()
+    assert torch.equal(measured, got[rt.choices[key]])
     torch.testing.assert_close(got[True], got[False], atol=2e-2 * float(ref.abs().max()), rtol=0)
 
 

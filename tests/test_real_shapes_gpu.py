@@ -3,12 +3,15 @@ vocabulary and two layers so that the plain implementation stays affordable on t
 implementation: a prompt in portions, then decoded tokens, alone and beside a second request.  In float32,
 in bfloat16 with the float32 checkpoint (weights stored in 32 bits stay so) and in bfloat16 with a bfloat16
 checkpoint ("bfloat16w"): the serving kernels (few-rows products and their cuts along k, partial sums, the
-one-kernel decode attention, prompt attention, the library product) at the shapes they serve."""
+one-kernel decode attention, prompt attention, the library product) at the shapes they serve.  At these
+widths N(0, 0.02) weights already make attention peaked: a pass without rotation or scale leaves the bfloat16
+tolerance several times over (tests/test_tolerances.py shows it for the 1.5B sizes)."""
 import pytest
 import torch
 
 import traces
 from plain import qwen2_plain as plain
+from tolerances import BF16_REL_MEAN, BF16_REL_WORST
 
 pytestmark = pytest.mark.gpu
 
@@ -84,4 +87,4 @@ def test_real_layer_shapes_match_plain(model, dtype):
         assert worst <= 3e-4 * max(1.0, scale), where
     else:
         assert engine.graph_replays > 10
-        assert worst <= 0.06 * scale and mean <= 0.012 * scale, where
+        assert worst <= BF16_REL_WORST * scale and mean <= BF16_REL_MEAN * scale, where

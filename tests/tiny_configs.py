@@ -29,9 +29,13 @@ SEEDS = {"A": 0, "B": 1, "C": 2}
 NOISY_NORMS = {"A": False, "B": True, "C": True}
 
 
-def write_tiny(folder, name, dtype=None):
+SHARP_STD = 0.1     # weights this wide make attention peaked: a wrong rotation or scale moves the logits by their whole size
+
+
+def write_tiny(folder, name, dtype=None, std=0.02):
     """Write config.json and model.safetensors of a tiny configuration with the engine's
-    random-weights mode; returns the folder."""
+    random-weights mode; returns the folder.  ``std`` is the width of the matrices and biases
+    (SHARP_STD for the "sharp" variants of the tests)."""
     import torch
     from zedinfer_amd.config import Qwen2Config
     from zedinfer_amd.models import expected_weights
@@ -40,7 +44,7 @@ def write_tiny(folder, name, dtype=None):
     cfg = Qwen2Config.from_dict(CONFIGS[name])
     fc = qwen2_forward_config(cfg)
     write_model_folder(folder, cfg, expected_weights(fc), seed=SEEDS[name], dtype=dtype or torch.float32,
-                       noisy_norms=NOISY_NORMS[name])
+                       noisy_norms=NOISY_NORMS[name], std=std)
     # keep the keys of the test's dict exactly (eos list and so on)
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(CONFIGS[name], f, indent=1)

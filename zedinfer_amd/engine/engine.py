@@ -139,6 +139,24 @@ class Engine:
         other.steps_run = other.graph_replays = 0
         return other
 
+    # ---- decisions made outside of steps ---------------------------------------------
+    def warm_up(self, step_sizes: Sequence[int] = (), choices: Optional[Dict[tuple, object]] = None
+                ) -> Dict[tuple, object]:
+        """Let every part decide, for steps of the given numbers of tokens, between ways of computing the
+        same thing that differ in speed and by rounding (``Part.tune``); nothing of the kind is decided
+        while a step runs.  ``choices`` (what an earlier call returned) are taken as they are, which makes
+        a run repeat another's bits.  Returns all decisions in force."""
+        if choices:
+            self.rt.choices.update(choices)
+        for n in step_sizes:
+            for part in self.model.parts:
+                part_tune = getattr(part, "tune", None)
+                if part_tune is not None:
+                    part_tune(int(n))
+        if step_sizes:
+            torch.cuda.synchronize(self.device)
+        return dict(self.rt.choices)
+
     # ---- requests ------------------------------------------------------------------
     def open(self, request_id, expected_tokens: int = 0) -> SequenceCache:
         return self.cache.open(request_id, expected_tokens)

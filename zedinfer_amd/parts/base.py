@@ -34,6 +34,10 @@ class Runtime:
         self._buffers: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
         self._views: Dict[tuple, torch.Tensor] = {}     # (name, dtype, shape) -> the view handed out last time
         self._outgrown: list = []                       # allocations that captured graphs may still use
+        # Decisions between equivalent ways of computing something (which differ by rounding), by a key
+        # the deciding part chooses.  They are made outside of steps (``Part.tune``, ``Engine.warm_up``)
+        # or given by the caller, never while a step runs: a run with the same choices gives the same bits.
+        self.choices: Dict[tuple, object] = {}
 
     def buffer(self, name: str, shape: Tuple[int, ...], dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         dtype = dtype or self.dtype
@@ -154,6 +158,11 @@ class Part:
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         self.spec = spec
         self.rt = rt
+
+    def tune(self, num_tokens: int) -> None:
+        """Measure, outside of any step, which of several equivalent ways is faster for steps of
+        ``num_tokens`` tokens and record the decision in ``rt.choices`` (``Engine.warm_up`` calls this).
+        ``forward`` only reads ``rt.choices``; without an entry it takes a fixed default."""
 
 
 class Mixer(Part):

@@ -40,56 +40,68 @@ class SwiGLU(FeedForward):
     graph_safe = True
     # For many rows the gate/up product is the library's, and at some sizes it makes the transposed
     # result, W . x^T, faster than x . W^T (measured at the 1.5B sizes: 100 against 119 us at 2,048 rows,
-    # 31 against 37 at 512, 73 against 67 at 1,024).  Which one is taken for (rows, 2I, H) is measured once,
-    # the first time that many rows come: three runs each of product plus activation; the transposed one
-    # must win by 5% (two runs of a program then seldom choose differently; their results differ by
-    # rounding only; ZEDINFER_GATE_UP_TRANSPOSED=0 or 1 fixes the choice instead).  The transposed result
-    # goes through the activation kernel that turns it back.
+    # 31 against 37 at 512, 73 against 67 at 1,024).  The transposed result goes through the activation
+    # kernel that turns it back; the two ways differ by rounding.  Which one a step of n rows takes is
+    # read from ``rt.choices[("gate_up_transposed", n, 2I, H)]``: absent, the straight product (or what
+    # ZEDINFER_GATE_UP_TRANSPOSED=0/1 says).  ``tune(n)`` measures both outside of any step and records
+    # the winner there; nothing is measured while a step runs.
     TRANSPOSED_MIN_ROWS = 128
-    _transposed_wins: Dict[tuple, bool] = {}
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
         H, I = int(spec.params["hidden_size"]), int(spec.params["intermediate_size"])
         return {"gate": WeightSpec((I, H)), "up": WeightSpec((I, H)), "down": WeightSpec((H, I))}
 
+    def _choice_key(self, n: int) -> tuple:
+        return ("gate_up_transposed", int(n), 2 * self.inter, self.hidden)
+
+    def _can_transpose(self, n: int) -> bool:
+        return (self.interleave == GATE_UP_BLOCK and self.rt.dtype == torch.bfloat16
+                and n >= self.TRANSPOSED_MIN_ROWS and n % 8 == 0 and n > ops.FEW_ROWS)
+
+    def _gate_up_straight(self, x: torch.Tensor, act: torch.Tensor) -> None:
+        gu = self.rt.buffer("ffn_gate_up", (x.shape[0], 2 * self.inter))
+        ops.linear(x, self.gate_up, out=gu)
+        ops.swiglu(gu, out=act, interleave=self.interleave)
+
+    def _gate_up_transposed(self, x: torch.Tensor, act: torch.Tensor) -> None:
+        n, I = x.shape[0], self.inter
+        gut = self.rt.buffer("ffn_gate_up", (n, 2 * I)).view(-1)[:2 * I * n].view(2 * I, n)      # the same memory
+        ops.linear_transposed(x, self.gate_up, out=gut)
+        ops.swiglu_t(gut, out=act)
+
     def _gate_up_many_rows(self, x: torch.Tensor, act: torch.Tensor) -> None:
         """act = swiglu of the gate/up product of x, bfloat16, interleaved weights, more rows than the
         few-rows kernels take."""
-        n, I = x.shape[0], self.inter
-        gu = self.rt.buffer("ffn_gate_up", (n, 2 * I))
+        n = x.shape[0]
+        if self._can_transpose(n) and x.is_contiguous():
+            wins = self.rt.choices.get(self._choice_key(n))
+            if wins is None:
+                wins = os.environ.get("ZEDINFER_GATE_UP_TRANSPOSED", "") == "1"
+            if wins:
+                return self._gate_up_transposed(x, act)
+        return self._gate_up_straight(x, act)
 
-        def straight():
-            ops.linear(x, self.gate_up, out=gu)
-            ops.swiglu(gu, out=act, interleave=self.interleave)
+    def tune(self, num_tokens: int) -> None:
+        """Decide the orientation of the gate/up product for steps of ``num_tokens`` rows: three runs each
+        of product plus activation; the transposed one must win by 5 %."""
+        n, key = int(num_tokens), self._choice_key(num_tokens)
+        forced = os.environ.get("ZEDINFER_GATE_UP_TRANSPOSED", "")
+        if key in self.rt.choices or not self._can_transpose(n) or forced in ("0", "1"):
+            return
+        x = self.rt.buffer("norm_out", (n, self.hidden))
+        act = self.rt.buffer("ffn_act", (n, self.inter))
 
-        if n < self.TRANSPOSED_MIN_ROWS or n % 8 or not x.is_contiguous():
-            return straight()
-        gut = gu.view(-1)[:2 * I * n].view(2 * I, n)      # the same memory
-
-        def transposed():
-            ops.linear_transposed(x, self.gate_up, out=gut)
-            ops.swiglu_t(gut, out=act)
-
-        key = (n, 2 * I, self.hidden)
-        wins = SwiGLU._transposed_wins.get(key)
-        forced = os.environ.get("ZEDINFER_GATE_UP_TRANSPOSED", "")      # "0" / "1": no measurement, always that way
-        if wins is None and forced in ("0", "1"):
-            wins = SwiGLU._transposed_wins[key] = forced == "1"
-        if wins is None and torch.cuda.is_current_stream_capturing():
-            return straight()           # nothing can be measured while a graph is recorded
-        if wins is None:
-            def clock(fn):
-                fn()
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                for _ in range(3):
-                    fn()
-                b.record()
-                b.synchronize()
-                return a.elapsed_time(b)
-            wins = SwiGLU._transposed_wins[key] = clock(transposed) < 0.95 * clock(straight)
-        return transposed() if wins else straight()
+        def clock(fn):
+            fn(x, act)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(3):
+                fn(x, act)
+            b.record()
+            b.synchronize()
+            return a.elapsed_time(b)
+        self.rt.choices[key] = bool(clock(self._gate_up_transposed) < 0.95 * clock(self._gate_up_straight))
 
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         super().__init__(spec, weights, rt)
