@@ -57,7 +57,7 @@ class SwiGLU(FeedForward):
 
     def _can_transpose(self, n: int) -> bool:
         return (self.interleave == GATE_UP_BLOCK and self.rt.dtype == torch.bfloat16
-                and n >= self.TRANSPOSED_MIN_ROWS and n % 8 == 0 and n > ops.FEW_ROWS)
+                and n >= self.TRANSPOSED_MIN_ROWS and n % 8 == 0)
 
     def _gate_up_straight(self, x: torch.Tensor, act: torch.Tensor) -> None:
         gu = self.rt.buffer("ffn_gate_up", (x.shape[0], 2 * self.inter))
