@@ -12,6 +12,8 @@
 // the probability's bit pattern (non-negative floats order like their bits);
 // equal probabilities are ordered by rising token id.  One workgroup per row.
 #include "zi_common.h"
+#include "zi_no_alloc.h"
+#include <mutex>
 
 #define SAMPLE_THREADS 1024
 
@@ -129,6 +131,66 @@ extern "C" int zi_argmax(int32_t* out_idx, float* out_val, const void* logits, i
         argmax_kernel<T><<<rows, SAMPLE_THREADS, 0, stream>>>(out_idx, out_val, (const T*)logits, ld, vocab);
     });
     return zi_check_launch("argmax");
+}
+
+// ---- the argmax that allocates nothing ------------------------------------------------------------
+// The parts' (value, index) pairs live in this array instead of a workspace.  In host code the array's
+// name is only a stand-in for the symbol; the memory's address on a device comes from
+// hipGetSymbolAddress, once per device, with that device current (every GPU has its own copy).
+static __device__ __align__(256) unsigned char scratch[ZI_ARGMAX_STATIC_MAX_PARTS * 8];
+
+#define ZI_MAX_DEVICES 64
+static void* scratch_of_device[ZI_MAX_DEVICES];
+static std::mutex scratch_lock;
+
+// The address of `scratch` on the current device; nullptr (with the error set) when it cannot be had.
+static void* scratch_address() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= ZI_MAX_DEVICES) {
+        zi_fail("argmax_static: no current device (%s, device %d)", hipGetErrorString(e), dev);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_of_device[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            zi_fail("argmax_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        scratch_of_device[dev] = ptr;
+    }
+    return scratch_of_device[dev];
+}
+
+extern "C" int zi_argmax_static_max_parts() { return ZI_ARGMAX_STATIC_MAX_PARTS; }
+
+extern "C" int zi_argmax_static(int32_t* out_idx, float* out_val, const void* logits, int dt, int rows, int vocab,
+                                int64_t ld, hipStream_t stream) {
+    ZI_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "argmax_static: bad sizes rows=%d vocab=%d", rows, vocab);
+    ZI_REQUIRE(out_idx && logits, "argmax_static: null argument");
+    if (rows == 0) return 0;
+    const int parts = (vocab + ARGMAX_PART - 1) / ARGMAX_PART;
+    if (parts == 1) {      // short rows need no memory beside the result
+        ZI_DISPATCH_DTYPE(dt, T, {
+            argmax_kernel<T><<<rows, SAMPLE_THREADS, 0, stream>>>(out_idx, out_val, (const T*)logits, ld, vocab);
+        });
+        return zi_check_launch("argmax_static");
+    }
+    ZI_REQUIRE((int64_t)rows * parts <= ZI_ARGMAX_STATIC_MAX_PARTS && rows <= 65535,
+               "argmax_static: %d rows of %d values are %lld parts, the library's array holds %d "
+               "(use zi_argmax with a workspace)", rows, vocab, (long long)rows * parts, ZI_ARGMAX_STATIC_MAX_PARTS);
+    void* ptr = scratch_address();
+    if (!ptr) return 1;
+    float* pv = reinterpret_cast<float*>(ptr);
+    int32_t* pi = reinterpret_cast<int32_t*>(pv + (int64_t)rows * parts);
+    ZI_DISPATCH_DTYPE(dt, T, {
+        argmax_part_kernel<T><<<dim3(rows, parts), SAMPLE_THREADS, 0, stream>>>(pv, pi, (const T*)logits, ld, vocab,
+                                                                                ARGMAX_PART);
+    });
+    argmax_merge_kernel<<<rows, ZI_WAVE, 0, stream>>>(out_idx, out_val, pv, pi, parts);
+    return zi_check_launch("argmax_static");
 }
 
 // Sum and count of the probabilities whose bit pattern is >= tau.
