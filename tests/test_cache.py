@@ -75,6 +75,27 @@ def test_ensure_is_all_or_nothing():
     m.check()
 
 
+def test_undo_gives_back_what_an_ensure_took():
+    """A step that cannot grow one of its requests undoes the growth of the others (Engine.step does)."""
+    m = manager(pages=6, window=6)
+    a, b = m.open("a"), m.open("b")
+    m.ensure(a, 5)
+    m.commit(a, 5)
+    before = (list(a.pages[0]), list(a.pages[1]), a.held[:], a.promised[:],
+              m.groups[0].pool.num_free, m.groups[1].pool.num_free, m.groups[0].pool.committed)
+    growth = m.ensure(a, 14)
+    assert growth.taken and a.held[0] > before[2][0]
+    with pytest.raises(OutOfPages):
+        m.ensure(b, 20)
+    m.undo(a, growth)
+    assert before == (a.pages[0], a.pages[1], a.held, a.promised, m.groups[0].pool.num_free,
+                      m.groups[1].pool.num_free, m.groups[0].pool.committed)
+    m.check()
+    m.ensure(a, 14)                                  # and it can be taken again
+    m.commit(a, 14)
+    m.check()
+
+
 def test_window_gives_pages_back():
     m = manager(pages=6, page_size=4, window=6)
     s = m.open("a")

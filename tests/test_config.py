@@ -71,6 +71,13 @@ def test_forward_config_is_built_from_config_alone():
     assert [l.mixer.params["window"] for l in fc.layers] == [0, 20, 20]
 
 
+def test_window_keys_can_be_ignored_as_the_reference_does(monkeypatch):
+    """The reference parses the window keys and never uses them (src/frontend/models/base.cpp:807-813)."""
+    monkeypatch.setenv("ZEDINFER_IGNORE_SLIDING_WINDOW", "1")
+    fc = qwen2_forward_config(Qwen2Config.from_dict(tiny_configs.TINY_C))
+    assert [l.mixer.params["window"] for l in fc.layers] == [0, 0, 0]
+
+
 def test_schedule_validation():
     import dataclasses
     fc = qwen2_forward_config(Qwen2Config.from_dict(tiny_configs.TINY_A))

@@ -102,3 +102,27 @@ def test_replay_tool(tiny, dtype, tmp_path):
     folder, engine_dtype, _ = variant(tiny, dtype)
     out = traces.run_tool(folder, engine_dtype, steps, str(tmp_path / "out"), traces.max_live_tokens(steps))
     check(tiny, dtype, steps, out)
+
+
+@pytest.mark.parametrize("how", ["options", "trace"])
+def test_replay_tool_with_the_configuration_s_own_pages(tiny, how, tmp_path):
+    """The pool geometry given to the tool, on the command line or as the trace's first line: the page
+    size of the configuration (8 for B and C), at most four live requests, and so few pages that the
+    tool reports more handed out than the pool has."""
+    import re
+    steps = traces.mixed(tiny["requests"], seed=5)
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    folder, engine_dtype, _ = variant(tiny, "bfloat16ws")
+    need = traces.max_live_tokens(steps)
+    log = str(tmp_path / "stderr.txt")
+    if how == "options":
+        out = traces.run_tool(folder, engine_dtype, steps, str(tmp_path / "out"), need,
+                              options=["--kv-block-size", ps, "--max-live", 4], stderr_to=log)
+    else:
+        out = traces.run_tool(folder, engine_dtype, steps, str(tmp_path / "out"), need,
+                              geometry={"kv_block_size": ps, "num_kv_blocks": need // ps, "max_live": 4}, stderr_to=log)
+    check(tiny, "bfloat16ws", steps, out)
+    said = open(log).read()
+    assert f"{need // ps} pages of {ps} tokens" in said and "up to 4 live requests" in said
+    groups = re.findall(r"cache group \d+ \(\w+\): (\d+) pages, (\d+) handed out", said)
+    assert groups and all(int(total) == need // ps and int(takes) > int(total) for total, takes in groups), said

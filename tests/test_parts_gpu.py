@@ -49,12 +49,12 @@ def spec(kind, params=None, weights=None):
     return PartSpec(kind, params or {}, weights or {})
 
 
-def one_sequence_batch(cache, seq, tokens_or_n, vocab=1 << 30):
+def one_sequence_batch(cache, seq, tokens_or_n, vocab=1 << 30, planners=()):
     """The device batch of one entry that brings n tokens to ``seq``."""
     from zedinfer_amd.engine.batch import StepEntry, build_device_batch
     toks = list(tokens_or_n) if not isinstance(tokens_or_n, int) else [0] * tokens_or_n
     cache.ensure(seq, seq.length + len(toks))
-    return build_device_batch([StepEntry(seq, toks, [])], cache, vocab, cache.device)
+    return build_device_batch([StepEntry(seq, toks, [])], cache, vocab, cache.device, planners=planners)
 
 
 # ---- norm -------------------------------------------------------------------------------------
@@ -208,7 +208,7 @@ def test_attention_part_in_portions(dtype, nh, nkv, d, window, bias):
     seq = cache.open("s")
     got, i = [], 0
     for n in [23, 2, 1, 9, 1, 1, 3, 20, 1]:
-        batch = one_sequence_batch(cache, seq, n)
+        batch = one_sequence_batch(cache, seq, n, planners=[mixer.planner()])
         got.append(as_rows(mixer.forward(x[i:i + n].cuda(), batch, mem)).cpu())
         cache.commit(seq, seq.length + n)
         i += n
@@ -269,6 +269,27 @@ def _define_toy():
                 memory.state[int(slot)] = s
             return (out @ self.wout.t()).to(x.dtype)
 
+    @register_mixer("toy_decayed_sum_on_device")
+    class DecayedSumOnDevice(DecayedSum):
+        """The same mixer with nothing but launches over device arrays, so that its steps can be captured
+        as graphs.  It keeps state per request, so padding would advance it: ``padding_safe`` stays False
+        (the default) and the engine must not pad its steps."""
+
+        graph_safe = True
+
+        def forward(self, x, batch, memory):
+            u = x.float() @ self.win.t()                                        # [n, S]
+            t = torch.arange(batch.num_tokens, device=x.device)
+            entry = batch.tok_seq.long()
+            j = (batch.positions - batch.entry_past[entry]).float()             # place of the token in its entry
+            same = (entry[:, None] == entry[None, :]) & (t[None, :] <= t[:, None])
+            m = torch.where(same, self.decay ** (t[:, None] - t[None, :]).clamp(min=0).float(), 0.0)
+            s0 = memory.state[batch.entry_slot.long()][entry]                   # every token's starting state
+            s = m @ u + (self.decay ** (j + 1.0))[:, None] * s0
+            last = (batch.entry_start + batch.entry_len - 1).long()
+            memory.state.index_copy_(0, batch.entry_slot.long(), s[last])
+            return (s @ self.wout.t()).to(x.dtype)
+
     @dataclass(frozen=True)
     class ToyConfig(ModelConfig):
         toy_state_size: int = 8
@@ -283,13 +304,13 @@ def _define_toy():
             cfg.validate()
             return cfg
 
-    def toy_forward_config(cfg: ToyConfig) -> ModelForwardConfig:
+    def toy_forward_config(cfg: ToyConfig, kind: str = "toy_decayed_sum") -> ModelForwardConfig:
         H, nh, nkv, d = cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
         layers = []
         for L in range(cfg.num_hidden_layers):
             p = f"model.layers.{L}."
             if L % 2 == 0:
-                mixer = PartSpec("toy_decayed_sum", {"hidden_size": H, "state_size": cfg.toy_state_size,
+                mixer = PartSpec(kind, {"hidden_size": H, "state_size": cfg.toy_state_size,
                                                      "decay": cfg.toy_decay},
                                  {"win": p + "toy.win.weight", "wout": p + "toy.wout.weight"})
             else:
@@ -314,6 +335,8 @@ def _define_toy():
                              {"weight": "lm_head.weight"}))
 
     register_architecture("ToyStateForCausalLM", ToyConfig, toy_forward_config)
+    register_architecture("ToyStateOnDeviceForCausalLM", ToyConfig,
+                          lambda cfg: toy_forward_config(cfg, "toy_decayed_sum_on_device"))
 
 
 TOY = dict(architectures=["ToyStateForCausalLM"], model_type="toy_state", hidden_size=48, intermediate_size=80,
@@ -377,6 +400,61 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
             assert worst <= 0.08 * scale and mean <= 0.015 * scale, where
     # slots were reused by later requests and started from a zero state each time
     assert engine.cache.slots.takes > engine.cache.slots.total
+
+
+def test_steps_of_a_stateful_mixer_are_not_padded(tmp_path, monkeypatch):
+    """A mixer with state per request that can be captured as a graph: decode steps replay as graphs, but
+    prompt portions, whose graphs need padding, run as they are, because the mixer does not say that
+    padding is harmless to it.  With the flag forced the padding tokens advance the state and the logits
+    are wrong, which is what the flag is for."""
+    _define_toy()
+    from zedinfer_amd.config import SchedulerConfig, load_config
+    from zedinfer_amd.engine import Engine, StepEntry
+    from zedinfer_amd.models import expected_weights
+    from zedinfer_amd.parts import MIXERS
+    from zedinfer_amd.weights import write_model_folder
+    toy = dict(TOY, architectures=["ToyStateOnDeviceForCausalLM"], model_type="toy_state_on_device")
+    folder = str(tmp_path / "toy")
+    os.makedirs(folder)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(toy, f)
+    arch, cfg = load_config(folder)
+    write_model_folder(folder, cfg, expected_weights(arch.forward_config(cfg)), seed=5, dtype=torch.float32,
+                       std=0.08, noisy_norms=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(toy, f)
+    pcfg, w = plain.load_folder(folder)
+    toks = {r: traces.random_tokens(toy["vocab_size"], 150, seed=60 + i) for i, r in enumerate("abc")}
+    ref = {r: toy_plain_forward(pcfg, w, t) for r, t in toks.items()}
+
+    def run(engine):
+        """Portions of 35 tokens (a shape that recurs: it would be padded to 64 and recorded), then single
+        tokens; the worst difference from the plain implementation."""
+        seqs = {r: engine.open(r) for r in toks}
+        fed = {r: 0 for r in toks}
+        worst = 0.0
+        plan = [[(r, 35)] for _ in range(3) for r in "abc"] + [[("a", 1), ("b", 1), ("c", 1)]] * 20
+        for step in plan:
+            out = engine.step([StepEntry(seqs[r], toks[r][fed[r]:fed[r] + n], [n - 1]) for r, n in step])
+            for i, (r, n) in enumerate(step):
+                fed[r] += n
+                worst = max(worst, float((out[i].cpu() - ref[r][fed[r] - 1]).abs().max()))
+        for s in seqs.values():
+            engine.close(s)
+        return worst
+
+    sched = SchedulerConfig(num_kv_blocks=80, kv_block_size=8, max_batch_requests=4)
+    engine = Engine.from_folder(folder, "float32", sched)
+    assert engine.use_graphs and not engine.padding_safe
+    assert run(engine) <= 2e-4
+    assert engine.prompt_graph_replays == 0 and engine.graph_replays >= 10
+    # the same with the mixer claiming that padding is harmless: the portions are padded, recorded and replayed,
+    # the padding tokens advance the state, and the logits that follow are wrong
+    monkeypatch.setattr(MIXERS.get("toy_decayed_sum_on_device"), "padding_safe", True)
+    padded = Engine.from_folder(folder, "float32", sched)
+    assert padded.padding_safe
+    assert run(padded) > 1e-2
+    assert padded.prompt_graph_replays > 0
 
 
 # ---- a second toy architecture: routed feed-forward, another position encoding, a run order that is data ----
@@ -590,3 +668,158 @@ def test_toy_architecture_with_routing_pairs_rotation_and_a_shared_cache(tmp_pat
             # a token whose two best experts are nearly as probable may go to the other one in bfloat16:
             # the mean stays small, single rows may not
             assert mean <= 0.02 * scale, (mean, scale, where)
+
+
+# ---- a third toy architecture: a position encoding with two axes ----------------------------------
+def _define_toy_two_axes():
+    """A position encoding that reads two positions per token (as an encoding of image patches reads a
+    row and a column): the first half of every head's pairs turns by the position on axis 0, the second
+    half by the position on axis 1.  Registered from here; the step's entries may bring positions of
+    their own."""
+    from zedinfer_amd import ops
+    from zedinfer_amd.config.forward_config import LayerSpec, ModelForwardConfig, PartSpec, default_schedule
+    from zedinfer_amd.config.model_config import ModelConfig
+    from zedinfer_amd.config.registry import register_architecture, registered_architectures
+    from zedinfer_amd.parts import PositionEncoding, register_position_encoding
+
+    if "ToyTwoAxesForCausalLM" in registered_architectures():
+        return
+
+    @register_position_encoding("toy_rope_two_axes")
+    class RopeTwoAxes(PositionEncoding):
+        position_axes = 2
+        graph_safe = True       # launches over device arrays only
+
+        def __init__(self, spec, weights, rt):
+            super().__init__(spec, weights, rt)
+            d = int(spec.params["head_dim"])
+            k = torch.arange(d // 2, dtype=torch.float32, device=rt.device)
+            self.inv = 1.0 / torch.pow(torch.tensor(float(spec.params["theta"]), device=rt.device), 2.0 * k / d)
+
+        def turn(self, x, positions, heads, d):
+            assert positions.shape == (x.shape[0], 2)
+            half = d // 2
+            axis = (torch.arange(half, device=x.device) >= half // 2).long()          # pair -> axis
+            ang = positions.float()[:, axis] * self.inv[None, :]                       # [n, d/2]
+            c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+            t = x.float().view(x.shape[0], heads, d)
+            a, b = t[..., :half], t[..., half:]
+            return torch.cat([a * c - b * s, b * c + a * s], dim=-1).view(x.shape[0], heads * d).to(x.dtype)
+
+        def rotate_and_store(self, q, k, v, positions, slots, memory, nh, nkv, d):
+            q.copy_(self.turn(q, positions, nh, d))
+            if memory.writes:
+                kk = self.turn(k, positions, nkv, d)
+                ops.rope_kv_store(q, kk, v.contiguous(), positions[:, 0].contiguous(), slots, None, memory.k,
+                                  memory.v, nh, nkv, d)
+
+    def forward_config(cfg) -> ModelForwardConfig:
+        H, nh, nkv, d = cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim
+        layers = []
+        for L in range(cfg.num_hidden_layers):
+            p = f"model.layers.{L}."
+            mixer = PartSpec("attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                                           "qkv_bias": False, "window": 0,
+                                           "position": PartSpec("toy_rope_two_axes", {"head_dim": d, "theta": cfg.rope_theta})},
+                             {"q": p + "self_attn.q_proj.weight", "k": p + "self_attn.k_proj.weight",
+                              "v": p + "self_attn.v_proj.weight", "o": p + "self_attn.o_proj.weight"})
+            ffn = PartSpec("swiglu", {"hidden_size": H, "intermediate_size": cfg.intermediate_size},
+                           {"gate": p + "mlp.gate_proj.weight", "up": p + "mlp.up_proj.weight",
+                            "down": p + "mlp.down_proj.weight"})
+            norms = {"input": PartSpec("rmsnorm", {"dim": H, "eps": cfg.rms_norm_eps}, {"weight": p + "input_layernorm.weight"}),
+                     "post_mixer": PartSpec("rmsnorm", {"dim": H, "eps": cfg.rms_norm_eps},
+                                            {"weight": p + "post_attention_layernorm.weight"})}
+            layers.append(LayerSpec("prenorm", mixer, ffn, norms))
+        return ModelForwardConfig(
+            architecture="ToyTwoAxesForCausalLM", hidden_size=H, vocab_size=cfg.vocab_size,
+            embedding=PartSpec("token", {"vocab_size": cfg.vocab_size, "hidden_size": H}, {"weight": "model.embed_tokens.weight"}),
+            layers=tuple(layers), schedule=default_schedule(cfg.num_hidden_layers),
+            final_norm=PartSpec("rmsnorm", {"dim": H, "eps": cfg.rms_norm_eps}, {"weight": "model.norm.weight"}),
+            lm_head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": H, "tied_to": None},
+                             {"weight": "lm_head.weight"}))
+
+    register_architecture("ToyTwoAxesForCausalLM", ModelConfig, forward_config)
+
+
+TOY_TWO_AXES = dict(architectures=["ToyTwoAxesForCausalLM"], model_type="toy_two_axes", hidden_size=40, intermediate_size=56,
+                    vocab_size=211, max_position_embeddings=256, num_hidden_layers=2, num_attention_heads=2,
+                    num_key_value_heads=1, head_dim=24, rope_theta=100.0, rms_norm_eps=1e-6)
+
+
+def toy_two_axes_plain_forward(cfg, w, ids, pos2):
+    """``pos2`` [T, 2]: the position of every token on both axes."""
+    w = {k: v.float() for k, v in w.items()}
+    T = len(ids)
+    eps, nh, nkv, d = cfg["rms_norm_eps"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    half = d // 2
+    inv = 1.0 / torch.pow(torch.tensor(cfg["rope_theta"]), 2.0 * torch.arange(half, dtype=torch.float32) / d)
+    ang = torch.cat([pos2[:, :1].float().expand(T, half // 2), pos2[:, 1:].float().expand(T, half - half // 2)], 1) * inv
+
+    def turn(x, heads):
+        t = x.view(T, heads, d)
+        c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        a, b = t[..., :half], t[..., half:]
+        return torch.cat([a * c - b * s, b * c + a * s], dim=-1)
+
+    h = plain.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    for L in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{L}."
+        x = plain.rms_norm(h, w[p + "input_layernorm.weight"], eps)
+        q = turn(plain.linear(x, w[p + "self_attn.q_proj.weight"]), nh)
+        k = turn(plain.linear(x, w[p + "self_attn.k_proj.weight"]), nkv)
+        v = plain.linear(x, w[p + "self_attn.v_proj.weight"]).view(T, nkv, d)
+        a = plain.causal_gqa_attention(q, k, v, 1.0 / math.sqrt(d))
+        h = h + plain.linear(a.reshape(T, nh * d), w[p + "self_attn.o_proj.weight"])
+        x = plain.rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
+        h = h + plain.mlp_block(x, w, p)
+    return plain.linear(plain.rms_norm(h, w["model.norm.weight"], eps), w["lm_head.weight"])
+
+
+def test_toy_architecture_with_positions_on_two_axes(tmp_path):
+    """The step carries positions on as many axes as the model's position encodings read.  Entries that
+    bring none get their tokens' indices on every axis; entries may bring their own (here: a grid whose
+    rows are 7 wide, so that axis 1 runs 0..6 again and again while the cache index goes on counting).
+    Prompt portions, single tokens (replayed as graphs when they bring no positions) and both mixed."""
+    _define_toy_two_axes()
+    from zedinfer_amd.config import SchedulerConfig, load_config
+    from zedinfer_amd.engine import Engine, StepEntry
+    from zedinfer_amd.models import expected_weights
+    from zedinfer_amd.weights import write_model_folder
+    folder = str(tmp_path / "toy_two_axes")
+    os.makedirs(folder)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(TOY_TWO_AXES, f)
+    arch, cfg = load_config(folder)
+    write_model_folder(folder, cfg, expected_weights(arch.forward_config(cfg)), seed=3, dtype=torch.float32, std=0.15,
+                       noisy_norms=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(TOY_TWO_AXES, f)
+    pcfg, w = plain.load_folder(folder)
+    T = 90
+    toks = {r: traces.random_tokens(TOY_TWO_AXES["vocab_size"], T, seed=20 + i) for i, r in enumerate("gs")}
+    idx = torch.arange(T)
+    grid = torch.stack([idx // 7, idx % 7], dim=1)                  # request "g": rows and columns of a grid
+    seqn = torch.stack([idx, idx], dim=1)                           # request "s": brings no positions
+    ref = {"g": toy_two_axes_plain_forward(pcfg, w, toks["g"], grid),
+           "s": toy_two_axes_plain_forward(pcfg, w, toks["s"], seqn)}
+    assert float((ref["g"] - toy_two_axes_plain_forward(pcfg, w, toks["g"], seqn)).abs().max()) > 0.05   # the axes matter
+    engine = Engine.from_folder(folder, "float32", SchedulerConfig(num_kv_blocks=40, kv_block_size=8, max_batch_requests=4))
+    assert engine.position_axes == 2
+    seqs = {r: engine.open(r) for r in toks}
+    fed = {r: 0 for r in toks}
+    worst = 0.0
+    plan = [[("g", 20)], [("s", 33), ("g", 9)], [("g", 1), ("s", 1)], [("g", 17), ("s", 1)]] + [[("s", 1), ("g", 1)]] * 8 \
+        + [[("s", 1)]] * 12 + [[("g", 30)], [("s", 20), ("g", 5)]]
+    for step in plan:
+        entries = []
+        for r, n in step:
+            pos = grid[fed[r]:fed[r] + n].tolist() if r == "g" else None
+            entries.append(StepEntry(seqs[r], toks[r][fed[r]:fed[r] + n], list(range(n)), positions=pos))
+        out = engine.step(entries).cpu()
+        row = 0
+        for r, n in step:
+            worst = max(worst, float((out[row:row + n] - ref[r][fed[r]:fed[r] + n]).abs().max()))
+            fed[r], row = fed[r] + n, row + n
+    assert worst <= 2e-4, worst
+    with pytest.raises(ValueError, match="positions"):
+        engine.step([StepEntry(seqs["g"], [5, 6], [0], positions=[[0, 0]])])

@@ -124,13 +124,18 @@ def run_in_process(engine, steps):
     return out
 
 
-def run_tool(model_dir, dtype, steps, out_dir, max_tokens, timeout=600):
-    """Drive bin/trace_run as a child process, one step at a time, waiting for each 'done'."""
+def run_tool(model_dir, dtype, steps, out_dir, max_tokens, timeout=600, options=(), geometry=None, stderr_to=None):
+    """Drive bin/trace_run as a child process, one step at a time, waiting for each 'done'.  ``options``
+    are further command-line options, ``geometry`` a dict sent as the trace's geometry line;
+    ``stderr_to`` is a file path that receives what the tool says on standard error."""
     os.makedirs(out_dir, exist_ok=True)
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir, "--dtype", dtype,
-           "--out", out_dir, "--max-tokens", str(max_tokens)]
-    p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+           "--out", out_dir, "--max-tokens", str(max_tokens)] + [str(o) for o in options]
+    err = open(stderr_to, "w") if stderr_to else None
+    p = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, stderr=err, text=True)
     try:
+        if geometry is not None:
+            p.stdin.write(json.dumps({"geometry": geometry}) + "\n")
         for st in steps:
             p.stdin.write(json.dumps(st) + "\n")
             p.stdin.flush()
@@ -141,6 +146,8 @@ def run_tool(model_dir, dtype, steps, out_dir, max_tokens, timeout=600):
     finally:
         if p.poll() is None:
             p.kill()
+        if err:
+            err.close()
     out = {}
     for st in steps:
         n = sum(len(e["want"]) for e in st["entries"])

@@ -59,6 +59,15 @@ class CacheGroup:
         return max(0, length - self.window + 1) // self.page_size
 
 
+@dataclass
+class Growth:
+    """What one ``CacheManager.ensure`` took for a sequence."""
+
+    taken: List[Tuple[int, int]]      # (group, logical page) of every page taken
+    grown: List[int]                  # promises added per group, beyond what admission promised
+    old_lens: List[int]               # the block tables' lengths before
+
+
 class SequenceCache:
     """What one live request holds: a state slot and, per group, its block table."""
 
@@ -171,17 +180,16 @@ class CacheManager:
                     seq.held[gi] -= 1
                     seq.version += 1
 
-    def ensure(self, seq: SequenceCache, new_len: int) -> None:
+    def ensure(self, seq: SequenceCache, new_len: int) -> "Growth":
         """Make sure pages exist for every position below ``new_len`` that a token at or after
-        ``seq.length`` can see.  All or nothing: on OutOfPages nothing has changed."""
+        ``seq.length`` can see.  All or nothing: on OutOfPages nothing has changed.  Returns what was
+        taken, which ``undo`` gives back (a step that cannot grow a later request undoes the earlier ones)."""
         if seq.closed:
             raise ValueError(f"request {seq.request_id!r} is closed")
         if new_len < seq.length:
             raise ValueError("a cache cannot shrink")
         self._release_passed(seq)
-        taken: List[Tuple[int, int]] = []
-        grown: List[int] = [0] * len(self.groups)
-        old_lens = [len(t) for t in seq.pages]
+        growth = Growth(taken=[], grown=[0] * len(self.groups), old_lens=[len(t) for t in seq.pages])
         try:
             for gi, g in enumerate(self.groups):
                 table = seq.pages[gi]
@@ -198,23 +206,29 @@ class CacheManager:
                                 f"and all {g.pool.total} are promised")
                         g.pool.commit(1)
                         seq.promised[gi] += 1
-                        grown[gi] += 1
+                        growth.grown[gi] += 1
                     table[i] = g.pool.take()
                     seq.held[gi] += 1
                     seq.version += 1
-                    taken.append((gi, i))
+                    growth.taken.append((gi, i))
         except OutOfPages:
-            for gi, i in taken:
-                self.groups[gi].pool.give_back(seq.pages[gi][i])
-                seq.pages[gi][i] = -1
-                seq.held[gi] -= 1
-            for gi, n in enumerate(grown):
-                self.groups[gi].pool.uncommit(n)
-                seq.promised[gi] -= n
-            for gi, n in enumerate(old_lens):
-                del seq.pages[gi][n:]
-            seq.version += 1
+            self.undo(seq, growth)
             raise
+        return growth
+
+    def undo(self, seq: SequenceCache, growth: "Growth") -> None:
+        """Give back what one ``ensure`` took (pages, promises beyond the admission's, table rows), before
+        anything was committed on top of it."""
+        for gi, i in growth.taken:
+            self.groups[gi].pool.give_back(seq.pages[gi][i])
+            seq.pages[gi][i] = -1
+            seq.held[gi] -= 1
+        for gi, n in enumerate(growth.grown):
+            self.groups[gi].pool.uncommit(n)
+            seq.promised[gi] -= n
+        for gi, n in enumerate(growth.old_lens):
+            del seq.pages[gi][n:]
+        seq.version += 1
 
     def commit(self, seq: SequenceCache, new_len: int) -> None:
         """The tokens below ``new_len`` are in the cache now; give back what no later token sees."""

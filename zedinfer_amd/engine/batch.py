@@ -5,31 +5,36 @@ its prompt, or one decoded token) and the places among them whose logits are
 wanted.  All entries are flattened into one token list without padding
 (reference: src/zedinfer/batch_context.cpp:21-85 builds the same flattened
 ids/positions; there decode rows must come first, here any order works).
+
+Nothing here knows a mixer.  What a mixer's kernels need beyond these arrays (how
+attention divides the tokens between its kernels, for instance) comes from the
+mixer's own ``StepPlanner``: its index arrays are packed into the same host buffer
+and travel in the same copy.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import List, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, SequenceCache
 from ..ops.staging import StagingRing
-
-
-SHORT_ENTRY = 4     # entries of up to this many tokens are attended token by token, split over the keys
-LONG_TILE = 64      # longer entries are cut into tiles of this many queries for the prompt kernel
+from ..parts.base import HostBatch, StepPlan, StepPlanner
 
 
 @dataclass
 class StepEntry:
     """``tokens`` continue the sequence whose cache is ``seq`` at position ``seq.length``;
-    ``want`` lists the places among ``tokens`` whose logits are returned."""
+    ``want`` lists the places among ``tokens`` whose logits are returned.  ``positions`` (optional, for
+    models whose position encoding has several axes): for each token its position on every axis;
+    None: the token's index in its sequence on every axis."""
 
     seq: SequenceCache
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    positions: Optional[Sequence[Sequence[int]]] = None
 
 
 @dataclass
@@ -46,7 +51,7 @@ class DeviceBatch:
     num_entries: int
     num_logit_rows: int
     token_ids: torch.Tensor      # [n]
-    positions: torch.Tensor      # [n] absolute position of each token in its sequence
+    positions: torch.Tensor      # [n] index of each token in its sequence (its place in the cache)
     tok_seq: torch.Tensor        # [n] entry index of each token
     logit_rows: torch.Tensor     # [rows] flat token indices
     entry_start: torch.Tensor    # [entries] first flat token index of the entry
@@ -54,25 +59,17 @@ class DeviceBatch:
     entry_past: torch.Tensor     # [entries] tokens of the entry already in the cache
     entry_slot: torch.Tensor     # [entries] state slot of the entry
     groups: List[GroupView] = field(default_factory=list)
-    # Tokens of entries that bring at most SHORT_ENTRY tokens ("decode" tokens) and the rest, as
-    # lists of flat token indices; None when the list would be all tokens or is empty.
-    short_idx: Optional[torch.Tensor] = None
-    long_idx: Optional[torch.Tensor] = None
-    num_short: int = 0
-    num_long: int = 0
-    max_short_keys: int = 0      # largest position + 1 among the short entries' tokens
-    max_long_keys: int = 0
-    # The long entries cut into tiles of LONG_TILE queries, the tile that sees most keys first:
-    # tile i covers tokens [tile_off[i], tile_off[i] + LONG_TILE) of entry tile_entry[i].
-    tile_entry: Optional[torch.Tensor] = None
-    tile_off: Optional[torch.Tensor] = None
-    num_tiles: int = 0
+    # what position encodings with several axes read: [n, axes]; with one axis it is ``positions`` itself
+    position_ids: Optional[torch.Tensor] = None
+    # the plans of the mixers' planners, by planner key
+    plans: Dict[tuple, StepPlan] = field(default_factory=dict)
     # host copies, for parts that plan their launches on the host
     host_start: Optional[np.ndarray] = None
     host_len: Optional[np.ndarray] = None
     host_past: Optional[np.ndarray] = None
     host_slot: Optional[np.ndarray] = None
     host_image: Optional[np.ndarray] = None      # all index arrays as they were copied to the device
+    device_image: Optional[torch.Tensor] = None  # the device buffer that holds them (every array is a view of it)
     # every entry brings exactly one token (a pure decode step): no token's keys are written by
     # another token of the step, so a mixer may store and attend in one kernel
     single_tokens: bool = False
@@ -83,25 +80,33 @@ class DeviceBatch:
     shared: dict = field(default_factory=dict)
 
 
+FIXED_PIECES = 8      # token ids, positions, tok_seq, logit rows, entry start / len / past / slot
+
+
 def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
                        device: torch.device, staging: Optional[StagingRing] = None,
                        table_widths: Optional[Sequence[int]] = None,
                        static: Optional[torch.Tensor] = None, pad_to: int = 0, pad_entries: int = 0,
-                       pad_rows: int = 0) -> DeviceBatch:
+                       pad_rows: int = 0, planners: Sequence[StepPlanner] = (), position_axes: int = 1,
+                       bound_single: int = 0, bound_multi: int = 0) -> DeviceBatch:
     """Check the entries, then pack every index array into one host buffer and copy it over once.
 
-    ``pad_to``: every entry that brings more than SHORT_ENTRY tokens is run as if it brought a multiple of
-    that many.  The tokens past its own are token 0 at the positions that follow; they have no place in the cache
+    ``pad_to``: every entry that brings more than one token is run as if it brought a multiple of that
+    many.  The tokens past its own are token 0 at the positions that follow; they have no place in the cache
     (slot -1: nothing is stored for them) and no real token sees them, so they change nothing but the
     shapes, which then recur from step to step.  ``pad_entries`` adds that many entries of one token that
-    belong to no request (token 0 at position 0, no slot, an empty block table, state slot 0: only for
-    models without per-request state), ``pad_rows`` that many wanted rows after the real ones (the first
-    token's), to the same end.
+    belong to no request (token 0 at position 0, no slot, an empty block table, state slot 0),
+    ``pad_rows`` that many wanted rows after the real ones (the first token's), to the same end.  Only for
+    models whose mixers all say ``padding_safe``.
 
     ``table_widths`` pads each group's block table to a given width; ``static`` is a device buffer
     the arrays are copied into instead of a fresh one (the layout depends only on the number of
-    tokens, entries, wanted rows and tiles and on the table widths, so a captured graph that reads
-    the arrays finds them at the same addresses every step)."""
+    tokens, entries and wanted rows, on the table widths and on the sizes of the planners' arrays, so a
+    captured graph that reads the arrays finds them at the same addresses every step; the buffer of a
+    step built without ``static`` is ``device_image`` of the result and can serve as ``static`` for the
+    next steps of the same shape).  ``planners``:
+    the planners of the model's mixers, one per key; ``bound_single`` / ``bound_multi`` are handed to
+    them (``HostBatch``).  ``position_axes``: the axes of the model's position encodings."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     seen = set()
@@ -118,12 +123,15 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
         for w in e.want:
             if not (0 <= w < n):
                 raise ValueError(f"request {e.seq.request_id!r}: wanted place {w} is outside its {n} tokens")
+        if e.positions is not None and (position_axes <= 1 or len(e.positions) != n):
+            raise ValueError(f"request {e.seq.request_id!r}: positions need one row of {position_axes} axes for each "
+                             f"of its {n} tokens, and a model whose position encoding has several axes")
         lens.append(n)
     E = len(entries) + int(pad_entries)
     lens = lens + [1] * int(pad_entries)
     real = list(lens)
     if pad_to:
-        lens = [-(-n // int(pad_to)) * int(pad_to) if n > SHORT_ENTRY else n for n in lens]
+        lens = [-(-n // int(pad_to)) * int(pad_to) if n > 1 else n for n in lens]
     N = int(sum(lens))
     starts = np.zeros(E, dtype=np.int32)
     starts[1:] = np.cumsum(lens)[:-1]
@@ -160,24 +168,27 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
         group_tables.append(t)
         widths.append(width)
 
-    short_tok = np.repeat(lens_a <= SHORT_ENTRY, lens)
-    flat = np.arange(N, dtype=np.int32)
-    short_idx, long_idx = flat[short_tok], flat[~short_tok]
-    n_short, n_long = int(short_idx.size), int(long_idx.size)
-    ends = past + lens_a
-    max_short = int(ends[lens_a <= SHORT_ENTRY].max()) if n_short else 0
-    max_long = int(ends[lens_a > SHORT_ENTRY].max()) if n_long else 0
+    single = bool((lens_a == 1).all())
+    hb = HostBatch(num_tokens=N, num_entries=E, entry_start=starts, entry_len=lens_a, entry_past=past,
+                   single_tokens=single, bound_single=int(bound_single), bound_multi=int(bound_multi))
+    plans = {pl.key: pl.plan(hb) for pl in planners}
 
-    tiles = [(int(past[i]) + off + min(LONG_TILE, int(lens_a[i]) - off), i, off)
-             for i in range(E) if lens_a[i] > SHORT_ENTRY for off in range(0, int(lens_a[i]), LONG_TILE)]
-    tiles.sort(key=lambda t: -t[0])
-    tile_entry = np.array([t[1] for t in tiles], dtype=np.int32)
-    tile_off = np.array([t[2] for t in tiles], dtype=np.int32)
-
-    pieces = [token_ids.astype(np.int32), positions, tok_seq, logit_rows, starts, lens_a, past, slot,
-              short_idx, long_idx, tile_entry, tile_off]
+    pieces = [token_ids.astype(np.int32), positions, tok_seq, logit_rows, starts, lens_a, past, slot]
     for g in range(G):
         pieces += [group_slots[g], group_tables[g].reshape(-1)]
+    if position_axes > 1:
+        pos_ids = np.repeat(positions[:, None], position_axes, axis=1)
+        for e, s, r in zip(entries, starts, real):
+            if e.positions is not None:
+                pos_ids[s:s + r] = np.asarray(e.positions, dtype=np.int32).reshape(r, position_axes)
+        pieces.append(pos_ids.reshape(-1))
+    plan_names = []
+    for key, plan in plans.items():
+        for name, a in plan.arrays.items():
+            if a.dtype != np.int32:
+                raise TypeError(f"planner {key}: array '{name}' must be int32")
+            pieces.append(a.reshape(-1))
+            plan_names.append((key, name, a.shape))
     sizes = [p.size for p in pieces]
     total = max(1, sum(sizes))
     host = staging.acquire(total) if staging is not None else torch.empty(
@@ -202,16 +213,20 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     for s in sizes:
         views.append(dev[off:off + s])
         off += s
-    groups = [GroupView(views[12 + 2 * g], views[13 + 2 * g].view(E, widths[g])) for g in range(G)]
+    groups = [GroupView(views[FIXED_PIECES + 2 * g], views[FIXED_PIECES + 1 + 2 * g].view(E, widths[g]))
+              for g in range(G)]
+    nxt = FIXED_PIECES + 2 * G
+    position_ids = views[1]
+    if position_axes > 1:
+        position_ids = views[nxt].view(N, position_axes)
+        nxt += 1
+    for i, (key, name, shape) in enumerate(plan_names):
+        plans[key].dev[name] = views[nxt + i].view(shape)
     return DeviceBatch(num_tokens=N, num_entries=E, num_logit_rows=R, token_ids=views[0], positions=views[1],
                        tok_seq=views[2], logit_rows=views[3], entry_start=views[4], entry_len=views[5],
-                       entry_past=views[6], entry_slot=views[7], groups=groups,
-                       short_idx=views[8] if 0 < n_short < N else None,
-                       long_idx=views[9] if 0 < n_long < N else None, num_short=n_short, num_long=n_long,
-                       max_short_keys=max_short, max_long_keys=max_long, tile_entry=views[10], tile_off=views[11],
-                       num_tiles=len(tiles), host_start=starts,
-                       host_len=lens_a, host_past=past, host_slot=slot, host_image=image,
-                       single_tokens=bool((lens_a == 1).all()),
+                       entry_past=views[6], entry_slot=views[7], groups=groups, position_ids=position_ids,
+                       plans=plans, host_start=starts, host_len=lens_a, host_past=past, host_slot=slot,
+                       host_image=image, device_image=dev, single_tokens=single,
                        all_rows_wanted=bool(R == N and (logit_rows == np.arange(N, dtype=np.int32)).all()))
 
 
@@ -220,21 +235,33 @@ class DecodeImage:
 
     While the same sequences go on decoding, only the token ids, the positions and the cache slots
     change, and a block table row when its sequence took or gave back a page: ``refresh`` rewrites
-    just those in place instead of packing everything anew.  The layout is the one
-    ``build_device_batch`` makes for the same entries and table widths."""
+    just those in place instead of packing everything anew (and the arrays of planners that do not say
+    ``fixed_for_single_tokens``).  The layout is the one ``build_device_batch`` makes for the same
+    entries and table widths."""
 
     def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, device: torch.device,
-                 staging: StagingRing, widths: Sequence[int], static: torch.Tensor):
+                 staging: StagingRing, widths: Sequence[int], static: Optional[torch.Tensor],
+                 planners: Sequence[StepPlanner] = (), position_axes: int = 1, bound_single: int = 0):
         self.cache, self.vocab_size, self.staging, self.static = cache, vocab_size, staging, static
         self.widths = tuple(int(w) for w in widths)
-        self.batch = build_device_batch(entries, cache, vocab_size, device, staging, widths, static)
+        self.planners, self.axes, self.bound_single = tuple(planners), int(position_axes), int(bound_single)
+        self.batch = build_device_batch(entries, cache, vocab_size, device, staging, widths, static,
+                                        planners=planners, position_axes=position_axes, bound_single=bound_single)
+        self.static = self.batch.device_image       # the buffer given, or the one this step made
         E, R = len(entries), self.batch.num_logit_rows
         self.seqs = [e.seq for e in entries]
         self.wants = tuple(len(e.want) for e in entries)
         self.versions = [e.seq.version for e in entries]
-        sizes = [E, E, E, R, E, E, E, E, E, 0, 0, 0]
+        sizes = [E, E, E, R, E, E, E, E]
         for w in self.widths:
             sizes += [E, E * w]
+        if self.axes > 1:
+            sizes.append(E * self.axes)
+        self.plan_pieces = {}          # (planner key, array name) -> index of its piece
+        for key, plan in self.batch.plans.items():
+            for name, a in plan.arrays.items():
+                self.plan_pieces[(key, name)] = len(sizes)
+                sizes.append(int(a.size))
         self.total = sum(sizes)
         self.offsets = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
         self.image = np.empty(max(self.total, 1), dtype=np.int32)
@@ -249,7 +276,8 @@ class DecodeImage:
         if len(entries) != len(self.seqs):
             return False
         for e, s, w in zip(entries, self.seqs, self.wants):
-            if e.seq is not s or len(e.tokens) != 1 or len(e.want) != w or (w and e.want[0] != 0):
+            if (e.seq is not s or len(e.tokens) != 1 or len(e.want) != w or (w and e.want[0] != 0)
+                    or e.positions is not None):
                 return False
         return True
 
@@ -264,8 +292,9 @@ class DecodeImage:
         self.piece(0)[:] = toks
         self.piece(1)[:] = pos
         self.piece(6)[:] = pos
+        G = len(self.widths)
         for g, w in enumerate(self.widths):
-            table = self.piece(13 + 2 * g).reshape(E, w)
+            table = self.piece(FIXED_PIECES + 1 + 2 * g).reshape(E, w)
             for i, s in enumerate(self.seqs):
                 if s.version != self.versions[i]:
                     pg = s.pages[g]
@@ -277,9 +306,26 @@ class DecodeImage:
             pages = table[self.rows, pos // ps]
             if (pages < 0).any():
                 raise RuntimeError("a decoded token's position has no page")
-            self.piece(12 + 2 * g)[:] = pages * ps + pos % ps
+            self.piece(FIXED_PIECES + 2 * g)[:] = pages * ps + pos % ps
+        if self.axes > 1:
+            self.piece(FIXED_PIECES + 2 * G)[:] = np.repeat(pos, self.axes)
         for i, s in enumerate(self.seqs):
             self.versions[i] = s.version
+        moving = [pl for pl in self.planners if not pl.fixed_for_single_tokens]
+        if moving:
+            hb = HostBatch(num_tokens=E, num_entries=E, entry_start=self.batch.host_start,
+                           entry_len=self.batch.host_len, entry_past=pos, single_tokens=True,
+                           bound_single=self.bound_single)
+            for pl in moving:
+                plan = pl.plan(hb)
+                old = self.batch.plans[pl.key]
+                if plan.sizes != old.sizes:
+                    raise RuntimeError(f"planner {pl.key}: launch sizes moved under a recorded step")
+                for name, a in plan.arrays.items():
+                    piece = self.piece(self.plan_pieces[(pl.key, name)])
+                    if a.size != piece.size:
+                        raise RuntimeError(f"planner {pl.key}: array '{name}' changed its size under a recorded step")
+                    piece[:] = a.reshape(-1)
         host = self.staging.acquire(self.total)
         host.numpy()[:] = self.image[:self.total]
         self.static[:self.total].copy_(host, non_blocking=True)

@@ -21,7 +21,7 @@ from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
 from ..sampling.sampler import default_sampling
 from ..weights import load_weights, random_weights
-from .batch import SHORT_ENTRY, DecodeImage, StagingRing, StepEntry, build_device_batch
+from .batch import DecodeImage, StagingRing, StepEntry, build_device_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
            "f32": torch.float32}
@@ -83,7 +83,11 @@ class Engine:
         self.prompt_graph_limit = 128    # shapes held; the one used longest ago goes first
         self._prompt_graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.prompt_graph_replays = 0
-        self._has_state = bool(self.model.state_requests())
+        # what the batch is built with: the planners of the mixers' launches, the axes of the position
+        # encodings, and whether steps may be padded (every mixer must say that padding is harmless to it)
+        self.planners = self.model.planners()
+        self.position_axes = self.model.position_axes()
+        self.padding_safe = self.model.padding_safe()
 
     # ---- construction ------------------------------------------------------------
     @classmethod
@@ -182,14 +186,21 @@ class Engine:
             if (token_source.dtype != torch.int32 or token_source.device != self.device
                     or token_source.shape != (len(entries),)):
                 raise ValueError(f"token_source must be an int32 tensor [{len(entries)}] on {self.device}")
-        for e in entries:
-            self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
+        grown = []
+        try:
+            for e in entries:
+                grown.append((e.seq, self.cache.ensure(e.seq, e.seq.length + len(e.tokens))))
+        except Exception:
+            for seq, growth in reversed(grown):      # nothing of a step that cannot run stays
+                self.cache.undo(seq, growth)
+            raise
         if self.use_graphs and 0 < len(entries) <= self.graph_max_entries and single:
             logits = self._graph_step(entries, token_source)
         elif self.use_graphs and token_source is None and self._one_portion(entries):
             logits = self._prompt_graph_step(entries)
         else:
-            batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging)
+            batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging,
+                                       planners=self.planners, position_axes=self.position_axes)
             if token_source is not None:
                 batch.token_ids.copy_(token_source, non_blocking=True)
             logits = self.model.run(batch, self.memories)
@@ -209,26 +220,26 @@ class Engine:
         R = sum(len(e.want) for e in entries)
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
-        max_keys = max(e.seq.length for e in entries) + 1
-        keys_bucket = _pow2_at_least(max_keys, 256)
-        key = (E, R, widths, keys_bucket)
+        # a bound, the same for many steps, of the tokens any sequence holds after this step: the
+        # mixers' planners size their launches by it
+        bound = _pow2_at_least(max(e.seq.length for e in entries) + 1, 256)
+        key = (E, R, widths, bound)
         dg = self._graphs.pop(key, None)
         if dg is not None:
             self._graphs[key] = dg              # used last: the last to go
         else:
             if len(self._graphs) >= self.graph_limit:
                 self._drop_oldest(self._graphs)
-            size = 8 * E + 2 * R + sum(E * (w + 1) for w in widths) + 64
-            dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
-            self._graphs[key] = dg
+            dg = self._graphs[key] = _DecodeGraph()
         if dg.image is not None and dg.image.matches(entries):
             batch = dg.image.refresh(entries)      # the same sequences go on: only what changed is rewritten
         else:
-            dg.image = DecodeImage(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer)
+            dg.image = DecodeImage(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
+                                   planners=self.planners, position_axes=self.position_axes, bound_single=bound)
+            dg.buffer = dg.image.static         # the first step's buffer serves all later ones of the shape
             batch = dg.image.batch
         if token_source is not None:
             batch.token_ids.copy_(token_source, non_blocking=True)
-        batch.max_short_keys = keys_bucket
         if dg.graph is not None:
             dg.graph.replay()
             self.graph_replays += 1
@@ -258,20 +269,23 @@ class Engine:
     PROMPT_GRAPH_STEP = 64
 
     def _one_portion(self, entries: Sequence[StepEntry]) -> bool:
-        """Portions of prompts (more than SHORT_ENTRY tokens each) of a size worth a graph together, beside
-        any number of single decoded tokens; at most one row wanted of each."""
+        """Portions of prompts (entries of several tokens) of a size worth a graph together, beside any
+        number of single decoded tokens; at most one row wanted of each.  Such steps are padded, so every
+        mixer must have said that padding is harmless to it."""
+        if not self.padding_safe:
+            return False
         total = 0
         for e in entries:
             n = len(e.tokens)
-            if len(e.want) > 1 or 1 < n <= SHORT_ENTRY:
+            if len(e.want) > 1 or e.positions is not None:
                 return False
             if n > 1:
                 total += -(-n // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
         return 0 < total <= self.prompt_graph_max_tokens and len(entries) <= self.graph_max_entries
 
     def _prompt_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
-        """A step of one portion of a prompt (more than SHORT_ENTRY tokens) beside single decoded tokens,
-        with the portion run as if it brought a multiple of PROMPT_GRAPH_STEP tokens (see
+        """A step of portions of prompts (entries of several tokens) beside single decoded tokens,
+        with every portion run as if it brought a multiple of PROMPT_GRAPH_STEP tokens (see
         ``build_device_batch``): the first step of a kind runs eagerly, the second is captured, later
         ones replay."""
         step = self.PROMPT_GRAPH_STEP
@@ -279,7 +293,7 @@ class Engine:
         padded = sum(-(-len(e.tokens) // step) * step for e in portions)      # tokens of all portions, padded
         wanted = sum(len(e.want) for e in entries)
         E, R, more_entries = len(entries), wanted, 0
-        if E > 1 and not self._has_state:
+        if E > 1:
             # the numbers of portions and of decoding requests move from step to step: the entries are brought
             # to a multiple of 8 with entries that belong to no request, and a row is wanted of every entry
             more_entries = -(-E // 8) * 8 - E
@@ -297,15 +311,12 @@ class Engine:
         else:
             if len(self._prompt_graphs) >= self.prompt_graph_limit:
                 self._drop_oldest(self._prompt_graphs)
-            N = padded + singles
-            size = 8 * N + R + 8 * E + sum(N + E * w for w in widths) + 64
-            dg = _DecodeGraph(torch.zeros((size,), dtype=torch.int32, device=self.device))
-            self._prompt_graphs[key] = dg
+            dg = self._prompt_graphs[key] = _DecodeGraph()
         batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
-                                   pad_to=step, pad_entries=more_entries, pad_rows=R - wanted)
-        batch.max_long_keys = long_bucket
-        if singles:
-            batch.max_short_keys = short_bucket
+                                   pad_to=step, pad_entries=more_entries, pad_rows=R - wanted,
+                                   planners=self.planners, position_axes=self.position_axes,
+                                   bound_single=short_bucket if singles else 0, bound_multi=long_bucket)
+        dg.buffer = batch.device_image          # the first step's buffer serves all later ones of the shape
         if dg.graph is not None:
             dg.graph.replay()
             self.prompt_graph_replays += 1
@@ -326,8 +337,8 @@ class Engine:
 
 
 class _DecodeGraph:
-    def __init__(self, buffer: torch.Tensor):
-        self.buffer = buffer
+    def __init__(self):
+        self.buffer: Optional[torch.Tensor] = None      # the device buffer of the step's index arrays
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
         self.warm = False

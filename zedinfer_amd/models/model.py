@@ -105,6 +105,23 @@ class DecoderModel:
                 out[st.cache] = req
         return out
 
+    def planners(self) -> tuple:
+        """The planners of the mixers' launches, one per key, in the order of the layers."""
+        out = {}
+        for b in self.blocks:
+            pl = b.mixer.planner()
+            if pl is not None and pl.key not in out:
+                out[pl.key] = pl
+        return tuple(out.values())
+
+    def position_axes(self) -> int:
+        """The axes the step's positions need: the most any position encoding of the model reads."""
+        return max([int(getattr(p, "position_axes", 1)) for p in self.parts] + [1])
+
+    def padding_safe(self) -> bool:
+        """Whether steps may be padded to recurring shapes: every mixer says that padding is harmless to it."""
+        return all(getattr(b.mixer, "padding_safe", False) for b in self.blocks)
+
     def graph_safe(self) -> bool:
         """Whether a step's launches can be captured and replayed: every part says so."""
         return all(getattr(p, "graph_safe", False) for p in self.parts)

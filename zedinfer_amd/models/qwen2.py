@@ -9,12 +9,21 @@ src/frontend/models/forward_config.hpp:176-192 with the ``model.`` prefix the
 checkpoint carries, src/frontend/models/base.cpp:1386-1410).
 
 Sliding window.  The reference parses ``use_sliding_window``, ``sliding_window``
-and ``max_window_layers`` and never reads them (reference: base.cpp:807-813).
-Here they select the mixer per layer: with ``use_sliding_window`` the layers
-from ``max_window_layers`` on see only the last ``sliding_window`` keys, the
-first ``max_window_layers`` layers see all keys.
+and ``max_window_layers`` and never reads them (reference: base.cpp:807-813):
+it attends over all keys in every layer whatever they say.  Here they select
+the mixer per layer, by the meaning the keys have in the Qwen2 configuration
+format ("max_window_layers: the first that many layers use full attention, the
+layers after them the sliding window"): with ``use_sliding_window`` the layers
+from ``max_window_layers`` on see only the last ``sliding_window`` keys.  So for
+a configuration with ``use_sliding_window: true`` this engine's logits differ
+from the reference's as soon as a sequence is longer than the window; no file of
+the reference pins the windowed case.  ``ZEDINFER_IGNORE_SLIDING_WINDOW=1`` in
+the environment makes every layer attend over all keys, as the reference does.
+All configurations of the benchmarks say ``use_sliding_window: false``.
 """
 from __future__ import annotations
+
+import os
 
 from ..config.forward_config import (LayerSpec, ModelForwardConfig, PartSpec, default_schedule)
 from ..config.model_config import Qwen2Config
@@ -22,6 +31,9 @@ from ..config.registry import register_architecture
 
 
 def layer_window(cfg: Qwen2Config, layer: int) -> int:
+    """Keys layer ``layer`` sees (0: all of them)."""
+    if os.environ.get("ZEDINFER_IGNORE_SLIDING_WINDOW", "0") not in ("", "0"):
+        return 0        # the reference's behaviour: the window keys are parsed and not used
     if cfg.use_sliding_window and layer >= cfg.max_window_layers:
         return cfg.sliding_window
     return 0

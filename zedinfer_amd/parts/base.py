@@ -7,7 +7,7 @@ runtime) and never learns which model it sits in.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable, Dict, Optional, Tuple
 
 import torch
@@ -165,6 +165,54 @@ class Part:
         ``forward`` only reads ``rt.choices``; without an entry it takes a fixed default."""
 
 
+@dataclass
+class HostBatch:
+    """A step as a planner sees it, on the host: entry e brings ``entry_len[e]`` tokens (those added as
+    padding included), the flat tokens ``entry_start[e]...``, after ``entry_past[e]`` tokens already in
+    the cache.
+
+    ``bound_single`` / ``bound_multi``: when a step is to be replayed as a graph, launch sizes must recur
+    from step to step, so the engine gives upper bounds that do: no entry of one token (of several
+    tokens) holds more than this many tokens once the step has run.  0: no bound is given, exact sizes
+    are fine."""
+
+    num_tokens: int
+    num_entries: int
+    entry_start: "np.ndarray"
+    entry_len: "np.ndarray"
+    entry_past: "np.ndarray"
+    single_tokens: bool
+    bound_single: int = 0
+    bound_multi: int = 0
+
+
+@dataclass
+class StepPlan:
+    """What a planner makes of a step: int32 index arrays, which travel to the device with the step's
+    other arrays in the same copy (``dev`` then holds them under the same names), and launch sizes the
+    host needs."""
+
+    arrays: Dict[str, "np.ndarray"] = field(default_factory=dict)
+    sizes: Dict[str, int] = field(default_factory=dict)
+    dev: Dict[str, torch.Tensor] = field(default_factory=dict)
+
+
+class StepPlanner:
+    """Plans a mixer's launches for one step on the host.  A mixer whose kernels need index arrays or
+    launch sizes derived from the step's entries returns one from ``Mixer.planner()``; planners with
+    equal ``key`` are run once per step and share the plan (``batch.plans[key]``).  The names, the order
+    and, for steps of equal (tokens, entries), the sizes of ``arrays`` must not depend on the step's
+    contents beyond what ``sizes`` reports: a captured graph reads them at fixed places."""
+
+    key: tuple = ()
+    # In steps in which every entry brings one token the arrays depend on the number of entries only:
+    # they need not be made again while the same requests go on decoding.
+    fixed_for_single_tokens: bool = False
+
+    def plan(self, hb: HostBatch) -> StepPlan:
+        raise NotImplementedError
+
+
 class Mixer(Part):
     """Mixes information across the tokens of a sequence.
 
@@ -174,6 +222,19 @@ class Mixer(Part):
     the few-rows matrix product leaves when it is cut along k).  ``batch`` is the step's
     device-side description (``engine.batch.DeviceBatch``); ``memory`` is this run's
     ``LayerMemory``."""
+
+    # To make the shapes of steps recur (so that they can be replayed as graphs) the engine may run an
+    # entry of several tokens as if it brought more: tokens of id 0 at the positions that follow, with no
+    # place in the cache (slot -1), whose results nobody reads; and it may add entries of one such token
+    # that belong to no request (state slot 0, an empty block table).  A mixer for which that changes
+    # nothing any real token sees sets this; one that keeps state per request must leave it False, or
+    # the padding would advance its state.  One mixer that leaves it False keeps the whole model's steps
+    # unpadded.
+    padding_safe: bool = False
+
+    def planner(self) -> Optional[StepPlanner]:
+        """The planner of this mixer's launches, or None when its kernels need no more than the batch."""
+        return None
 
     def cache_request(self) -> Optional[KVCacheRequest]:
         return None
@@ -218,7 +279,13 @@ class PositionEncoding(Part):
     is a rotation of pairs (k, k + R/2) of the first R dims of every head returns the step's angles
     as a float32 tensor [n, R/2, 2] of (cos, sin), computed once per step and kept in
     ``batch.shared``; an encoding that does nothing returns the string "none"; every other encoding
-    returns None (the default), and the mixer calls ``rotate_and_store*``."""
+    returns None (the default), and the mixer calls ``rotate_and_store*``.
+
+    ``positions`` is what the step gives for each token: int32 [n], the token's index in its sequence,
+    when ``position_axes`` is 1; with more axes int32 [n, position_axes], every axis the index in the
+    sequence unless the caller of the step gave the entry positions of its own (``StepEntry.positions``)."""
+
+    position_axes: int = 1
 
     def step_table(self, batch):
         return None

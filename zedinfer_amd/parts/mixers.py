@@ -4,13 +4,62 @@ from __future__ import annotations
 import math
 from typing import Dict, Optional
 
+import numpy as np
 import torch
 
 from .. import ops
 from ..config.forward_config import PartSpec
 from ..weights.loader import WeightSpec
-from .base import (KVCacheRequest, LayerMemory, Mixer, POSITION_ENCODINGS, Runtime, register_mixer)
+from .base import (HostBatch, KVCacheRequest, LayerMemory, Mixer, POSITION_ENCODINGS, Runtime, StepPlan, StepPlanner,
+                   register_mixer)
 from .feed_forward import stack_rows
+
+SHORT_ENTRY = 4     # entries of up to this many tokens are attended token by token, split over the keys
+LONG_TILE = 64      # longer entries are cut into tiles of this many queries for the prompt kernel
+
+
+class AttentionPlanner(StepPlanner):
+    """How the attention kernels divide a step: tokens of entries that bring at most SHORT_ENTRY tokens
+    ("decoded" tokens) go, one by one, to the kernel that splits a query's keys over many wavefronts;
+    longer entries are cut into tiles of LONG_TILE queries for the prompt kernel, the tile that sees
+    most keys first.
+
+    arrays: ``short_idx`` / ``long_idx``, the flat indices of the tokens of either kind; ``tile_entry`` /
+    ``tile_off``: tile i covers tokens [tile_off[i], tile_off[i] + LONG_TILE) of entry tile_entry[i].
+    sizes: ``num_short``, ``num_long``, ``num_tiles``; ``max_short_keys`` / ``max_long_keys``: an upper
+    bound of the keys a token of either kind sees (its position + 1), which sizes the launches."""
+
+    key = ("attention", SHORT_ENTRY, LONG_TILE)
+    fixed_for_single_tokens = True
+
+    def plan(self, hb: HostBatch) -> StepPlan:
+        lens, past = hb.entry_len, hb.entry_past
+        short = lens <= SHORT_ENTRY
+        short_tok = np.repeat(short, lens)
+        flat = np.arange(hb.num_tokens, dtype=np.int32)
+        short_idx, long_idx = flat[short_tok], flat[~short_tok]
+        ends = past + lens
+        max_short = int(ends[short].max()) if short_idx.size else 0
+        max_long = int(ends[~short].max()) if long_idx.size else 0
+        if short_idx.size and (hb.bound_single or hb.bound_multi):
+            # bounds that recur from step to step (the step is replayed as a graph)
+            several = bool((lens[short] > 1).any())
+            max_short = max(hb.bound_single if bool((lens[short] == 1).any()) else 0,
+                            hb.bound_multi if several else 0, 1)
+        if long_idx.size and hb.bound_multi:
+            max_long = hb.bound_multi
+        tiles = [(int(past[i]) + off + min(LONG_TILE, int(lens[i]) - off), i, off)
+                 for i in range(hb.num_entries) if not short[i] for off in range(0, int(lens[i]), LONG_TILE)]
+        tiles.sort(key=lambda t: -t[0])
+        return StepPlan(
+            arrays={"short_idx": short_idx, "long_idx": long_idx,
+                    "tile_entry": np.array([t[1] for t in tiles], dtype=np.int32),
+                    "tile_off": np.array([t[2] for t in tiles], dtype=np.int32)},
+            sizes={"num_short": int(short_idx.size), "num_long": int(long_idx.size), "num_tiles": len(tiles),
+                   "max_short_keys": max_short, "max_long_keys": max_long})
+
+
+_ATTENTION_PLANNER = AttentionPlanner()
 
 
 @register_mixer("attention")
@@ -27,6 +76,7 @@ class Attention(Mixer):
     scale (default 1/sqrt(head_dim)), position (a PartSpec of a position encoding)."""
 
     graph_safe = True
+    padding_safe = True      # padding has no place in the cache, and causal attention lets no real token see it
     # Every workgroup of the fused kernel adds and rotates its token's query again (one per chunk of
     # 256 keys), which costs more than the separate rotary kernel once many tokens decode together:
     # measured faster at 1 and 8 tokens, slower at 64.
@@ -55,8 +105,7 @@ class Attention(Mixer):
         self.nh, self.nkv, self.d = int(p["num_heads"]), int(p["num_kv_heads"]), int(p["head_dim"])
         if self.nh % self.nkv:
             raise ValueError(f"attention: {self.nh} heads are not a multiple of {self.nkv} key/value heads")
-        if self.d % 16:
-            raise ValueError(f"attention: head_dim {self.d} must be a multiple of 16")
+        # any head size: the matrix-core kernels take multiples of 16 up to 128, the plain ones the rest
         self.window = int(p.get("window", 0) or 0)
         self.scale = float(p.get("scale") or 1.0 / math.sqrt(self.d))
         self.qd, self.kvd = self.nh * self.d, self.nkv * self.d
@@ -82,27 +131,37 @@ class Attention(Mixer):
         not take goes to the plain one."""
         args = (memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
                 self.scale)
-        n_long = batch.num_long
-        if batch.num_short:
+        plan = batch.plans[_ATTENTION_PLANNER.key]
+        n_short, n_long, N = plan.sizes["num_short"], plan.sizes["num_long"], batch.num_tokens
+        if n_short:
             if ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
-                ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(batch.num_short, self.nh, self.d),),
+                ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n_short, self.nh, self.d),),
                                     torch.float32)
-                ops.attention_decode(q, *args, batch.max_short_keys, self.window, out=att,
-                                     tok_index=batch.short_idx, workspace=ws)
+                ops.attention_decode(q, *args, plan.sizes["max_short_keys"], self.window, out=att,
+                                     tok_index=plan.dev["short_idx"] if n_short < N else None, workspace=ws)
             else:
                 n_long = -1      # everything through the plain kernel
         if n_long < 0:
             ops.attention(q, *args, self.window, out=att)
         elif n_long > 0:
             if ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
-                need = ops.attention_prefill_workspace(q.shape[0], self.nh, self.d, batch.max_long_keys, self.window)
+                max_keys = plan.sizes["max_long_keys"]
+                need = ops.attention_prefill_workspace(q.shape[0], self.nh, self.d, max_keys, self.window)
                 ws = self.rt.buffer("attn_prompt_split", (need,), torch.float32) if need else None
-                ops.attention_prefill(q, memory.k, memory.v, batch.tile_entry, batch.tile_off, batch.entry_start,
-                                      batch.entry_len, batch.entry_past, view.block_tables, self.nh, self.nkv,
-                                      self.d, self.scale, self.window, out=att, max_keys=batch.max_long_keys,
+                ops.attention_prefill(q, memory.k, memory.v, plan.dev["tile_entry"], plan.dev["tile_off"],
+                                      batch.entry_start, batch.entry_len, batch.entry_past, view.block_tables, self.nh,
+                                      self.nkv, self.d, self.scale, self.window, out=att, max_keys=max_keys,
                                       workspace=ws)
             else:
-                ops.attention(q, *args, self.window, out=att, tok_index=batch.long_idx)
+                ops.attention(q, *args, self.window, out=att, tok_index=plan.dev["long_idx"] if n_long < N else None)
+
+    def planner(self) -> StepPlanner:
+        return _ATTENTION_PLANNER
+
+    def positions_of(self, batch) -> torch.Tensor:
+        """What the position encoding is given: every token's index in its sequence, or the step's
+        positions on several axes when the encoding has more than one."""
+        return batch.position_ids if self.position.position_axes > 1 else batch.positions
 
     def cache_request(self) -> Optional[KVCacheRequest]:
         return KVCacheRequest("window" if self.window > 0 else "full", self.nkv, self.d, self.window)
@@ -119,7 +178,7 @@ class Attention(Mixer):
             if out is not None:
                 return out
             q = self.rt.buffer("attn_q", (n, self.qd))
-            self.position.rotate_and_store_sums(sums, self.bias, q, batch.positions, view.slots, memory, self.nh,
+            self.position.rotate_and_store_sums(sums, self.bias, q, self.positions_of(batch), view.slots, memory, self.nh,
                                                 self.nkv, self.d)
         else:
             qkv = self.rt.buffer("attn_qkv", (n, self.qd + 2 * self.kvd))
@@ -129,7 +188,8 @@ class Attention(Mixer):
             else:
                 for dst, m, b in zip((q, k, v), self.mats, self.biases or (None, None, None)):
                     ops.linear(x, m, b, out=dst)
-            self.position.rotate_and_store(q, k, v, batch.positions, view.slots, memory, self.nh, self.nkv, self.d)
+            self.position.rotate_and_store(q, k, v, self.positions_of(batch), view.slots, memory, self.nh, self.nkv,
+                                           self.d)
         att = self.rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
         return self.project(att, n)
@@ -154,20 +214,21 @@ class Attention(Mixer):
         rot = 0 if isinstance(table, str) else 2 * table.shape[1]
         S, n, width = sums.shape
         ps = memory.k.shape[2]
+        max_keys = batch.plans[_ATTENTION_PLANNER.key].sizes["max_short_keys"]
         if not ops.attention_decode_fused_supported(memory.k.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
             return None
         ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
         # every entry brings one token: token t is of entry t
         args = (sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None, memory.k, memory.v,
                 None, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale,
-                batch.max_short_keys, self.window)
+                max_keys, self.window)
         if (self.o.numel() * self.o.element_size() <= self.PROJECT_FROM_CHUNKS_MAX_BYTES
                 and ops.attention_decode_project_supported(self.o, n, self.nh, self.d)):
             ops.attention_decode_fused(*args, workspace=ws, write_kv=memory.writes, leave_chunks=True)
             out = self.rt.buffer("attn_proj_heads", (ops.attention_decode_project_splits(self.nh), n, self.hidden),
                                  torch.float32)
-            return ops.attention_decode_project(ws, self.o, batch.positions, self.nh, self.d, batch.max_short_keys,
-                                                self.window, out=out)
+            return ops.attention_decode_project(ws, self.o, batch.positions, self.nh, self.d, max_keys, self.window,
+                                                out=out)
         att = self.rt.buffer("attn_out", (n, self.qd))
         ops.attention_decode_fused(*args, out=att, workspace=ws, write_kv=memory.writes)
         return self.project(att, n)

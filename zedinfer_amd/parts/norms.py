@@ -21,7 +21,9 @@ class RMSNorm(Norm):
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((int(spec.params["dim"]),))}
+        # a gain: 1 in random-weights mode (0 when the norm multiplies by 1 + w)
+        return {"weight": WeightSpec((int(spec.params["dim"]),),
+                                     init="zeros" if spec.params.get("add_one", False) else "ones")}
 
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         super().__init__(spec, weights, rt)

@@ -14,6 +14,7 @@ bfloat16.  In the float32 engine everything floating is widened to float32
 """
 from __future__ import annotations
 
+import sys
 from dataclasses import dataclass
 from typing import Dict, List, Mapping, Optional, Tuple
 
@@ -39,6 +40,9 @@ class WeightSpec:
     shape: Tuple[int, ...]
     kind: str = "float"              # "float" or "int"
     fallback: Optional[str] = None   # tensor to alias when this one is absent (tied head)
+    # what the random-weights mode fills it with: "normal" (N(0, std)), "ones" (a gain: 1, or 1 + N(0, std)
+    # with noisy gains) or "zeros"
+    init: str = "normal"
 
 
 def canonical_name(name: str) -> str:
@@ -108,6 +112,13 @@ def load_weights(folder: str, expected: Mapping[str, WeightSpec], engine_dtype: 
         for name, spec in expected.items():
             if name not in out:
                 out[name] = out[_expected_name(expected, spec.fallback)]
+        if engine_dtype == torch.bfloat16:
+            wide = [n for n, t in out.items() if t.dtype == torch.float32 and t.dim() >= 2]
+            if wide:
+                # said once per load: such a model runs, but far from the speed of a bfloat16 checkpoint
+                print(f"[zedinfer_amd] {len(wide)} of {len(out)} tensors in {folder} are stored in 32 bits and stay so "
+                      f"(first: {wide[0]}); their matrix products take the plain 32-bit kernel, not the matrix cores. "
+                      "Store the checkpoint in bfloat16 for serving speed.", file=sys.stderr, flush=True)
         return out
     finally:
         st.close()

@@ -2,9 +2,12 @@
 
 The reference has no such mode; benchmarks and tests here need models without
 a checkpoint.  A tensor's values depend only on (seed, tensor name), so the
-order in which tensors are made does not matter.  Matrices and biases are
-N(0, std); norm weights are 1, or 1 + N(0, std) when ``noisy_norms`` is set so
-that a forgotten weight multiply shows.
+order in which tensors are made does not matter.  What a tensor is filled with
+is the part's word (``WeightSpec.init``), not guessed from its name: "normal"
+tensors (matrices, biases) are N(0, std); "ones" (the gains of norms) are 1, or
+1 + N(0, std) when ``noisy_norms`` is set so that a forgotten weight multiply
+shows; "zeros" (gains that are added to 1) are 0, or N(0, std) with
+``noisy_norms``.
 """
 from __future__ import annotations
 
@@ -23,10 +26,6 @@ def _tensor_seed(seed: int, name: str) -> int:
     return int.from_bytes(h[:8], "little") & 0x7FFF_FFFF_FFFF_FFFF
 
 
-def _is_norm(name: str, spec: WeightSpec) -> bool:
-    return len(spec.shape) == 1 and ("norm" in name) and name.endswith("weight")
-
-
 def random_weights(expected: Mapping[str, WeightSpec], seed: int, dtype: torch.dtype,
                    device: torch.device | str = "cpu", std: float = 0.02,
                    noisy_norms: bool = False, tied: bool = True) -> Dict[str, torch.Tensor]:
@@ -42,12 +41,18 @@ def random_weights(expected: Mapping[str, WeightSpec], seed: int, dtype: torch.d
         if spec.kind == "int":
             out[name] = torch.zeros(spec.shape, dtype=torch.int32, device=device)
             continue
-        if _is_norm(name, spec):
+        if spec.init == "ones":
             t = torch.ones(spec.shape, dtype=torch.float32, device=device)
             if noisy_norms:
                 t += torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
-        else:
+        elif spec.init == "zeros":
+            t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
+            if noisy_norms:
+                t += torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
+        elif spec.init == "normal":
             t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
+        else:
+            raise ValueError(f"tensor '{name}': unknown init '{spec.init}' (normal, ones, zeros)")
         out[name] = t.to(dtype)
     for name, spec in expected.items():
         if name not in out:
