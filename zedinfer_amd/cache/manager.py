@@ -68,6 +68,9 @@ class Growth:
     old_lens: List[int]               # the block tables' lengths before
 
 
+NO_GROWTH = Growth(taken=[], grown=[], old_lens=[])      # what ``ensure`` returns when it took nothing
+
+
 class SequenceCache:
     """What one live request holds: a state slot and, per group, its block table."""
 
@@ -183,22 +186,29 @@ class CacheManager:
     def ensure(self, seq: SequenceCache, new_len: int) -> "Growth":
         """Make sure pages exist for every position below ``new_len`` that a token at or after
         ``seq.length`` can see.  All or nothing: on OutOfPages nothing has changed.  Returns what was
-        taken, which ``undo`` gives back (a step that cannot grow a later request undoes the earlier ones)."""
+        taken, which ``undo`` gives back (a step that cannot grow a later request undoes the earlier ones);
+        NO_GROWTH when nothing was (a decoded token inside its page: most calls, which therefore make no
+        objects)."""
         if seq.closed:
             raise ValueError(f"request {seq.request_id!r} is closed")
         if new_len < seq.length:
             raise ValueError("a cache cannot shrink")
         self._release_passed(seq)
-        growth = Growth(taken=[], grown=[0] * len(self.groups), old_lens=[len(t) for t in seq.pages])
+        growth = None
         try:
             for gi, g in enumerate(self.groups):
                 table = seq.pages[gi]
                 last = (new_len - 1) // g.page_size if new_len > 0 else -1
-                while len(table) <= last:
-                    table.append(-1)
+                if len(table) <= last:
+                    if growth is None:
+                        growth = Growth(taken=[], grown=[0] * len(self.groups), old_lens=[len(t) for t in seq.pages])
+                    while len(table) <= last:
+                        table.append(-1)
                 for i in range(g.first_live_page(seq.length), last + 1):
                     if table[i] >= 0:
                         continue
+                    if growth is None:
+                        growth = Growth(taken=[], grown=[0] * len(self.groups), old_lens=[len(t) for t in seq.pages])
                     if seq.held[gi] + 1 > seq.promised[gi]:
                         if g.pool.uncommitted < 1:
                             raise OutOfPages(
@@ -214,11 +224,13 @@ class CacheManager:
         except OutOfPages:
             self.undo(seq, growth)
             raise
-        return growth
+        return growth if growth is not None else NO_GROWTH
 
     def undo(self, seq: SequenceCache, growth: "Growth") -> None:
         """Give back what one ``ensure`` took (pages, promises beyond the admission's, table rows), before
         anything was committed on top of it."""
+        if growth is NO_GROWTH:
+            return
         for gi, i in growth.taken:
             self.groups[gi].pool.give_back(seq.pages[gi][i])
             seq.pages[gi][i] = -1

@@ -1,7 +1,7 @@
 // out[M,N] = x[M,K] . w[N,K]^T (+ bias) for 17..64 rows of x: decoding at larger batches, still bound
 // by the one pass over the weights.
 //
-// A workgroup of four wavefronts owns 64 weight rows (16 a wavefront) and a range of k.  It walks its
+// A workgroup of four to eight wavefronts owns 16 weight rows a wavefront and a range of k.  It walks its
 // k-blocks of 128: the block's slice of x (up to 64 rows x 128 values) is staged in LDS once for the four
 // wavefronts, each wavefront reads its own 16 weight rows from memory as whole cache lines, turns them
 // into matrix-core operands through a piece of LDS of its own (v_mfma_f32_16x16x32_bf16, float32
@@ -20,11 +20,12 @@ typedef __attribute__((ext_vector_type(4))) float gm_f32x4_t;
 // them that is only copied stays in memory instead of registers
 typedef __attribute__((ext_vector_type(4))) unsigned gm_u32x4_t;
 
-#define GM_WAVES 4
-#define GM_ROWS 64          // weight rows per workgroup
+#define GM_MIN_WAVES 4      // wavefronts of a workgroup: 4 .. 8, 16 weight rows each
+#define GM_MAX_WAVES 8
+#define GM_STAGERS 256      // threads that stage the block's x slice (the first four wavefronts)
 #define GM_KB 128
 #define GM_XS GM_KB         // LDS row stride, in elements: rows of 16 pieces of 16 bytes, piece c of row r at place c xor (r mod 16)
-#define GM_TARGET_WGS 384
+#define GM_CUS 256          // compute units the cut is balanced over
 
 #define GM_MODE_PLAIN 0
 #define GM_MODE_PARTIAL 1
@@ -42,7 +43,7 @@ __device__ __forceinline__ gm_u32x4_t gm_keep(gm_u32x4_t v, bool keep) {
     return v & mask;
 }
 
-template <int MT, int GM_RING>
+template <int MT, int GM_RING, int GM_WAVES>
 __global__ void __launch_bounds__(GM_WAVES* ZI_WAVE)
 gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __restrict__ x,
                 const zi_bf16* __restrict__ w, const zi_bf16* __restrict__ bias, int M, int N, int K, int64_t ldx,
@@ -55,7 +56,7 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     const int kb_total = (K + GM_KB - 1) / GM_KB;
     const int kb_lo = split * kb_per_split;
     const int kb_hi = (kb_lo + kb_per_split < kb_total) ? kb_lo + kb_per_split : kb_total;
-    const int n0 = blockIdx.x * GM_ROWS + wave * 16;
+    const int n0 = (blockIdx.x * GM_WAVES + wave) * 16;
     // Weights are read as whole cache lines: a load instruction takes 4 rows x 256 bytes (lane l: row
     // l / 16 of the four, 16-byte piece l % 16), four instructions a tile of 16 rows x 128 values.
     // Loads in the matrix-core operand layout (16 rows x 64 bytes an instruction) were measured a fifth
@@ -70,8 +71,10 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     // LDS rows are not padded but swizzled (16-byte reads in operand order then run at the full LDS rate)
     uint16_t* const wt_w = &wt[wave][0];
 
-    // what this thread stages of a block's x slice: MT pieces of 16 bytes (row srow + 16 * t, piece spc)
-    const int srow = tid / 16, spc = tid % 16;
+    // what this thread stages of a block's x slice: MT pieces of 16 bytes (row srow + 16 * t, piece spc);
+    // the first GM_STAGERS threads stage, the others' loads go to the same places and are dropped
+    const int srow = (tid % GM_STAGERS) / 16, spc = tid % 16;
+    const bool stager = tid < GM_STAGERS;
     // the weights of GM_RING k-blocks are in flight at once (a ring of register buffers); the x slice of
     // the next block is fetched while this one is worked on
     gm_u32x4_t ring[GM_RING][4], xring[GM_RING][MT];
@@ -97,6 +100,7 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
         for (int c = 0; c < 4; ++c) ring[slot][c] = *reinterpret_cast<const gm_u32x4_t*>(wrow[c] + (k < K ? k : K - 8));
     };
     auto stash = [&](const int slot, int b) __attribute__((always_inline)) {
+        if (GM_WAVES * ZI_WAVE > GM_STAGERS && !stager) return;
 #pragma unroll
         for (int t = 0; t < MT; ++t)
             *reinterpret_cast<gm_u32x4_t*>(&xs[b][(t * 16 + srow) * GM_XS + (spc ^ srow) * 8]) = xring[slot][t];
@@ -232,30 +236,62 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     }
 }
 
-// Splits of k and k-blocks per split for a weight matrix [N, K]: enough workgroups to fill the chip,
-// at least two k-blocks a workgroup where K allows, at most 16 splits (what the consumers add at once).
-void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split) {
-    const int groups = (N + GM_ROWS - 1) / GM_ROWS;
+// How the product with a weight matrix [N, K] is cut: wavefronts a workgroup (16 weight rows each), splits
+// of k over workgroups (at most 16: what the consumers add at once) and k-blocks per split.  A function of
+// N and K alone.
+//
+// A compute unit works through the wavefronts it is given at a fixed rate (measured: 280 workgroups of
+// four wavefronts on 256 compute units take almost twice as long as 140, because 24 units hold two), so
+// what counts is the most work any unit gets when workgroups are dealt out in turn: rounds = ceil(workgroups
+// / units), each of `waves * k-blocks` wavefront-blocks plus a start-up worth about ten of them.  Among
+// the cuts the cheapest by that measure is taken, then the one with the fewest splits, then the fewest
+// wavefronts.  A matrix with many times more rows than that keeps the units busy whatever the cut (its
+// workgroups follow each other, two to a unit): four wavefronts, no split (measured on the 151,936 rows of
+// the output head: 108 against 119 us with eight).
+void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split, int* waves) {
+    const int tiles = (N + 15) / 16;
     const int kb_total = (K + GM_KB - 1) / GM_KB;
-    int s = (GM_TARGET_WGS + groups / 2) / groups;    // to the nearest: 280 groups are enough by themselves
-    if (s > 16) s = 16;
-    if (s > kb_total / 2) s = kb_total / 2;
-    if (s < 1) s = 1;
-    const int per = (kb_total + s - 1) / s;
-    *kb_per_split = per;
-    *splits = (kb_total + per - 1) / per;
+    int64_t best_cost = -1;
+    int best_s = 1, best_w = GM_MIN_WAVES, best_per = kb_total;
+    const bool many = (tiles + GM_MIN_WAVES - 1) / GM_MIN_WAVES > 4 * GM_CUS;
+    for (int w = GM_MIN_WAVES; w <= (many ? GM_MIN_WAVES : GM_MAX_WAVES); ++w) {
+        const int groups = (tiles + w - 1) / w;
+        for (int s0 = 1; s0 <= (many ? 1 : 16) && s0 <= (kb_total > 1 ? kb_total / 2 : 1); ++s0) {
+            const int per = (kb_total + s0 - 1) / s0;
+            const int s = (kb_total + per - 1) / per;
+            if (s != s0) continue;      // the same cut under another name
+            const int64_t wgs = (int64_t)groups * s;
+            const int64_t rounds = (wgs + GM_CUS - 1) / GM_CUS;
+            const int64_t cost = rounds * ((int64_t)w * per + 10);
+            if (best_cost < 0 || cost < best_cost || (cost == best_cost && s < best_s)) {
+                best_cost = cost; best_s = s; best_w = w; best_per = per;
+            }
+        }
+    }
+    *splits = best_s;
+    *kb_per_split = best_per;
+    *waves = best_w;
 }
 
 // The launch; the checks are the caller's (zi_gemm_skinny).
 int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const zi_bf16* w, const zi_bf16* bias, int M,
                        int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int vec_out, hipStream_t stream) {
-    int splits, per;
-    zi_gemm_mid_plan(N, K, &splits, &per);
-    const dim3 grid((N + GM_ROWS - 1) / GM_ROWS, splits);
+    int splits, per, waves;
+    zi_gemm_mid_plan(N, K, &splits, &per, &waves);
+    const int tiles = (N + 15) / 16;
+    const dim3 grid((tiles + waves - 1) / waves, splits);
     const int mt = (M + 15) / 16;
-#define ZI_GM(MT)                                                                                            \
-    gemm_mid_kernel<MT, 3><<<grid, GM_WAVES * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, \
-                                                                    ldw, ldo, per, vec_out)
+#define ZI_GM2(MT, WV)                                                                                            \
+    gemm_mid_kernel<MT, 3, WV><<<grid, WV * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, ldw, \
+                                                                  ldo, per, vec_out)
+#define ZI_GM(MT)                               \
+    switch (waves) {                            \
+        case 4: ZI_GM2(MT, 4); break;           \
+        case 5: ZI_GM2(MT, 5); break;           \
+        case 6: ZI_GM2(MT, 6); break;           \
+        case 7: ZI_GM2(MT, 7); break;           \
+        default: ZI_GM2(MT, 8); break;          \
+    }
     switch (mt) {
         case 1: ZI_GM(1); break;
         case 2: ZI_GM(2); break;
@@ -263,5 +299,6 @@ int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const
         default: ZI_GM(4); break;
     }
 #undef ZI_GM
+#undef ZI_GM2
     return zi_check_launch("gemm_mid");
 }

@@ -284,15 +284,15 @@ extern "C" int zi_gemm_skinny_supported(int M, int N, int K, int64_t ldx, int64_
 }
 
 // The kernel for 17..64 rows (gemm_mid.hip): its cut and its launch.
-void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split);
+void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split, int* waves);
 int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const zi_bf16* w, const zi_bf16* bias, int M,
                        int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int vec_out, hipStream_t stream);
 
 // Splits of k for M rows against a weight matrix [N, K]: the leading dimension of the partial sums.  A
 // function of N, K and of whether M is at most 16 (the two kernels cut differently).
 extern "C" int zi_gemm_skinny_splits(int M, int N, int K) {
-    int kpw, s, tpw;
-    if (M > 16) zi_gemm_mid_plan(N, K, &s, &tpw);
+    int kpw, s, tpw, waves;
+    if (M > 16) zi_gemm_mid_plan(N, K, &s, &tpw, &waves);
     else skinny_plan(N, K, &kpw, &s, &tpw);
     return s;
 }
@@ -331,9 +331,9 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
     ZI_REQUIRE(mode >= 0 && mode <= 2, "gemm_skinny: unknown mode %d", mode);
     ZI_REQUIRE(ldx >= K && ldw >= K, "gemm_skinny: leading dimension too small");
     ZI_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny: x and w must be 16-byte aligned");
-    int kpw = 1, splits, tpw;
+    int kpw = 1, splits, tpw, mid_waves;
     const int mt = (M + 15) / 16;
-    if (mt > 1) zi_gemm_mid_plan(N, K, &splits, &tpw);    // more than 16 rows: the kernel that stages x in LDS
+    if (mt > 1) zi_gemm_mid_plan(N, K, &splits, &tpw, &mid_waves);    // more than 16 rows: the kernel that stages x in LDS
     else skinny_plan(N, K, &kpw, &splits, &tpw);
     const int tiles = (N + SK_ROWS - 1) / SK_ROWS;
     const dim3 grid((tiles + tpw - 1) / tpw, splits);

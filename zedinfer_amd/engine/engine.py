@@ -15,7 +15,7 @@ from typing import Dict, Optional, Sequence
 import torch
 
 from .. import ops
-from ..cache.manager import CacheManager, SequenceCache
+from ..cache.manager import NO_GROWTH, CacheManager, SequenceCache
 from ..config import ModelConfig, ModelForwardConfig, SchedulerConfig, load_config
 from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
@@ -189,7 +189,9 @@ class Engine:
         grown = []
         try:
             for e in entries:
-                grown.append((e.seq, self.cache.ensure(e.seq, e.seq.length + len(e.tokens))))
+                growth = self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
+                if growth is not NO_GROWTH:
+                    grown.append((e.seq, growth))
         except Exception:
             for seq, growth in reversed(grown):      # nothing of a step that cannot run stays
                 self.cache.undo(seq, growth)

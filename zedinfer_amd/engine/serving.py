@@ -156,6 +156,13 @@ class InferenceEngine:
     def __init__(self, engine: Engine):
         self.engine = engine
         self._loop = ServingLoop(engine, engine.fc.eos_token_ids)
+        # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
+        # taken out of the garbage collector's passes, a full collection in the middle of serving costs
+        # little (measured: one of 50 ms among decode steps of 6.5 ms without this).
+        if os.environ.get("ZEDINFER_GC_FREEZE", "1") not in ("", "0"):
+            import gc
+            gc.collect()
+            gc.freeze()
 
     @classmethod
     def create(cls, model_path: str, dtype="bfloat16", scheduler_config: Optional[SchedulerConfig] = None
