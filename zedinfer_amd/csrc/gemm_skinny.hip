@@ -288,11 +288,20 @@ void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split, int* waves);
 int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const zi_bf16* w, const zi_bf16* bias, int M,
                        int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int vec_out, hipStream_t stream);
 
+// From how many rows of x on the kernel that stages x in LDS (gemm_mid.hip) is taken.  It must be taken
+// beyond 16 rows (the kernel in this file holds one matrix-core tile of x); below, the choice is by speed.
+static int g_mid_min_rows = 1;
+extern "C" int zi_gemm_skinny_mid_min_rows(int rows) {
+    const int before = g_mid_min_rows;
+    if (rows >= 1 && rows <= 17) g_mid_min_rows = rows;
+    return before;
+}
+
 // Splits of k for M rows against a weight matrix [N, K]: the leading dimension of the partial sums.  A
-// function of N, K and of whether M is at most 16 (the two kernels cut differently).
+// function of N, K and of which of the two kernels takes M rows (they cut differently).
 extern "C" int zi_gemm_skinny_splits(int M, int N, int K) {
     int kpw, s, tpw, waves;
-    if (M > 16) zi_gemm_mid_plan(N, K, &s, &tpw, &waves);
+    if (M >= g_mid_min_rows) zi_gemm_mid_plan(N, K, &s, &tpw, &waves);
     else skinny_plan(N, K, &kpw, &s, &tpw);
     return s;
 }
@@ -333,7 +342,8 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
     ZI_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny: x and w must be 16-byte aligned");
     int kpw = 1, splits, tpw, mid_waves;
     const int mt = (M + 15) / 16;
-    if (mt > 1) zi_gemm_mid_plan(N, K, &splits, &tpw, &mid_waves);    // more than 16 rows: the kernel that stages x in LDS
+    const bool mid = M >= g_mid_min_rows;
+    if (mid) zi_gemm_mid_plan(N, K, &splits, &tpw, &mid_waves);    // more than 16 rows: the kernel that stages x in LDS
     else skinny_plan(N, K, &kpw, &splits, &tpw);
     const int tiles = (N + SK_ROWS - 1) / SK_ROWS;
     const dim3 grid((tiles + tpw - 1) / tpw, splits);
@@ -363,7 +373,7 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
     else if (kmode == SK_MODE_SWIGLU) vec_out = ldo % 4 == 0 && ((uintptr_t)dst % 8) == 0;
     else vec_out = ldo % 4 == 0 && ((uintptr_t)dst % (out_dt == ZI_F32 ? 16 : 8)) == 0;
     const int of32 = out_dt == ZI_F32;
-    if (mt > 1) {
+    if (mid) {
         const int rc = zi_gemm_mid_launch(dst, of32, kmode, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo,
                                           vec_out, stream);
         if (rc) return rc;
