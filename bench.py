@@ -9,7 +9,8 @@ A step is one decode step of the serving loop (schedule, model, sampling) with `
 requests that each hold a 2,048-token prompt.  Prints ONE JSON line.  Besides the decode speed it
 reports a 2,048-token prefill (tokens a second and the fraction of the bf16 matrix peak), the
 decode step against the HBM roofline (bytes that must be read: every weight once and the cache of
-the live requests), and decode at batch 1 and 64.  Weights are seeded random, token ids seeded
+the live requests), decode at batch 1 and 64, and (under "further") the same architecture at the
+Qwen2.5-7B sizes: decode at batch 8 and 64 requests batched continuously.  Weights are seeded random, token ids seeded
 uniform random in [100, vocab-100] as in the reference's own benchmark
 (reference: src/zedinfer/profiler.cpp:79-84, docs/perf/benchmark_v0.1.0.md:3-11).
 """
@@ -152,6 +153,45 @@ def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT, warm=1):
     return sum(times[warm:]) / rounds * 1000.0
 
 
+def further_7b(args):
+    """Decode at batch 8 (2,048-token prompts) and 64 requests batched continuously, at the Qwen2.5-7B sizes:
+    each figure with its sizes and, for the decode step, its fraction of the HBM roofline."""
+    import torch
+    from zedinfer_amd.config import Qwen2Config, SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    shape = dict(SHAPE, **SHAPES["7B"])
+    cfg = Qwen2Config.from_dict(shape)
+    L, el, batch, steps, warm = shape["num_hidden_layers"], 2, 8, min(args.steps, 48), min(args.warmup, 8)
+    holder = {}
+
+    def decode_engine():
+        tokens = PROMPT + warm + steps + 2 * batch + 64
+        sched = SchedulerConfig(num_kv_blocks=batch * (-(-tokens // 16)) + 16, kv_block_size=16, max_batch_requests=batch,
+                                max_batch_tokens=PROMPT + batch, max_prefill_tokens=PROMPT, max_seq_len=8192)
+        holder["e"] = Engine.from_config(cfg, "Qwen2ForCausalLM", args.dtype, seed=0, sched=sched)
+        return holder["e"]
+    tps, ms_step, ctx_mid = measure_decode(decode_engine, batch, steps, warm, cfg.vocab_size, PROMPT)
+    need = decode_bytes(shape, L, batch, ctx_mid, el)
+    achieved = need / (ms_step / 1000.0) / 1e9
+    res = {"config": {"model": "Qwen2.5-7B shape", "num_layers": L, "layers_run": L, "hidden": cfg.hidden_size,
+                      "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                      "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": False,
+                      "kv_page_tokens": 16, "context_len": 8192, "dtype": args.dtype},
+           "decode_b8": {"value": round(tps, 2), "unit": "tok/s", "ms_per_step": round(ms_step, 4), "seq_len": PROMPT,
+                         "steps": steps, "roofline_achieved_gbs": round(achieved, 1),
+                         "roofline_frac": round(achieved / HBM_PEAK_GBS, 4)}}
+
+    def mix_engine():
+        sched = SchedulerConfig(num_kv_blocks=64 * (-(-(4096 + 256 + 64) // 16)) + 16, kv_block_size=16,
+                                max_batch_requests=64, max_batch_tokens=2048 + 64, max_prefill_tokens=2048, max_seq_len=8192)
+        return holder["e"].with_cache(sched)
+    gen, pre, secs, ptoks = measure_mix(mix_engine, 64, cfg.vocab_size)
+    res["mix64"] = {"value": round(gen, 1), "unit": "generated tok/s", "requests": 64, "prompt_tokens": ptoks,
+                    "prompt_lens": "uniform 128..4096", "new_tokens_each": 256, "prefill_chunk": 2048,
+                    "seconds": round(secs, 3), "prompt_tok_s": round(pre, 1)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -167,6 +207,7 @@ def main():
                     help="instead: continuous batching of R requests, prompts uniform in [128, 4096], 256 greedy "
                          "tokens each, prompts cut at 2,048 tokens a step")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--no-further", action="store_true", help="skip the figures at the 7B sizes")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
     args = ap.parse_args()
@@ -258,6 +299,11 @@ def main():
         short = measure_prefill(factory(1, 128), V, tokens=128, warm=2)
         points["prefill_128"] = round(128 / short * 1000.0, 1)
         out["points"] = points
+        if args.shape == "1.5B" and args.layers == FULL_LAYERS and not args.no_further:
+            # the same architecture at the Qwen2.5-7B sizes: decode at batch 8 and the continuous-batching mix
+            weights_cache.clear()
+            torch.cuda.empty_cache()
+            out["further"] = further_7b(args)
     out["choices"] = CHOICES
     print(json.dumps(out))
     return 0
