@@ -1,5 +1,5 @@
-// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for 17..64 rows of x: decoding at larger batches, still bound
-// by the one pass over the weights.
+// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for 1..64 rows of x: the decode-time products, bound by the one
+// pass over the weights (the entry points are in gemm_skinny.hip).
 //
 // A workgroup of four to eight wavefronts owns 16 weight rows a wavefront and a range of k.  It walks its
 // k-blocks of 128: the block's slice of x (up to 64 rows x 128 values) is staged in LDS once for the four

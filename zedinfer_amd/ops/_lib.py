@@ -45,7 +45,6 @@ _PROTOTYPES = {
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
     "zi_gemm_skinny": [P, I, I, P, P, P, I, I, I, L, L, L, P, L, P],
     "zi_gemm_skinny_splits": [I, I, I],
-    "zi_gemm_skinny_mid_min_rows": [I],
     "zi_reduce_splits": [P, I, P, P, I, I, L, I, P],
     "zi_rope_kv_store_split": [P, I, L, P, I, L, L, P, I, I, P, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_gemm_skinny_supported": [I, I, I, L, L],

@@ -722,8 +722,7 @@ def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
 
 
 def linear_splits(M: int, N: int, K: int) -> int:
-    """Partial sums the few-rows product of M rows with a weight matrix [N, K] leaves: a function of N, K
-    and of whether M is at most 16 (two kernels, two cuts)."""
+    """Partial sums the few-rows product with a weight matrix [N, K] leaves: a function of N and K alone."""
     return int(_lib.load().zi_gemm_skinny_splits(int(M), int(N), int(K)))
 
 
