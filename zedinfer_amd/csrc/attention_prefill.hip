@@ -756,6 +756,9 @@ extern "C" int zi_attention_prefill_supported(int dt, int nh, int nkv, int d, in
 
 extern "C" int zi_attention_prefill_tile() { return PF_BM; }
 
+// Keys one workgroup walks at most: tiles are cut at absolute multiples of this.
+extern "C" int zi_attention_prefill_chunk_keys() { return PF_CHUNK; }
+
 // Tile i covers the queries [tile_off[i], tile_off[i] + 64) of entry tile_entry[i] (fewer at the
 // entry's end); entry e brings entry_len[e] tokens that start at row entry_start[e] of q and at
 // position entry_past[e] of its sequence, whose block table is row e of block_tables.

@@ -42,6 +42,7 @@ _PROTOTYPES = {
     "zi_attention_prefill_variant": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],
     "zi_attention_prefill_tile": [],
+    "zi_attention_prefill_chunk_keys": [],
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
     "zi_gemm_skinny": [P, I, I, P, P, P, I, I, I, L, L, L, P, L, P],
     "zi_gemm_skinny_splits": [I, I, I],

@@ -578,8 +578,8 @@ def attention_prefill_workspace(rows: int, nh: int, d: int, max_keys: int, windo
 
 
 def _prefill_chunks(max_keys: int, window: int) -> int:
-    if window > 0:      # a windowed tile's keys span at most the window, a tile and a block
-        max_keys = min(max_keys, window + PREFILL_TILE + 128) + 2047
+    if window > 0:      # a windowed tile's keys span at most the window, a tile and a block, from anywhere in a cut
+        max_keys = min(max_keys, window + PREFILL_TILE + 128) + int(_lib.load().zi_attention_prefill_chunk_keys()) - 1
     return int(_lib.load().zi_attention_prefill_chunks(int(max_keys)))
 
 
