@@ -28,14 +28,15 @@
 // bfloat16 only; head_dim a multiple of 16 up to 128; group size up to 16; page size
 // a multiple of 8.  Other shapes are the plain kernel's.
 #include "zi_common.h"
+#include "zi_paging.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 dec_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float dec_f32x4_t;
 
-#define DEC_MAXC 64       // most chunks of one token
-#define DEC_CHUNK 256     // keys of the smallest chunk
-#define DEC_WAVES 4
-#define DEC_BLOCK 64      // keys a wavefront handles at a time
+#define DEC_MAXC ZI_DEC_MAXC       // most chunks of one token
+#define DEC_CHUNK ZI_DEC_CHUNK     // keys of the smallest chunk
+#define DEC_WAVES ZI_DEC_WAVES
+#define DEC_BLOCK ZI_DEC_BLOCK     // keys a wavefront handles at a time
 
 union dec_pack {
     uint4 u;
@@ -43,21 +44,7 @@ union dec_pack {
     uint16_t h[8];
 };
 
-// The cut of a token's keys: first key seen, first key of chunk 0 (a multiple of 8),
-// keys per chunk, number of chunks.
-struct DecSplit {
-    int lo, lo_al, len, count;
-};
-__host__ __device__ __forceinline__ DecSplit dec_split(int p, int window) {
-    DecSplit s;
-    s.lo = (window > 0 && p - window + 1 > 0) ? p - window + 1 : 0;
-    s.lo_al = s.lo & ~7;
-    const int nk = p - s.lo_al + 1;
-    s.len = DEC_CHUNK;
-    while (nk > s.len * DEC_MAXC) s.len *= 2;
-    s.count = (nk + s.len - 1) / s.len;
-    return s;
-}
+// The cut of a token's keys (DecSplit, dec_split) and every place in the cache come from zi_paging.h.
 
 // The projections of the step's tokens as they leave the matrix product, for the kernel variant that
 // rotates and stores them itself (FUSED): row t of `sums` holds the query heads, then the key heads, then
@@ -113,8 +100,8 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     const int32_t* bt = block_tables + (int64_t)(tok_seq ? tok_seq[t] : t) * max_pages;   // no list: token t is of sequence t
     const int ps_shift = (ps & (ps - 1)) == 0 ? __ffs(ps) - 1 : -1;   // no division for the usual page sizes
     const int quarter = sp.len / DEC_WAVES;
-    const int k_begin = sp.lo_al + chunk * sp.len + wave * quarter;
-    const int k_end = (k_begin + quarter < p + 1) ? k_begin + quarter : p + 1;   // one past the wavefront's last key
+    int k_begin, k_end;      // the wavefront's keys; k_end is one past the last
+    zi_dec_wave_keys(sp, chunk, wave, p, &k_begin, &k_end);
     const int p8 = p & ~7, pi_last = max_pages - 1;
 
     // FUSED: eight consecutive columns of the token's projection row (splits added in rising order, then
@@ -239,21 +226,21 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
             qop[dk] = w.b;
         }
         if (owner) {
-            const int slot = pj.slots[t];
-            const bool inside = slot >= 0 && slot < pj.cache_slots;   // the host checks the range; never write outside the pool
-            const int64_t page = inside ? slot / ps : 0, off = inside ? slot % ps : 0;
+            const ZiSlotPlace place = zi_slot_place(pj.slots[t], pj.cache_slots, ps);   // the host checks the range; never write outside the pool
+            const bool inside = place.ok;
+            const int64_t page = place.page, off = place.off;
 #pragma unroll
             for (int dk = 0; dk < DK; ++dk) {
                 knew[dk] = sk[dk][j];
                 if (inside && r == r_p && dk * 32 + j * 8 < D)
-                    *reinterpret_cast<uint4*>(const_cast<zi_bf16*>(kcache) + ((page * nkv + kvh) * ps + off) * D + dk * 32 + j * 8) = knew[dk];
+                    *reinterpret_cast<uint4*>(const_cast<zi_bf16*>(kcache) + zi_key_offset(page, kvh, (int)off, nkv, ps, D) + dk * 32 + j * 8) = knew[dk];
             }
 #pragma unroll
             for (int dd = 0; dd < DT; ++dd) {
                 const int dim = dd * 16 + r;
                 const uint32_t hv = sv[dim];
                 if (inside && j == j_p)
-                    const_cast<zi_bf16*>(vcache)[((page * nkv + kvh) * D + dim) * ps + off].bits = (uint16_t)hv;
+                    const_cast<zi_bf16*>(vcache)[zi_value_offset(page, kvh, dim, (int)off, nkv, ps, D)].bits = (uint16_t)hv;
                 vnew[dd / 2] = (dd & 1) ? (vnew[dd / 2] | (hv << 16)) : hv;
             }
         }
@@ -282,32 +269,28 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         int kpage[4], kslot[4], vpage[2], vslot[2];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-            const int key = base + (tt / 2) * 32 + (r / 4) * 8 + (tt % 2) * 4 + (r % 4);
-            const int kc = key < p ? key : p;
-            int pi = ps_shift >= 0 ? kc >> ps_shift : kc / ps;
-            kslot[tt] = kc - pi * ps;
-            kpage[tt] = bt[pi < pi_last ? pi : pi_last];
+            const ZiTablePlace at = zi_table_place(zi_dec_tile_key(base, tt, r), p, ps, ps_shift, pi_last);
+            kslot[tt] = at.slot;
+            kpage[tt] = bt[at.index];
         }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
-            const int key0 = base + b * 32 + j * 8;
-            const int kc = key0 < p8 ? key0 : p8;
-            int pi = ps_shift >= 0 ? kc >> ps_shift : kc / ps;
-            vslot[b] = kc - pi * ps;
-            vpage[b] = bt[pi < pi_last ? pi : pi_last];
+            const ZiTablePlace at = zi_table_place(zi_dec_value_key0(base, b, j), p8, ps, ps_shift, pi_last);
+            vslot[b] = at.slot;
+            vpage[b] = bt[at.index];
         }
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-            const int page = (unsigned)kpage[tt] < (unsigned)num_pages ? kpage[tt] : 0;   // a window may have freed it
-            const zi_bf16* kr = kcache + (((int64_t)page * nkv + kvh) * ps + kslot[tt]) * D;
+            const int page = zi_page_or_zero(kpage[tt], num_pages);   // a window may have freed it
+            const zi_bf16* kr = kcache + zi_key_offset(page, kvh, kslot[tt], nkv, ps, D);
 #pragma unroll
             for (int dk = 0; dk < DK; ++dk)
                 kop[tt][dk].u = *reinterpret_cast<const uint4*>(kr + ((D % 32 == 0 || dk * 32 + j * 8 < D) ? dk * 32 + j * 8 : 0));
         }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
-            const int page = (unsigned)vpage[b] < (unsigned)num_pages ? vpage[b] : 0;
-            const zi_bf16* vr = vcache + (((int64_t)page * nkv + kvh) * D + r) * ps + vslot[b];
+            const int page = zi_page_or_zero(vpage[b], num_pages);
+            const zi_bf16* vr = vcache + zi_value_offset(page, kvh, r, vslot[b], nkv, ps, D);
 #pragma unroll
             for (int dd = 0; dd < DT; ++dd) vop[dd][b].u = *reinterpret_cast<const uint4*>(vr + (int64_t)dd * 16 * ps);
         }
@@ -324,7 +307,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         if (base < sp.lo || base + DEC_BLOCK > k_end) {
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
-                const int key0 = base + b * 32 + j * 8;
+                const int key0 = zi_dec_value_key0(base, b, j);
                 unsigned keep[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -379,7 +362,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         for (int tt = 0; tt < 4; ++tt)
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const int key = base + (tt / 2) * 32 + j * 8 + (tt % 2) * 4 + e;
+                const int key = zi_dec_score_key(base, tt, j, e);
                 const float v = (whole || (key >= sp.lo && key < k_end)) ? s[tt][e] * scale_log2 : -INFINITY;
                 s[tt][e] = v;
                 mx = fmaxf(mx, v);
@@ -436,7 +419,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     }
     const bool final = sp.count == 1 && !leave_parts;
     const float inv = final ? 1.f / L : 1.f;
-    const int64_t slot = ((int64_t)x * nh + kvh * G + r) * DEC_MAXC + chunk;
+    const int64_t slot = zi_dec_part_slot(x, nh, kvh * G + r, chunk);
     for (int dd = wave; dd < DT; dd += DEC_WAVES) {
         dec_f32x4_t acc = dec_f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -469,7 +452,7 @@ attention_decode_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const floa
     const int t = tok_index ? tok_index[x] : x;
     const DecSplit sp = dec_split(tok_pos[t], window);
     if (sp.count == 1 || sp.count > max_chunks) return;
-    const int64_t slot0 = ((int64_t)x * nh + h) * DEC_MAXC;
+    const int64_t slot0 = zi_dec_part_slot(x, nh, h, 0);
     // chunk c's (m, l) sit in lane c
     const float mc = lane < sp.count ? part_ml[(slot0 + lane) * 2] : -INFINITY;
     const float lc = lane < sp.count ? part_ml[(slot0 + lane) * 2 + 1] : 0.f;
@@ -540,7 +523,7 @@ attention_decode_project_kernel(float* __restrict__ sums, const float* __restric
         for (int e = 0; e < 8; ++e) v[e] = 0.f;
         const int q = tid & 15, mtc = mt < n ? mt : n - 1;
         const int count = dec_split(tok_pos[mtc], window).count;
-        const int64_t slot0 = ((int64_t)mtc * nh + h) * DEC_MAXC;
+        const int64_t slot0 = zi_dec_part_slot(mtc, nh, h, 0);
         const float2* ml = reinterpret_cast<const float2*>(part_ml) + slot0;
         const float* po0 = part_o + slot0 * D + (d0 < D ? d0 : 0);
         float2 mlq[DEC_MAXC / 16];
@@ -631,9 +614,7 @@ attention_decode_project_kernel(float* __restrict__ sums, const float* __restric
 }
 
 // Floats of workspace the split kernel needs for n tokens.
-extern "C" int64_t zi_attention_decode_workspace(int n, int nh, int d) {
-    return (int64_t)n * nh * DEC_MAXC * (d + 2);
-}
+extern "C" int64_t zi_attention_decode_workspace(int n, int nh, int d) { return zi_dec_workspace_floats(n, nh, d); }
 
 // Chunks the launch must cover when no token sees more than `keys` keys (position + 1, or the window).
 extern "C" int zi_attention_decode_chunks(int keys) {

@@ -33,17 +33,19 @@
 // padded with zeros for the score product); page size a power of two from 8.
 // Other shapes are the plain kernel's.
 #include "zi_common.h"
+#include "zi_paging.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float pf_f32x4_t;
 
 #define PF_KH 2                  // wavefronts that share a query sub-tile, each with its own 64 keys of a block
 #define PF_WAVES (4 * PF_KH)
-#define PF_BM 64                 // queries per workgroup
+#define PF_BM ZI_PF_BM           // queries per workgroup
 #define PF_BN 64                 // keys per wavefront and block
 #define PF_BS (PF_BN * PF_KH)    // keys per block
-#define PF_CHUNK 2048            // keys one workgroup walks at most: a tile with more is cut over several
-#define PF_MAXC 64               // most such cuts of one tile
+#define PF_CHUNK ZI_PF_CHUNK     // keys one workgroup walks at most: a tile with more is cut over several
+#define PF_MAXC ZI_PF_MAXC       // most such cuts of one tile
+static_assert(PF_BS == ZI_PF_BS, "the block of keys is the one the shared cut is made for");
 
 union pf_pack {
     uint4 u;
@@ -87,14 +89,11 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
     const int r = lane & 15, j = lane >> 4;
     const int32_t* bt = block_tables + (int64_t)e * max_pages;
     const int pos0 = past + off;            // position of the tile's first query
-    const int kmax = pos0 + count - 1;      // last key any query of the tile sees
-    const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-    const int kb_first = (lo_tile / PF_BS) * PF_BS;
-    // this workgroup's cut of the tile's keys: [kb_begin, khi], inside chunk c of absolute multiples of PF_CHUNK
-    const int c0 = kb_first / PF_CHUNK, nc = kmax / PF_CHUNK - c0 + 1, c = c0 + blockIdx.y;
-    if (c * PF_CHUNK > kmax) return;
-    const int kb_begin = (c * PF_CHUNK > kb_first) ? c * PF_CHUNK : kb_first;
-    const int khi = ((c + 1) * PF_CHUNK - 1 < kmax) ? (c + 1) * PF_CHUNK - 1 : kmax;
+    // this workgroup's cut of the tile's keys: [kb_begin, khi], between absolute multiples of PF_CHUNK
+    const PfCut cut = zi_pf_cut(pos0, count, window, blockIdx.y);
+    if (!cut.live) return;
+    const int kmax = cut.kmax;              // last key any query of the tile sees
+    const int nc = cut.nc, kb_begin = cut.kb_begin, khi = cut.khi;
 
     // this wavefront's queries (sub-tile qs) and its share of every block's keys (kh)
     const int qs = wave % 4, kh = wave / 4;
@@ -370,7 +369,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                     for (int x = 0; x < 4; ++x) zi_store(out + (int64_t)(start + off + row) * ldo + (int64_t)h * D + dd * 16 + j * 4 + x, NAN);
             return;
         }
-        const int64_t slot = ((int64_t)(start + off + row) * nh + h) * max_chunks + blockIdx.y;
+        const int64_t slot = zi_pf_part_slot(start + off + row, nh, h, max_chunks, blockIdx.y);
 #pragma unroll
         for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = o[dd];
         if (j == 0) {
@@ -439,13 +438,9 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     const int r = lane & 15, j = lane >> 4;
     const int32_t* bt = block_tables + (int64_t)e * max_pages;
     const int pos0 = past + off;
-    const int kmax = pos0 + count - 1;
-    const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-    const int kb_first = (lo_tile / PF_BS) * PF_BS;
-    const int c0 = kb_first / PF_CHUNK, nc = kmax / PF_CHUNK - c0 + 1, c = c0 + blockIdx.y;
-    if (c * PF_CHUNK > kmax) return;
-    const int kb_begin = (c * PF_CHUNK > kb_first) ? c * PF_CHUNK : kb_first;
-    const int khi = ((c + 1) * PF_CHUNK - 1 < kmax) ? (c + 1) * PF_CHUNK - 1 : kmax;
+    const PfCut cut = zi_pf_cut(pos0, count, window, blockIdx.y);
+    if (!cut.live) return;
+    const int kmax = cut.kmax, nc = cut.nc, kb_begin = cut.kb_begin, khi = cut.khi;
 
     const int qs = wave % 4, kh = wave / 4;
     const int row = qs * 16 + r;
@@ -677,7 +672,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
                     for (int x = 0; x < 4; ++x) zi_store(out + (int64_t)(start + off + row) * ldo + (int64_t)h * D + dd * 16 + j * 4 + x, NAN);
             return;
         }
-        const int64_t slot = ((int64_t)(start + off + row) * nh + h) * max_chunks + blockIdx.y;
+        const int64_t slot = zi_pf_part_slot(start + off + row, nh, h, max_chunks, blockIdx.y);
 #pragma unroll
         for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = o[dd];
         if (j == 0) {
@@ -710,12 +705,10 @@ attention_prefill_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const flo
     const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
     const int count = (len - off < PF_BM) ? len - off : PF_BM;
     if (qi >= count) return;
-    const int pos0 = past + off, kmax = pos0 + count - 1;
-    const int lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
-    const int c0 = ((lo_tile / PF_BS) * PF_BS) / PF_CHUNK, nc = kmax / PF_CHUNK - c0 + 1;
+    const int nc = zi_pf_cut(past + off, count, window, 0).nc;
     if (nc == 1 || nc > max_chunks) return;
     const int64_t row = start + off + qi;
-    const int64_t slot0 = (row * nh + h) * max_chunks;
+    const int64_t slot0 = zi_pf_part_slot(row, nh, h, max_chunks, 0);
     // cut c's (m, l) sit in lane c; a cut none of whose keys this query sees left m = -inf, l = 0
     const float mc = lane < nc ? part_ml[(slot0 + lane) * 2] : -INFINITY;
     const float lc = lane < nc ? part_ml[(slot0 + lane) * 2 + 1] : 0.f;
@@ -737,7 +730,7 @@ attention_prefill_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const flo
 
 // Floats of workspace a launch over `rows` query rows needs when tiles are cut into up to `max_chunks`.
 extern "C" int64_t zi_attention_prefill_workspace(int rows, int nh, int d, int max_chunks) {
-    return max_chunks > 1 ? (int64_t)rows * nh * max_chunks * (d + 2) : 0;
+    return zi_pf_workspace_floats(rows, nh, d, max_chunks);
 }
 
 // Cuts the launch must cover when no query sees more than `keys` keys (position + 1; with a window: the

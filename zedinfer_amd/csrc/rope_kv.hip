@@ -15,6 +15,7 @@
 // the P.V product.  Token slot s lives in page s / page_size at offset s % page_size.
 // A negative slot skips the write.
 #include "zi_common.h"
+#include "zi_paging.h"
 
 template <typename T>
 __global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
@@ -44,14 +45,15 @@ __global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k,
         zi_store(base + j + half, b * c + a * s);
     }
     if (!write_kv) return;
-    const int slot = slots[t];
-    if (slot < 0 || slot >= cache_slots) return;  // the host checks the range; never write outside the pool
-    const int64_t page = slot / page_size, off = slot % page_size;
+    const ZiSlotPlace place = zi_slot_place(slots[t], cache_slots, page_size);
+    if (!place.ok) return;  // padding, or out of range (the host checks the range; never write outside the pool)
+    const int64_t page = place.page;
+    const int off = place.off;
     const T* kr = k + t * ldk;
     const T* vr = v + t * ldv;
     for (int i = threadIdx.x; i < nkv * d; i += blockDim.x) {
         const int h = i / d, j = i % d;
-        const int64_t dst = ((page * nkv + h) * page_size + off) * d + j;
+        const int64_t dst = zi_key_offset(page, h, off, nkv, page_size, d) + j;
         float kv;
         if (j < half) {
             kv = zi_load(kr + h * d + j) * cs[j] - zi_load(kr + h * d + j + half) * cs[half + j];
@@ -62,7 +64,7 @@ __global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k,
             kv = zi_load(kr + h * d + j);
         }
         zi_store(kcache + dst, kv);
-        vcache[((page * nkv + h) * d + j) * page_size + off] = vr[h * d + j];
+        vcache[zi_value_offset(page, h, j, off, nkv, page_size, d)] = vr[h * d + j];
     }
 }
 
@@ -132,9 +134,10 @@ rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k
     const int dp = d / 8;
     for (int i = tid; i < nt * nkv * dp; i += 256) {
         const int tt = i / (nkv * dp), rem = i % (nkv * dp), h = rem / dp, j0 = (rem % dp) * 8;
-        const int slot = slots[t0 + tt];
-        if (slot < 0 || slot >= cache_slots) continue;     // the host checks the range; never write outside the pool
-        const int64_t page = slot / page_size, off = slot % page_size;
+        const ZiSlotPlace place = zi_slot_place(slots[t0 + tt], cache_slots, page_size);
+        if (!place.ok) continue;     // the host checks the range; never write outside the pool
+        const int64_t page = place.page;
+        const int off = place.off;
         const zi_bf16* kr = k + (int64_t)(t0 + tt) * ldk + (int64_t)h * d;
         float a[8], o8[8];
         unpack(*reinterpret_cast<const uint4*>(kr + j0), a);
@@ -151,7 +154,7 @@ rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k
 #pragma unroll
             for (int x = 0; x < 8; ++x) o8[x] = a[x];
         }
-        *reinterpret_cast<uint4*>(kcache + ((page * nkv + h) * page_size + off) * d + j0) = pack(o8);
+        *reinterpret_cast<uint4*>(kcache + zi_key_offset(page, h, off, nkv, page_size, d) + j0) = pack(o8);
     }
     // values: transposed.  Eight tokens in eight consecutive slots from a multiple of eight: one run per dim.
     bool run = nt == RKT_TOKENS;
@@ -170,15 +173,14 @@ rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k
             u.y = (uint32_t)vt[2 * kvd + i] | ((uint32_t)vt[3 * kvd + i] << 16);
             u.z = (uint32_t)vt[4 * kvd + i] | ((uint32_t)vt[5 * kvd + i] << 16);
             u.w = (uint32_t)vt[6 * kvd + i] | ((uint32_t)vt[7 * kvd + i] << 16);
-            *reinterpret_cast<uint4*>(vcache + ((page * nkv + h) * d + dim) * page_size + off) = u;
+            *reinterpret_cast<uint4*>(vcache + zi_value_offset(page, h, dim, (int)off, nkv, page_size, d)) = u;
         }
     } else {
         for (int i = tid; i < nt * kvd; i += 256) {
             const int tt = i / kvd, col = i % kvd, h = col / d, dim = col % d;
-            const int slot = slots[t0 + tt];
-            if (slot < 0 || slot >= cache_slots) continue;
-            const int64_t page = slot / page_size, off = slot % page_size;
-            vcache[((page * nkv + h) * d + dim) * page_size + off].bits = vt[i];
+            const ZiSlotPlace place = zi_slot_place(slots[t0 + tt], cache_slots, page_size);
+            if (!place.ok) continue;
+            vcache[zi_value_offset(place.page, h, dim, place.off, nkv, page_size, d)].bits = vt[i];
         }
     }
 }
@@ -264,11 +266,10 @@ rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __re
     if (is_q) {
         dst = q_out + t * ldq + (int64_t)hs * d;
     } else {
-        const int slot = slots[t];
-        if (slot < 0 || slot >= cache_slots) return;  // the host checks the range; never write outside the pool
-        const int64_t page = slot / page_size, off = slot % page_size;
-        dst = kcache + ((page * nkv + g) * page_size + off) * d;
-        vbase = (page * nkv + g) * d * page_size + off;
+        const ZiSlotPlace place = zi_slot_place(slots[t], cache_slots, page_size);
+        if (!place.ok) return;  // the host checks the range; never write outside the pool
+        dst = kcache + zi_key_offset(place.page, g, place.off, nkv, page_size, d);
+        vbase = zi_value_offset(place.page, g, 0, place.off, nkv, page_size, d);
         store_v = true;
     }
     for (int j = lane; j < half; j += ZI_WAVE) {
