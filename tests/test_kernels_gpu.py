@@ -658,6 +658,22 @@ def test_attention_prefill(ops, nh, nkv, d, ps, window, portions):
                               dev([e[2] for e in entries]), bt, nh, nkv, d, scale, window, out=out2)
         n0 = entries[0][1]
         assert bool((out2[:n0] == 7.0).all()) and torch.equal(out2[n0:], out[n0:])
+    # head sizes 64 and 128 take tiles of 128 queries too (a staged block of keys serves twice the queries): the
+    # same bits, a query's walk over its keys does not depend on the tile it rides in
+    wide = ops.attention_prefill_tile(dtype, d)
+    assert wide == (128 if d in (64, 128) else 64)
+    if wide == 128:
+        te2, to2 = prefill_tiles(entries, tile=128)
+        out4 = torch.full((n_tok, nh * d), 7.0, dtype=dtype, device="cuda")
+        ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, te2, to2, dev([e[0] for e in entries]),
+                              dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale,
+                              window, out=out4, tile=128)
+        assert torch.equal(out4, out)
+    else:
+        with pytest.raises(ValueError, match="tiles of 128"):
+            ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, te, to, dev([e[0] for e in entries]),
+                                  dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale,
+                                  window, out=out, tile=128)
     # head sizes 64 and 128 have a second kernel (keys and values straight into LDS): the same bits
     if d in (64, 128):
         before = ops.attention_prefill_variant(0)

@@ -182,20 +182,21 @@ def test_decode_walk_reports_what_is_broken(model):
     assert model.pm_check_store(1, ptr(out), ctypes.c_int64(m.num_pages * ps), m.num_pages, 2, 32, ps, st) != 0
 
 
-def prefill(pm, plan, hb, real, tables, num_pages, nh, nkv, d, ps, window, max_chunks, workspace=None):
+def prefill(pm, plan, hb, real, tables, num_pages, nh, nkv, d, ps, window, max_chunks, workspace=None, tile=64):
     rows = hb.num_tokens
     ws = pm.pm_prefill_workspace(rows, nh, d, max_chunks) if workspace is None else workspace
     stats = (ctypes.c_int64 * 3)()
     rc = pm.pm_check_prefill(plan.sizes["num_tiles"], ptr(plan.arrays["tile_entry"]), ptr(plan.arrays["tile_off"]),
                              ptr(hb.entry_start), ptr(hb.entry_len), ptr(hb.entry_past), ptr(real), hb.num_entries,
                              ptr(tables), tables.shape[1], num_pages, nh, nkv, d, ps, window, rows, max_chunks,
-                             ctypes.c_int64(ws), stats)
+                             ctypes.c_int64(ws), tile, stats)
     return rc, pm.pm_last_error().decode(), list(stats)
 
 
+@pytest.mark.parametrize("tile", [64, 128])
 @pytest.mark.parametrize("window", [0, 24, 100])
 @pytest.mark.parametrize("seed", range(5))
-def test_prefill_walk_under_random_traffic(model, seed, window):
+def test_prefill_walk_under_random_traffic(model, seed, window, tile):
     """Portions of prompts after whatever the sequences hold, cut into tiles by the attention's own planner;
     once as they are, once padded to multiples of 64 tokens as recorded steps run them."""
     m, live, rng = traffic(seed + 20, window, pages=400, ps=8)
@@ -218,21 +219,24 @@ def test_prefill_walk_under_random_traffic(model, seed, window):
         starts[1:] = np.cumsum(lens)[:-1]
         past = np.array([s.length for s, _ in portions], dtype=np.int32)
         hb = HostBatch(int(lens.sum()), len(portions), starts, lens, past, False)
-        plan = AttentionPlanner().plan(hb)
-        assert plan.sizes["num_long"] == int(lens.sum())
+        planner = AttentionPlanner(tile, heads=6)
+        planner.FILL = 1 if tile == 128 else planner.FILL        # take the wide tiles however small the step
+        plan = planner.plan(hb)
+        assert plan.sizes["num_long"] == int(lens.sum()) and plan.sizes["tile"] == tile
         for g, group in enumerate(m.groups):
             tables = padded_tables([s for s, _ in portions], g, pow2(max(len(s.pages[g]) for s, _ in portions), 8))
             keys = plan.sizes["max_long_keys"]
             if group.window:
-                keys = min(keys, group.window + 64 + 128) + 2047
+                keys = min(keys, group.window + 128 + 128) + 2047
             chunks = model.pm_prefill_chunks(keys)
             rc, err, stats = prefill(model, plan, hb, real, tables, m.num_pages, 6, 2, 32, group.page_size, group.window,
-                                     chunks)
+                                     chunks, tile=tile)
             assert rc == 0, err
             assert stats[0] > 0 and stats[2] == 0
 
 
-def test_prefill_walk_of_a_long_prompt_and_what_is_broken(model):
+@pytest.mark.parametrize("tile", [64, 128])
+def test_prefill_walk_of_a_long_prompt_and_what_is_broken(model, tile):
     """One portion that continues a long sequence: its tiles are cut along the keys every 2,048, and the cuts'
     partial results have places of their own in the workspace."""
     m = CacheManager({0: KVCacheRequest("full", 2, 32)}, {}, 700, 8, 2, torch.bfloat16, None, max_step_tokens=2048)
@@ -242,18 +246,21 @@ def test_prefill_walk_of_a_long_prompt_and_what_is_broken(model):
     m.ensure(s, 4100 + 300)
     hb = HostBatch(300, 1, np.array([0], dtype=np.int32), np.array([300], dtype=np.int32),
                    np.array([4100], dtype=np.int32), False)
-    plan = AttentionPlanner().plan(hb)
+    planner = AttentionPlanner(tile, heads=4)
+    planner.FILL = 1
+    plan = planner.plan(hb)
+    assert plan.sizes["tile"] == tile
     tables = padded_tables([s], 0, pow2(len(s.pages[0]), 8))
     chunks = model.pm_prefill_chunks(plan.sizes["max_long_keys"])
     assert chunks == 3
-    rc, err, stats = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, chunks)
+    rc, err, stats = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, chunks, tile=tile)
     assert rc == 0, err
     assert stats[0] == sum(4100 + i + 1 for i in range(300)) and stats[1] == 300 * 4 * 3
-    rc, err, _ = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, chunks, workspace=1000)
+    rc, err, _ = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, chunks, workspace=1000, tile=tile)
     assert rc != 0 and "workspace" in err
     broken = tables.copy()
     broken[0, 300] = -1
-    rc, err, _ = prefill(model, plan, hb, None, broken, m.num_pages, 4, 2, 32, 8, 0, chunks)
+    rc, err, _ = prefill(model, plan, hb, None, broken, m.num_pages, 4, 2, 32, 8, 0, chunks, tile=tile)
     assert rc != 0 and "page entry" in err
-    rc, err, stats = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, 2)    # sized for fewer cuts
+    rc, err, stats = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, 2, tile=tile)    # sized for fewer cuts
     assert rc == 0 and stats[2] == plan.sizes["num_tiles"]

@@ -88,3 +88,42 @@ def test_real_layer_shapes_match_plain(model, dtype):
     else:
         assert engine.graph_replays > 10
         assert worst <= BF16_REL_WORST * scale and mean <= BF16_REL_MEAN * scale, where
+
+
+def test_wide_prompt_tiles_give_the_same_logits(model, monkeypatch):
+    """The prompt kernel's tiles of 128 queries (taken by the planner for steps that fill the chip) against its
+    tiles of 64, through the engine: a query's walk over its keys does not depend on the tile it rides in, so the
+    logits agree bit for bit, portions beside each other and at a page's edge included."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    from zedinfer_amd.parts.mixers import AttentionPlanner
+    reqs = model["requests"]
+    p, q = reqs["p"], reqs["q"]
+    want = lambda n: list(range(n))   # noqa: E731
+    steps = [
+        {"step": 0, "entries": [{"id": "p", "tokens": p[:200], "want": want(200)}], "end": []},
+        {"step": 1, "entries": [{"id": "p", "tokens": p[200:329], "want": want(129)},
+                                {"id": "q", "tokens": q[:65], "want": want(65)}], "end": ["p", "q"]},
+    ]
+    seen, outs = [], []
+    plan = AttentionPlanner.plan
+
+    def recording(self, hb):
+        made = plan(self, hb)
+        seen.append(made.sizes["tile"])
+        return made
+
+    monkeypatch.setattr(AttentionPlanner, "plan", recording)
+    for fill in (AttentionPlanner.FILL, 1):
+        monkeypatch.setattr(AttentionPlanner, "FILL", fill)
+        engine = Engine.from_folder(model["folder16"], "bfloat16",
+                                    SchedulerConfig(num_kv_blocks=40, kv_block_size=16, max_batch_requests=4))
+        assert engine.planners[0].wide_tile == 128
+        seen.clear()
+        outs.append(traces.run_in_process(engine, steps))
+        assert set(seen) == ({64} if fill > 1 else {128}), seen
+    for s in (0, 1):
+        assert torch.equal(torch.as_tensor(outs[0][s]), torch.as_tensor(outs[1][s])), s
+    worst, mean, scale, rows, where = traces.compare(steps, outs[1], model["reference16"], reqs)
+    assert rows == 329 + 65
+    assert worst <= BF16_REL_WORST * scale and mean <= BF16_REL_MEAN * scale, where

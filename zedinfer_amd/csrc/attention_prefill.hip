@@ -406,7 +406,9 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 // cleaned in LDS.  Keys need no such care: their scores are masked.
 __device__ __attribute__((aligned(16))) const unsigned pf_zero16[4] = {0u, 0u, 0u, 0u};
 
-template <int D>
+// QW: sub-tiles of 16 queries a wavefront owns: 1 (tiles of 64 queries) or 2 (tiles of 128: every block of keys and
+// values that is brought into LDS, and every operand read from there, serves twice the queries).
+template <int D, int QW>
 __global__ void __launch_bounds__(PF_WAVES* ZI_WAVE)
 attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* __restrict__ q, int64_t ldq,
                              const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,
@@ -416,6 +418,9 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
                              int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale,
                              float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks) {
     static_assert(D == 64 || D == 128, "this variant takes head sizes 64 and 128");
+    static_assert(QW == 1 || QW == 2, "16 or 32 queries a wavefront");
+    constexpr int BM = PF_BM * QW;                   // queries of a tile
+    constexpr int QR = 16 * QW;                      // queries of a wavefront
     constexpr int DK = D / 32, DT = D / 16;
     constexpr int KC = D / 8;                        // 16-byte pieces of a key row
     constexpr int VC = PF_BS / 8;                    // and of a row of the transposed value tile: 16
@@ -423,17 +428,19 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     constexpr int THREADS = PF_WAVES * ZI_WAVE;
     constexpr int KI = KCH / THREADS, VI = VCH / THREADS;   // load instructions a wavefront issues per tile
     constexpr int KSW = 16 / KC;                     // key rows that share 256 bytes of LDS (and one swizzle)
-    __shared__ __attribute__((aligned(16))) uint4 k_a[KCH];
-    __shared__ __attribute__((aligned(16))) uint4 k_b[KCH];
-    __shared__ __attribute__((aligned(16))) uint4 v_a[VCH];
-    __shared__ __attribute__((aligned(16))) uint4 v_b[VCH];
+    __shared__ __attribute__((aligned(16))) uint4 k_ab[2 * KCH];
+    __shared__ __attribute__((aligned(16))) uint4 v_ab[2 * VCH];
+    uint4* const k_a = k_ab;
+    uint4* const k_b = k_ab + KCH;
+    uint4* const v_a = v_ab;
+    uint4* const v_b = v_ab + VCH;
     __shared__ int32_t bt_lds[PF_CHUNK / 8 + 8];     // the pages of this workgroup's keys (page size >= 8)
 
     const int tile = blockIdx.x / nh, h = blockIdx.x % nh;
     const int g = h / (nh / nkv);
     const int e = tile_entry[tile], off = tile_off[tile];
     const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
-    const int count = (len - off < PF_BM) ? len - off : PF_BM;
+    const int count = (len - off < BM) ? len - off : BM;
     const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
     const int r = lane & 15, j = lane >> 4;
     const int32_t* bt = block_tables + (int64_t)e * max_pages;
@@ -442,30 +449,41 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     if (!cut.live) return;
     const int kmax = cut.kmax, nc = cut.nc, kb_begin = cut.kb_begin, khi = cut.khi;
 
+    // wavefront (qs, kh): queries qs * QR .. + QR - 1 of the tile (sub-tile u: 16 of them), half kh of every block
     const int qs = wave % 4, kh = wave / 4;
-    const int row = qs * 16 + r;
-    const bool wave_active = qs * 16 < count;
-    const bool qvalid = row < count;
-    const int qrow = qvalid ? row : count - 1;
-    const int qpos = pos0 + qrow;
-    const int wave_first = pos0 + ((qs * 16 < count) ? qs * 16 : count - 1);
-    const int wave_last = pos0 + ((qs * 16 + 15 < count) ? qs * 16 + 15 : count - 1);
+    int row[QW], qpos[QW];
+    bool qvalid[QW];
+#pragma unroll
+    for (int u = 0; u < QW; ++u) {
+        row[u] = qs * QR + u * 16 + r;
+        qvalid[u] = row[u] < count;
+        qpos[u] = pos0 + (qvalid[u] ? row[u] : count - 1);
+    }
+    const bool wave_active = qs * QR < count;
+    const int wave_first = pos0 + ((qs * QR < count) ? qs * QR : count - 1);
+    const int wave_last = pos0 + ((qs * QR + QR - 1 < count) ? qs * QR + QR - 1 : count - 1);
     const float scale_log2 = scale * 1.4426950408889634f;
-    const int wave_lo = (window > 0 && pos0 + qs * 16 - window + 1 > 0) ? pos0 + qs * 16 - window + 1 : 0;
-    pf_bf16x8_t qop[DK];
-    {
-        const zi_bf16* qr = q + (int64_t)(start + off + qrow) * ldq + (int64_t)h * D + j * 8;
+    const int wave_lo = (window > 0 && pos0 + qs * QR - window + 1 > 0) ? pos0 + qs * QR - window + 1 : 0;
+    pf_bf16x8_t qop[QW][DK];
+#pragma unroll
+    for (int u = 0; u < QW; ++u) {
+        const zi_bf16* qr = q + (int64_t)(start + off + (qvalid[u] ? row[u] : count - 1)) * ldq + (int64_t)h * D + j * 8;
 #pragma unroll
         for (int dk = 0; dk < DK; ++dk) {
             pf_pack p;
             p.u = *reinterpret_cast<const uint4*>(qr + dk * 32);
-            qop[dk] = p.b;
+            qop[u][dk] = p.b;
         }
     }
-    pf_f32x4_t o[DT];
+    pf_f32x4_t o[QW][DT];
+    float m[QW], lsum[QW];
 #pragma unroll
-    for (int dd = 0; dd < DT; ++dd) o[dd] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
-    float m = -INFINITY, lsum = 0.f;
+    for (int u = 0; u < QW; ++u) {
+#pragma unroll
+        for (int dd = 0; dd < DT; ++dd) o[u][dd] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
+        m[u] = -INFINITY;
+        lsum[u] = 0.f;
+    }
 
     // the block table's entries for keys [kb_begin, khi], once
     const int ps = 1 << ps_shift, ps_mask = ps - 1;
@@ -536,67 +554,73 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     auto work = [&](int kb0, const uint4* kl, const uint4* vl) {
         const int kb = kb0 + kh * PF_BN;      // this wavefront's 64 keys of the block
         if (wave_active && kb <= wave_last && kb + PF_BN > wave_lo) {
-        pf_f32x4_t s[4];
+        pf_f32x4_t s[QW][4];
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            s[t] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < QW; ++u) s[u][t] = pf_f32x4_t{0.f, 0.f, 0.f, 0.f};
             const int rho = kh * PF_BN + t * 16 + r;
 #pragma unroll
             for (int dk = 0; dk < DK; ++dk) {
                 pf_pack a;
                 a.u = kl[rho * KC + ((dk * 4 + j) ^ ((rho / KSW) & (KC - 1)))];
-                s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, qop[dk], s[t], 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < QW; ++u)      // one read of the keys' operand serves every sub-tile
+                    s[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, qop[u][dk], s[u][t], 0, 0, 0);
             }
         }
         const bool whole = kb + PF_BN - 1 <= wave_first && (window <= 0 || kb > wave_last - window);
-        float mx = -INFINITY;
-        if (whole) {
+        pf_pack pb[QW][2];
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+        for (int u = 0; u < QW; ++u) {
+            float mx = -INFINITY;
+            if (whole) {
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    s[t][x] *= scale_log2;
-                    mx = fmaxf(mx, s[t][x]);
-                }
-        } else {
+                for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+                    for (int x = 0; x < 4; ++x) {
+                        s[u][t][x] *= scale_log2;
+                        mx = fmaxf(mx, s[u][t][x]);
+                    }
+            } else {
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
-                    const bool vis = key <= qpos && (window <= 0 || key > qpos - window);
-                    const float v = vis ? s[t][x] * scale_log2 : -INFINITY;
-                    s[t][x] = v;
-                    mx = fmaxf(mx, v);
-                }
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
-        const float m_new = fmaxf(m, mx);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float corr = __builtin_amdgcn_exp2f(m - m_use);
-        m = m_new;
-        float psum = 0.f;
+                for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                s[t][x] = __builtin_amdgcn_exp2f(s[t][x] - m_use);
-                psum += s[t][x];
+                    for (int x = 0; x < 4; ++x) {
+                        const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
+                        const bool vis = key <= qpos[u] && (window <= 0 || key > qpos[u] - window);
+                        const float v = vis ? s[u][t][x] * scale_log2 : -INFINITY;
+                        s[u][t][x] = v;
+                        mx = fmaxf(mx, v);
+                    }
             }
-        pf_pack pb[2];
+            mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
+            const float m_new = fmaxf(m[u], mx);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float corr = __builtin_amdgcn_exp2f(m[u] - m_use);
+            m[u] = m_new;
+            float psum = 0.f;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            pb[b].u.x = zi_pack_bf16x2(s[2 * b][0], s[2 * b][1]);
-            pb[b].u.y = zi_pack_bf16x2(s[2 * b][2], s[2 * b][3]);
-            pb[b].u.z = zi_pack_bf16x2(s[2 * b + 1][0], s[2 * b + 1][1]);
-            pb[b].u.w = zi_pack_bf16x2(s[2 * b + 1][2], s[2 * b + 1][3]);
-        }
-        lsum = lsum * corr + psum;
-        if (__any(corr != 1.f)) {
+            for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int dd = 0; dd < DT; ++dd) {
-                o[dd][0] *= corr; o[dd][1] *= corr; o[dd][2] *= corr; o[dd][3] *= corr;
+                for (int x = 0; x < 4; ++x) {
+                    s[u][t][x] = __builtin_amdgcn_exp2f(s[u][t][x] - m_use);
+                    psum += s[u][t][x];
+                }
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                pb[u][b].u.x = zi_pack_bf16x2(s[u][2 * b][0], s[u][2 * b][1]);
+                pb[u][b].u.y = zi_pack_bf16x2(s[u][2 * b][2], s[u][2 * b][3]);
+                pb[u][b].u.z = zi_pack_bf16x2(s[u][2 * b + 1][0], s[u][2 * b + 1][1]);
+                pb[u][b].u.w = zi_pack_bf16x2(s[u][2 * b + 1][2], s[u][2 * b + 1][3]);
+            }
+            lsum[u] = lsum[u] * corr + psum;
+            if (__any(corr != 1.f)) {
+#pragma unroll
+                for (int dd = 0; dd < DT; ++dd) {
+                    o[u][dd][0] *= corr; o[u][dd][1] *= corr; o[u][dd][2] *= corr; o[u][dd][3] *= corr;
+                }
             }
         }
 #pragma unroll
@@ -606,7 +630,9 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             for (int b = 0; b < 2; ++b) {
                 pf_pack a;
                 a.u = vl[dim * VC + ((kh * 8 + b * 4 + j) ^ (dim & (VC - 1)))];
-                o[dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[b].b, o[dd], 0, 0, 0);
+#pragma unroll
+                for (int u = 0; u < QW; ++u)      // and one read of the values' operand
+                    o[u][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[u][b].b, o[u][dd], 0, 0, 0);
             }
         }
         }
@@ -631,64 +657,79 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
         kb0 += PF_BS;
     }
     __syncthreads();
-    float l = lsum;
-    l += __shfl_xor(l, 16, ZI_WAVE);
-    l += __shfl_xor(l, 32, ZI_WAVE);
-    {
-        // the two wavefronts of a query sub-tile merge their (maximum, sum, output) through LDS; nobody reads
-        // the tiles any more
-        float* mo = reinterpret_cast<float*>(k_a);                   // [qs][DT][64][4]: as large as a key tile
-        float* ml = reinterpret_cast<float*>(v_a);                   // [qs][64][2]
-        static_assert(sizeof(float) * 4 * DT * ZI_WAVE * 4 <= sizeof(uint4) * KCH, "the key tile holds the merge");
-        if (kh > 0) {
-            float* dst = mo + qs * (DT * ZI_WAVE * 4);
+    float l[QW];
 #pragma unroll
-            for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(dst + (dd * ZI_WAVE + lane) * 4) = o[dd];
-            ml[(qs * ZI_WAVE + lane) * 2] = m;
-            ml[(qs * ZI_WAVE + lane) * 2 + 1] = l;
+    for (int u = 0; u < QW; ++u) {
+        l[u] = lsum[u];
+        l[u] += __shfl_xor(l[u], 16, ZI_WAVE);
+        l[u] += __shfl_xor(l[u], 32, ZI_WAVE);
+    }
+    {
+        // the two wavefronts of a query group merge their (maximum, sum, output) through LDS; nobody reads
+        // the tiles any more
+        float* mo = reinterpret_cast<float*>(k_ab);                  // [qs][QW][DT][64][4]: within the two key tiles
+        float* ml = reinterpret_cast<float*>(v_ab);                  // [qs][QW][64][2]
+        static_assert(sizeof(float) * 4 * QW * DT * ZI_WAVE * 4 <= sizeof(uint4) * 2 * KCH, "the key tiles hold the merge");
+        if (kh > 0) {
+#pragma unroll
+            for (int u = 0; u < QW; ++u) {
+                float* dst = mo + (qs * QW + u) * (DT * ZI_WAVE * 4);
+#pragma unroll
+                for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(dst + (dd * ZI_WAVE + lane) * 4) = o[u][dd];
+                ml[((qs * QW + u) * ZI_WAVE + lane) * 2] = m[u];
+                ml[((qs * QW + u) * ZI_WAVE + lane) * 2 + 1] = l[u];
+            }
         }
         __syncthreads();
         if (kh > 0) return;
-        const float* src = mo + qs * (DT * ZI_WAVE * 4);
-        const float m2 = ml[(qs * ZI_WAVE + lane) * 2];
-        const float l2 = ml[(qs * ZI_WAVE + lane) * 2 + 1];
-        const float mm = fmaxf(m, m2);
-        const float mu = (mm == -INFINITY) ? 0.f : mm;
-        const float a1 = __builtin_amdgcn_exp2f(m - mu), a2 = __builtin_amdgcn_exp2f(m2 - mu);
-        l = l * a1 + l2 * a2;
-        m = mm;
+#pragma unroll
+        for (int u = 0; u < QW; ++u) {
+            const float* src = mo + (qs * QW + u) * (DT * ZI_WAVE * 4);
+            const float m2 = ml[((qs * QW + u) * ZI_WAVE + lane) * 2];
+            const float l2 = ml[((qs * QW + u) * ZI_WAVE + lane) * 2 + 1];
+            const float mm = fmaxf(m[u], m2);
+            const float mu = (mm == -INFINITY) ? 0.f : mm;
+            const float a1 = __builtin_amdgcn_exp2f(m[u] - mu), a2 = __builtin_amdgcn_exp2f(m2 - mu);
+            l[u] = l[u] * a1 + l2 * a2;
+            m[u] = mm;
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) {
+                const pf_f32x4_t v = *reinterpret_cast<const pf_f32x4_t*>(src + (dd * ZI_WAVE + lane) * 4);
+                o[u][dd][0] = o[u][dd][0] * a1 + v[0] * a2; o[u][dd][1] = o[u][dd][1] * a1 + v[1] * a2;
+                o[u][dd][2] = o[u][dd][2] * a1 + v[2] * a2; o[u][dd][3] = o[u][dd][3] * a1 + v[3] * a2;
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < QW; ++u) {
+        if (!qvalid[u]) continue;
+        if (nc > 1) {
+            // one of several cuts of this tile's keys: leave (maximum, sum, unnormalised output) for the merge
+            if (nc > max_chunks) {
+                if (blockIdx.y == 0)
+                    for (int dd = 0; dd < DT; ++dd)
+                        for (int x = 0; x < 4; ++x)
+                            zi_store(out + (int64_t)(start + off + row[u]) * ldo + (int64_t)h * D + dd * 16 + j * 4 + x, NAN);
+                continue;
+            }
+            const int64_t slot = zi_pf_part_slot(start + off + row[u], nh, h, max_chunks, blockIdx.y);
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = o[u][dd];
+            if (j == 0) {
+                part_ml[slot * 2] = m[u];
+                part_ml[slot * 2 + 1] = l[u];
+            }
+            continue;
+        }
+        const float inv = 1.f / l[u];
+        zi_bf16* orow = out + (int64_t)(start + off + row[u]) * ldo + (int64_t)h * D;
 #pragma unroll
         for (int dd = 0; dd < DT; ++dd) {
-            const pf_f32x4_t v = *reinterpret_cast<const pf_f32x4_t*>(src + (dd * ZI_WAVE + lane) * 4);
-            o[dd][0] = o[dd][0] * a1 + v[0] * a2; o[dd][1] = o[dd][1] * a1 + v[1] * a2;
-            o[dd][2] = o[dd][2] * a1 + v[2] * a2; o[dd][3] = o[dd][3] * a1 + v[3] * a2;
+            uint2 w;
+            w.x = zi_pack_bf16x2(o[u][dd][0] * inv, o[u][dd][1] * inv);
+            w.y = zi_pack_bf16x2(o[u][dd][2] * inv, o[u][dd][3] * inv);
+            *reinterpret_cast<uint2*>(orow + dd * 16 + j * 4) = w;
         }
-    }
-    if (!qvalid) return;
-    if (nc > 1) {
-        if (nc > max_chunks) {
-            if (blockIdx.y == 0)
-                for (int dd = 0; dd < DT; ++dd)
-                    for (int x = 0; x < 4; ++x) zi_store(out + (int64_t)(start + off + row) * ldo + (int64_t)h * D + dd * 16 + j * 4 + x, NAN);
-            return;
-        }
-        const int64_t slot = zi_pf_part_slot(start + off + row, nh, h, max_chunks, blockIdx.y);
-#pragma unroll
-        for (int dd = 0; dd < DT; ++dd) *reinterpret_cast<pf_f32x4_t*>(part_o + slot * D + dd * 16 + j * 4) = o[dd];
-        if (j == 0) {
-            part_ml[slot * 2] = m;
-            part_ml[slot * 2 + 1] = l;
-        }
-        return;
-    }
-    const float inv = 1.f / l;
-    zi_bf16* orow = out + (int64_t)(start + off + row) * ldo + (int64_t)h * D;
-#pragma unroll
-    for (int dd = 0; dd < DT; ++dd) {
-        uint2 w;
-        w.x = zi_pack_bf16x2(o[dd][0] * inv, o[dd][1] * inv);
-        w.y = zi_pack_bf16x2(o[dd][2] * inv, o[dd][3] * inv);
-        *reinterpret_cast<uint2*>(orow + dd * 16 + j * 4) = w;
     }
 }
 
@@ -699,11 +740,11 @@ attention_prefill_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const flo
                                const float* __restrict__ part_ml, const int32_t* __restrict__ tile_entry,
                                const int32_t* __restrict__ tile_off, const int32_t* __restrict__ entry_start,
                                const int32_t* __restrict__ entry_len, const int32_t* __restrict__ entry_past, int nh,
-                               int D, int window, int max_chunks) {
-    const int tile = blockIdx.x / PF_BM, qi = blockIdx.x % PF_BM, h = blockIdx.y, lane = threadIdx.x;
+                               int D, int window, int max_chunks, int bm) {
+    const int tile = blockIdx.x / bm, qi = blockIdx.x % bm, h = blockIdx.y, lane = threadIdx.x;
     const int e = tile_entry[tile], off = tile_off[tile];
     const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
-    const int count = (len - off < PF_BM) ? len - off : PF_BM;
+    const int count = (len - off < bm) ? len - off : bm;
     if (qi >= count) return;
     const int nc = zi_pf_cut(past + off, count, window, 0).nc;
     if (nc == 1 || nc > max_chunks) return;
@@ -747,14 +788,6 @@ extern "C" int zi_attention_prefill_supported(int dt, int nh, int nkv, int d, in
     return page_size >= 8 && (page_size & (page_size - 1)) == 0;
 }
 
-extern "C" int zi_attention_prefill_tile() { return PF_BM; }
-
-// Keys one workgroup walks at most: tiles are cut at absolute multiples of this.
-extern "C" int zi_attention_prefill_chunk_keys() { return PF_CHUNK; }
-
-// Tile i covers the queries [tile_off[i], tile_off[i] + 64) of entry tile_entry[i] (fewer at the
-// entry's end); entry e brings entry_len[e] tokens that start at row entry_start[e] of q and at
-// position entry_past[e] of its sequence, whose block table is row e of block_tables.
 // Which kernel head sizes 64 and 128 take: 1 (the default) loads keys and values straight into LDS, 0 stages
 // them through registers like the other head sizes.  For measurements and tests.
 static int pf_variant = 1;
@@ -764,13 +797,28 @@ extern "C" int zi_attention_prefill_variant(int variant) {
     return before;
 }
 
+// Queries of a tile: 64, or 128 where the kernel that loads straight into LDS serves (head sizes 64 and 128):
+// there a block of keys and values in LDS, and an operand read from it, serves twice the queries.  The caller
+// cuts its entries into tiles of this many queries (zi_attention_prefill takes either size for those shapes).
+extern "C" int zi_attention_prefill_tile(int dt, int d) {
+    return (dt == ZI_BF16 && pf_variant == 1 && (d == 64 || d == 128)) ? 2 * PF_BM : PF_BM;
+}
+
+// Keys one workgroup walks at most: tiles are cut at absolute multiples of this.
+extern "C" int zi_attention_prefill_chunk_keys() { return PF_CHUNK; }
+
+// Tile i covers the queries [tile_off[i], tile_off[i] + tile) of entry tile_entry[i] (fewer at the
+// entry's end; `tile` is 64, or 128 for head sizes 64 and 128); entry e brings entry_len[e] tokens that start at row entry_start[e] of q and at
+// position entry_past[e] of its sequence, whose block table is row e of block_tables.
 extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
                                     const void* kcache, const void* vcache, const int32_t* tile_entry,
                                     const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
                                     const int32_t* entry_past, const int32_t* block_tables, int max_pages,
                                     int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
-                                    int rows, int max_chunks, float* workspace, int64_t workspace_floats,
+                                    int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
                                     hipStream_t stream) {
+    ZI_REQUIRE(tile == PF_BM || (tile == 2 * PF_BM && pf_variant == 1 && (d == 64 || d == 128)),
+               "attention_prefill: tiles of %d queries (64, or 128 for head sizes 64 and 128)", tile);
     ZI_REQUIRE(zi_attention_prefill_supported(dt, nh, nkv, d, page_size),
                "attention_prefill: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, page size a power "
                "of two from 8): dtype %d heads %d kv_heads %d head_dim %d page %d", dt, nh, nkv, d, page_size);
@@ -787,7 +835,7 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
                                    workspace_floats >= zi_attention_prefill_workspace(rows, nh, d, max_chunks)),
                "attention_prefill: workspace of %lld floats is too small or not aligned", (long long)workspace_floats);
     if (num_tiles == 0) return 0;
-    ZI_REQUIRE((int64_t)num_tiles * nh < (1ll << 31) && (int64_t)num_tiles * PF_BM < (1ll << 31), "attention_prefill: too many tiles");
+    ZI_REQUIRE((int64_t)num_tiles * nh < (1ll << 31) && (int64_t)num_tiles * tile < (1ll << 31), "attention_prefill: too many tiles");
     const dim3 grid(num_tiles * nh, max_chunks);
     int ps_shift = 0;
     while ((1 << ps_shift) < page_size) ++ps_shift;
@@ -798,13 +846,15 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
         window, scale, po, pml, max_chunks)
-#define ZI_PF_DMA(DD)                                                                                          \
-    attention_prefill_dma_kernel<DD><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                                 \
+#define ZI_PF_DMA(DD, QW)                                                                                      \
+    attention_prefill_dma_kernel<DD, QW><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                             \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
         window, scale, po, pml, max_chunks)
-    if (pf_variant == 1 && d == 128) ZI_PF_DMA(128);
-    else if (pf_variant == 1 && d == 64) ZI_PF_DMA(64);
+    if (pf_variant == 1 && d == 128 && tile == 2 * PF_BM) ZI_PF_DMA(128, 2);
+    else if (pf_variant == 1 && d == 64 && tile == 2 * PF_BM) ZI_PF_DMA(64, 2);
+    else if (pf_variant == 1 && d == 128) ZI_PF_DMA(128, 1);
+    else if (pf_variant == 1 && d == 64) ZI_PF_DMA(64, 1);
     else
     switch (d) {
         case 16: ZI_PF(16); break;
@@ -819,7 +869,8 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
 #undef ZI_PF
 #undef ZI_PF_DMA
     if (max_chunks > 1)
-        attention_prefill_merge_kernel<<<dim3(num_tiles * PF_BM, nh), ZI_WAVE, 0, stream>>>(
-            (zi_bf16*)out, ldo, po, pml, tile_entry, tile_off, entry_start, entry_len, entry_past, nh, d, window, max_chunks);
+        attention_prefill_merge_kernel<<<dim3(num_tiles * tile, nh), ZI_WAVE, 0, stream>>>(
+            (zi_bf16*)out, ldo, po, pml, tile_entry, tile_off, entry_start, entry_len, entry_past, nh, d, window, max_chunks,
+            tile);
     return zi_check_launch("attention_prefill");
 }

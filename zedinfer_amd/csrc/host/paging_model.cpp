@@ -154,7 +154,8 @@ extern "C" int pm_check_decode(int n_idx, const int* tok_index, const int* tok_s
 }
 
 // The prompt attention launch (attention_prefill kernels): grid (tiles * nh, cuts), eight wavefronts: four
-// groups of 16 queries, each shared by two wavefronts that take alternate halves of every block of 128 keys.
+// groups of tile / 4 queries (tile = 64 or 128 queries), each shared by two wavefronts that take alternate
+// halves of every block of 128 keys.
 // stats[0] = (query, key) pairs covered, stats[1] = workspace slots written, stats[2] = tiles given NaN.
 // `entry_real` (or null): the tokens of each entry that are its own; the rest are padding, whose queries'
 // results nobody reads and whose keys are nowhere: they are checked for bounds only.
@@ -162,8 +163,10 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
                                 const int* entry_len, const int* entry_past, const int* entry_real, int num_entries,
                                 const int* block_tables,
                                 int max_pages, int num_pages, int nh, int nkv, int d, int ps, int window, int rows,
-                                int max_chunks, int64_t workspace_floats, int64_t* stats) {
+                                int max_chunks, int64_t workspace_floats, int tile_queries, int64_t* stats) {
     PM_CHECK(nkv > 0 && nh % nkv == 0 && ps >= 8 && (ps & (ps - 1)) == 0 && max_pages > 0, "prefill: bad sizes");
+    PM_CHECK(tile_queries == ZI_PF_BM || tile_queries == 2 * ZI_PF_BM, "prefill: tiles of %d queries", tile_queries);
+    const int BM = tile_queries, QR = tile_queries / 4;
     const int ps_shift = shift_of(ps), pi_last = max_pages - 1;
     const int64_t pool = zi_pool_elements(num_pages, nkv, ps, d);
     const int64_t ml_base = (int64_t)rows * nh * max_chunks * d;
@@ -175,8 +178,8 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
         const int e = tile_entry[tile], off = tile_off[tile];
         PM_CHECK(e >= 0 && e < num_entries, "prefill: tile %d names entry %d of %d", tile, e, num_entries);
         const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
-        PM_CHECK(off >= 0 && off < len && off % ZI_PF_BM == 0, "prefill: tile %d starts at %d of %d tokens", tile, off, len);
-        const int count = (len - off < ZI_PF_BM) ? len - off : ZI_PF_BM;
+        PM_CHECK(off >= 0 && off < len && off % BM == 0, "prefill: tile %d starts at %d of %d tokens", tile, off, len);
+        const int count = (len - off < BM) ? len - off : BM;
         const int real = entry_real ? entry_real[e] - off : count;      // queries of the tile that are real
         PM_CHECK(start + off + count <= rows, "prefill: tile %d covers rows up to %d of %d", tile, start + off + count, rows);
         const int* bt = block_tables + (int64_t)e * max_pages;
@@ -219,14 +222,14 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
                 }
                 // which wavefronts work on which half of the block, and the pairs they cover
                 for (int qs = 0; qs < 4; ++qs) {
-                    if (qs * 16 >= count) continue;
-                    const int wave_last = pos0 + ((qs * 16 + 15 < count) ? qs * 16 + 15 : count - 1);
-                    const int wave_lo = (window > 0 && pos0 + qs * 16 - window + 1 > 0) ? pos0 + qs * 16 - window + 1 : 0;
+                    if (qs * QR >= count) continue;
+                    const int wave_last = pos0 + ((qs * QR + QR - 1 < count) ? qs * QR + QR - 1 : count - 1);
+                    const int wave_lo = (window > 0 && pos0 + qs * QR - window + 1 > 0) ? pos0 + qs * QR - window + 1 : 0;
                     for (int kh = 0; kh < 2; ++kh) {
                         const int kb2 = kb + kh * 64;
                         if (!(kb2 <= wave_last && kb2 + 64 > wave_lo)) continue;
-                        for (int r = 0; r < 16 && qs * 16 + r < count; ++r) {
-                            const int q = qs * 16 + r, qpos = pos0 + q;
+                        for (int r = 0; r < QR && qs * QR + r < count; ++r) {
+                            const int q = qs * QR + r, qpos = pos0 + q;
                             for (int k = 0; k < 64; ++k) {
                                 const int key = kb2 + k;
                                 if (key <= qpos && (window <= 0 || key > qpos - window)) {

@@ -37,11 +37,11 @@ _PROTOTYPES = {
     "zi_attention_decode_project_heads": [I],
     "zi_rope_table": [P, P, P, I, I, P],
     "zi_attention_decode_chunks": [I],
-    "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, P],
+    "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, P],
     "zi_attention_prefill_chunks": [I],
     "zi_attention_prefill_variant": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],
-    "zi_attention_prefill_tile": [],
+    "zi_attention_prefill_tile": [I, I],
     "zi_attention_prefill_chunk_keys": [],
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
     "zi_gemm_skinny": [P, I, I, P, P, P, I, I, I, L, L, L, P, L, P],

@@ -561,7 +561,18 @@ def attention_prefill_variant(variant: int = -1) -> int:
     return int(_lib.load().zi_attention_prefill_variant(int(variant)))
 
 
-PREFILL_TILE = 64     # queries one workgroup of the prompt kernel takes
+PREFILL_TILE = 64     # queries one workgroup of the prompt kernel takes, at least
+PREFILL_TILE_MAX = 128
+
+
+def attention_prefill_tile(dtype: torch.dtype, d: int) -> int:
+    """Queries of a tile of ``attention_prefill`` for this head size: 64, or 128 where the kernel that loads keys
+    and values straight into LDS serves (a staged block then serves twice the queries).  The caller cuts its
+    entries into tiles of this many queries."""
+    if dtype not in _CODES:
+        return PREFILL_TILE
+    return int(_lib.load().zi_attention_prefill_tile(_CODES[dtype], int(d)))
+
 
 
 def attention_prefill_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, page_size: int) -> bool:
@@ -579,7 +590,7 @@ def attention_prefill_workspace(rows: int, nh: int, d: int, max_keys: int, windo
 
 def _prefill_chunks(max_keys: int, window: int) -> int:
     if window > 0:      # a windowed tile's keys span at most the window, a tile and a block, from anywhere in a cut
-        max_keys = min(max_keys, window + PREFILL_TILE + 128) + int(_lib.load().zi_attention_prefill_chunk_keys()) - 1
+        max_keys = min(max_keys, window + PREFILL_TILE_MAX + 128) + int(_lib.load().zi_attention_prefill_chunk_keys()) - 1
     return int(_lib.load().zi_attention_prefill_chunks(int(max_keys)))
 
 
@@ -587,14 +598,14 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
                       tile_off: torch.Tensor, entry_start: torch.Tensor, entry_len: torch.Tensor,
                       entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, out: Optional[torch.Tensor] = None, max_keys: int = 0,
-                      workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      workspace: Optional[torch.Tensor] = None, tile: int = PREFILL_TILE) -> torch.Tensor:
     """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
     of 16 up to 128, page size a power of two from 8).
 
     Entry e brings ``entry_len[e]`` tokens, rows ``entry_start[e]...`` of q, that continue a sequence
     holding ``entry_past[e]`` tokens whose block table is row e of ``block_tables``.  Tile i covers the
-    queries [tile_off[i], tile_off[i] + PREFILL_TILE) of entry ``tile_entry[i]``; rows of ``out`` that no
-    tile covers are left alone.  ``max_keys`` is an upper bound, known on the host, of the keys any query
+    queries [tile_off[i], tile_off[i] + tile) of entry ``tile_entry[i]`` (``tile``: 64, or what
+    ``attention_prefill_tile`` says for the head size); rows of ``out`` that no tile covers are left alone.  ``max_keys`` is an upper bound, known on the host, of the keys any query
     sees (its position + 1; 0: what the block tables could hold): tiles that see more than 2,048 keys are
     cut over several workgroups and merged, which needs ``workspace`` (``attention_prefill_workspace``
     entries of float32; allocated here when not given).  A bound that is too low leaves NaN in the rows
@@ -617,8 +628,8 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
     if (block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous()
             or block_tables.shape[0] < E):
         raise ValueError("attention_prefill: block_tables must be a contiguous int32 [entries, max_pages] tensor")
-    if _lib.load().zi_attention_prefill_tile() != PREFILL_TILE:
-        raise _lib.KernelLibraryError("the kernel library was built for another prompt tile size")
+    if tile not in (PREFILL_TILE, attention_prefill_tile(q.dtype, d)):
+        raise ValueError(f"attention_prefill: tiles of {tile} queries are not taken for head size {d}")
     if out is None:
         out = torch.empty((n, nh * d), dtype=q.dtype, device=q.device)
     ldo, wo = _rows(out, "attention_prefill out")
@@ -636,7 +647,7 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
     _lib.call("zi_attention_prefill", _p(out), _p(q), _code(q, "attention_prefill"), num_tiles, ldq, ldo, _p(kcache),
               _p(vcache), _p(tile_entry), _p(tile_off), _p(entry_start), _p(entry_len), _p(entry_past),
               _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), n,
-              max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, _stream())
+              max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, int(tile), _stream())
     return out
 
 

@@ -15,22 +15,33 @@ from .base import (HostBatch, KVCacheRequest, LayerMemory, Mixer, POSITION_ENCOD
 from .feed_forward import stack_rows
 
 SHORT_ENTRY = 4     # entries of up to this many tokens are attended token by token, split over the keys
-LONG_TILE = 64      # longer entries are cut into tiles of this many queries for the prompt kernel
+LONG_TILE = 64      # longer entries are cut into tiles of this many queries for the prompt kernel (or 128: see below)
 
 
 class AttentionPlanner(StepPlanner):
     """How the attention kernels divide a step: tokens of entries that bring at most SHORT_ENTRY tokens
     ("decoded" tokens) go, one by one, to the kernel that splits a query's keys over many wavefronts;
-    longer entries are cut into tiles of LONG_TILE queries for the prompt kernel, the tile that sees
-    most keys first.
+    longer entries are cut into tiles of queries for the prompt kernel, the tile that sees most keys first.
+
+    Tiles hold LONG_TILE queries, or ``wide_tile`` (twice as many, where the mixer's prompt kernel takes them:
+    a block of keys staged on the chip then serves twice the queries) when the step is large enough to fill
+    the chip with those: measured with 28 layers of the 1.5B sizes (12 heads), 16,384 tokens of one prompt run
+    88 against 99 ms with the wide tiles, 8,192 tokens 33.7 against 37.0, 3,072 tokens 12.8 against 13.3, and
+    2,048 tokens 9.2 against 9.1 ms; with 28 heads 2,048 tokens gain 2%.  The choice is a function of the entries' (padded) lengths
+    and of the bound of their keys, so that a recorded step meets the same one again.
 
     arrays: ``short_idx`` / ``long_idx``, the flat indices of the tokens of either kind; ``tile_entry`` /
-    ``tile_off``: tile i covers tokens [tile_off[i], tile_off[i] + LONG_TILE) of entry tile_entry[i].
-    sizes: ``num_short``, ``num_long``, ``num_tiles``; ``max_short_keys`` / ``max_long_keys``: an upper
+    ``tile_off``: tile i covers tokens [tile_off[i], tile_off[i] + tile) of entry tile_entry[i].
+    sizes: ``num_short``, ``num_long``, ``num_tiles``, ``tile``; ``max_short_keys`` / ``max_long_keys``: an upper
     bound of the keys a token of either kind sees (its position + 1), which sizes the launches."""
 
-    key = ("attention", SHORT_ENTRY, LONG_TILE)
     fixed_for_single_tokens = True
+    FILL = 384          # workgroups of wide tiles from which they pay (one and a half a compute unit)
+    CUT_KEYS = 2048     # a tile's keys are cut over several workgroups every so many
+
+    def __init__(self, wide_tile: int = LONG_TILE, heads: int = 1):
+        self.wide_tile, self.heads = int(wide_tile), int(heads)
+        self.key = ("attention", SHORT_ENTRY, self.wide_tile, self.heads)
 
     def plan(self, hb: HostBatch) -> StepPlan:
         lens, past = hb.entry_len, hb.entry_past
@@ -48,18 +59,30 @@ class AttentionPlanner(StepPlanner):
                             hb.bound_multi if several else 0, 1)
         if long_idx.size and hb.bound_multi:
             max_long = hb.bound_multi
-        tiles = [(int(past[i]) + off + min(LONG_TILE, int(lens[i]) - off), i, off)
-                 for i in range(hb.num_entries) if not short[i] for off in range(0, int(lens[i]), LONG_TILE)]
+        tile = LONG_TILE
+        if self.wide_tile > LONG_TILE and long_idx.size:
+            wide = int(sum(-(-int(n) // self.wide_tile) for n in lens[~short]))
+            if wide * -(-max_long // self.CUT_KEYS) * self.heads >= self.FILL:
+                tile = self.wide_tile
+        tiles = [(int(past[i]) + off + min(tile, int(lens[i]) - off), i, off)
+                 for i in range(hb.num_entries) if not short[i] for off in range(0, int(lens[i]), tile)]
         tiles.sort(key=lambda t: -t[0])
         return StepPlan(
             arrays={"short_idx": short_idx, "long_idx": long_idx,
                     "tile_entry": np.array([t[1] for t in tiles], dtype=np.int32),
                     "tile_off": np.array([t[2] for t in tiles], dtype=np.int32)},
             sizes={"num_short": int(short_idx.size), "num_long": int(long_idx.size), "num_tiles": len(tiles),
-                   "max_short_keys": max_short, "max_long_keys": max_long})
+                   "tile": tile, "max_short_keys": max_short, "max_long_keys": max_long})
 
 
-_ATTENTION_PLANNER = AttentionPlanner()
+_PLANNERS: Dict[tuple, AttentionPlanner] = {}
+
+
+def attention_planner(wide_tile: int, heads: int) -> AttentionPlanner:
+    """One planner per (widest tile, heads): mixers that agree in both share a plan."""
+    if (wide_tile, heads) not in _PLANNERS:
+        _PLANNERS[(wide_tile, heads)] = AttentionPlanner(wide_tile, heads)
+    return _PLANNERS[(wide_tile, heads)]
 
 
 @register_mixer("attention")
@@ -124,6 +147,9 @@ class Attention(Mixer):
             else:
                 self.biases = bs
         self.o = weights["o"]
+        # the widest prompt tile the prompt kernel of this head size takes (the planner chooses step by step)
+        self.wide_tile = ops.attention_prefill_tile(rt.dtype, self.d) if rt.device.type == "cuda" else LONG_TILE
+        self.plan_key = attention_planner(self.wide_tile, self.nh).key
 
     def attend(self, q, att, batch, view, memory: LayerMemory) -> None:
         """Tokens of short entries (decoded tokens) go to the kernel that splits one query's keys over
@@ -131,7 +157,7 @@ class Attention(Mixer):
         not take goes to the plain one."""
         args = (memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
                 self.scale)
-        plan = batch.plans[_ATTENTION_PLANNER.key]
+        plan = batch.plans[self.plan_key]
         n_short, n_long, N = plan.sizes["num_short"], plan.sizes["num_long"], batch.num_tokens
         if n_short:
             if ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
@@ -151,12 +177,12 @@ class Attention(Mixer):
                 ops.attention_prefill(q, memory.k, memory.v, plan.dev["tile_entry"], plan.dev["tile_off"],
                                       batch.entry_start, batch.entry_len, batch.entry_past, view.block_tables, self.nh,
                                       self.nkv, self.d, self.scale, self.window, out=att, max_keys=max_keys,
-                                      workspace=ws)
+                                      workspace=ws, tile=plan.sizes["tile"])
             else:
                 ops.attention(q, *args, self.window, out=att, tok_index=plan.dev["long_idx"] if n_long < N else None)
 
     def planner(self) -> StepPlanner:
-        return _ATTENTION_PLANNER
+        return attention_planner(self.wide_tile, self.nh)
 
     def positions_of(self, batch) -> torch.Tensor:
         """What the position encoding is given: every token's index in its sequence, or the step's
@@ -214,7 +240,7 @@ class Attention(Mixer):
         rot = 0 if isinstance(table, str) else 2 * table.shape[1]
         S, n, width = sums.shape
         ps = memory.k.shape[2]
-        max_keys = batch.plans[_ATTENTION_PLANNER.key].sizes["max_short_keys"]
+        max_keys = batch.plans[self.plan_key].sizes["max_short_keys"]
         if not ops.attention_decode_fused_supported(memory.k.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
             return None
         ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
