@@ -381,7 +381,7 @@ def test_decode_graphs_replay_what_eager_steps_compute(tiny, dtype, tmp_path):
         dtype = "bfloat16"
     fast, slow = engine(tiny, dtype).engine, engine(tiny, dtype).engine
     assert fast.use_graphs
-    slow.use_graphs = False
+    slow.use_graphs = slow.use_tapes = False       # every step part by part
     toks = {r: traces.random_tokens(V, 150, seed=60 + i) for i, r in enumerate("abcd")}
     fed = {r: 0 for r in toks}
     seqs = {}
@@ -438,7 +438,7 @@ def test_prompt_portions_replay_as_graphs(tiny, dtype, tmp_path):
         dtype = "bfloat16"
     fast, slow = engine(tiny, dtype, num_kv_blocks=1000).engine, engine(tiny, dtype, num_kv_blocks=1000).engine
     assert fast.use_graphs
-    slow.use_graphs = False
+    slow.use_graphs = slow.use_tapes = False       # every step part by part
     toks = {r: traces.random_tokens(V, 1800, seed=80 + i) for i, r in enumerate("abcd")}
     fed = {r: 0 for r in toks}
     seqs = {}
@@ -497,7 +497,7 @@ def test_graphs_that_are_dropped_and_recorded_again(tiny):
     from zedinfer_amd.engine import StepEntry
     V = tiny["cfg"]["vocab_size"]
     fast, slow = engine(tiny, num_kv_blocks=300).engine, engine(tiny, num_kv_blocks=300).engine
-    slow.use_graphs = False
+    slow.use_graphs = slow.use_tapes = False       # every step part by part
     fast.graph_limit = fast.prompt_graph_limit = 2
     toks = {r: traces.random_tokens(V, 900, seed=90 + i) for i, r in enumerate("abc")}
     fed = {r: 0 for r in toks}
@@ -533,7 +533,7 @@ def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatc
     tiny16 = dict(tiny, folder=folder16, weights=plain.load_folder(folder16)[1])
     one, two = engine(tiny16, "bfloat16").engine, engine(tiny16, "bfloat16").engine
     for eng in (one, two):
-        eng.use_graphs = False
+        eng.use_graphs = eng.use_tapes = False       # every step part by part: the calls are counted
     toks = {r: traces.random_tokens(V, 120, seed=70 + i) for i, r in enumerate("abc")}
     fed = {r: 0 for r in toks}
     seqs = {(e, r): e.open(r) for e in (one, two) for r in toks}
@@ -585,26 +585,22 @@ def test_decode_graphs_with_the_library_product(tiny, requests, monkeypatch, tmp
     tiny16 = dict(tiny, folder=folder16, weights=plain.load_folder(folder16)[1])
     fast = engine(tiny16, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
     slow = engine(tiny16, "bfloat16", max_batch_requests=requests + 4, num_kv_blocks=8 * requests).engine
-    slow.use_graphs = False
+    slow.use_graphs = slow.use_tapes = False       # every step part by part
     # steps with prompt portions run as they are in both engines (padded to a graph's shape they would take
     # other kernels and round differently, and so would every later step that reads what they stored)
     fast.prompt_graph_max_tokens = 0
+    fast.use_tapes = False
     names = [f"r{i}" for i in range(requests)]
     toks = {r: traces.random_tokens(V, 40, seed=80 + i) for i, r in enumerate(names)}
     seqs = {(e, r): e.open(r) for e in (fast, slow) for r in names}
     fed = {r: 0 for r in names}
     calls = {}
-    real_call, real_mm = _lib.call, torch.mm
+    real_call = _lib.call
 
     def counted_call(name, *a):
         calls[name] = calls.get(name, 0) + 1
         return real_call(name, *a)
-
-    def counted_mm(*a, **k):
-        calls["library"] = calls.get("library", 0) + 1
-        return real_mm(*a, **k)
     monkeypatch.setattr(_lib, "call", counted_call)
-    monkeypatch.setattr(torch, "mm", counted_mm)
 
     def both(plan):
         outs = []
@@ -628,9 +624,9 @@ def test_decode_graphs_with_the_library_product(tiny, requests, monkeypatch, tmp
     assert first.get("zi_gemm_generic", 0) == 0, first
     assert first.get("zi_attention_decode", 0) > 0 and first.get("zi_attention_decode_fused", 0) == 0, first
     if requests <= 64:
-        assert first.get("zi_gemm_skinny", 0) > 0 and first.get("library", 0) == 0, first
+        assert first.get("zi_gemm_skinny", 0) > 0 and first.get("zi_gemm_lt", 0) == 0, first
     else:
-        assert first.get("library", 0) > 0, first
+        assert first.get("zi_gemm_lt", 0) > 0, first
     worst = mean = scale = 0.0
     for i, r in enumerate(names):
         ref = plain.forward(tiny["cfg"], tiny16["weights"], toks[r][:fed[r]])[-1]

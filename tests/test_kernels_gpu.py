@@ -297,6 +297,49 @@ def test_linear(ops, xdt, wdt, odt, M, N, K):
     assert float(wide[:, :4].abs().max()) == 0 and float(wide[:, N + 4:].abs().max()) == 0
 
 
+@pytest.mark.parametrize("M,N,K", [(65, 136, 72), (200, 2048, 1536), (130, 1536, 8960), (1000, 152, 264)])
+def test_linear_by_the_library(ops, M, N, K):
+    """The many-rows products that go to the library (straight with and without bias, into rows of a wider
+    buffer, with float32 results, transposed) against a float64 product; then with an algorithm chosen by
+    timing, and with one fixed by its number."""
+    x, w, b = rnd(M, K, dtype=torch.bfloat16, seed=1), rnd(N, K, dtype=torch.bfloat16, scale=0.05, seed=2), \
+        rnd(N, dtype=torch.bfloat16, seed=3)
+    ref = torch.nn.functional.linear(x.double(), w.double()).float()
+    ref_b = ref + b.float()
+    calls = []
+    real = ops._lib.call
+    ops._lib.call = lambda name, *a: (calls.append(name), real(name, *a))[1]
+    try:
+        t = dict(atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(ops.linear(x, w, b).float(), ref_b, **t)
+        torch.testing.assert_close(ops.linear(x, w).float(), ref, **t)
+        torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32), ref, atol=1e-3, rtol=1e-3)
+        wide = torch.zeros(M, N + 16, dtype=torch.bfloat16, device="cuda")
+        ops.linear(x, w, b, out=wide[:, 8:N + 8])
+        torch.testing.assert_close(wide[:, 8:N + 8].float(), ref_b, **t)
+        assert float(wide[:, :8].abs().max()) == 0 and float(wide[:, N + 8:].abs().max()) == 0
+        xw = torch.zeros(M, K + 8, dtype=torch.bfloat16, device="cuda")
+        xw[:, :K] = x
+        torch.testing.assert_close(ops.linear(xw[:, :K], w, b).float(), ref_b, **t)
+        torch.testing.assert_close(ops.linear_transposed(x, w).float(), ref.t(), **t)
+        assert calls == ["zi_gemm_lt"] * 6, calls
+        before = ops.linear(x, w, b)
+        for kwargs in (dict(bias=b), dict(transposed=True), dict(out_dtype=torch.float32)):
+            chosen, proposed, us = ops.linear_tune(x, w, candidates=8, rounds=2, **kwargs)
+            assert 0 <= chosen < proposed and us > 0
+            assert ops.linear_tune(x, w, candidates=8, rounds=2, **kwargs)[0] == chosen       # a shape is tuned once
+        torch.testing.assert_close(ops.linear(x, w, b).float(), ref_b, **t)
+        torch.testing.assert_close(ops.linear_transposed(x, w).float(), ref.t(), **t)
+        torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32), ref, atol=1e-3, rtol=1e-3)
+        ops.linear_choose(x, w, 0, bias=b)
+        assert torch.equal(ops.linear(x, w, b), before)         # the library's first proposal again
+        with pytest.raises(ops.KernelLibraryError, match="proposal"):
+            ops.linear_choose(x, w, 10 ** 6, bias=b)
+    finally:
+        ops._lib.call = real
+    assert ops.linear_tune(x[:8], w) is None and ops.linear_tune(x.float(), w.float()) is None
+
+
 def test_linear_skinny_row_does_not_depend_on_batch(ops):
     """The decode-time product cuts k by the weight's shape alone: a row's result is bit-identical
     whether 1, 8 or 64 rows ride along."""

@@ -1,0 +1,137 @@
+"""The step tape: library calls recorded once and made again from native code.  The tape alone (recorded
+operators on buffers whose contents change), then the engine: steps that run from tapes against the same
+steps part by part, bit for bit, and against the plain implementation."""
+import pytest
+import torch
+
+import tiny_configs
+import traces
+from plain import qwen2_plain as plain
+from tolerances import F32_TOL, bf16_within
+
+pytestmark = pytest.mark.gpu
+
+
+def test_a_tape_repeats_its_calls_on_new_contents():
+    from zedinfer_amd import ops
+    from zedinfer_amd.ops.tape import Recording
+    torch.manual_seed(0)
+    n, H, N = 6, 200, 136
+    x = torch.randn(n, H, device="cuda").bfloat16()
+    w = (torch.randn(N, H, device="cuda") * 0.05).bfloat16()
+    g = torch.randn(H, device="cuda").bfloat16()
+    resid = torch.randn(n, H, device="cuda")
+    normed, y = torch.empty_like(x), torch.empty(n, N, device="cuda", dtype=torch.float32)
+
+    def step():
+        ops.add_rms_norm(resid, x, g, 1e-5, out=normed)          # resid += x; normed = norm(resid) * g
+        ops.linear(normed, w, out=y)
+
+    keep = resid.clone()
+    step()                                   # workspaces get their sizes
+    resid.copy_(keep)
+    with Recording(torch.device("cuda", 0)) as rec:
+        step()
+    assert rec.allocations == 0 and [c[0] for c in rec.calls] == ["zi_add_rmsnorm", "zi_gemm_skinny"]
+    tape = rec.tape()
+    assert tape.length == 2
+    first = y.clone()
+    for seed in (1, 2):                      # new contents in the same buffers
+        torch.manual_seed(seed)
+        x.copy_(torch.randn(n, H, device="cuda").bfloat16())
+        resid.copy_(torch.randn(n, H, device="cuda"))
+        keep = resid.clone()
+        tape.run()
+        got, got_resid = y.clone(), resid.clone()
+        resid.copy_(keep)
+        step()
+        assert torch.equal(got, y) and torch.equal(got_resid, resid) and not torch.equal(got, first)
+
+
+def test_a_tape_refuses_what_it_cannot_hold():
+    import ctypes
+    from zedinfer_amd.ops import _lib
+    from zedinfer_amd.ops.tape import Recording, Tape
+    with pytest.raises(_lib.KernelLibraryError, match="not an entry point"):
+        Tape([("zi_gemm_lt_choose", (1, 0, 0, 1, 1, 1, 1, 1, 1, 1, 0))])
+    lib = _lib.load()
+    handle = ctypes.c_void_p(lib.zi_tape_new())
+    words = (ctypes.c_int64 * 3)(1, 2, 3)
+    with pytest.raises(_lib.KernelLibraryError, match="takes 9 arguments, 3 were recorded"):
+        _lib.call("zi_tape_record", handle, b"zi_embedding", ctypes.cast(words, ctypes.c_void_p), 3)
+    lib.zi_tape_free(handle)
+    # a call that fails on replay is reported with its place in the tape
+    with Recording() as rec:
+        pass
+    assert rec.tape() is None
+    bad = Tape([("zi_add", (ctypes.c_void_p(0), 1, ctypes.c_void_p(0), 1, ctypes.c_void_p(0), 1, 0, ctypes.c_void_p(0))),
+                ("zi_add", (ctypes.c_void_p(0), 99, ctypes.c_void_p(0), 1, ctypes.c_void_p(0), 1, 8, ctypes.c_void_p(0)))])
+    with pytest.raises(_lib.KernelLibraryError, match="call 1 of a tape of 2"):
+        bad.run()
+    with pytest.raises(RuntimeError, match="already"):
+        with Recording():
+            with Recording():
+                pass
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("B", "bfloat16"), ("C", "bfloat16")])
+def test_steps_from_tapes_equal_steps_part_by_part(name, dtype, tmp_path, monkeypatch):
+    """Three requests with prompts of 128 tokens in portions of 64 (a shape that recurs: its second step is
+    recorded, the later ones run from the tape), then decoded together token by token, on an engine that runs
+    from tapes alone (no graphs) and on one that runs every step part by part: the same bits, and both within
+    the tolerance of the plain implementation.  Portions that are multiples of the padding step are taken so
+    that both engines launch the same kernels."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), name, dtype=store, std=tiny_configs.SHARP_STD)
+    cfg, w = plain.load_folder(folder)
+    V = cfg["vocab_size"]
+    ps = tiny_configs.PAGE_SIZES[name]
+
+    def make(tapes):
+        e = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=3 * (200 // ps + 2), kv_block_size=ps,
+                                                              max_batch_requests=4))
+        e.use_graphs = False
+        e.use_tapes = tapes
+        return e
+    taped, plainly = make(True), make(False)
+    assert taped.model.tape_safe()
+    toks = {r: traces.random_tokens(V, 150, seed=60 + i) for i, r in enumerate("abc")}
+    seqs = {(e, r): e.open(r) for e in (taped, plainly) for r in toks}
+    fed = {r: 0 for r in toks}
+
+    def both(plan):
+        outs = [e.step([StepEntry(seqs[(e, r)], toks[r][fed[r]:fed[r] + n], [n - 1]) for r, n in plan])
+                for e in (taped, plainly)]
+        for r, n in plan:
+            fed[r] += n
+        assert torch.equal(outs[0], outs[1]), plan
+        return outs[0]
+
+    for r in "abc":
+        both([(r, 64)])
+    for r in "abc":
+        both([(r, 64)])
+    runs_after_prompts = taped.tape_runs
+    assert runs_after_prompts >= 2              # the third request's portions, at the least
+    for _ in range(22):
+        last = both([(r, 1) for r in "abc"])
+    assert taped.tape_runs >= runs_after_prompts + 15 and plainly.tape_runs == 0
+    worst = mean = scale = 0.0
+    for i, r in enumerate("abc"):
+        ref = plain.forward(cfg, w, toks[r][:fed[r]])[-1]
+        d = (last[i].cpu() - ref).abs()
+        worst, mean, scale = max(worst, float(d.max())), mean + float(d.mean()) / 3, max(scale, float(ref.abs().max()))
+    if dtype == "float32":
+        assert worst <= F32_TOL * max(1.0, scale)
+    else:
+        assert bf16_within(worst, mean, scale)
+    for e in (taped, plainly):
+        for r in toks:
+            e.close(seqs[(e, r)])
+        e.cache.check()
+    # without tapes and graphs nothing is padded and nothing recorded
+    monkeypatch.setenv("ZEDINFER_DISABLE_TAPES", "1")
+    off = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=32, kv_block_size=ps, max_batch_requests=4))
+    assert not off.use_tapes

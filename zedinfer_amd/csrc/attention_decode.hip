@@ -28,6 +28,7 @@
 // bfloat16 only; head_dim a multiple of 16 up to 128; group size up to 16; page size
 // a multiple of 8.  Other shapes are the plain kernel's.
 #include "zi_common.h"
+#include "zi_api.h"
 #include "zi_paging.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 dec_bf16x8_t;

@@ -15,6 +15,7 @@
 // batch.  The faster kernels cover the common shapes; this one covers the rest
 // and the float32 path.
 #include "zi_common.h"
+#include "zi_api.h"
 
 #define ATTN_MAX_D 512
 #define ATTN_ACC (ATTN_MAX_D / ZI_WAVE)

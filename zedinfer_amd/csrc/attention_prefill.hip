@@ -33,6 +33,7 @@
 // padded with zeros for the score product); page size a power of two from 8.
 // Other shapes are the plain kernel's.
 #include "zi_common.h"
+#include "zi_api.h"
 #include "zi_paging.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8_t;

@@ -32,6 +32,8 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-unknown-warning-option",
 ]
+# The library matrix product (gemm_lt.hip) is hipBLASLt's.
+LINK_LIBS = ["-lhipblaslt"]
 
 
 def sources() -> List[str]:
@@ -44,7 +46,7 @@ def headers() -> List[str]:
 
 def source_hash() -> str:
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + LINK_LIBS).encode())
     for f in sources() + headers():
         h.update(f.encode())
         with open(os.path.join(CSRC, f), "rb") as fh:
@@ -148,7 +150,7 @@ def build(verbose: bool = True, force: bool = True, jobs: Optional[int] = None) 
         with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
             objs = list(ex.map(compile_one, srcs))
         tmp_lib = os.path.join(obj_dir, LIB_NAME + f".{os.getpid()}")
-        cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp_lib] + objs
+        cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp_lib] + objs + LINK_LIBS
         r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
         if r.returncode != 0:
             raise RuntimeError(f"linking the kernel library failed:\n{r.stderr[-4000:]}")

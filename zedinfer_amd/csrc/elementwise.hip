@@ -1,6 +1,7 @@
 // Row gathers and elementwise ops: embedding lookup, row gather, residual add,
 // SwiGLU.  Arithmetic is done in float32 and rounded once on store.
 #include "zi_common.h"
+#include "zi_api.h"
 
 // out[i,:] = table[ids[i],:]   (reference: src/backend/ops/embedding/cpu/embedding_cpu.cpp:10-23).
 // An id outside [0, V) writes NaN into the row so that the fault shows.

@@ -8,6 +8,7 @@
 // any layer whose checkpoint tensor is stored in 32-bit.
 // (reference: src/backend/ops/linear/cpu/linear_cpu.cpp:26-85.)
 #include "zi_common.h"
+#include "zi_api.h"
 
 #define GT 64   // output tile edge
 #define GK 16   // k step

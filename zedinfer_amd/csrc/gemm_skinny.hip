@@ -17,6 +17,7 @@
 // other one's cut was balanced; since then it was slower at every size from one row on (1.5B gate/up at 8 rows
 // 12.9 against 11.7 us, 32B gate/up 111 against 95 us) and is gone.
 #include "zi_common.h"
+#include "zi_api.h"
 
 #define SK_MODE_PLAIN 0
 #define SK_MODE_PARTIAL 1

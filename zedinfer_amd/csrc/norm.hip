@@ -5,6 +5,7 @@
 // Sum of squares, rstd and the products are float32; one workgroup per row, so
 // a row's result does not depend on which other rows are in the batch.
 #include "zi_common.h"
+#include "zi_api.h"
 
 #define NORM_THREADS 256
 

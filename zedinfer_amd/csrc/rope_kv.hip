@@ -15,6 +15,7 @@
 // the P.V product.  Token slot s lives in page s / page_size at offset s % page_size.
 // A negative slot skips the write.
 #include "zi_common.h"
+#include "zi_api.h"
 #include "zi_paging.h"
 
 template <typename T>

@@ -12,6 +12,7 @@
 // the probability's bit pattern (non-negative floats order like their bits);
 // equal probabilities are ordered by rising token id.  One workgroup per row.
 #include "zi_common.h"
+#include "zi_api.h"
 #include "zi_no_alloc.h"
 #include <mutex>
 

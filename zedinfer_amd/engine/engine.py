@@ -21,6 +21,7 @@ from ..models import DecoderModel, expected_weights
 from ..parts import Runtime
 from ..sampling.sampler import default_sampling
 from ..weights import load_weights, random_weights
+from ..ops.tape import Recording
 from .batch import DecodeImage, StagingRing, StepEntry, build_device_batch
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
@@ -70,6 +71,12 @@ class Engine:
         # (entries, wanted rows, block-table widths, attention launch size).
         self.use_graphs = (self.device.type == "cuda" and self.model.graph_safe()
                            and os.environ.get("ZEDINFER_DISABLE_GRAPHS", "0") in ("", "0"))
+        # Before a shape has a graph (or when graphs are off, or for prompt portions too long to be worth one) its
+        # second and later steps run from a tape of the first's library calls: the host then spends what the
+        # launches cost, not the interpreter's time for every part (about 5 ms for 28 layers).
+        self.use_tapes = (self.device.type == "cuda" and self.model.tape_safe()
+                          and os.environ.get("ZEDINFER_DISABLE_TAPES", "0") in ("", "0"))
+        self.tape_runs = 0
         self.graph_max_entries = 256     # measured: 128 requests decode 77% faster as a graph, 256 37%
         self.graph_limit = 48
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
@@ -196,9 +203,9 @@ class Engine:
             for seq, growth in reversed(grown):      # nothing of a step that cannot run stays
                 self.cache.undo(seq, growth)
             raise
-        if self.use_graphs and 0 < len(entries) <= self.graph_max_entries and single:
+        if (self.use_graphs or self.use_tapes) and 0 < len(entries) <= self.graph_max_entries and single:
             logits = self._graph_step(entries, token_source)
-        elif self.use_graphs and token_source is None and self._one_portion(entries):
+        elif (self.use_graphs or self.use_tapes) and token_source is None and self._one_portion(entries):
             logits = self._prompt_graph_step(entries)
         else:
             batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging,
@@ -246,6 +253,8 @@ class Engine:
             dg.graph.replay()
             self.graph_replays += 1
             return dg.logits
+        if not self.use_graphs:
+            return self._run_or_replay(dg, batch)
         logits = self.model.run(batch, self.memories)      # allocates every workspace; its result is this step's
         if dg.warm:
             # the second step of this kind: capture (nothing runs), to be replayed from the third on
@@ -259,6 +268,25 @@ class Engine:
         dg.warm = True
         return logits
 
+    def _run_or_replay(self, dg: "_DecodeGraph", batch) -> Optional[torch.Tensor]:
+        """A step of a shape that has no graph: from the shape's tape when it has one, else part by part, and
+        then (once the workspaces have their sizes: not at the shape's first step, which may still allocate)
+        recorded as its tape.  The batch lives in the shape's own buffer, as for a graph."""
+        if dg.tape is not None:
+            dg.tape.run()
+            self.tape_runs += 1
+            return dg.logits
+        if not self.use_tapes or dg.no_tape or not dg.ran:
+            dg.ran = True
+            return self.model.run(batch, self.memories)
+        with Recording(self.device) as rec:
+            logits = self.model.run(batch, self.memories)
+        if rec.allocations:
+            dg.no_tape = True       # memory taken during the step would be another's at the next
+        else:
+            dg.tape, dg.logits = rec.tape(), logits
+        return logits
+
 
     def _drop_oldest(self, graphs: Dict[tuple, "_DecodeGraph"]) -> None:
         """Forget the first graph of the dictionary.  One that was recorded may still be running, and with
@@ -269,6 +297,7 @@ class Engine:
 
     # ---- one portion of one prompt as a graph -------------------------------------------
     PROMPT_GRAPH_STEP = 64
+    TAPE_MAX_TOKENS = 8192      # padded tokens of the portions of a step that is still run from a tape
 
     def _one_portion(self, entries: Sequence[StepEntry]) -> bool:
         """Portions of prompts (entries of several tokens) of a size worth a graph together, beside any
@@ -283,7 +312,8 @@ class Engine:
                 return False
             if n > 1:
                 total += -(-n // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
-        return 0 < total <= self.prompt_graph_max_tokens and len(entries) <= self.graph_max_entries
+        most = max(self.prompt_graph_max_tokens if self.use_graphs else 0, self.TAPE_MAX_TOKENS if self.use_tapes else 0)
+        return 0 < total <= most and len(entries) <= self.graph_max_entries
 
     def _prompt_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """A step of portions of prompts (entries of several tokens) beside single decoded tokens,
@@ -292,7 +322,8 @@ class Engine:
         ones replay."""
         step = self.PROMPT_GRAPH_STEP
         portions = [e for e in entries if len(e.tokens) > 1]
-        padded = sum(-(-len(e.tokens) // step) * step for e in portions)      # tokens of all portions, padded
+        sizes = tuple(sorted(-(-len(e.tokens) // step) * step for e in portions))     # tokens of the portions, padded
+        padded = sum(sizes)
         wanted = sum(len(e.want) for e in entries)
         E, R, more_entries = len(entries), wanted, 0
         if E > 1:
@@ -306,7 +337,9 @@ class Engine:
         long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions), 2048)
         short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
         singles = len(entries) - len(portions) + more_entries
-        key = (E, singles, padded, R, widths, long_bucket, short_bucket)
+        # everything the launches' sizes depend on: the portions' sizes one by one (the planners cut each into
+        # tiles by rules of their own), not their sum
+        key = (E, singles, sizes, R, widths, long_bucket, short_bucket)
         dg = self._prompt_graphs.pop(key, None)
         if dg is not None:
             self._prompt_graphs[key] = dg       # used last: the last to go
@@ -323,11 +356,12 @@ class Engine:
             dg.graph.replay()
             self.prompt_graph_replays += 1
             return dg.logits[:wanted] if wanted else None
-        logits = self.model.run(batch, self.memories)
+        logits = self._run_or_replay(dg, batch)
         dg.seen += 1
-        # Recording costs about as much as ten steps: a portion alone is recorded the second time its shape
-        # comes, a shape with decoded tokens beside the portion only the third time.
-        if dg.seen >= (2 if len(entries) == 1 else 3):
+        # Capturing a graph costs about as much as ten steps: a portion alone is captured the second time its
+        # shape comes, a shape with decoded tokens beside the portion only the third time; portions too long
+        # to be worth a graph (the GPU needs longer for them than the host) stay with their tape.
+        if self.use_graphs and padded <= self.prompt_graph_max_tokens and dg.seen >= (2 if len(entries) == 1 else 3):
             torch.cuda.synchronize(self.device)
             first = logits.clone() if logits is not None else None
             g = torch.cuda.CUDAGraph()
@@ -345,6 +379,9 @@ class _DecodeGraph:
         self.logits: Optional[torch.Tensor] = None
         self.warm = False
         self.seen = 0
+        self.ran = False                                # a step of the shape has run part by part
+        self.tape = None                                # the library calls of one step of the shape
+        self.no_tape = False                            # a step of the shape cannot be recorded
         self.image: Optional[DecodeImage] = None
 
 

@@ -156,6 +156,10 @@ class InferenceEngine:
     def __init__(self, engine: Engine):
         self.engine = engine
         self._loop = ServingLoop(engine, engine.fc.eos_token_ids)
+        # The size of a full portion of a prompt is the one many-rows step that recurs: its products' algorithms
+        # (and other choices of the parts) are measured now, once (ZEDINFER_WARM_UP=0: the defaults).
+        if os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and engine.device.type == "cuda":
+            engine.warm_up([engine.sched.max_prefill_tokens])
         # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
         # taken out of the garbage collector's passes, a full collection in the middle of serving costs
         # little (measured: one of 50 ms among decode steps of 6.5 ms without this).

@@ -126,6 +126,10 @@ class DecoderModel:
         """Whether a step's launches can be captured and replayed: every part says so."""
         return all(getattr(p, "graph_safe", False) for p in self.parts)
 
+    def tape_safe(self) -> bool:
+        """Whether a step's device work is calls into the kernel library alone: every part says so."""
+        return all(getattr(p, "graph_safe", False) and getattr(p, "tape_safe", False) for p in self.parts)
+
     # ---- one step -------------------------------------------------------------
     def run(self, batch, memories: Sequence[LayerMemory]) -> Optional[torch.Tensor]:
         """Run the tokens of ``batch`` through the schedule; float32 logits [wanted, vocab]

@@ -7,7 +7,7 @@ add, argmax, embedding, linear, rms_norm, rope, swiglu).
 """
 from .functional import (add, add_rms_norm, argmax, attention, attention_decode, attention_decode_supported, attention_decode_workspace, attention_decode_fused, attention_decode_fused_supported, attention_decode_project, attention_decode_project_splits, attention_decode_project_supported, rope_table, attention_prefill, attention_prefill_variant, attention_prefill_workspace, attention_prefill_tile,
                          attention_prefill_supported, embedding, gather_rows, has_cuda, has_gpu,
-                         linear, linear_splits, linear_sums, linear_transposed, linear_sums_supported, linear_swiglu,
+                         linear, linear_tune, linear_choose, linear_splits, linear_sums, linear_transposed, linear_sums_supported, linear_swiglu,
                          linear_swiglu_supported, reduce_sums, rms_norm, rope, rope_kv_store, rope_kv_store_sums,
                          rope_inv_freq, sample, swiglu, swiglu_t,
                          device_synchronize)
@@ -16,7 +16,7 @@ from ._lib import KernelLibraryError, library_path, load
 __all__ = [
     "add", "add_rms_norm", "argmax", "attention", "attention_decode", "attention_decode_supported", "attention_decode_workspace", "attention_decode_fused", "attention_decode_fused_supported", "attention_decode_project", "attention_decode_project_splits", "attention_decode_project_supported", "rope_table", "attention_prefill", "attention_prefill_variant", "attention_prefill_workspace", "attention_prefill_tile",
     "attention_prefill_supported", "embedding", "gather_rows", "has_cuda", "has_gpu", "linear",
-    "linear_splits", "linear_sums", "linear_transposed", "linear_sums_supported", "linear_swiglu", "linear_swiglu_supported", "reduce_sums",
+    "linear_tune", "linear_choose", "linear_splits", "linear_sums", "linear_transposed", "linear_sums_supported", "linear_swiglu", "linear_swiglu_supported", "reduce_sums",
     "rms_norm", "rope", "rope_kv_store", "rope_kv_store_sums", "rope_inv_freq", "sample", "swiglu", "swiglu_t", "device_synchronize",
     "KernelLibraryError", "library_path", "load",
 ]

@@ -5,6 +5,7 @@ There is no fallback: when the library cannot be loaded, every op raises.
 from __future__ import annotations
 
 import ctypes
+import struct
 import threading
 from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p
 from typing import Optional
@@ -46,11 +47,17 @@ _PROTOTYPES = {
     "zi_gemm_generic": [P, I, P, I, P, I, P, I, I, I, I, L, L, L, P],
     "zi_gemm_skinny": [P, I, I, P, P, P, I, I, I, L, L, L, P, L, P],
     "zi_gemm_skinny_splits": [I, I, I],
+    "zi_gemm_lt": [P, I, P, P, P, I, L, L, L, L, L, L, P, L, P],
+    "zi_gemm_lt_tune": [P, I, P, P, P, I, L, L, L, L, L, L, P, L, I, I, P, P, P, P],
+    "zi_gemm_lt_choose": [I, I, I, L, L, L, L, L, L, L, I],
     "zi_reduce_splits": [P, I, P, P, I, I, L, I, P],
     "zi_rope_kv_store_split": [P, I, L, P, I, L, L, P, I, I, P, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_gemm_skinny_supported": [I, I, I, L, L],
     "zi_argmax": [P, P, P, I, I, I, L, P, L, P],
     "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],
+    "zi_tape_record": [P, c_char_p, P, I],
+    "zi_tape_run": [P, P],
+    "zi_tape_length": [P],
 }
 
 
@@ -92,8 +99,16 @@ def load() -> ctypes.CDLL:
         lib.zi_attention_prefill_workspace.restype = c_int64
         lib.zi_argmax_workspace.argtypes = [I, I]
         lib.zi_argmax_workspace.restype = c_int64
+        lib.zi_tape_new.argtypes = []
+        lib.zi_tape_new.restype = c_void_p
+        lib.zi_tape_free.argtypes = [P]
+        lib.zi_tape_free.restype = None
         _lib, _lib_path = lib, path
         return lib
+
+
+# The calls made while a tape records (``ops.tape.Recording``): a list of (name, arguments), or None.
+_recorded: Optional[list] = None
 
 
 def call(name: str, *args) -> None:
@@ -101,3 +116,25 @@ def call(name: str, *args) -> None:
     rc = getattr(lib, name)(*args)
     if rc != 0:
         raise KernelLibraryError(lib.zi_last_error().decode("utf-8", "replace"))
+    if _recorded is not None:
+        _recorded.append((name, args))
+
+
+def argument_words(name: str, args) -> list:
+    """The arguments of a call as the 64-bit words a tape holds: integers and pointers by value, floats as
+    the bits of a double."""
+    kinds = _PROTOTYPES[name]
+    if len(kinds) != len(args):
+        raise KernelLibraryError(f"{name} takes {len(kinds)} arguments, {len(args)} were given")
+    words = []
+    for kind, a in zip(kinds, args):
+        if kind is F:
+            words.append(struct.unpack("<q", struct.pack("<d", float(a.value if isinstance(a, c_float) else a)))[0])
+        elif kind is P:
+            v = a.value if isinstance(a, c_void_p) else a
+            if v is not None and not isinstance(v, int):
+                raise KernelLibraryError(f"{name}: an argument of a kind a tape cannot hold ({type(a).__name__})")
+            words.append(int(v or 0))
+        else:
+            words.append(int(a.value if hasattr(a, "value") else a))
+    return words

@@ -1,7 +1,8 @@
 """Checked launches of the HIP kernels on torch tensors."""
 from __future__ import annotations
 
-from ctypes import c_void_p
+import ctypes
+from ctypes import c_float, c_int, c_void_p
 from typing import Optional, Tuple
 
 import numpy as np
@@ -677,10 +678,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
         return out
     bf = torch.bfloat16
     all_bf = x.dtype == bf and weight.dtype == bf and (bias is None or bias.dtype == bf)
-    if all_bf and out.dtype == torch.float32 and M > SKINNY_MAX_ROWS and bias is None and out.is_contiguous():
+    if all_bf and out.dtype == torch.float32 and M > SKINNY_MAX_ROWS and bias is None and _library_ok(x, weight, out):
         # float32 output for many rows (logits of a large decode batch or of every place of a prompt): the
         # library's product with float32 results, one pass over the weights instead of one per 64 rows
-        torch.mm(x, weight.t(), out_dtype=torch.float32, out=out)
+        _library_product(out, x, weight, None, False)
         return out
     if all_bf and (M <= FEW_ROWS or out.dtype == torch.float32) and _skinny_ok(x, weight, K, ldx, ldw):
         # few rows (decoding), or float32 output (logits): the hand-written matrix-core kernel
@@ -692,11 +693,8 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
             _lib.call("zi_gemm_skinny", _p(out[m0:m0 + m]), _code(out, "linear out"), 0, _p(x[m0:m0 + m]), _p(weight),
                       _p(bias), m, N, K, ldx, ldw, ldo, _p(ws), need, _stream())
         return out
-    if all_bf and out.dtype == bf and out.is_contiguous():
-        if bias is not None:
-            torch.addmm(bias, x, weight.t(), out=out)
-        else:
-            torch.mm(x, weight.t(), out=out)
+    if all_bf and out.dtype == bf and _library_ok(x, weight, out):
+        _library_product(out, x, weight, bias, False)
         return out
     _lib.call("zi_gemm_generic", _p(out), _code(out, "linear out"), _p(x), _code(x, "linear x"), _p(weight),
               _code(weight, "linear weight"), _p(bias), _code(bias, "linear bias") if bias is not None else F32,
@@ -717,8 +715,62 @@ def linear_transposed(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch
         out = torch.empty((N, M), dtype=torch.bfloat16, device=x.device)
     if tuple(out.shape) != (N, M) or out.dtype != torch.bfloat16 or not out.is_contiguous():
         raise ValueError(f"linear_transposed: out must be a contiguous bfloat16 [{N}, {M}] tensor")
-    torch.mm(weight, x.t(), out=out)
+    _library_product(out, x, weight, None, True)
     return out
+
+
+LIBRARY_WORKSPACE_BYTES = 64 << 20     # what an algorithm of the library's product may use beside its operands
+_LIBRARY_WORKSPACES = {}
+
+
+def _library_ok(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> bool:
+    """Rows one element apart in memory and 16-byte aligned: what the library's product is given."""
+    return all(t.stride(1) == 1 and t.data_ptr() % 16 == 0 and t.stride(0) % 8 == 0 for t in (x, weight)) \
+        and out.stride(1) == 1 and out.data_ptr() % 16 == 0
+
+
+def _library_args(out, x, weight, bias, transposed):
+    ws = _LIBRARY_WORKSPACES.get(x.device)
+    if ws is None:
+        ws = _LIBRARY_WORKSPACES[x.device] = torch.empty((LIBRARY_WORKSPACE_BYTES,), dtype=torch.uint8, device=x.device)
+    return (_p(out), _code(out, "linear out"), _p(x), _p(weight), _p(bias), int(transposed), x.shape[0], weight.shape[0],
+            x.shape[1], x.stride(0), weight.stride(0), out.stride(0), _p(ws), LIBRARY_WORKSPACE_BYTES)
+
+
+def _library_product(out, x, weight, bias, transposed) -> None:
+    _lib.call("zi_gemm_lt", *_library_args(out, x, weight, bias, transposed), _stream())
+
+
+def linear_tune(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, transposed: bool = False,
+                out_dtype: Optional[torch.dtype] = None, candidates: int = 16, rounds: int = 5):
+    """Let the library time its proposals for the product ``linear`` (``linear_transposed``) makes of these operands
+    and keep the fastest for every later call of the shape; returns (chosen, proposed, microseconds), or None when
+    the product is not the library's (few rows, float32 operands).  Waits for the device."""
+    bf = torch.bfloat16
+    M, N = x.shape[0], weight.shape[0]
+    out_dtype = out_dtype or bf
+    if x.dtype != bf or weight.dtype != bf or (bias is not None and bias.dtype != bf):
+        return None
+    if M <= (SKINNY_MAX_ROWS if out_dtype == torch.float32 else FEW_ROWS) or (out_dtype == torch.float32 and bias is not None):
+        return None
+    out = torch.empty((N, M) if transposed else (M, N), dtype=out_dtype, device=x.device)
+    if not _library_ok(x, weight, out):
+        return None
+    chosen, proposed, us = c_int(0), c_int(0), c_float(0.0)
+    _lib.call("zi_gemm_lt_tune", *_library_args(out, x, weight, bias, transposed), int(candidates), int(rounds),
+              ctypes.byref(chosen), ctypes.byref(proposed), ctypes.byref(us), _stream())
+    return chosen.value, proposed.value, us.value
+
+
+def linear_choose(x: torch.Tensor, weight: torch.Tensor, which: int, bias: Optional[torch.Tensor] = None,
+                  transposed: bool = False, out_dtype: Optional[torch.dtype] = None) -> None:
+    """Fix the library's algorithm for the product of these operands to proposal ``which`` (what ``linear_tune``
+    returned in an earlier run) without timing anything."""
+    _gpu("linear_choose", x, weight, bias)
+    M, N, K = x.shape[0], weight.shape[0], x.shape[1]
+    code = F32 if out_dtype == torch.float32 else BF16
+    _lib.call("zi_gemm_lt_choose", code, int(bias is not None), int(transposed), M, N, K, x.stride(0), weight.stride(0),
+              M if transposed else N, LIBRARY_WORKSPACE_BYTES, int(which))
 
 
 def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:

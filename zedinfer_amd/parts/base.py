@@ -7,6 +7,7 @@ runtime) and never learns which model it sits in.
 """
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass, field
 from typing import Callable, Dict, Optional, Tuple
 
@@ -38,6 +39,25 @@ class Runtime:
         # the deciding part chooses.  They are made outside of steps (``Part.tune``, ``Engine.warm_up``)
         # or given by the caller, never while a step runs: a run with the same choices gives the same bits.
         self.choices: Dict[tuple, object] = {}
+
+    def tune_linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                    transposed: bool = False, out_dtype: Optional[torch.dtype] = None) -> None:
+        """Outside of any step: let the library choose, by timing its proposals, the algorithm of the product
+        ``ops.linear`` (``ops.linear_transposed``) makes of operands of these shapes, and record the choice in
+        ``choices``; a choice already recorded there (an earlier run's) is put in force instead.  Nothing happens
+        for products that are not the library's (few rows, float32) or with ZEDINFER_TUNE_LIBRARY=0."""
+        if os.environ.get("ZEDINFER_TUNE_LIBRARY", "1") == "0" or x.device.type != "cuda":
+            return
+        from .. import ops
+        key = ("library_product", int(x.shape[0]), int(weight.shape[0]), int(x.shape[1]), bias is not None,
+               bool(transposed), "float32" if out_dtype == torch.float32 else "bfloat16")
+        known = self.choices.get(key)
+        if known is not None:
+            ops.linear_choose(x, weight, int(known), bias, transposed, out_dtype)
+            return
+        found = ops.linear_tune(x, weight, bias, transposed, out_dtype)
+        if found is not None:
+            self.choices[key] = found[0]
 
     def buffer(self, name: str, shape: Tuple[int, ...], dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         dtype = dtype or self.dtype
@@ -149,6 +169,11 @@ class Part:
     # calls) may set this.  When every part of a model does, steps of decoded tokens are captured as
     # graphs and replayed; a part that leaves the default keeps the whole model on eager launches.
     graph_safe: bool = False
+    # A graph-safe part all of whose device work is calls into the kernel library (``ops``) with outputs in
+    # buffers of the runtime, none through torch operators, may set this too.  When every part of a model
+    # does, the library calls of a step are recorded the first time a shape comes and made again from native
+    # code when it recurs, before (or without) a graph.
+    tape_safe: bool = False
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:

@@ -15,6 +15,7 @@ class PreNormBlock(Block):
     float32 and every add into it happens inside the norm that follows it."""
 
     graph_safe = True
+    tape_safe = True
 
     norm_names = ("input", "post_mixer")
 

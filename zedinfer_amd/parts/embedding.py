@@ -17,6 +17,7 @@ class TokenEmbedding(Part):
     (reference: src/frontend/models/transformer_forward.cpp:54-60).  params: vocab_size, hidden_size."""
 
     graph_safe = True
+    tape_safe = True
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -40,6 +41,7 @@ class LinearHead(Part):
     params: vocab_size, hidden_size, tied_to (tensor name or None)."""
 
     graph_safe = True
+    tape_safe = True
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:

@@ -38,6 +38,7 @@ class SwiGLU(FeedForward):
     params: hidden_size, intermediate_size."""
 
     graph_safe = True
+    tape_safe = True
     # For many rows the gate/up product is the library's, and at some sizes it makes the transposed
     # result, W . x^T, faster than x . W^T (measured at the 1.5B sizes: 100 against 119 us at 2,048 rows,
     # 31 against 37 at 512, 73 against 67 at 1,024).  The transposed result goes through the activation
@@ -83,14 +84,21 @@ class SwiGLU(FeedForward):
         return self._gate_up_straight(x, act)
 
     def tune(self, num_tokens: int) -> None:
-        """Decide the orientation of the gate/up product for steps of ``num_tokens`` rows: three runs each
-        of product plus activation; the transposed one must win by 5 %."""
+        """For steps of ``num_tokens`` rows: the library's algorithms for the gate/up and down products, then the
+        orientation of the gate/up product: three runs each of product plus activation; the transposed one must
+        win by 5 %."""
         n, key = int(num_tokens), self._choice_key(num_tokens)
+        x = self.rt.buffer("norm_out", (n, self.hidden))
+        act = self.rt.buffer("ffn_act", (n, self.inter))
+        # first the library's algorithm for each product, then the way round with those
+        if self.gate_up is not None:
+            self.rt.tune_linear(x, self.gate_up)
+            if self._can_transpose(n):
+                self.rt.tune_linear(x, self.gate_up, transposed=True)
+        self.rt.tune_linear(act, self.down)
         forced = os.environ.get("ZEDINFER_GATE_UP_TRANSPOSED", "")
         if key in self.rt.choices or not self._can_transpose(n) or forced in ("0", "1"):
             return
-        x = self.rt.buffer("norm_out", (n, self.hidden))
-        act = self.rt.buffer("ffn_act", (n, self.inter))
 
         def clock(fn):
             fn(x, act)

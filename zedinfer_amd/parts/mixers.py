@@ -99,6 +99,7 @@ class Attention(Mixer):
     scale (default 1/sqrt(head_dim)), position (a PartSpec of a position encoding)."""
 
     graph_safe = True
+    tape_safe = True
     padding_safe = True      # padding has no place in the cache, and causal attention lets no real token see it
     # Every workgroup of the fused kernel adds and rotates its token's query again (one per chunk of
     # 256 keys), which costs more than the separate rotary kernel once many tokens decode together:
@@ -219,6 +220,17 @@ class Attention(Mixer):
         att = self.rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
         return self.project(att, n)
+
+    def tune(self, num_tokens: int) -> None:
+        """The library's algorithms for the projections of a step of ``num_tokens`` rows."""
+        n = int(num_tokens)
+        x = self.rt.buffer("norm_out", (n, self.hidden))
+        if self.qkv is not None:
+            self.rt.tune_linear(x, self.qkv, self.bias)
+        else:
+            for m, b in zip(self.mats, self.biases or (None, None, None)):
+                self.rt.tune_linear(x, m, b)
+        self.rt.tune_linear(self.rt.buffer("attn_out", (n, self.qd)), self.o)
 
     def project(self, att: torch.Tensor, n: int) -> torch.Tensor:
         if ops.linear_sums_supported(att, self.o):

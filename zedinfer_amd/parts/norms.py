@@ -18,6 +18,7 @@ class RMSNorm(Norm):
     params: dim, eps, add_one (default False)."""
 
     graph_safe = True
+    tape_safe = True
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:

@@ -19,6 +19,7 @@ class RopeNeox(PositionEncoding):
     params: head_dim, theta, rotary_dim (default head_dim)."""
 
     graph_safe = True
+    tape_safe = True
 
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         super().__init__(spec, weights, rt)
@@ -57,6 +58,7 @@ class NoPosition(PositionEncoding):
     """No encoding: keys and values are stored as they are."""
 
     graph_safe = True
+    tape_safe = True
 
     def step_table(self, batch):
         return "none"
