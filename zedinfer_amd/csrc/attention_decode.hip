@@ -82,7 +82,9 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     __shared__ uint4 sk[DK][4];        // FUSED: the token's own key, in pieces (k-step, j)
     __shared__ uint16_t sv[D];         // and its value
 
-    const int x = blockIdx.x, kvh = blockIdx.y, chunk = blockIdx.z;
+    // a token's chunks are neighbours in the launch order: those past its count leave at once, beside chunks
+    // that stream, and do not gather at the launch's end
+    const int x = blockIdx.z, kvh = blockIdx.y, chunk = blockIdx.x;
     const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
     const int r = lane & 15, j = lane >> 4;
     const int t = tok_index ? tok_index[x] : x;
@@ -658,7 +660,8 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
                "%s: workspace of %lld floats is too small or not aligned", who, (long long)workspace_floats);
     float* po = workspace;
     float* pml = workspace ? workspace + (int64_t)n_idx * nh * DEC_MAXC * d : nullptr;
-    const dim3 grid(n_idx, nkv, max_chunks);
+    ZI_REQUIRE(n_idx <= 65535, "%s: at most 65535 tokens a launch, got %d", who, n_idx);
+    const dim3 grid(max_chunks, nkv, n_idx);
     const int G = nh / nkv;
     const DecProjection none = {};
 #define ZI_DEC(DD)                                                                                                   \

@@ -231,7 +231,7 @@ class Engine:
                        for g in range(len(self.cache.groups)))
         # a bound, the same for many steps, of the tokens any sequence holds after this step: the
         # mixers' planners size their launches by it
-        bound = _pow2_at_least(max(e.seq.length for e in entries) + 1, 256)
+        bound = _bucket_at_least(max(e.seq.length for e in entries) + 1, 256)
         key = (E, R, widths, bound)
         dg = self._graphs.pop(key, None)
         if dg is not None:
@@ -335,7 +335,7 @@ class Engine:
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
         long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions), 2048)
-        short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
+        short_bucket = _bucket_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
         singles = len(entries) - len(portions) + more_entries
         # everything the launches' sizes depend on: the portions' sizes one by one (the planners cut each into
         # tiles by rules of their own), not their sum
@@ -383,6 +383,17 @@ class _DecodeGraph:
         self.tape = None                                # the library calls of one step of the shape
         self.no_tape = False                            # a step of the shape cannot be recorded
         self.image: Optional[DecodeImage] = None
+
+
+def _bucket_at_least(n: int, floor: int = 1) -> int:
+    """A bound of the tokens a decoding sequence holds that many steps share: a power of two up to 1,024, then
+    the next multiple of 512 (of 2,048 beyond 8,192).  The attention launch is sized by it, and workgroups
+    for keys that no sequence has yet cost time: with powers of two alone a batch just past 2,048 tokens
+    launched twice the workgroups it needed."""
+    if n <= 1024:
+        return _pow2_at_least(n, floor)
+    step = 512 if n <= 8192 else 2048
+    return max(-(-n // step) * step, floor)
 
 
 def _pow2_at_least(n: int, floor: int = 1) -> int:
