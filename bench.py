@@ -15,6 +15,7 @@ uniform random in [100, vocab-100] as in the reference's own benchmark
 (reference: src/zedinfer/profiler.cpp:79-84, docs/perf/benchmark_v0.1.0.md:3-11).
 """
 import argparse
+import gc
 import json
 import os
 import random
@@ -289,8 +290,14 @@ def main():
         out["prefill"] = {"value": round(PF / pms * 1000.0, 1), "tokens": PF, "ms": round(pms, 3),
                           "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}
         points = {}
+        per_token = 2 * args.layers * cfg.num_key_value_heads * cfg.head_dim * el      # cache bytes of one token
         for b, st in ((1, min(args.steps, 64)), (64, min(args.steps, 32)), (256, min(args.steps, 16))):
+            gc.collect()
             torch.cuda.empty_cache()
+            tokens = args.prompt_len + args.warmup + args.steps + 2 * b + 64
+            if b * tokens * per_token > 0.9 * torch.cuda.mem_get_info()[0]:
+                points[f"decode_b{b}"] = None       # the requests' keys and values do not fit beside the weights
+                continue
             t, _, _ = measure_decode(factory(b), b, st, min(args.warmup, 8), V, args.prompt_len)
             points[f"decode_b{b}"] = round(t, 2)
         # the reference's own short run (its bench -p 128): a prompt step of this size replays as a graph
