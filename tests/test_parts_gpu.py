@@ -97,12 +97,14 @@ def test_swiglu_part(dtype, n):
 
 
 @pytest.mark.parametrize("n,H,I", [(256, 72, 200), (136, 96, 72), (1024, 128, 344)])
-def test_swiglu_part_both_orientations_of_the_product(n, H, I):
+def test_swiglu_part_both_orientations_of_the_product(n, H, I, monkeypatch):
     """Many rows in bfloat16: the library may make the gate/up product faster transposed.  Both ways,
     chosen here through the runtime's recorded choices, give the plain result (and nearly each other's);
     without a choice the forward pass takes the straight one and measures nothing; ``tune`` measures
-    outside of a step, records its decision, and the forward pass then follows it."""
+    outside of a step, records its decision, and the forward pass then follows it.  (The library keeps its
+    first algorithm for every product here, so that bits can be compared before and after ``tune``.)"""
     from zedinfer_amd.parts import FEED_FORWARDS
+    monkeypatch.setenv("ZEDINFER_TUNE_LIBRARY", "0")
     dtype = torch.bfloat16
     w = {"gate": rnd(I, H, seed=1, scale=0.2), "up": rnd(I, H, seed=2, scale=0.2), "down": rnd(H, I, seed=3, scale=0.2)}
     x = rnd(n, H, seed=4)
@@ -129,6 +131,49 @@ def test_swiglu_part_both_orientations_of_the_product(n, H, I):
     measured = as_rows(part.forward(x.to(dtype).cuda())).cpu()
     assert torch.equal(measured, got[rt.choices[key]])
     torch.testing.assert_close(got[True], got[False], atol=2e-2 * float(ref.abs().max()), rtol=0)
+
+
+def test_library_algorithms_are_chosen_at_warm_up_and_can_be_repeated(tmp_path, monkeypatch):
+    """``Engine.warm_up`` lets the parts time the library's proposals for their many-rows products and records
+    what was taken; a second engine given those choices puts them in force without timing; with
+    ZEDINFER_TUNE_LIBRARY=0 nothing is timed or recorded.  Steps of that many rows agree with the plain
+    implementation whatever was chosen."""
+    import tiny_configs
+    import traces
+    from plain import qwen2_plain as plain_model
+    from tolerances import bf16_within
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    from zedinfer_amd.ops import _lib
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "B", dtype=torch.bfloat16, std=tiny_configs.SHARP_STD)
+    cfg, w = plain_model.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["B"]
+    sched = SchedulerConfig(num_kv_blocks=64, kv_block_size=ps, max_batch_requests=4)
+    calls = []
+    real = _lib.call
+    monkeypatch.setattr(_lib, "call", lambda name, *a: (calls.append(name), real(name, *a))[1])
+    first = Engine.from_folder(folder, "bfloat16", sched)
+    choices = first.warm_up([192])
+    products = {k: v for k, v in choices.items() if k[0] == "library_product"}
+    assert len(products) >= 4 and all(k[1] == 192 and isinstance(v, int) for k, v in products.items()), choices
+    assert calls.count("zi_gemm_lt_tune") == len(products)      # a shape is timed once; later layers take the record
+    calls.clear()
+    second = Engine.from_folder(folder, "bfloat16", sched)
+    assert second.warm_up([192], choices=choices) == choices
+    assert calls.count("zi_gemm_lt_choose") >= len(products) and "zi_gemm_lt_tune" not in calls
+    toks = traces.random_tokens(cfg["vocab_size"], 192, seed=3)
+    ref = plain_model.forward(cfg, w, toks)
+    for e in (first, second):
+        seq = e.open("r")
+        got = e.step([StepEntry(seq, toks, list(range(192)))]).cpu()
+        d = (got - ref).abs()
+        assert bf16_within(float(d.max()), float(d.mean()), float(ref.abs().max()))
+        e.close(seq)
+    monkeypatch.setenv("ZEDINFER_TUNE_LIBRARY", "0")
+    calls.clear()
+    third = Engine.from_folder(folder, "bfloat16", sched)
+    assert not [k for k in third.warm_up([320]) if k[0] == "library_product"]
+    assert "zi_gemm_lt_tune" not in calls
 
 
 # ---- embedding and head -----------------------------------------------------------------------
