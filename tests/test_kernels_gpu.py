@@ -323,16 +323,20 @@ def test_linear_by_the_library(ops, M, N, K):
         torch.testing.assert_close(ops.linear(xw[:, :K], w, b).float(), ref_b, **t)
         torch.testing.assert_close(ops.linear_transposed(x, w).float(), ref.t(), **t)
         assert calls == ["zi_gemm_lt"] * 6, calls
-        before = ops.linear(x, w, b)
+        # a shape that has been served keeps its algorithm (the library's first proposal); one that has not is timed
+        assert ops.linear_tune(x, w, bias=b, candidates=8, rounds=2)[0] == 0
+        x2 = rnd(M + 8, K, dtype=torch.bfloat16, seed=5)
+        ref2 = torch.nn.functional.linear(x2.double(), w.double()).float()
         for kwargs in (dict(bias=b), dict(transposed=True), dict(out_dtype=torch.float32)):
-            chosen, proposed, us = ops.linear_tune(x, w, candidates=8, rounds=2, **kwargs)
+            chosen, proposed, us = ops.linear_tune(x2, w, candidates=8, rounds=2, **kwargs)
             assert 0 <= chosen < proposed and us > 0
-            assert ops.linear_tune(x, w, candidates=8, rounds=2, **kwargs)[0] == chosen       # a shape is tuned once
-        torch.testing.assert_close(ops.linear(x, w, b).float(), ref_b, **t)
-        torch.testing.assert_close(ops.linear_transposed(x, w).float(), ref.t(), **t)
-        torch.testing.assert_close(ops.linear(x, w, out_dtype=torch.float32), ref, atol=1e-3, rtol=1e-3)
+            assert ops.linear_tune(x2, w, candidates=8, rounds=2, **kwargs)[0] == chosen       # a shape is timed once
+        torch.testing.assert_close(ops.linear(x2, w, b).float(), ref2 + b.float(), **t)
+        torch.testing.assert_close(ops.linear_transposed(x2, w).float(), ref2.t(), **t)
+        torch.testing.assert_close(ops.linear(x2, w, out_dtype=torch.float32), ref2, atol=1e-3, rtol=1e-3)
+        before = ops.linear(x, w, b)
         ops.linear_choose(x, w, 0, bias=b)
-        assert torch.equal(ops.linear(x, w, b), before)         # the library's first proposal again
+        assert torch.equal(ops.linear(x, w, b), before)
         with pytest.raises(ops.KernelLibraryError, match="proposal"):
             ops.linear_choose(x, w, 10 ** 6, bias=b)
     finally:

@@ -13,8 +13,9 @@
 //
 // One plan per shape (sizes, strides, output type, with or without bias, which way round) holds the
 // library's descriptors and the algorithm: the first of the library's own proposals until
-// zi_gemm_lt_tune has timed a number of them on the caller's operands and kept the fastest.  Plans live
-// until the process ends.  The calls are serialised by a mutex; the handle belongs to one device, the
+// zi_gemm_lt_tune has timed a number of them on the caller's operands and kept the fastest.  Plans, and
+// with them the choices, belong to the process (every engine in it gets the same bits for a shape) and live
+// until it ends.  The calls are serialised by a mutex; the handle belongs to one device, the
 // one that was current at the first call.
 #include "zi_common.h"
 #include "zi_api.h"
@@ -31,6 +32,7 @@ struct LtPlan {
     hipblasLtMatrixLayout_t a = nullptr, b = nullptr, c = nullptr;
     std::vector<hipblasLtMatmulHeuristicResult_t> proposals;
     int chosen = 0;          // index into proposals
+    int used = 0;            // a product of this shape has run outside of tuning
     int tuned = 0;
     float tuned_us = 0.f;
 };
@@ -154,13 +156,15 @@ extern "C" int zi_gemm_lt(void* out, int out_dt, const void* x, const void* weig
     if (lt_ready()) return 1;
     LtPlan* p = nullptr;
     if (lt_plan(LtKey{M, N, K, ldx, ldw, ldo, out_dt, bias != nullptr, transposed != 0}, (uint64_t)workspace_bytes, &p)) return 1;
+    p->used = 1;
     return lt_run(p, p->chosen, out, x, weight, bias, transposed, workspace, (uint64_t)workspace_bytes, stream);
 }
 
 // Time up to `candidates` of the library's proposals for this product on the given operands (`rounds` runs each
 // after one that does not count; `out` is overwritten) and keep the fastest for every later call of the shape
 // (the first proposal, unless another is at least 3 % faster).
-// Waits for the stream.  A shape is tuned once: later calls return what the first found.
+// Waits for the stream.  A shape is tuned once: later calls return what the first found, and a shape that
+// zi_gemm_lt has already served keeps the algorithm it was served with.
 // chosen / proposed / microseconds may be null.
 extern "C" int zi_gemm_lt_tune(void* out, int out_dt, const void* x, const void* weight, const void* bias, int transposed,
                                int64_t M, int64_t N, int64_t K, int64_t ldx, int64_t ldw, int64_t ldo, void* workspace,
@@ -172,6 +176,11 @@ extern "C" int zi_gemm_lt_tune(void* out, int out_dt, const void* x, const void*
     if (lt_ready()) return 1;
     LtPlan* p = nullptr;
     if (lt_plan(LtKey{M, N, K, ldx, ldw, ldo, out_dt, bias != nullptr, transposed != 0}, (uint64_t)workspace_bytes, &p)) return 1;
+    if (!p->tuned && p->used) {
+        // products of this shape have run with the first proposal: it stays, so that no engine of the process
+        // sees its rounding change in the middle of its life
+        p->tuned = 1;
+    }
     if (!p->tuned) {
         hipEvent_t e0 = nullptr, e1 = nullptr;
         if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return zi_fail("gemm_lt_tune: no events");
