@@ -350,18 +350,24 @@ def test_generation_config_of_the_model_folder_is_the_default(tiny, tmp_path, mo
 
 def test_command_lines(tiny, tmp_path):
     env = dict(os.environ, PYTHONPATH=ROOT)
-    run = lambda *a: subprocess.run([sys.executable, *a], capture_output=True, text=True, env=env, timeout=300)  # noqa: E731
+    run = lambda *a: subprocess.run([sys.executable, *a], capture_output=True, text=True, env=env, timeout=300,  # noqa: E731
+                                    cwd=str(tmp_path))
     ps = str(tiny_configs.PAGE_SIZES[tiny["name"]])
     prompt = traces.random_tokens(tiny["cfg"]["vocab_size"], 9, seed=3)
     r = run(os.path.join(ROOT, "bin", "ping"), tiny["folder"], "--dtype", "fp32", "--prompt-ids",
             ",".join(map(str, prompt)), "--max-new-tokens", "5", "--ignore-eos", "--num-kv-blocks", "32",
-            "--kv-block-size", ps)
+            "--kv-block-size", ps, "--log-file", str(tmp_path / "p.log"), "--log-level", "debug")
     assert r.returncode == 0, r.stderr
     want = plain.greedy_generate(tiny["cfg"], tiny["weights"], prompt, 5)
     assert "output_ids: " + ",".join(map(str, want)) in r.stdout and "finish_reason: length" in r.stdout
+    logged = (tmp_path / "p.log").read_text()
+    assert "Engine initialized" in logged and "Engine initialized" in r.stderr and "choices made at warm-up" in logged
     r = run(os.path.join(ROOT, "bin", "bench"), tiny["folder"], "-p", "32", "-d", "8", "-r", "1",
-            "--num-kv-blocks", "32", "--kv-block-size", ps)
+            "--num-kv-blocks", "32", "--kv-block-size", ps, "--no-log-to-console")
     assert r.returncode == 0 and "Prefill:" in r.stdout and "tok/s" in r.stdout, r.stderr
+    assert "Engine initialized" not in r.stderr and "Engine initialized" in (tmp_path / "logs" / "bench.log").read_text()
+    r = run(os.path.join(ROOT, "bin", "bench"), tiny["folder"], "--log-append", "--log-overwrite")
+    assert r.returncode == 1 and "mutually exclusive" in r.stderr
     r = run(os.path.join(ROOT, "bin", "batch_bench"), tiny["folder"], "-b", "3", "-p", "20", "-d", "6",
             "--num-kv-blocks", "64", "--kv-block-size", ps, "--random-weights", "--seed", "4")
     assert r.returncode == 0 and "Throughput" in r.stdout and "18 tokens generated" in r.stdout, r.stderr + r.stdout

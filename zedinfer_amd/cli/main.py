@@ -35,6 +35,21 @@ def _common(p: argparse.ArgumentParser) -> None:
     p.add_argument("--max-seq-len", type=int, default=16384)
 
 
+def _logging(p: argparse.ArgumentParser, name: str):
+    from .logging_options import add_logging_arguments
+    add_logging_arguments(p, f"logs/{name}.log")
+
+
+def _init_logging(args) -> bool:
+    from .logging_options import init_logger
+    try:
+        init_logger(args)
+        return True
+    except ValueError as e:
+        print(e, file=sys.stderr)
+        return False
+
+
 def _sampling(p: argparse.ArgumentParser) -> None:
     p.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
     p.add_argument("--top-k", type=int, default=0)
@@ -55,9 +70,13 @@ def _engine(args):
         eng = Engine.from_config(cfg, arch.name, args.dtype, args.seed, sched)
     else:
         eng = Engine.from_folder(args.model_path, args.dtype, sched)
-    print(f"Engine initialized in {(time.perf_counter() - t0) * 1000:.0f} ms "
-          f"({eng.cache.num_pages} pages of {eng.cache.page_size} tokens)", file=sys.stderr)
-    return InferenceEngine(eng)
+    import logging
+    log = logging.getLogger("zedinfer_amd")
+    log.info("Engine initialized in %.0f ms (%d pages of %d tokens)", (time.perf_counter() - t0) * 1000,
+             eng.cache.num_pages, eng.cache.page_size)
+    ie = InferenceEngine(eng)
+    log.debug("choices made at warm-up: %s", eng.rt.choices)
+    return ie
 
 
 def ping(argv: Optional[List[str]] = None) -> int:
@@ -70,7 +89,10 @@ def ping(argv: Optional[List[str]] = None) -> int:
                    help="Maximum number of new tokens to generate (0 = unlimited)")
     p.add_argument("--stream", action="store_true", help="Print token ids as they are generated")
     p.add_argument("--ignore-eos", action="store_true")
+    _logging(p, "ping")
     args = p.parse_args(argv)
+    if not _init_logging(args):
+        return 1
     if args.max_new_tokens < 0:
         print("--max-new-tokens/--max-tokens must be >= 0", file=sys.stderr)
         return 1
@@ -96,7 +118,10 @@ def bench(argv: Optional[List[str]] = None) -> int:
     p.add_argument("-p", "--prefill-len", type=int, default=128)
     p.add_argument("-d", "--decode-len", "--max-tokens", type=int, default=128, dest="decode_len")
     p.add_argument("-r", "--rounds", type=int, default=3)
+    _logging(p, "bench")
     args = p.parse_args(argv)
+    if not _init_logging(args):
+        return 1
     if args.decode_len <= 0:
         print("--decode-len/--max-tokens must be > 0 for benchmark runs", file=sys.stderr)
         return 1
@@ -130,7 +155,10 @@ def batch_bench(argv: Optional[List[str]] = None) -> int:
     p.add_argument("--no-warmup", action="store_true",
                    help="count the first batch too (it records the decode graphs and measures the matrix products' "
                         "way round once; the reference has no such first-time costs and no warm-up round)")
+    _logging(p, "batch_bench")
     args = p.parse_args(argv)
+    if not _init_logging(args):
+        return 1
     if args.decode_len <= 0:
         print("--decode-len/--max-tokens must be > 0 for benchmark runs", file=sys.stderr)
         return 1
