@@ -716,7 +716,22 @@ def test_attention_prefill(ops, nh, nkv, d, ps, window, portions):
                               dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale,
                               window, out=out4, tile=128)
         assert torch.equal(out4, out)
+        # workgroups of four wavefronts that walk blocks of 64 keys (for launches of many tiles): another order of
+        # a query's keys, so another rounding, the same for both tile sizes
+        alone = {}
+        for tile, (ta, tb) in ((64, (te, to)), (128, (te2, to2))):
+            alone[tile] = torch.full((n_tok, nh * d), 7.0, dtype=dtype, device="cuda")
+            ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, ta, tb, dev([e[0] for e in entries]),
+                                  dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale,
+                                  window, out=alone[tile], tile=tile, alone=True)
+            assert not torch.isnan(alone[tile]).any()
+            torch.testing.assert_close(alone[tile].view(n_tok, nh, d).float(), ref, atol=2e-2, rtol=2e-2)
+        assert torch.equal(alone[64], alone[128])
     else:
+        with pytest.raises(ValueError, match="four wavefronts"):
+            ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, te, to, dev([e[0] for e in entries]),
+                                  dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale,
+                                  window, out=out, alone=True)
         with pytest.raises(ValueError, match="tiles of 128"):
             ops.attention_prefill(q.view(n_tok, nh * d), kc, vc, te, to, dev([e[0] for e in entries]),
                                   dev([e[1] for e in entries]), dev([e[2] for e in entries]), bt, nh, nkv, d, scale,

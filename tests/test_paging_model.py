@@ -183,17 +183,19 @@ def test_decode_walk_reports_what_is_broken(model):
 
 
 def prefill(pm, plan, hb, real, tables, num_pages, nh, nkv, d, ps, window, max_chunks, workspace=None, tile=64):
+    """``tile``: 64, 128, or -128 for tiles of 128 queries in workgroups of four wavefronts (blocks of 64 keys)."""
+    alone, tile = int(tile < 0), abs(tile)
     rows = hb.num_tokens
     ws = pm.pm_prefill_workspace(rows, nh, d, max_chunks) if workspace is None else workspace
     stats = (ctypes.c_int64 * 3)()
     rc = pm.pm_check_prefill(plan.sizes["num_tiles"], ptr(plan.arrays["tile_entry"]), ptr(plan.arrays["tile_off"]),
                              ptr(hb.entry_start), ptr(hb.entry_len), ptr(hb.entry_past), ptr(real), hb.num_entries,
                              ptr(tables), tables.shape[1], num_pages, nh, nkv, d, ps, window, rows, max_chunks,
-                             ctypes.c_int64(ws), tile, stats)
+                             ctypes.c_int64(ws), tile, alone, stats)
     return rc, pm.pm_last_error().decode(), list(stats)
 
 
-@pytest.mark.parametrize("tile", [64, 128])
+@pytest.mark.parametrize("tile", [64, 128, -128])
 @pytest.mark.parametrize("window", [0, 24, 100])
 @pytest.mark.parametrize("seed", range(5))
 def test_prefill_walk_under_random_traffic(model, seed, window, tile):
@@ -219,10 +221,12 @@ def test_prefill_walk_under_random_traffic(model, seed, window, tile):
         starts[1:] = np.cumsum(lens)[:-1]
         past = np.array([s.length for s, _ in portions], dtype=np.int32)
         hb = HostBatch(int(lens.sum()), len(portions), starts, lens, past, False)
-        planner = AttentionPlanner(tile, heads=6)
-        planner.FILL = 1 if tile == 128 else planner.FILL        # take the wide tiles however small the step
+        planner = AttentionPlanner(abs(tile), heads=6)
+        planner.FILL = 1 if abs(tile) == 128 else planner.FILL   # take the wide tiles however small the step
+        planner.FILL_ALONE = 1 if tile < 0 else 10 ** 9
         plan = planner.plan(hb)
-        assert plan.sizes["num_long"] == int(lens.sum()) and plan.sizes["tile"] == tile
+        assert plan.sizes["num_long"] == int(lens.sum()) and plan.sizes["tile"] == abs(tile)
+        assert plan.sizes["alone"] == (tile < 0)
         for g, group in enumerate(m.groups):
             tables = padded_tables([s for s, _ in portions], g, pow2(max(len(s.pages[g]) for s, _ in portions), 8))
             keys = plan.sizes["max_long_keys"]
@@ -235,7 +239,7 @@ def test_prefill_walk_under_random_traffic(model, seed, window, tile):
             assert stats[0] > 0 and stats[2] == 0
 
 
-@pytest.mark.parametrize("tile", [64, 128])
+@pytest.mark.parametrize("tile", [64, 128, -128])
 def test_prefill_walk_of_a_long_prompt_and_what_is_broken(model, tile):
     """One portion that continues a long sequence: its tiles are cut along the keys every 2,048, and the cuts'
     partial results have places of their own in the workspace."""
@@ -246,10 +250,11 @@ def test_prefill_walk_of_a_long_prompt_and_what_is_broken(model, tile):
     m.ensure(s, 4100 + 300)
     hb = HostBatch(300, 1, np.array([0], dtype=np.int32), np.array([300], dtype=np.int32),
                    np.array([4100], dtype=np.int32), False)
-    planner = AttentionPlanner(tile, heads=4)
+    planner = AttentionPlanner(abs(tile), heads=4)
     planner.FILL = 1
+    planner.FILL_ALONE = 1 if tile < 0 else 10 ** 9
     plan = planner.plan(hb)
-    assert plan.sizes["tile"] == tile
+    assert plan.sizes["tile"] == abs(tile) and plan.sizes["alone"] == (tile < 0)
     tables = padded_tables([s], 0, pow2(len(s.pages[0]), 8))
     chunks = model.pm_prefill_chunks(plan.sizes["max_long_keys"])
     assert chunks == 3

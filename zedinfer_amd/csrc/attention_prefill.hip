@@ -256,10 +256,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    s[t][x] *= scale_log2;
-                    mx = fmaxf(mx, s[t][x]);
-                }
+                for (int x = 0; x < 4; ++x) mx = fmaxf(mx, s[t][x]);
         } else {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
@@ -267,14 +264,16 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                 for (int x = 0; x < 4; ++x) {
                     const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
                     const bool vis = key <= qpos && (window <= 0 || key > qpos - window);
-                    const float v = vis ? s[t][x] * scale_log2 : -INFINITY;
+                    const float v = vis ? s[t][x] : -INFINITY;
                     s[t][x] = v;
                     mx = fmaxf(mx, v);
                 }
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
         mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
-        const float m_new = fmaxf(m, mx);
+        // the scale is positive (the host checks): the largest scaled score is the largest score, scaled; the
+        // scaling of every score is then one fused multiply-add with the subtraction of the maximum
+        const float m_new = fmaxf(m, mx * scale_log2);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float corr = __builtin_amdgcn_exp2f(m - m_use);      // 2^(-inf) = 0 before the first key
         m = m_new;
@@ -283,7 +282,7 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                s[t][x] = __builtin_amdgcn_exp2f(s[t][x] - m_use);    // 0 for masked keys
+                s[t][x] = __builtin_amdgcn_exp2f(fmaf(s[t][x], scale_log2, -m_use));    // 0 for masked keys
                 psum += s[t][x];
             }
         pf_pack pb[2];
@@ -409,8 +408,13 @@ __device__ __attribute__((aligned(16))) const unsigned pf_zero16[4] = {0u, 0u, 0
 
 // QW: sub-tiles of 16 queries a wavefront owns: 1 (tiles of 64 queries) or 2 (tiles of 128: every block of keys and
 // values that is brought into LDS, and every operand read from there, serves twice the queries).
-template <int D, int QW>
-__global__ void __launch_bounds__(PF_WAVES* ZI_WAVE)
+// KH: wavefronts that share a query group, each with its own 64 keys of a block: 2 (eight wavefronts, blocks of
+// 128 keys, one workgroup on a compute unit) or 1 (four wavefronts, blocks of 64 keys, half the LDS: two
+// workgroups on a compute unit, which are not in step with each other, so that one's matrix instructions run
+// beside the other's softmax and loads; a tile's walk is one wavefront's per query group, so it takes longer:
+// for launches with many tiles).
+template <int D, int QW, int KH>
+__global__ void __launch_bounds__(4 * KH * ZI_WAVE, KH == 1 ? 2 : 1)
 attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* __restrict__ q, int64_t ldq,
                              const zi_bf16* __restrict__ kcache, const zi_bf16* __restrict__ vcache,
                              const int32_t* __restrict__ tile_entry, const int32_t* __restrict__ tile_off,
@@ -424,9 +428,13 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     constexpr int QR = 16 * QW;                      // queries of a wavefront
     constexpr int DK = D / 32, DT = D / 16;
     constexpr int KC = D / 8;                        // 16-byte pieces of a key row
-    constexpr int VC = PF_BS / 8;                    // and of a row of the transposed value tile: 16
-    constexpr int KCH = PF_BS * KC, VCH = D * VC;    // pieces of the two tiles
-    constexpr int THREADS = PF_WAVES * ZI_WAVE;
+    static_assert(KH == 1 || KH == 2, "one or two wavefronts a query group");
+    constexpr int WAVES = 4 * KH;
+    constexpr int BS = PF_BN * KH;                   // keys of a block
+    constexpr int VC = BS / 8;                       // and of a row of the transposed value tile: 8 or 16
+    constexpr int VSW = 16 / VC;                     // value rows that share 256 bytes of LDS (and one swizzle)
+    constexpr int KCH = BS * KC, VCH = D * VC;       // pieces of the two tiles
+    constexpr int THREADS = WAVES * ZI_WAVE;
     constexpr int KI = KCH / THREADS, VI = VCH / THREADS;   // load instructions a wavefront issues per tile
     constexpr int KSW = 16 / KC;                     // key rows that share 256 bytes of LDS (and one swizzle)
     __shared__ __attribute__((aligned(16))) uint4 k_ab[2 * KCH];
@@ -506,11 +514,11 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     for (int i = 0; i < VI; ++i) {
         const int L = (wave * VI + i) * ZI_WAVE + lane;
         v_dim[i] = L / VC;
-        v_key[i] = ((L % VC) ^ (v_dim[i] & (VC - 1))) * 8;
+        v_key[i] = ((L % VC) ^ ((v_dim[i] / VSW) & (VC - 1))) * 8;
     }
-    const zi_bf16* kbase = kcache + (int64_t)g * ps * D;
-    const zi_bf16* vbase = vcache + (int64_t)g * D * ps;
-    const int64_t page_stride = (int64_t)nkv * ps * D;
+    const uint4* kbase16 = reinterpret_cast<const uint4*>(kcache + (int64_t)g * ps * D);
+    const uint4* vbase16 = reinterpret_cast<const uint4*>(vcache + (int64_t)g * D * ps);
+    const uint32_t page_pieces = (uint32_t)nkv * ps * D / 8;      // 16-byte pieces of one page
     const int khi8 = khi & ~7;
     __syncthreads();      // the table is in LDS
 
@@ -521,8 +529,10 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             const int kc = key <= khi ? key : khi;
             const int pg = bt_lds[(kc >> ps_shift) - pi_first];
             const int page = (unsigned)pg < (unsigned)num_pages ? pg : 0;     // not held: a window has passed it
-            const zi_bf16* src = kbase + page * page_stride + (int64_t)(kc & ps_mask) * D + k_piece[i] * 8;
-            __builtin_amdgcn_global_load_lds(src, kl + (wave * KI + i) * ZI_WAVE, 16, 0, 0);
+            // places in the pool as 32-bit counts of 16-byte pieces (the host checks that the pool has fewer
+            // than 2^32 of them): one shift-and-add makes the address
+            const uint32_t at = (uint32_t)page * page_pieces + (uint32_t)(kc & ps_mask) * KC + k_piece[i];
+            __builtin_amdgcn_global_load_lds(kbase16 + at, kl + (wave * KI + i) * ZI_WAVE, 16, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < VI; ++i) {
@@ -530,19 +540,22 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             const int kc = key0 <= khi ? key0 : khi8;
             const int pg = bt_lds[(kc >> ps_shift) - pi_first];
             const bool ok = key0 <= kmax && (unsigned)pg < (unsigned)num_pages;
-            const zi_bf16* src = ok ? vbase + pg * page_stride + ((int64_t)v_dim[i] << ps_shift) + (kc & ps_mask)
-                                    : reinterpret_cast<const zi_bf16*>(pf_zero16);
+            // the address is made for every lane (of page 0 where there is none) and replaced afterwards: a
+            // choice between two ways of making it would become a branch
+            const uint32_t at = (uint32_t)(ok ? pg : 0) * page_pieces + ((((uint32_t)v_dim[i] << ps_shift) + (kc & ps_mask)) >> 3);
+            const uint4* there = vbase16 + at;
+            const uint4* src = ok ? there : reinterpret_cast<const uint4*>(pf_zero16);
             __builtin_amdgcn_global_load_lds(src, vl + (wave * VI + i) * ZI_WAVE, 16, 0, 0);
         }
     };
     // The piece of every value row that holds the last key and keys past it: what lies past is cleared
     // (those slots of the page may hold anything).  Only in the block that holds the last key.
     auto clean = [&](int kb, uint4* vl) {
-        if (kb + PF_BS - 1 > kmax && ((kmax + 1) & 7) != 0) {
+        if (kb + BS - 1 > kmax && ((kmax + 1) & 7) != 0) {
             if (tid < D) {
                 const int piece = (kmax - kb) / 8, keep = (kmax + 1) & 7;
                 pf_pack val;
-                uint4* at = vl + tid * VC + (piece ^ (tid & (VC - 1)));
+                uint4* at = vl + tid * VC + (piece ^ ((tid / VSW) & (VC - 1)));
                 val.u = *at;
 #pragma unroll
                 for (int x = 0; x < 8; ++x)
@@ -579,10 +592,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        s[u][t][x] *= scale_log2;
-                        mx = fmaxf(mx, s[u][t][x]);
-                    }
+                    for (int x = 0; x < 4; ++x) mx = fmaxf(mx, s[u][t][x]);
             } else {
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
@@ -590,14 +600,14 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
                     for (int x = 0; x < 4; ++x) {
                         const int key = kb + (t / 2) * 32 + j * 8 + (t % 2) * 4 + x;
                         const bool vis = key <= qpos[u] && (window <= 0 || key > qpos[u] - window);
-                        const float v = vis ? s[u][t][x] * scale_log2 : -INFINITY;
+                        const float v = vis ? s[u][t][x] : -INFINITY;
                         s[u][t][x] = v;
                         mx = fmaxf(mx, v);
                     }
             }
             mx = fmaxf(mx, __shfl_xor(mx, 16, ZI_WAVE));
             mx = fmaxf(mx, __shfl_xor(mx, 32, ZI_WAVE));
-            const float m_new = fmaxf(m[u], mx);
+            const float m_new = fmaxf(m[u], mx * scale_log2);      // the scale is positive
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
             const float corr = __builtin_amdgcn_exp2f(m[u] - m_use);
             m[u] = m_new;
@@ -606,7 +616,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int x = 0; x < 4; ++x) {
-                    s[u][t][x] = __builtin_amdgcn_exp2f(s[u][t][x] - m_use);
+                    s[u][t][x] = __builtin_amdgcn_exp2f(fmaf(s[u][t][x], scale_log2, -m_use));
                     psum += s[u][t][x];
                 }
 #pragma unroll
@@ -630,7 +640,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
 #pragma unroll
             for (int b = 0; b < 2; ++b) {
                 pf_pack a;
-                a.u = vl[dim * VC + ((kh * 8 + b * 4 + j) ^ (dim & (VC - 1)))];
+                a.u = vl[dim * VC + ((kh * 8 + b * 4 + j) ^ ((dim / VSW) & (VC - 1)))];
 #pragma unroll
                 for (int u = 0; u < QW; ++u)      // and one read of the values' operand
                     o[u][dd] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb[u][b].b, o[u][dd], 0, 0, 0);
@@ -645,17 +655,17 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
     int kb0 = kb_begin;
     while (true) {
         __syncthreads();
-        if (kb0 + PF_BS <= khi) issue(kb0 + PF_BS, k_b, v_b);
+        if (kb0 + BS <= khi) issue(kb0 + BS, k_b, v_b);
         clean(kb0, v_a);
         work(kb0, k_a, v_a);
-        if (kb0 + PF_BS > khi) break;
-        kb0 += PF_BS;
+        if (kb0 + BS > khi) break;
+        kb0 += BS;
         __syncthreads();
-        if (kb0 + PF_BS <= khi) issue(kb0 + PF_BS, k_a, v_a);
+        if (kb0 + BS <= khi) issue(kb0 + BS, k_a, v_a);
         clean(kb0, v_b);
         work(kb0, k_b, v_b);
-        if (kb0 + PF_BS > khi) break;
-        kb0 += PF_BS;
+        if (kb0 + BS > khi) break;
+        kb0 += BS;
     }
     __syncthreads();
     float l[QW];
@@ -665,7 +675,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
         l[u] += __shfl_xor(l[u], 16, ZI_WAVE);
         l[u] += __shfl_xor(l[u], 32, ZI_WAVE);
     }
-    {
+    if constexpr (KH > 1) {
         // the two wavefronts of a query group merge their (maximum, sum, output) through LDS; nobody reads
         // the tiles any more
         float* mo = reinterpret_cast<float*>(k_ab);                  // [qs][QW][DT][64][4]: within the two key tiles
@@ -802,7 +812,7 @@ extern "C" int zi_attention_prefill_variant(int variant) {
 // there a block of keys and values in LDS, and an operand read from it, serves twice the queries.  The caller
 // cuts its entries into tiles of this many queries (zi_attention_prefill takes either size for those shapes).
 extern "C" int zi_attention_prefill_tile(int dt, int d) {
-    return (dt == ZI_BF16 && pf_variant == 1 && (d == 64 || d == 128)) ? 2 * PF_BM : PF_BM;
+    return (dt == ZI_BF16 && pf_variant >= 1 && (d == 64 || d == 128)) ? 2 * PF_BM : PF_BM;
 }
 
 // Keys one workgroup walks at most: tiles are cut at absolute multiples of this.
@@ -810,15 +820,17 @@ extern "C" int zi_attention_prefill_chunk_keys() { return PF_CHUNK; }
 
 // Tile i covers the queries [tile_off[i], tile_off[i] + tile) of entry tile_entry[i] (fewer at the
 // entry's end; `tile` is 64, or 128 for head sizes 64 and 128); entry e brings entry_len[e] tokens that start at row entry_start[e] of q and at
-// position entry_past[e] of its sequence, whose block table is row e of block_tables.
+// position entry_past[e] of its sequence, whose block table is row e of block_tables.  `alone` (head sizes 64 and
+// 128): workgroups of four wavefronts that walk blocks of 64 keys, two to a compute unit, for launches of many
+// tiles; a query's keys are then added in another order, so the result differs by rounding.
 extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
                                     const void* kcache, const void* vcache, const int32_t* tile_entry,
                                     const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
                                     const int32_t* entry_past, const int32_t* block_tables, int max_pages,
                                     int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
                                     int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
-                                    hipStream_t stream) {
-    ZI_REQUIRE(tile == PF_BM || (tile == 2 * PF_BM && pf_variant == 1 && (d == 64 || d == 128)),
+                                    int alone, hipStream_t stream) {
+    ZI_REQUIRE(tile == PF_BM || (tile == 2 * PF_BM && pf_variant >= 1 && (d == 64 || d == 128)),
                "attention_prefill: tiles of %d queries (64, or 128 for head sizes 64 and 128)", tile);
     ZI_REQUIRE(zi_attention_prefill_supported(dt, nh, nkv, d, page_size),
                "attention_prefill: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, page size a power "
@@ -830,6 +842,10 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
                    ((uintptr_t)vcache % 16) == 0,
                "attention_prefill: q, out and the caches must be aligned to 16 bytes");
     ZI_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
+    ZI_REQUIRE(scale > 0.f, "attention_prefill: the scale must be positive, got %g", (double)scale);
+    ZI_REQUIRE((int64_t)num_pages * nkv * page_size * d / 8 < (1ll << 32),
+               "attention_prefill: a cache pool of %lld pages is more than this kernel addresses (64 GiB a tensor)",
+               (long long)num_pages);
     ZI_REQUIRE(max_chunks >= 1 && max_chunks <= PF_MAXC, "attention_prefill: max_chunks %d outside 1..%d (contexts up to %d keys)",
                max_chunks, PF_MAXC, PF_MAXC * PF_CHUNK);
     ZI_REQUIRE(max_chunks == 1 || (workspace && ((uintptr_t)workspace % 16) == 0 &&
@@ -847,15 +863,22 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
         window, scale, po, pml, max_chunks)
-#define ZI_PF_DMA(DD, QW)                                                                                      \
-    attention_prefill_dma_kernel<DD, QW><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                             \
+#define ZI_PF_DMA(DD, QW, KH)                                                                                  \
+    attention_prefill_dma_kernel<DD, QW, KH><<<grid, 4 * KH * ZI_WAVE, 0, stream>>>(                           \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
         window, scale, po, pml, max_chunks)
-    if (pf_variant == 1 && d == 128 && tile == 2 * PF_BM) ZI_PF_DMA(128, 2);
-    else if (pf_variant == 1 && d == 64 && tile == 2 * PF_BM) ZI_PF_DMA(64, 2);
-    else if (pf_variant == 1 && d == 128) ZI_PF_DMA(128, 1);
-    else if (pf_variant == 1 && d == 64) ZI_PF_DMA(64, 1);
+    const bool dma = pf_variant >= 1 && (d == 64 || d == 128);
+    const bool wide = tile == 2 * PF_BM;
+    ZI_REQUIRE(!alone || dma, "attention_prefill: workgroups of four wavefronts are for head sizes 64 and 128");
+    if (dma && d == 128 && wide && alone) ZI_PF_DMA(128, 2, 1);
+    else if (dma && d == 128 && wide) ZI_PF_DMA(128, 2, 2);
+    else if (dma && d == 128 && alone) ZI_PF_DMA(128, 1, 1);
+    else if (dma && d == 128) ZI_PF_DMA(128, 1, 2);
+    else if (dma && d == 64 && wide && alone) ZI_PF_DMA(64, 2, 1);
+    else if (dma && d == 64 && wide) ZI_PF_DMA(64, 2, 2);
+    else if (dma && d == 64 && alone) ZI_PF_DMA(64, 1, 1);
+    else if (dma && d == 64) ZI_PF_DMA(64, 1, 2);
     else
     switch (d) {
         case 16: ZI_PF(16); break;

@@ -155,7 +155,7 @@ extern "C" int pm_check_decode(int n_idx, const int* tok_index, const int* tok_s
 
 // The prompt attention launch (attention_prefill kernels): grid (tiles * nh, cuts), eight wavefronts: four
 // groups of tile / 4 queries (tile = 64 or 128 queries), each shared by two wavefronts that take alternate
-// halves of every block of 128 keys.
+// halves of every block of 128 keys; or (`alone`) four wavefronts, one a group, and blocks of 64 keys.
 // stats[0] = (query, key) pairs covered, stats[1] = workspace slots written, stats[2] = tiles given NaN.
 // `entry_real` (or null): the tokens of each entry that are its own; the rest are padding, whose queries'
 // results nobody reads and whose keys are nowhere: they are checked for bounds only.
@@ -163,10 +163,11 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
                                 const int* entry_len, const int* entry_past, const int* entry_real, int num_entries,
                                 const int* block_tables,
                                 int max_pages, int num_pages, int nh, int nkv, int d, int ps, int window, int rows,
-                                int max_chunks, int64_t workspace_floats, int tile_queries, int64_t* stats) {
+                                int max_chunks, int64_t workspace_floats, int tile_queries, int alone, int64_t* stats) {
     PM_CHECK(nkv > 0 && nh % nkv == 0 && ps >= 8 && (ps & (ps - 1)) == 0 && max_pages > 0, "prefill: bad sizes");
     PM_CHECK(tile_queries == ZI_PF_BM || tile_queries == 2 * ZI_PF_BM, "prefill: tiles of %d queries", tile_queries);
     const int BM = tile_queries, QR = tile_queries / 4;
+    const int KH = alone ? 1 : 2, BS = 64 * KH;      // wavefronts that share a query group, keys of a block
     const int ps_shift = shift_of(ps), pi_last = max_pages - 1;
     const int64_t pool = zi_pool_elements(num_pages, nkv, ps, d);
     const int64_t ml_base = (int64_t)rows * nh * max_chunks * d;
@@ -200,8 +201,8 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
             const int pi_first = cut.kb_begin >> ps_shift, n_entries = (cut.khi >> ps_shift) - pi_first + 1;
             PM_CHECK(n_entries <= ZI_PF_CHUNK / 8 + 8 && n_entries <= 8 * 64, "prefill: %d block table entries for one cut",
                      n_entries);
-            for (int kb = cut.kb_begin; kb <= cut.khi; kb += ZI_PF_BS) {
-                for (int k = 0; k < ZI_PF_BS; ++k) {
+            for (int kb = cut.kb_begin; kb <= cut.khi; kb += BS) {
+                for (int k = 0; k < BS; ++k) {
                     const int key = kb + k, kc = key <= cut.khi ? key : cut.khi;
                     const int idx = (kc >> ps_shift) - pi_first;
                     PM_CHECK(idx >= 0 && idx < n_entries, "prefill: key %d reads staged table entry %d of %d", key, idx,
@@ -225,7 +226,7 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
                     if (qs * QR >= count) continue;
                     const int wave_last = pos0 + ((qs * QR + QR - 1 < count) ? qs * QR + QR - 1 : count - 1);
                     const int wave_lo = (window > 0 && pos0 + qs * QR - window + 1 > 0) ? pos0 + qs * QR - window + 1 : 0;
-                    for (int kh = 0; kh < 2; ++kh) {
+                    for (int kh = 0; kh < KH; ++kh) {
                         const int kb2 = kb + kh * 64;
                         if (!(kb2 <= wave_last && kb2 + 64 > wave_lo)) continue;
                         for (int r = 0; r < QR && qs * QR + r < count; ++r) {

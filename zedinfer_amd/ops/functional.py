@@ -599,7 +599,7 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
                       tile_off: torch.Tensor, entry_start: torch.Tensor, entry_len: torch.Tensor,
                       entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, out: Optional[torch.Tensor] = None, max_keys: int = 0,
-                      workspace: Optional[torch.Tensor] = None, tile: int = PREFILL_TILE) -> torch.Tensor:
+                      workspace: Optional[torch.Tensor] = None, tile: int = PREFILL_TILE, alone: bool = False) -> torch.Tensor:
     """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
     of 16 up to 128, page size a power of two from 8).
 
@@ -610,7 +610,8 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
     sees (its position + 1; 0: what the block tables could hold): tiles that see more than 2,048 keys are
     cut over several workgroups and merged, which needs ``workspace`` (``attention_prefill_workspace``
     entries of float32; allocated here when not given).  A bound that is too low leaves NaN in the rows
-    concerned."""
+    concerned.  ``alone`` (where the head size has tiles of 128): workgroups of four wavefronts, two to a compute
+    unit, which pays for launches of many tiles; the result differs by rounding."""
     _gpu("attention_prefill", q, kcache, vcache, tile_entry, tile_off, entry_start, entry_len, entry_past,
          block_tables, out)
     ldq, wq = _rows(q, "attention_prefill q")
@@ -631,6 +632,8 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
         raise ValueError("attention_prefill: block_tables must be a contiguous int32 [entries, max_pages] tensor")
     if tile not in (PREFILL_TILE, attention_prefill_tile(q.dtype, d)):
         raise ValueError(f"attention_prefill: tiles of {tile} queries are not taken for head size {d}")
+    if alone and attention_prefill_tile(q.dtype, d) == PREFILL_TILE:
+        raise ValueError(f"attention_prefill: workgroups of four wavefronts are not made for head size {d}")
     if out is None:
         out = torch.empty((n, nh * d), dtype=q.dtype, device=q.device)
     ldo, wo = _rows(out, "attention_prefill out")
@@ -648,7 +651,8 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
     _lib.call("zi_attention_prefill", _p(out), _p(q), _code(q, "attention_prefill"), num_tiles, ldq, ldo, _p(kcache),
               _p(vcache), _p(tile_entry), _p(tile_off), _p(entry_start), _p(entry_len), _p(entry_past),
               _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), n,
-              max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, int(tile), _stream())
+              max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, int(tile), int(bool(alone)),
+              _stream())
     return out
 
 

@@ -27,16 +27,19 @@ class AttentionPlanner(StepPlanner):
     a block of keys staged on the chip then serves twice the queries) when the step is large enough to fill
     the chip with those: measured with 28 layers of the 1.5B sizes (12 heads), 16,384 tokens of one prompt run
     88 against 99 ms with the wide tiles, 8,192 tokens 33.7 against 37.0, 3,072 tokens 12.8 against 13.3, and
-    2,048 tokens 9.2 against 9.1 ms; with 28 heads 2,048 tokens gain 2%.  The choice is a function of the entries' (padded) lengths
+    2,048 tokens 9.2 against 9.1 ms; with 28 heads 2,048 tokens gain 2%.  Larger steps still take the wide tiles
+    in workgroups of four wavefronts, two to a compute unit (``alone``: 16,384 tokens 81.6 against 86.4 ms, 4,096
+    tokens 16.0 against 16.4; the result differs by rounding).  The choice is a function of the entries' (padded) lengths
     and of the bound of their keys, so that a recorded step meets the same one again.
 
     arrays: ``short_idx`` / ``long_idx``, the flat indices of the tokens of either kind; ``tile_entry`` /
     ``tile_off``: tile i covers tokens [tile_off[i], tile_off[i] + tile) of entry tile_entry[i].
-    sizes: ``num_short``, ``num_long``, ``num_tiles``, ``tile``; ``max_short_keys`` / ``max_long_keys``: an upper
+    sizes: ``num_short``, ``num_long``, ``num_tiles``, ``tile``, ``alone``; ``max_short_keys`` / ``max_long_keys``: an upper
     bound of the keys a token of either kind sees (its position + 1), which sizes the launches."""
 
     fixed_for_single_tokens = True
     FILL = 384          # workgroups of wide tiles from which they pay (one and a half a compute unit)
+    FILL_ALONE = 768    # and from which workgroups of four wavefronts, two to a compute unit, pay (``alone``)
     CUT_KEYS = 2048     # a tile's keys are cut over several workgroups every so many
 
     def __init__(self, wide_tile: int = LONG_TILE, heads: int = 1):
@@ -59,11 +62,13 @@ class AttentionPlanner(StepPlanner):
                             hb.bound_multi if several else 0, 1)
         if long_idx.size and hb.bound_multi:
             max_long = hb.bound_multi
-        tile = LONG_TILE
+        tile, alone = LONG_TILE, False
         if self.wide_tile > LONG_TILE and long_idx.size:
             wide = int(sum(-(-int(n) // self.wide_tile) for n in lens[~short]))
-            if wide * -(-max_long // self.CUT_KEYS) * self.heads >= self.FILL:
+            groups = wide * -(-max_long // self.CUT_KEYS) * self.heads
+            if groups >= self.FILL:
                 tile = self.wide_tile
+                alone = groups >= self.FILL_ALONE
         tiles = [(int(past[i]) + off + min(tile, int(lens[i]) - off), i, off)
                  for i in range(hb.num_entries) if not short[i] for off in range(0, int(lens[i]), tile)]
         tiles.sort(key=lambda t: -t[0])
@@ -72,7 +77,7 @@ class AttentionPlanner(StepPlanner):
                     "tile_entry": np.array([t[1] for t in tiles], dtype=np.int32),
                     "tile_off": np.array([t[2] for t in tiles], dtype=np.int32)},
             sizes={"num_short": int(short_idx.size), "num_long": int(long_idx.size), "num_tiles": len(tiles),
-                   "tile": tile, "max_short_keys": max_short, "max_long_keys": max_long})
+                   "tile": tile, "alone": alone, "max_short_keys": max_short, "max_long_keys": max_long})
 
 
 _PLANNERS: Dict[tuple, AttentionPlanner] = {}
@@ -178,7 +183,7 @@ class Attention(Mixer):
                 ops.attention_prefill(q, memory.k, memory.v, plan.dev["tile_entry"], plan.dev["tile_off"],
                                       batch.entry_start, batch.entry_len, batch.entry_past, view.block_tables, self.nh,
                                       self.nkv, self.d, self.scale, self.window, out=att, max_keys=max_keys,
-                                      workspace=ws, tile=plan.sizes["tile"])
+                                      workspace=ws, tile=plan.sizes["tile"], alone=plan.sizes["alone"])
             else:
                 ops.attention(q, *args, self.window, out=att, tok_index=plan.dev["long_idx"] if n_long < N else None)
 
