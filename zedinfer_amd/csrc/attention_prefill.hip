@@ -516,9 +516,9 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
         v_dim[i] = L / VC;
         v_key[i] = ((L % VC) ^ ((v_dim[i] / VSW) & (VC - 1))) * 8;
     }
-    const uint4* kbase16 = reinterpret_cast<const uint4*>(kcache + (int64_t)g * ps * D);
-    const uint4* vbase16 = reinterpret_cast<const uint4*>(vcache + (int64_t)g * D * ps);
-    const uint32_t page_pieces = (uint32_t)nkv * ps * D / 8;      // 16-byte pieces of one page
+    const zi_bf16* kbase = kcache + (int64_t)g * ps * D;
+    const zi_bf16* vbase = vcache + (int64_t)g * D * ps;
+    const int64_t page_stride = (int64_t)nkv * ps * D;
     const int khi8 = khi & ~7;
     __syncthreads();      // the table is in LDS
 
@@ -529,10 +529,8 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             const int kc = key <= khi ? key : khi;
             const int pg = bt_lds[(kc >> ps_shift) - pi_first];
             const int page = (unsigned)pg < (unsigned)num_pages ? pg : 0;     // not held: a window has passed it
-            // places in the pool as 32-bit counts of 16-byte pieces (the host checks that the pool has fewer
-            // than 2^32 of them): one shift-and-add makes the address
-            const uint32_t at = (uint32_t)page * page_pieces + (uint32_t)(kc & ps_mask) * KC + k_piece[i];
-            __builtin_amdgcn_global_load_lds(kbase16 + at, kl + (wave * KI + i) * ZI_WAVE, 16, 0, 0);
+            const zi_bf16* src = kbase + page * page_stride + (int64_t)(kc & ps_mask) * D + k_piece[i] * 8;
+            __builtin_amdgcn_global_load_lds(src, kl + (wave * KI + i) * ZI_WAVE, 16, 0, 0);
         }
 #pragma unroll
         for (int i = 0; i < VI; ++i) {
@@ -540,11 +538,8 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             const int kc = key0 <= khi ? key0 : khi8;
             const int pg = bt_lds[(kc >> ps_shift) - pi_first];
             const bool ok = key0 <= kmax && (unsigned)pg < (unsigned)num_pages;
-            // the address is made for every lane (of page 0 where there is none) and replaced afterwards: a
-            // choice between two ways of making it would become a branch
-            const uint32_t at = (uint32_t)(ok ? pg : 0) * page_pieces + ((((uint32_t)v_dim[i] << ps_shift) + (kc & ps_mask)) >> 3);
-            const uint4* there = vbase16 + at;
-            const uint4* src = ok ? there : reinterpret_cast<const uint4*>(pf_zero16);
+            const zi_bf16* src = ok ? vbase + pg * page_stride + ((int64_t)v_dim[i] << ps_shift) + (kc & ps_mask)
+                                    : reinterpret_cast<const zi_bf16*>(pf_zero16);
             __builtin_amdgcn_global_load_lds(src, vl + (wave * VI + i) * ZI_WAVE, 16, 0, 0);
         }
     };
@@ -843,9 +838,6 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
                "attention_prefill: q, out and the caches must be aligned to 16 bytes");
     ZI_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
     ZI_REQUIRE(scale > 0.f, "attention_prefill: the scale must be positive, got %g", (double)scale);
-    ZI_REQUIRE((int64_t)num_pages * nkv * page_size * d / 8 < (1ll << 32),
-               "attention_prefill: a cache pool of %lld pages is more than this kernel addresses (64 GiB a tensor)",
-               (long long)num_pages);
     ZI_REQUIRE(max_chunks >= 1 && max_chunks <= PF_MAXC, "attention_prefill: max_chunks %d outside 1..%d (contexts up to %d keys)",
                max_chunks, PF_MAXC, PF_MAXC * PF_CHUNK);
     ZI_REQUIRE(max_chunks == 1 || (workspace && ((uintptr_t)workspace % 16) == 0 &&

@@ -28,7 +28,7 @@ class AttentionPlanner(StepPlanner):
     the chip with those: measured with 28 layers of the 1.5B sizes (12 heads), 16,384 tokens of one prompt run
     88 against 99 ms with the wide tiles, 8,192 tokens 33.7 against 37.0, 3,072 tokens 12.8 against 13.3, and
     2,048 tokens 9.2 against 9.1 ms; with 28 heads 2,048 tokens gain 2%.  Larger steps still take the wide tiles
-    in workgroups of four wavefronts, two to a compute unit (``alone``: 16,384 tokens 81.6 against 86.4 ms, 4,096
+    in workgroups of four wavefronts, two to a compute unit (``alone``: 16,384 tokens 83 against 86.4 ms, 4,096
     tokens 16.0 against 16.4; the result differs by rounding).  The choice is a function of the entries' (padded) lengths
     and of the bound of their keys, so that a recorded step meets the same one again.
 
