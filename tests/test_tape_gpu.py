@@ -135,3 +135,32 @@ def test_steps_from_tapes_equal_steps_part_by_part(name, dtype, tmp_path, monkey
     monkeypatch.setenv("ZEDINFER_DISABLE_TAPES", "1")
     off = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=32, kv_block_size=ps, max_batch_requests=4))
     assert not off.use_tapes
+
+
+def test_a_step_that_allocates_is_not_taped(tmp_path, monkeypatch):
+    """A part that takes device memory while a step runs (against what ``tape_safe`` promises) is noticed when the
+    step is recorded: the recording is dropped, the shape marked, and its steps go on part by part, with the
+    right results."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    from zedinfer_amd.parts.feed_forward import SwiGLU
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "A")
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["A"]
+    e = Engine.from_folder(folder, "float32", SchedulerConfig(num_kv_blocks=64, kv_block_size=ps, max_batch_requests=4))
+    e.use_graphs = False
+    real = SwiGLU.forward
+    kept = []
+
+    def leaky(self, x):
+        kept.append(torch.empty(1024, device=x.device))        # a fresh allocation every call
+        return real(self, x)
+    monkeypatch.setattr(SwiGLU, "forward", leaky)
+    toks = traces.random_tokens(cfg["vocab_size"], 40, seed=1)
+    ref = plain.forward(cfg, w, toks)
+    seq = e.open("r")
+    e.step([StepEntry(seq, toks[:8], [7])])
+    for i in range(8, 40):
+        got = e.step([StepEntry(seq, toks[i:i + 1], [0])]).cpu()
+        assert float((got[0] - ref[i]).abs().max()) < F32_TOL * max(1.0, float(ref.abs().max()))
+    assert e.tape_runs == 0 and any(dg.no_tape for dg in e._graphs.values())
