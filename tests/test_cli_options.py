@@ -1,4 +1,4 @@
-"""The command lines' logging options: the reference's names, levels and defaults
+"""The command lines' logging options (the reference's names, levels and defaults) and text prompts through a supplied tokenizer
 (reference: include/utils/logging_cli.hpp:11-63, include/utils/logging.hpp:56-84)."""
 import argparse
 import logging
@@ -44,3 +44,19 @@ def test_file_console_append_and_overwrite(tmp_path, capsys):
     quiet = init_logger(parser().parse_args(["--log-file", str(tmp_path / "none.log"), "--log-level", "none"]))
     quiet.critical("nothing")
     assert not (tmp_path / "none.log").exists()
+
+
+def test_text_prompts_through_a_supplied_tokenizer(tmp_path):
+    """``ping --prompt`` encodes with a tokenizer.json beside the model (the engine itself is ids in, ids out)."""
+    tokenizers = pytest.importorskip("tokenizers")
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+    from zedinfer_amd.cli.main import load_tokenizer
+    tok = tokenizers.Tokenizer(WordLevel({"[UNK]": 0, "a": 1, "token": 2, "in": 3, "out": 4}, unk_token="[UNK]"))
+    tok.pre_tokenizer = Whitespace()
+    tok.save(str(tmp_path / "tokenizer.json"))
+    loaded = load_tokenizer(str(tmp_path / "tokenizer.json"))
+    assert loaded.encode("a token in a token out").ids == [1, 2, 3, 1, 2, 4]
+    assert loaded.decode([2, 4]) == "token out"
+    with pytest.raises(OSError, match="no tokenizer file"):
+        load_tokenizer(str(tmp_path / "none.json"))

@@ -5,7 +5,8 @@ batch), plus ``random_model``, which writes a model folder with seeded random we
 Option names and meanings are the reference's where it has them (reference:
 examples/ping.cpp:29-115, examples/bench.cpp:23-60,86-145, examples/batch_bench.cpp:27-60,101-180).
 ``--nvidia`` is accepted and ignored: there is one backend.  Text prompts need a tokenizer, which
-this engine does not hold: ``ping`` takes token ids (``--prompt-ids``).
+this engine does not hold: ``ping`` takes token ids (``--prompt-ids``), or text (``--prompt``) when a
+tokenizer.json is supplied, which the `tokenizers` package then reads.
 """
 from __future__ import annotations
 
@@ -79,12 +80,26 @@ def _engine(args):
     return ie
 
 
+def load_tokenizer(path: str):
+    """A tokenizer from a tokenizer.json file, through the `tokenizers` package: a text front-end beside the
+    engine, which itself takes and gives token ids (the reference holds its own tokenizer:
+    src/frontend/tokenizer/base.hpp:17-20)."""
+    if not os.path.isfile(path):
+        raise OSError(f"no tokenizer file at {path}")
+    from tokenizers import Tokenizer
+    return Tokenizer.from_file(path)
+
+
 def ping(argv: Optional[List[str]] = None) -> int:
     p = argparse.ArgumentParser(prog="ping", description="Generate from one prompt")
     _common(p)
     _sampling(p)
     p.add_argument("--prompt-ids", default="1,2,3,4,5,6,7,8",
                    help="prompt as comma-separated token ids (the engine holds no tokenizer)")
+    p.add_argument("--prompt", default=None,
+                   help="prompt as text, for a model folder that holds a tokenizer.json (or with --tokenizer): encoded "
+                        "with the `tokenizers` package, the generated ids are decoded too")
+    p.add_argument("--tokenizer", default=None, help="a tokenizer.json file (default: the one in the model folder)")
     p.add_argument("--max-new-tokens", "--max-tokens", type=int, default=0, dest="max_new_tokens",
                    help="Maximum number of new tokens to generate (0 = unlimited)")
     p.add_argument("--stream", action="store_true", help="Print token ids as they are generated")
@@ -97,8 +112,18 @@ def ping(argv: Optional[List[str]] = None) -> int:
         print("--max-new-tokens/--max-tokens must be >= 0", file=sys.stderr)
         return 1
     from ..engine import GenerationConfig
+    tokenizer = None
+    if args.prompt is not None:
+        try:
+            tokenizer = load_tokenizer(args.tokenizer or os.path.join(args.model_path, "tokenizer.json"))
+        except (OSError, ImportError, ValueError) as e:
+            print(f"--prompt needs a tokenizer: {e}", file=sys.stderr)
+            return 1
     ie = _engine(args)
-    ids = [int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]
+    if tokenizer is not None:
+        ids = tokenizer.encode(args.prompt).ids
+    else:
+        ids = [int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]
     cb = (lambda t: print(t, end=" ", flush=True)) if args.stream else None
     cfg = GenerationConfig(max_new_tokens=args.max_new_tokens, temperature=args.temperature, top_k=args.top_k,
                            top_p=args.top_p, repetition_penalty=args.repetition_penalty, seed=args.seed,
@@ -107,6 +132,8 @@ def ping(argv: Optional[List[str]] = None) -> int:
     if args.stream:
         print()
     print("output_ids:", ",".join(str(t) for t in res.output_ids))
+    if tokenizer is not None:
+        print("output_text:", tokenizer.decode(list(res.output_ids)))
     print("finish_reason:", res.finish_reason)
     print(res.stats.summary())
     return 0
