@@ -365,3 +365,18 @@ def test_requests_without_sampling_options_take_the_default():
     r = req(3)
     s2.submit(r)
     assert r.sampler.params.greedy
+
+
+def test_bounds_that_many_decode_steps_share():
+    """The bound of the sequences' lengths that sizes a decode step's attention launch (and keys its graph):
+    never below the length, a power of two up to 1,024, then steps of 512 (of 2,048 beyond 8,192), so that a
+    batch just past a power of two does not launch twice the workgroups it needs."""
+    from zedinfer_amd.engine.engine import _bucket_at_least
+    assert [_bucket_at_least(n, 256) for n in (1, 256, 257, 600, 1024)] == [256, 256, 512, 1024, 1024]
+    assert [_bucket_at_least(n, 256) for n in (1025, 2049, 2560, 2561, 8192)] == [1536, 2560, 2560, 3072, 8192]
+    assert [_bucket_at_least(n, 256) for n in (8193, 10240, 10241, 32768)] == [10240, 10240, 12288, 32768]
+    last = 0
+    for n in range(1, 40000, 37):
+        b = _bucket_at_least(n, 256)
+        assert b >= n and b >= last and (n <= 1024 or (b - n) * 4 <= n)       # monotone; past 1,024 at most a quarter too wide
+        last = b
