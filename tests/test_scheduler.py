@@ -378,5 +378,5 @@ def test_bounds_that_many_decode_steps_share():
     last = 0
     for n in range(1, 40000, 37):
         b = _bucket_at_least(n, 256)
-        assert b >= n and b >= last and (n <= 1024 or (b - n) * 4 <= n)       # monotone; past 1,024 at most a quarter too wide
+        assert b >= n and b >= last and (n <= 1024 or b - n < (512 if n <= 8192 else 2048))       # monotone, one step at most
         last = b
