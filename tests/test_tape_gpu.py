@@ -164,3 +164,23 @@ def test_a_step_that_allocates_is_not_taped(tmp_path, monkeypatch):
         got = e.step([StepEntry(seq, toks[i:i + 1], [0])]).cpu()
         assert float((got[0] - ref[i]).abs().max()) < F32_TOL * max(1.0, float(ref.abs().max()))
     assert e.tape_runs == 0 and any(dg.no_tape for dg in e._graphs.values())
+
+
+def test_generation_from_tapes_alone(tmp_path, monkeypatch):
+    """The serving loop (continuous batching, chunked prefill, steps queued ahead) with graphs switched off: the
+    recurring steps run from tapes, and every request gets the plain implementation's greedy tokens."""
+    from zedinfer_amd import GenerationConfig, InferenceEngine, SchedulerConfig
+    monkeypatch.setenv("ZEDINFER_DISABLE_GRAPHS", "1")
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "B")
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["B"]
+    ie = InferenceEngine.create(folder, "float32", SchedulerConfig(num_kv_blocks=96, kv_block_size=ps, max_batch_requests=3,
+                                                                   max_prefill_tokens=64, max_batch_tokens=80))
+    assert not ie.engine.use_graphs and ie.engine.use_tapes
+    prompts = [traces.random_tokens(cfg["vocab_size"], n, seed=20 + i) for i, n in enumerate([130, 64, 7, 128, 50])]
+    results = ie.generate(prompts, GenerationConfig(max_new_tokens=24, ignore_eos=True))
+    for prompt, res in zip(prompts, results):
+        assert res.output_ids == plain.greedy_generate(cfg, w, prompt, 24)
+    assert ie.engine.tape_runs > 20 and ie.engine.graph_replays == 0
+    ie.engine.cache.check()
+    assert not ie.engine.cache.live
