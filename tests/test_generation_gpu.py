@@ -527,6 +527,35 @@ def test_graphs_that_are_dropped_and_recorded_again(tiny):
     assert fast.graph_replays >= 10 and fast.prompt_graph_replays >= 5
 
 
+def test_steps_of_many_rows_come_in_the_sizes_the_warm_up_measured(tmp_path):
+    """A serving engine on bfloat16 weights measures the library's algorithms for its many-rows products at every
+    multiple of 64 rows a step can bring; portions of prompts beside decoding requests then run with their
+    decoding entries filled up to a multiple of 64, so every such step's rows are among the measured sizes; the
+    tokens are the plain implementation's."""
+    from zedinfer_amd import GenerationConfig, InferenceEngine, SchedulerConfig
+    from zedinfer_amd.engine.engine import many_rows_step_sizes
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "B", dtype=torch.bfloat16, std=tiny_configs.SHARP_STD)
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["B"]
+    ie = InferenceEngine.create(folder, "bfloat16", SchedulerConfig(num_kv_blocks=160, kv_block_size=ps, max_batch_requests=4,
+                                                                    max_prefill_tokens=192, max_batch_tokens=256))
+    eng = ie.engine
+    measured = {k[1] for k in eng.rt.choices if k[0] == "library_product"}
+    assert measured == set(many_rows_step_sizes(192 + 4 + 64)) == {320, 256, 192, 128}
+    prompts = [traces.random_tokens(cfg["vocab_size"], n, seed=70 + i) for i, n in enumerate([250, 200, 130, 70])]
+    results = ie.generate(prompts, GenerationConfig(max_new_tokens=12, ignore_eos=True))
+    mixed = [k for k in eng._prompt_graphs if k[1] > 0]             # (entries, decoding entries, sizes of the portions, ...)
+    assert mixed and all(k[1] % 64 == 0 and (sum(k[2]) + k[1]) in measured for k in mixed), mixed
+    # bfloat16 may break a near tie the other way: every token that was generated must be, for the plain
+    # implementation fed the same tokens, the best or within the bfloat16 tolerance of the best
+    for prompt, res in zip(prompts, results):
+        assert len(res.output_ids) == 12
+        ref = plain.forward(cfg, w, list(prompt) + res.output_ids)[len(prompt) - 1:-1]
+        taken = ref[torch.arange(12), torch.tensor(res.output_ids)]
+        assert bool((taken >= ref.max(dim=1).values - 0.06 * float(ref.abs().max())).all()), (taken, ref.max(dim=1).values)
+    eng.cache.check()
+
+
 def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatch, tmp_path):
     """Pure decode steps of few tokens rotate, store and attend in one kernel.  With that path switched
     off the same steps give the same logits (the caches hold the same keys and values, so later steps

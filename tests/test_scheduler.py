@@ -380,3 +380,13 @@ def test_bounds_that_many_decode_steps_share():
         b = _bucket_at_least(n, 256)
         assert b >= n and b >= last and (n <= 1024 or b - n < (512 if n <= 8192 else 2048))       # monotone, one step at most
         last = b
+
+
+def test_sizes_at_which_a_serving_engine_measures_its_choices():
+    """The multiples of the step that portions of prompts are padded to, from 128 rows to the most a step can
+    bring, largest first."""
+    from zedinfer_amd.engine.engine import Engine, many_rows_step_sizes
+    assert Engine.PROMPT_GRAPH_STEP == 64
+    assert many_rows_step_sizes(300) == [320, 256, 192, 128]
+    assert many_rows_step_sizes(2112) == list(range(2112, 127, -64))
+    assert many_rows_step_sizes(64) == [] and many_rows_step_sizes(100) == [128]

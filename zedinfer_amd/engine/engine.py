@@ -10,7 +10,7 @@ block tables before the run and commits the new lengths after it.
 from __future__ import annotations
 
 import os
-from typing import Dict, Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -327,9 +327,13 @@ class Engine:
         wanted = sum(len(e.want) for e in entries)
         E, R, more_entries = len(entries), wanted, 0
         if E > 1:
-            # the numbers of portions and of decoding requests move from step to step: the entries are brought
-            # to a multiple of 8 with entries that belong to no request, and a row is wanted of every entry
-            more_entries = -(-E // 8) * 8 - E
+            # the numbers of portions and of decoding requests move from step to step: the decoding entries are
+            # brought to a multiple of PROMPT_GRAPH_STEP with entries that belong to no request, and a row is
+            # wanted of every entry.  The step's rows are then a multiple of that step as well: fewer shapes, and
+            # the many-rows products come in the numbers of rows that a warm-up has measured
+            # (``many_rows_step_sizes``).
+            decoding = E - len(portions)
+            more_entries = -(-decoding // step) * step - decoding
             E += more_entries
             R = E
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
@@ -383,6 +387,15 @@ class _DecodeGraph:
         self.tape = None                                # the library calls of one step of the shape
         self.no_tape = False                            # a step of the shape cannot be recorded
         self.image: Optional[DecodeImage] = None
+
+
+def many_rows_step_sizes(most_tokens: int, step: int = Engine.PROMPT_GRAPH_STEP, least: int = 128) -> List[int]:
+    """The numbers of rows that steps with portions of prompts come in, up to ``most_tokens`` tokens a step:
+    portions are run as multiples of ``step`` tokens and decoding entries beside them in multiples of ``step``
+    (``Engine._prompt_graph_step``), so these are the multiples of ``step`` (from ``least``: fewer rows go to
+    the few-rows kernels or are not worth measuring).  Largest first: workspaces get their final sizes at once."""
+    top = -(-int(most_tokens) // step) * step
+    return [n for n in range(top, 0, -step) if n >= least]
 
 
 def _bucket_at_least(n: int, floor: int = 1) -> int:

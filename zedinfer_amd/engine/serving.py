@@ -17,7 +17,7 @@ import torch
 from ..config import SchedulerConfig
 from ..ops.staging import StagingRing
 from ..sampling.sampler import Sampler
-from .engine import Engine
+from .engine import Engine, many_rows_step_sizes
 from .request import GenerationConfig, GenerationResult, InferenceRequest
 from .scheduler import ScheduledBatch, Scheduler
 
@@ -156,10 +156,15 @@ class InferenceEngine:
     def __init__(self, engine: Engine):
         self.engine = engine
         self._loop = ServingLoop(engine, engine.fc.eos_token_ids)
-        # The size of a full portion of a prompt is the one many-rows step that recurs: its products' algorithms
-        # (and other choices of the parts) are measured now, once (ZEDINFER_WARM_UP=0: the defaults).
+        # The products' algorithms (and other choices of the parts) for steps of many rows are measured now, once
+        # (ZEDINFER_WARM_UP=0: the defaults), at every number of rows that steps with portions of prompts come
+        # in: the library's first proposal for a shape can be a third slower than what timing finds, and what
+        # timing finds for one number of rows does not carry over to its neighbours (measured; see
+        # ``many_rows_step_sizes``).
         if os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and engine.device.type == "cuda":
-            engine.warm_up([engine.sched.max_prefill_tokens])
+            sched = engine.sched
+            most = min(sched.max_batch_tokens, sched.max_prefill_tokens + sched.max_batch_requests)
+            engine.warm_up(many_rows_step_sizes(most + Engine.PROMPT_GRAPH_STEP))       # a portion and the decoding entries are rounded up
         # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
         # taken out of the garbage collector's passes, a full collection in the middle of serving costs
         # little (measured: one of 50 ms among decode steps of 6.5 ms without this).
