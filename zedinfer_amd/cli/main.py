@@ -58,7 +58,9 @@ def _sampling(p: argparse.ArgumentParser) -> None:
     p.add_argument("--repetition-penalty", type=float, default=1.0)
 
 
-def _engine(args):
+def _engine(args, step_tokens: Optional[List[int]] = None):
+    """The serving engine the options describe.  ``step_tokens``: the program's steps of many tokens bring these
+    numbers of tokens only, so the engine measures its choices for them instead of for every size."""
     from ..config import SchedulerConfig, load_config
     from ..engine import Engine, InferenceEngine
     sched = SchedulerConfig(max_batch_tokens=args.max_batch_tokens, max_batch_requests=args.max_batch_requests,
@@ -75,7 +77,11 @@ def _engine(args):
     log = logging.getLogger("zedinfer_amd")
     log.info("Engine initialized in %.0f ms (%d pages of %d tokens)", (time.perf_counter() - t0) * 1000,
              eng.cache.num_pages, eng.cache.page_size)
-    ie = InferenceEngine(eng)
+    sizes = None
+    if step_tokens is not None:
+        step = Engine.PROMPT_GRAPH_STEP
+        sizes = sorted({-(-n // step) * step for n in step_tokens if n > step}, reverse=True)
+    ie = InferenceEngine(eng, warm_up_sizes=sizes)
     log.debug("choices made at warm-up: %s", eng.rt.choices)
     return ie
 
@@ -119,11 +125,12 @@ def ping(argv: Optional[List[str]] = None) -> int:
         except (OSError, ImportError, ValueError) as e:
             print(f"--prompt needs a tokenizer: {e}", file=sys.stderr)
             return 1
-    ie = _engine(args)
     if tokenizer is not None:
         ids = tokenizer.encode(args.prompt).ids
     else:
         ids = [int(t) for t in args.prompt_ids.replace(" ", "").split(",") if t]
+    # one prompt: its full portions and the last one are the only steps of many tokens
+    ie = _engine(args, [min(len(ids), args.max_prefill_tokens), len(ids) % max(args.max_prefill_tokens, 1)])
     cb = (lambda t: print(t, end=" ", flush=True)) if args.stream else None
     cfg = GenerationConfig(max_new_tokens=args.max_new_tokens, temperature=args.temperature, top_k=args.top_k,
                            top_p=args.top_p, repetition_penalty=args.repetition_penalty, seed=args.seed,
@@ -154,7 +161,7 @@ def bench(argv: Optional[List[str]] = None) -> int:
         return 1
     from ..engine.profiler import Profiler
     args.max_batch_tokens = max(args.max_batch_tokens, args.prefill_len)
-    ie = _engine(args)
+    ie = _engine(args, [args.prefill_len])          # the prompt enters in one step
     prof = Profiler(ie.engine)
     prof.warmup(args.prefill_len, args.decode_len)
     tp = td = 0.0

@@ -153,7 +153,9 @@ class ServingLoop:
 class InferenceEngine:
     """Everything for generation from one model folder."""
 
-    def __init__(self, engine: Engine):
+    def __init__(self, engine: Engine, warm_up_sizes: Optional[Sequence[int]] = None):
+        """``warm_up_sizes``: the numbers of rows to measure the parts' choices for (None: every size a step with
+        prompt portions can bring under the scheduler's limits; empty: none)."""
         self.engine = engine
         self._loop = ServingLoop(engine, engine.fc.eos_token_ids)
         # The products' algorithms (and other choices of the parts) for steps of many rows are measured now, once
@@ -164,7 +166,9 @@ class InferenceEngine:
         if os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and engine.device.type == "cuda":
             sched = engine.sched
             most = min(sched.max_batch_tokens, sched.max_prefill_tokens + sched.max_batch_requests)
-            engine.warm_up(many_rows_step_sizes(most + Engine.PROMPT_GRAPH_STEP))       # a portion and the decoding entries are rounded up
+            if warm_up_sizes is None:       # a portion and the decoding entries are rounded up: one more size
+                warm_up_sizes = many_rows_step_sizes(most + Engine.PROMPT_GRAPH_STEP)
+            engine.warm_up(list(warm_up_sizes))
         # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
         # taken out of the garbage collector's passes, a full collection in the middle of serving costs
         # little (measured: one of 50 ms among decode steps of 6.5 ms without this).
@@ -174,9 +178,9 @@ class InferenceEngine:
             gc.freeze()
 
     @classmethod
-    def create(cls, model_path: str, dtype="bfloat16", scheduler_config: Optional[SchedulerConfig] = None
-               ) -> "InferenceEngine":
-        return cls(Engine.from_folder(model_path, dtype, scheduler_config))
+    def create(cls, model_path: str, dtype="bfloat16", scheduler_config: Optional[SchedulerConfig] = None,
+               warm_up_sizes: Optional[Sequence[int]] = None) -> "InferenceEngine":
+        return cls(Engine.from_folder(model_path, dtype, scheduler_config), warm_up_sizes)
 
     @property
     def default_sampling(self):
