@@ -74,13 +74,14 @@ def rand_ids(rng, n, vocab):
     return [rng.randrange(100, vocab - 100) for _ in range(n)]
 
 
-def measure_decode(engine_factory, batch, steps, warmup, vocab, prompt_len=PROMPT):
+def measure_decode(engine_factory, batch, steps, warmup, vocab, prompt_len=PROMPT, warm_up_sizes=None):
     """tokens a second and ms a step of `steps` decode steps with `batch` running requests that each
-    hold a prompt of `prompt_len` tokens."""
+    hold a prompt of `prompt_len` tokens.  `warm_up_sizes`: the numbers of rows the serving engine measures its
+    choices for before (None: every size its steps can bring)."""
     import torch
     from zedinfer_amd import GenerationConfig, InferenceRequest
     from zedinfer_amd.engine import InferenceEngine
-    ie = InferenceEngine(engine_factory())
+    ie = InferenceEngine(engine_factory(), warm_up_sizes=warm_up_sizes)
     loop = ie.serving_loop()
     rng = random.Random(1234 + batch)
     reqs = [loop.submit_async(InferenceRequest(rand_ids(rng, prompt_len, vocab),
@@ -194,6 +195,50 @@ def further_7b(args):
     return res
 
 
+def further_32b(args):
+    """Decode at batch 8 with 8,192-token prompts and the prefill of one 16,384-token prompt in one step, at the
+    Qwen2.5-32B sizes (64 layers, 65 GB of weights)."""
+    import torch
+    from zedinfer_amd.config import Qwen2Config, SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    shape = dict(SHAPE, **SHAPES["32B"])
+    cfg = Qwen2Config.from_dict(shape)
+    L, el, batch, prompt, long_prompt = shape["num_hidden_layers"], 2, 8, 8192, 16384
+    steps, warm = min(args.steps, 24), min(args.warmup, 4)
+    holder = {}
+
+    def decode_engine():
+        tokens = prompt + warm + steps + 2 * batch + 64
+        sched = SchedulerConfig(num_kv_blocks=batch * (-(-tokens // 16)) + 16, kv_block_size=16, max_batch_requests=batch,
+                                max_batch_tokens=prompt + batch, max_prefill_tokens=prompt, max_seq_len=2 * prompt)
+        holder["e"] = Engine.from_config(cfg, "Qwen2ForCausalLM", args.dtype, seed=0, sched=sched)
+        return holder["e"]
+    # the prompts enter whole, alone or beside the requests that decode already: the two sizes of such steps
+    from zedinfer_amd.engine.engine import many_rows_size_at_least
+    tps, ms_step, ctx_mid = measure_decode(decode_engine, batch, steps, warm, cfg.vocab_size, prompt,
+                                           warm_up_sizes=[many_rows_size_at_least(prompt + 64), prompt])
+    need = decode_bytes(shape, L, batch, ctx_mid, el)
+    achieved = need / (ms_step / 1000.0) / 1e9
+    res = {"config": {"model": "Qwen2.5-32B shape", "num_layers": L, "layers_run": L, "hidden": cfg.hidden_size,
+                      "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                      "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": False,
+                      "kv_page_tokens": 16, "context_len": 2 * prompt, "dtype": args.dtype},
+           "decode_b8": {"value": round(tps, 2), "unit": "tok/s", "ms_per_step": round(ms_step, 4), "seq_len": prompt,
+                         "steps": steps, "roofline_achieved_gbs": round(achieved, 1),
+                         "roofline_frac": round(achieved / HBM_PEAK_GBS, 4)}}
+    torch.cuda.empty_cache()
+
+    def prefill_engine():
+        sched = SchedulerConfig(num_kv_blocks=long_prompt // 16 + 16, kv_block_size=16, max_batch_requests=1,
+                                max_batch_tokens=long_prompt + 1, max_prefill_tokens=long_prompt, max_seq_len=2 * long_prompt)
+        return holder["e"].with_cache(sched)
+    pms = measure_prefill(prefill_engine, cfg.vocab_size, rounds=2, tokens=long_prompt)
+    fl = prefill_flops(shape, L, long_prompt)
+    res["prefill_16384"] = {"value": round(long_prompt / pms * 1000.0, 1), "unit": "tok/s", "tokens": long_prompt,
+                            "ms": round(pms, 2), "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -209,7 +254,7 @@ def main():
                     help="instead: continuous batching of R requests, prompts uniform in [128, 4096], 256 greedy "
                          "tokens each, prompts cut at 2,048 tokens a step")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
-    ap.add_argument("--no-further", action="store_true", help="skip the figures at the 7B sizes")
+    ap.add_argument("--no-further", action="store_true", help="skip the figures at the 7B and 32B sizes")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
     args = ap.parse_args()
@@ -312,6 +357,9 @@ def main():
             weights_cache.clear()
             torch.cuda.empty_cache()
             out["further"] = further_7b(args)
+            gc.collect()
+            torch.cuda.empty_cache()
+            out["further_32b"] = further_32b(args)
     out["choices"] = CHOICES
     print(json.dumps(out))
     return 0

@@ -384,9 +384,16 @@ def test_bounds_that_many_decode_steps_share():
 
 def test_sizes_at_which_a_serving_engine_measures_its_choices():
     """The multiples of the step that portions of prompts are padded to, from 128 rows to the most a step can
-    bring, largest first."""
-    from zedinfer_amd.engine.engine import Engine, many_rows_step_sizes
+    bring, largest first; beyond 4,096 rows they lie further apart (32 an octave), and every number of rows has
+    one at most a 32nd above it."""
+    from zedinfer_amd.engine.engine import Engine, many_rows_size_at_least, many_rows_step_sizes
     assert Engine.PROMPT_GRAPH_STEP == 64
     assert many_rows_step_sizes(300) == [320, 256, 192, 128]
     assert many_rows_step_sizes(2112) == list(range(2112, 127, -64))
     assert many_rows_step_sizes(64) == [] and many_rows_step_sizes(100) == [128]
+    assert many_rows_step_sizes(4300)[:4] == [4352, 4224, 4096, 4032]
+    sizes = many_rows_step_sizes(20000)
+    assert sizes[0] == 20480 and len(sizes) == 63 + 32 + 32 + 8
+    for n in range(128, 20001, 7):
+        up = many_rows_size_at_least(n)
+        assert up in sizes and n <= up <= n + max(63, n // 32), n

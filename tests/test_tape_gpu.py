@@ -184,3 +184,35 @@ def test_generation_from_tapes_alone(tmp_path, monkeypatch):
     assert ie.engine.tape_runs > 20 and ie.engine.graph_replays == 0
     ie.engine.cache.check()
     assert not ie.engine.cache.live
+
+
+def test_a_large_step_is_brought_up_to_a_measured_size(tmp_path):
+    """Beyond 4,096 rows the sizes that a serving engine measures lie 128 rows apart: a step of 4,170 prompt tokens
+    beside one decoding request (4,224 + 64 rows) gets 64 more padding tokens behind the portion.  Nothing of a
+    request changes by that: the logits of the step and of the decode steps after it are the plain
+    implementation's."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    from zedinfer_amd.engine.engine import many_rows_size_at_least
+    assert [many_rows_size_at_least(n) for n in (4096, 4097, 4288, 8192, 8200)] == [4096, 4224, 4352, 8192, 8448]
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "A")
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["A"]
+    e = Engine.from_folder(folder, "float32", SchedulerConfig(num_kv_blocks=4400 // ps + 8, kv_block_size=ps, max_batch_requests=4,
+                                                              max_seq_len=8192))
+    e.use_graphs = False
+    long_toks = traces.random_tokens(cfg["vocab_size"], 4174, seed=5)
+    short_toks = traces.random_tokens(cfg["vocab_size"], 36, seed=6)
+    a, b = e.open("a"), e.open("b")
+    e.step([StepEntry(b, short_toks[:30], [])])
+    got = e.step([StepEntry(a, long_toks[:4170], [4169]), StepEntry(b, short_toks[30:31], [0])]).cpu()
+    keys = [k for k in e._prompt_graphs if k[1] > 0]
+    assert keys == [k for k in keys if k[2] == (4288,) and k[0] == 65], list(e._prompt_graphs)
+    ref_a, ref_b = plain.forward(cfg, w, long_toks), plain.forward(cfg, w, short_toks)
+    tol = F32_TOL * max(1.0, float(ref_a.abs().max()), float(ref_b.abs().max()))
+    assert float((got[0] - ref_a[4169]).abs().max()) < tol and float((got[1] - ref_b[30]).abs().max()) < tol
+    for i in range(4):
+        got = e.step([StepEntry(a, long_toks[4170 + i:4171 + i], [0]), StepEntry(b, short_toks[31 + i:32 + i], [0])]).cpu()
+        assert float((got[0] - ref_a[4170 + i]).abs().max()) < tol and float((got[1] - ref_b[31 + i]).abs().max()) < tol
+    assert a.length == 4174 and b.length == 35
+    e.cache.check()

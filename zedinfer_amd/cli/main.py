@@ -79,8 +79,8 @@ def _engine(args, step_tokens: Optional[List[int]] = None):
              eng.cache.num_pages, eng.cache.page_size)
     sizes = None
     if step_tokens is not None:
-        step = Engine.PROMPT_GRAPH_STEP
-        sizes = sorted({-(-n // step) * step for n in step_tokens if n > step}, reverse=True)
+        from ..engine.engine import many_rows_size_at_least
+        sizes = sorted({many_rows_size_at_least(n) for n in step_tokens if n > Engine.PROMPT_GRAPH_STEP}, reverse=True)
     ie = InferenceEngine(eng, warm_up_sizes=sizes)
     log.debug("choices made at warm-up: %s", eng.rt.choices)
     return ie

@@ -87,14 +87,15 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
                        device: torch.device, staging: Optional[StagingRing] = None,
                        table_widths: Optional[Sequence[int]] = None,
                        static: Optional[torch.Tensor] = None, pad_to: int = 0, pad_entries: int = 0,
-                       pad_rows: int = 0, planners: Sequence[StepPlanner] = (), position_axes: int = 1,
+                       pad_rows: int = 0, pad_more: int = 0, planners: Sequence[StepPlanner] = (), position_axes: int = 1,
                        bound_single: int = 0, bound_multi: int = 0) -> DeviceBatch:
     """Check the entries, then pack every index array into one host buffer and copy it over once.
 
     ``pad_to``: every entry that brings more than one token is run as if it brought a multiple of that
     many.  The tokens past its own are token 0 at the positions that follow; they have no place in the cache
     (slot -1: nothing is stored for them) and no real token sees them, so they change nothing but the
-    shapes, which then recur from step to step.  ``pad_entries`` adds that many entries of one token that
+    shapes, which then recur from step to step.  ``pad_more``: that many more such tokens behind the longest
+    entry's.  ``pad_entries`` adds that many entries of one token that
     belong to no request (token 0 at position 0, no slot, an empty block table, state slot 0),
     ``pad_rows`` that many wanted rows after the real ones (the first token's), to the same end.  Only for
     models whose mixers all say ``padding_safe``.
@@ -132,6 +133,11 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     real = list(lens)
     if pad_to:
         lens = [-(-n // int(pad_to)) * int(pad_to) if n > 1 else n for n in lens]
+    if pad_more:
+        longest = max(range(len(lens)), key=lambda i: lens[i])
+        if lens[longest] <= 1:
+            raise ValueError("more padding needs an entry of several tokens to stand behind")
+        lens[longest] += int(pad_more)
     N = int(sum(lens))
     starts = np.zeros(E, dtype=np.int32)
     starts[1:] = np.cumsum(lens)[:-1]

@@ -336,9 +336,16 @@ class Engine:
             more_entries = -(-decoding // step) * step - decoding
             E += more_entries
             R = E
+        # beyond 4,096 rows the measured sizes lie further apart: the step is brought up to the next one with
+        # more padding behind its longest portion (at most a 32nd more rows)
+        rows = padded + (E - len(portions))
+        more_tokens = many_rows_size_at_least(rows) - rows
+        if more_tokens:
+            sizes = tuple(sorted(sizes[:-1] + (sizes[-1] + more_tokens,)))
+            padded += more_tokens
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
-        long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions), 2048)
+        long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions) + more_tokens, 2048)
         short_bucket = _bucket_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
         singles = len(entries) - len(portions) + more_entries
         # everything the launches' sizes depend on: the portions' sizes one by one (the planners cut each into
@@ -352,7 +359,7 @@ class Engine:
                 self._drop_oldest(self._prompt_graphs)
             dg = self._prompt_graphs[key] = _DecodeGraph()
         batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
-                                   pad_to=step, pad_entries=more_entries, pad_rows=R - wanted,
+                                   pad_to=step, pad_more=more_tokens, pad_entries=more_entries, pad_rows=R - wanted,
                                    planners=self.planners, position_axes=self.position_axes,
                                    bound_single=short_bucket if singles else 0, bound_multi=long_bucket)
         dg.buffer = batch.device_image          # the first step's buffer serves all later ones of the shape
@@ -389,13 +396,34 @@ class _DecodeGraph:
         self.image: Optional[DecodeImage] = None
 
 
+def _many_rows_spacing(rows: int, step: int) -> int:
+    top, s = 64 * step, step
+    while rows > top:
+        top, s = 2 * top, 2 * s
+    return s
+
+
+def many_rows_size_at_least(rows: int, step: int = Engine.PROMPT_GRAPH_STEP) -> int:
+    """The number of rows a step of ``rows`` rows is run with: the next multiple of ``step`` up to 4,096 rows, of
+    2 x ``step`` up to 8,192, of 4 x ``step`` up to 16,384 and so on (32 sizes an octave: measuring every size
+    when an engine is made stays affordable, and a step gets at most a 32nd more rows)."""
+    rows = max(int(rows), 1)
+    s = _many_rows_spacing(rows, step)
+    return -(-rows // s) * s
+
+
 def many_rows_step_sizes(most_tokens: int, step: int = Engine.PROMPT_GRAPH_STEP, least: int = 128) -> List[int]:
     """The numbers of rows that steps with portions of prompts come in, up to ``most_tokens`` tokens a step:
-    portions are run as multiples of ``step`` tokens and decoding entries beside them in multiples of ``step``
-    (``Engine._prompt_graph_step``), so these are the multiples of ``step`` (from ``least``: fewer rows go to
-    the few-rows kernels or are not worth measuring).  Largest first: workspaces get their final sizes at once."""
-    top = -(-int(most_tokens) // step) * step
-    return [n for n in range(top, 0, -step) if n >= least]
+    portions are run as multiples of ``step`` tokens, decoding entries beside them in multiples of ``step``, and
+    large steps are brought up to sizes further apart (``Engine._prompt_graph_step``,
+    ``many_rows_size_at_least``).  From ``least`` rows on: fewer go to the few-rows kernels or are not worth
+    measuring.  Largest first: workspaces get their final sizes at once."""
+    sizes, n = [], many_rows_size_at_least(most_tokens, step)
+    while n >= least:
+        sizes.append(n)
+        s = _many_rows_spacing(n - 1, step)
+        n = (n - 1) // s * s
+    return sizes
 
 
 def _bucket_at_least(n: int, floor: int = 1) -> int:

@@ -746,12 +746,20 @@ def _library_product(out, x, weight, bias, transposed) -> None:
 
 
 def linear_tune(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None, transposed: bool = False,
-                out_dtype: Optional[torch.dtype] = None, candidates: int = 16, rounds: int = 5):
+                out_dtype: Optional[torch.dtype] = None, candidates: Optional[int] = None, rounds: Optional[int] = None):
     """Let the library time its proposals for the product ``linear`` (``linear_transposed``) makes of these operands
     and keep the fastest for every later call of the shape; returns (chosen, proposed, microseconds), or None when
-    the product is not the library's (few rows, float32 operands).  Waits for the device."""
+    the product is not the library's (few rows, float32 operands).  Waits for the device.  ``candidates``: how
+    many of the proposals are timed (None: the first 16, the first 8 of a product of about 250 us and more);
+    ``rounds``: timed runs of each (None: five of a short product, fewer of one that takes long enough for the
+    clock: three beyond about 50 us, two beyond 250)."""
     bf = torch.bfloat16
     M, N = x.shape[0], weight.shape[0]
+    about_us = 2.0 * M * N * x.shape[1] / 1e9        # at a petaflop a second
+    if rounds is None:
+        rounds = 5 if about_us < 50 else (3 if about_us < 250 else 2)
+    if candidates is None:
+        candidates = 16 if about_us < 250 else 8
     out_dtype = out_dtype or bf
     if x.dtype != bf or weight.dtype != bf or (bias is not None and bias.dtype != bf):
         return None
