@@ -297,7 +297,10 @@ class Engine:
 
     # ---- one portion of one prompt as a graph -------------------------------------------
     PROMPT_GRAPH_STEP = 64
-    TAPE_MAX_TOKENS = 8192      # padded tokens of the portions of a step that is still run from a tape
+    # padded tokens of the portions of a step that is still padded and run from a tape (a step of many tokens does
+    # not need the tape, the GPU takes far longer than the host, but its padded rows are a size whose library
+    # products can have been measured)
+    TAPE_MAX_TOKENS = 32768
 
     def _one_portion(self, entries: Sequence[StepEntry]) -> bool:
         """Portions of prompts (entries of several tokens) of a size worth a graph together, beside any

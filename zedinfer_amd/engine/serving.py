@@ -17,7 +17,7 @@ import torch
 from ..config import SchedulerConfig
 from ..ops.staging import StagingRing
 from ..sampling.sampler import Sampler
-from .engine import Engine, many_rows_step_sizes
+from .engine import Engine, many_rows_size_at_least, many_rows_step_sizes
 from .request import GenerationConfig, GenerationResult, InferenceRequest
 from .scheduler import ScheduledBatch, Scheduler
 
@@ -153,6 +153,8 @@ class ServingLoop:
 class InferenceEngine:
     """Everything for generation from one model folder."""
 
+    WARM_UP_EVERY_SIZE_UP_TO = 8192     # rows; measuring every size of longer steps would take minutes
+
     def __init__(self, engine: Engine, warm_up_sizes: Optional[Sequence[int]] = None):
         """``warm_up_sizes``: the numbers of rows to measure the parts' choices for (None: every size a step with
         prompt portions can bring under the scheduler's limits; empty: none)."""
@@ -167,7 +169,13 @@ class InferenceEngine:
             sched = engine.sched
             most = min(sched.max_batch_tokens, sched.max_prefill_tokens + sched.max_batch_requests)
             if warm_up_sizes is None:       # a portion and the decoding entries are rounded up: one more size
-                warm_up_sizes = many_rows_step_sizes(most + Engine.PROMPT_GRAPH_STEP)
+                step = Engine.PROMPT_GRAPH_STEP
+                warm_up_sizes = many_rows_step_sizes(min(most, self.WARM_UP_EVERY_SIZE_UP_TO) + step)
+                if most > self.WARM_UP_EVERY_SIZE_UP_TO:
+                    # of longer steps only the ones that recur: a full portion, alone and beside decoding requests
+                    full = sorted({many_rows_size_at_least(sched.max_prefill_tokens),
+                                   many_rows_size_at_least(min(most, sched.max_prefill_tokens + step) + step)}, reverse=True)
+                    warm_up_sizes = [n for n in full if n > warm_up_sizes[0]] + warm_up_sizes
             engine.warm_up(list(warm_up_sizes))
         # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
         # taken out of the garbage collector's passes, a full collection in the middle of serving costs
