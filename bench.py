@@ -198,8 +198,9 @@ def further_7b(args):
 
 
 def further_32b(args):
-    """Decode at batch 8 with 8,192-token prompts and the prefill of one 16,384-token prompt in one step, at the
-    Qwen2.5-32B sizes (64 layers, 65 GB of weights)."""
+    """Decode at batch 8 and 1 with 8,192-token prompts and the prefill of one 16,384-token prompt in one step, at
+    the Qwen2.5-32B sizes (64 layers, 65 GB of weights; batch 64 holds 139 GB of keys and values and takes half a
+    minute to prefill: `--shape 32B --batch 64 --prompt-len 8192` measures it)."""
     import torch
     from zedinfer_amd.config import Qwen2Config, SchedulerConfig
     from zedinfer_amd.engine import Engine
@@ -228,6 +229,12 @@ def further_32b(args):
            "decode_b8": {"value": round(tps, 2), "unit": "tok/s", "ms_per_step": round(ms_step, 4), "seq_len": prompt,
                          "steps": steps, "roofline_achieved_gbs": round(achieved, 1),
                          "roofline_frac": round(achieved / HBM_PEAK_GBS, 4)}}
+    torch.cuda.empty_cache()
+    one, _, _ = measure_decode(lambda: holder["e"].with_cache(SchedulerConfig(
+        num_kv_blocks=(prompt + warm + steps + 128) // 16 + 16, kv_block_size=16, max_batch_requests=1,
+        max_batch_tokens=prompt + 1, max_prefill_tokens=prompt, max_seq_len=2 * prompt)), 1, steps, warm, cfg.vocab_size,
+        prompt, warm_up_sizes=[prompt])
+    res["decode_b1"] = {"value": round(one, 2), "unit": "tok/s", "seq_len": prompt}
     torch.cuda.empty_cache()
 
     def prefill_engine():
