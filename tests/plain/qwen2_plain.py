@@ -103,12 +103,18 @@ def argmax_lowest_index(logits: torch.Tensor) -> int:
 # --------------------------------------------------------------------------
 def attention_block(x, w: Dict[str, torch.Tensor], p: str, cfg: dict, pos, window):
     """q/k/v projections with biases, rotation of q and k, attention, output projection
-    without bias (src/frontend/models/transformer_forward.cpp:71-78, :99-112)."""
+    without bias (src/frontend/models/transformer_forward.cpp:71-78, :99-112).  When the weights hold
+    ``self_attn.q_norm.weight`` and ``self_attn.k_norm.weight`` [head_dim], every query and key head is RMS-normed
+    over head_dim before the rotation (:80-96; Qwen2 checkpoints hold none)."""
     T = x.shape[0]
     nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
     q = linear(x, w[p + "self_attn.q_proj.weight"], w.get(p + "self_attn.q_proj.bias"))
     k = linear(x, w[p + "self_attn.k_proj.weight"], w.get(p + "self_attn.k_proj.bias"))
     v = linear(x, w[p + "self_attn.v_proj.weight"], w.get(p + "self_attn.v_proj.bias"))
+    if p + "self_attn.q_norm.weight" in w:
+        eps = cfg.get("rms_norm_eps", 1e-6)
+        q = rms_norm(q.view(T, nh, d), w[p + "self_attn.q_norm.weight"], eps).reshape(T, nh * d)
+        k = rms_norm(k.view(T, nkv, d), w[p + "self_attn.k_norm.weight"], eps).reshape(T, nkv * d)
     q = rope_neox(q.view(T, nh, d), pos, cfg["rope_theta"])
     k = rope_neox(k.view(T, nkv, d), pos, cfg["rope_theta"])
     a = causal_gqa_attention(q, k, v.view(T, nkv, d), 1.0 / math.sqrt(d), window)

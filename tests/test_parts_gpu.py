@@ -226,10 +226,13 @@ def test_rope_part_rotates_queries_and_stores_keys(dtype, rotary_dim):
 
 # ---- mixer ------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("nh,nkv,d,window,bias", [(6, 2, 32, 0, True), (5, 1, 48, 11, False), (4, 4, 64, 0, True)])
-def test_attention_part_in_portions(dtype, nh, nkv, d, window, bias):
+@pytest.mark.parametrize("nh,nkv,d,window,bias,qk_norm", [(6, 2, 32, 0, True, False), (5, 1, 48, 11, False, False),
+                                                          (4, 4, 64, 0, True, False), (6, 2, 32, 0, True, True),
+                                                          (5, 1, 48, 11, False, True)])
+def test_attention_part_in_portions(dtype, nh, nkv, d, window, bias, qk_norm):
     """The attention mixer alone, fed a sequence in portions (a long one, then short ones and single
-    tokens), against the plain attention block over the whole sequence."""
+    tokens), against the plain attention block over the whole sequence; also with every query and key head
+    normed before the rotation (an option of the part that the architecture built here does not use)."""
     from zedinfer_amd.cache.manager import CacheManager
     from zedinfer_amd.parts import MIXERS
     H, T, ps, theta = 88, 61, 8, 7e3
@@ -240,10 +243,14 @@ def test_attention_part_in_portions(dtype, nh, nkv, d, window, bias):
          "v_bias": rnd(nkv * d, seed=7, scale=0.5)}
     if not bias:
         w = {k: v for k, v in w.items() if not k.endswith("bias")}
+    eps = 3e-4
+    if qk_norm:
+        names.update({"q_norm": "qn", "k_norm": "kn"})
+        w.update({"q_norm": 1 + rnd(d, seed=11, scale=0.3), "k_norm": 1 + rnd(d, seed=12, scale=0.3)})
     w = {k: v.to(dtype) for k, v in w.items()}
     rt = runtime(dtype)
     sp = spec("attention", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d, "qkv_bias": bias,
-                            "window": window,
+                            "window": window, "qk_norm": qk_norm, "qk_norm_eps": eps,
                             "position": spec("rope_neox", {"head_dim": d, "theta": theta, "rotary_dim": d})}, names)
     mixer = MIXERS.get("attention")(sp, {k: v.cuda() for k, v in w.items()}, rt)
     cache = CacheManager({0: mixer.cache_request()}, {}, 16, ps, 2, dtype, rt.device, max_step_tokens=64)
@@ -258,9 +265,11 @@ def test_attention_part_in_portions(dtype, nh, nkv, d, window, bias):
         cache.commit(seq, seq.length + n)
         i += n
     assert i == T
-    cfg = {"num_attention_heads": nh, "num_key_value_heads": nkv, "head_dim": d, "rope_theta": theta}
+    cfg = {"num_attention_heads": nh, "num_key_value_heads": nkv, "head_dim": d, "rope_theta": theta, "rms_norm_eps": eps}
     wf = {"L.self_attn.q_proj.weight": w["q"], "L.self_attn.k_proj.weight": w["k"], "L.self_attn.v_proj.weight": w["v"],
           "L.self_attn.o_proj.weight": w["o"]}
+    if qk_norm:
+        wf.update({"L.self_attn.q_norm.weight": w["q_norm"], "L.self_attn.k_norm.weight": w["k_norm"]})
     if bias:
         wf.update({"L.self_attn.q_proj.bias": w["q_bias"], "L.self_attn.k_proj.bias": w["k_bias"],
                    "L.self_attn.v_proj.bias": w["v_bias"]})

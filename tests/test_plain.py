@@ -139,6 +139,38 @@ def test_attention_block_depends_on_distances_only():
     assert float((a0 - a2).abs().max()) > 1e-4
 
 
+def test_optional_norm_of_query_and_key_heads():
+    """With q_norm / k_norm gains among the weights every query and key head is normed over head_dim before the
+    rotation: the size of the projections then does not matter (a norm after the biases, before anything else),
+    the gains do, one per dim (which a norm placed after the rotation would pair differently), and gains of one
+    with unit-RMS heads change nothing."""
+    cfg, w = tiny_weights("B")
+    cfg = plain.normalized_config(dict(cfg, rms_norm_eps=1e-30))
+    p, d = "model.layers.0.", cfg["head_dim"]
+    x = torch.randn(9, 96, dtype=torch.float64)
+    w = dict(w)
+    w[p + "self_attn.q_norm.weight"] = 1 + 0.3 * torch.randn(d, dtype=torch.float64)
+    w[p + "self_attn.k_norm.weight"] = 1 + 0.3 * torch.randn(d, dtype=torch.float64)
+    a0 = plain.attention_block(x, w, p, cfg, torch.arange(9), None)
+    bigger = dict(w)
+    for name in ("q_proj.weight", "q_proj.bias", "k_proj.weight", "k_proj.bias"):
+        bigger[p + "self_attn." + name] = 5.0 * w[p + "self_attn." + name]
+    torch.testing.assert_close(plain.attention_block(x, bigger, p, cfg, torch.arange(9), None), a0, atol=1e-9, rtol=1e-9)
+    other = dict(w)
+    other[p + "self_attn.k_norm.weight"] = w[p + "self_attn.k_norm.weight"].flip(0)
+    assert float((plain.attention_block(x, other, p, cfg, torch.arange(9), None) - a0).abs().max()) > 1e-4
+    # the gain of dim k multiplies dim k of the normed head before the rotation mixes dims k and k + d/2: with the
+    # two halves' gains exchanged and the head's halves exchanged by hand the result differs, so the order matters
+    nh = cfg["num_attention_heads"]
+    q = plain.linear(x, w[p + "self_attn.q_proj.weight"], w[p + "self_attn.q_proj.bias"]).view(9, nh, d)
+    normed_then_rotated = plain.rope_neox(plain.rms_norm(q, w[p + "self_attn.q_norm.weight"], 1e-30), torch.arange(9), cfg["rope_theta"])
+    rotated_then_normed = plain.rms_norm(plain.rope_neox(q, torch.arange(9), cfg["rope_theta"]), w[p + "self_attn.q_norm.weight"], 1e-30)
+    assert float((normed_then_rotated - rotated_then_normed).abs().max()) > 1e-3
+    # without the gains among the weights nothing is normed
+    plainly = {k: v for k, v in w.items() if "_norm.weight" not in k or "layernorm" in k}
+    assert float((plain.attention_block(x, plainly, p, cfg, torch.arange(9), None) - a0).abs().max()) > 1e-4
+
+
 def test_model_norm_and_residual_placement():
     cfg, w = tiny_weights("A")
     ids = [5, 17, 3, 300, 5]

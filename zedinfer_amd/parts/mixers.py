@@ -101,7 +101,10 @@ class Attention(Mixer):
     The three projections are stacked into one [Qd + 2 KVd, H] matrix at load.
 
     params: hidden_size, num_heads, num_kv_heads, head_dim, qkv_bias, window (0: all keys),
-    scale (default 1/sqrt(head_dim)), position (a PartSpec of a position encoding)."""
+    scale (default 1/sqrt(head_dim)), position (a PartSpec of a position encoding), qk_norm (an RMS norm
+    over head_dim of every query and key head before the position encoding, gains ``q_norm`` and ``k_norm``
+    [head_dim], eps ``qk_norm_eps``; reference: transformer_forward.cpp:80-96.  The architecture built here
+    has none; the three projections then run one by one and the one-kernel decode path is not taken)."""
 
     graph_safe = True
     tape_safe = True
@@ -125,6 +128,8 @@ class Attention(Mixer):
         if p.get("qkv_bias", False):
             w.update({"q_bias": WeightSpec((nh * d,)), "k_bias": WeightSpec((nkv * d,)),
                       "v_bias": WeightSpec((nkv * d,))})
+        if p.get("qk_norm", False):
+            w.update({"q_norm": WeightSpec((d,), init="ones"), "k_norm": WeightSpec((d,), init="ones")})
         return w
 
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
@@ -153,6 +158,14 @@ class Attention(Mixer):
             else:
                 self.biases = bs
         self.o = weights["o"]
+        self.qk_norm = bool(p.get("qk_norm", False))
+        if self.qk_norm:
+            self.q_norm, self.k_norm = weights["q_norm"], weights["k_norm"]
+            self.qk_norm_eps = float(p.get("qk_norm_eps", 1e-6))
+            if self.qkv is not None:        # the projections run one by one, each into a buffer of its own
+                self.mats = [self.qkv[:self.qd], self.qkv[self.qd:self.qd + self.kvd], self.qkv[self.qd + self.kvd:]]
+                if self.bias is not None:
+                    self.biases = [self.bias[:self.qd], self.bias[self.qd:self.qd + self.kvd], self.bias[self.qd + self.kvd:]]
         # the widest prompt tile the prompt kernel of this head size takes (the planner chooses step by step)
         self.wide_tile = ops.attention_prefill_tile(rt.dtype, self.d) if rt.device.type == "cuda" else LONG_TILE
         self.plan_key = attention_planner(self.wide_tile, self.nh).key
@@ -201,7 +214,17 @@ class Attention(Mixer):
     def forward(self, x: torch.Tensor, batch, memory: LayerMemory) -> torch.Tensor:
         n = x.shape[0]
         view = batch.groups[memory.group]
-        if self.qkv is not None and ops.linear_sums_supported(x, self.qkv):
+        if self.qk_norm:
+            q, k, v = (self.rt.buffer(name, (n, width)) for name, width in
+                       (("attn_q", self.qd), ("attn_k", self.kvd), ("attn_v", self.kvd)))
+            for dst, m, b in zip((q, k, v), self.mats, self.biases or (None, None, None)):
+                ops.linear(x, m, b, out=dst)
+            # every head is a row of head_dim values: normed in place
+            ops.rms_norm(q.view(n * self.nh, self.d), self.q_norm, self.qk_norm_eps, out=q.view(n * self.nh, self.d))
+            ops.rms_norm(k.view(n * self.nkv, self.d), self.k_norm, self.qk_norm_eps, out=k.view(n * self.nkv, self.d))
+            self.position.rotate_and_store(q, k, v, self.positions_of(batch), view.slots, memory, self.nh, self.nkv,
+                                           self.d)
+        elif self.qkv is not None and ops.linear_sums_supported(x, self.qkv):
             # few rows: the projection leaves float32 partial sums; the rotary kernel adds them and the bias
             S = ops.linear_splits(n, self.qkv.shape[0], self.hidden)
             sums = self.rt.buffer("attn_qkv_sums", (S, n, self.qd + 2 * self.kvd), torch.float32)
@@ -230,7 +253,7 @@ class Attention(Mixer):
         """The library's algorithms for the projections of a step of ``num_tokens`` rows."""
         n = int(num_tokens)
         x = self.rt.buffer("norm_out", (n, self.hidden))
-        if self.qkv is not None:
+        if self.qkv is not None and not self.qk_norm:
             self.rt.tune_linear(x, self.qkv, self.bias)
         else:
             for m, b in zip(self.mats, self.biases or (None, None, None)):
