@@ -165,7 +165,10 @@ class InferenceEngine:
         # in: the library's first proposal for a shape can be a third slower than what timing finds, and what
         # timing finds for one number of rows does not carry over to its neighbours (measured; see
         # ``many_rows_step_sizes``).
-        if os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and engine.device.type == "cuda":
+        # (the reference's own switch for its warm-up is honoured too: ZEDINFER_DISABLE_WARMUP set,
+        # src/zedinfer/engine.cpp:506)
+        if (os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and "ZEDINFER_DISABLE_WARMUP" not in os.environ
+                and engine.device.type == "cuda"):
             sched = engine.sched
             most = min(sched.max_batch_tokens, sched.max_prefill_tokens + sched.max_batch_requests)
             if warm_up_sizes is None:       # a portion and the decoding entries are rounded up: one more size
