@@ -136,3 +136,60 @@ def test_wide_prompt_tiles_give_the_same_logits(model, monkeypatch):
     worst, mean, scale, rows, where = traces.compare(steps, alone, model["reference16"], reqs)
     assert rows == 329 + 65
     assert worst <= BF16_REL_WORST * scale and mean <= BF16_REL_MEAN * scale, where
+
+
+def test_graphs_that_hold_the_library_product_replay_right_at_real_widths(model):
+    """Steps whose many-rows products are the library's, with the algorithms a warm-up chose by timing, captured
+    as HIP graphs at the real widths and replayed several times with other work between the replays: prompt
+    portions of 200 tokens (run as 256 rows, one row wanted) and 70 requests decoding together.  Every replay is
+    held against the plain implementation, the decode steps also bit for bit against an engine that launches
+    every step part by part (a library algorithm that clears its workspace with a memset node, or anything
+    else that a graph does not repeat, would show from the second replay on)."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    pcfg, w16 = plain.load_folder(model["folder16"])
+    p = model["requests"]["p"]
+    sched = SchedulerConfig(num_kv_blocks=400, kv_block_size=16, max_batch_requests=80)
+    fast, slow = (Engine.from_folder(model["folder16"], "bfloat16", sched) for _ in range(2))
+    slow.use_graphs = slow.use_tapes = False
+    fast.warm_up([256])
+
+    def within(got, ref):
+        d = (got.float().cpu() - ref).abs()
+        scale = float(ref.abs().max())
+        return float(d.max()) <= BF16_REL_WORST * scale and float(d.mean()) <= BF16_REL_MEAN * scale
+
+    # ---- prompt portions: the first step of the shape runs part by part, the second is captured, the rest replay
+    other = fast.open("other")
+    fast.step([StepEntry(other, p[:40], [])])
+    for i in range(5):
+        toks = p[20 * i:20 * i + 200]
+        seq = fast.open(("prompt", i))
+        got = fast.step([StepEntry(seq, toks, [199])])
+        assert within(got[0], plain.forward(pcfg, w16, toks)[199]), i
+        fast.close(seq)
+        fast.step([StepEntry(other, p[40 + i:41 + i], [0])])          # eager work of another shape between the replays
+        torch.cuda.synchronize()
+    assert fast.prompt_graph_replays >= 3
+    fast.close(other)
+    # ---- 70 requests decode together: more than 64 rows, the library's product inside the decode graph
+    names = [f"d{i}" for i in range(70)]
+    seqs = {(e, r): e.open(r) for e in (fast, slow) for r in names}
+    # (the prompts enter part by part in both engines: padded to a graph's shape the products would have other
+    # numbers of rows, round differently, and so would every later step that reads what was stored)
+    fast.use_graphs = fast.use_tapes = False
+    for e in (fast, slow):
+        e.step([StepEntry(seqs[(e, r)], p[i:i + 8], []) for i, r in enumerate(names)])
+    fast.use_graphs = fast.use_tapes = True
+    before = fast.graph_replays
+    for k in range(6):
+        outs = [e.step([StepEntry(seqs[(e, r)], p[i + 8 + k:i + 9 + k], [0]) for i, r in enumerate(names)]) for e in (fast, slow)]
+        assert torch.equal(outs[0], outs[1]), k
+        torch.cuda.synchronize()
+    assert fast.graph_replays >= before + 4 and slow.graph_replays == 0
+    for i in (0, 33, 69):
+        assert within(outs[0][i], plain.forward(pcfg, w16, p[i:i + 14])[13]), i
+    for e in (fast, slow):
+        for r in names:
+            e.close(seqs[(e, r)])
+        e.cache.check()

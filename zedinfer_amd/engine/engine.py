@@ -308,15 +308,17 @@ class Engine:
         mixer must have said that padding is harmless to it."""
         if not self.padding_safe:
             return False
-        total = 0
+        total = real = 0
         for e in entries:
             n = len(e.tokens)
             if len(e.want) > 1 or e.positions is not None:
                 return False
             if n > 1:
                 total += -(-n // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
+                real += n
         most = max(self.prompt_graph_max_tokens if self.use_graphs else 0, self.TAPE_MAX_TOKENS if self.use_tapes else 0)
-        return 0 < total <= most and len(entries) <= self.graph_max_entries
+        # many very short portions would be padded to many times their tokens: such a step runs as it is
+        return 0 < total <= most and total <= 4 * real + self.PROMPT_GRAPH_STEP and len(entries) <= self.graph_max_entries
 
     def _prompt_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """A step of portions of prompts (entries of several tokens) beside single decoded tokens,
