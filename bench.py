@@ -85,10 +85,16 @@ def measure_decode(engine_factory, batch, steps, warmup, vocab, prompt_len=PROMP
     loop = ie.serving_loop()
     rng = random.Random(1234 + batch)
     reqs = [loop.submit_async(InferenceRequest(rand_ids(rng, prompt_len, vocab),
-                                               GenerationConfig(max_new_tokens=warmup + steps + 2 * batch + 8,
+                                               GenerationConfig(max_new_tokens=warmup + steps + 2 * batch + 32,
                                                                 ignore_eos=True)))
             for _ in range(batch)]
     while loop.pending_count() or any(r.phase.value != "decode" for r in reqs):
+        loop.step()
+    # set-up, like the prompts before: a kind of step is captured as a graph once it has come a few times
+    # (Engine.graph_after); the warm-up and the timed steps are steps of the serving loop's steady state
+    for _ in range(2 * ie.engine.graph_after + 2):
+        if ie.engine.graph_replays > 0:
+            break
         loop.step()
     for _ in range(warmup):
         loop.step()

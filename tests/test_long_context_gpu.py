@@ -28,6 +28,7 @@ def test_long_context_serving_kernels_agree_with_the_float32_path(tmp_path):
     for dtype in ("float32", "bfloat16"):
         eng = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=(T + decoded) // 16 + 8, kv_block_size=16,
                                                                  max_batch_requests=4, max_batch_tokens=4096))
+        eng.graph_after = 2
         seq = eng.open("long")
         rows = []
         for a in range(0, T, 2048):

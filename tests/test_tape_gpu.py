@@ -207,7 +207,7 @@ def test_a_large_step_is_brought_up_to_a_measured_size(tmp_path):
     e.step([StepEntry(b, short_toks[:30], [])])
     got = e.step([StepEntry(a, long_toks[:4170], [4169]), StepEntry(b, short_toks[30:31], [0])]).cpu()
     keys = [k for k in e._prompt_graphs if k[1] > 0]
-    assert keys == [k for k in keys if k[2] == (4288,) and k[0] == 65], list(e._prompt_graphs)
+    assert keys == [k for k in keys if k[2] == 4288 and k[0] == 65], list(e._prompt_graphs)
     ref_a, ref_b = plain.forward(cfg, w, long_toks), plain.forward(cfg, w, short_toks)
     tol = F32_TOL * max(1.0, float(ref_a.abs().max()), float(ref_b.abs().max()))
     assert float((got[0] - ref_a[4169]).abs().max()) < tol and float((got[1] - ref_b[30]).abs().max()) < tol
@@ -215,4 +215,96 @@ def test_a_large_step_is_brought_up_to_a_measured_size(tmp_path):
         got = e.step([StepEntry(a, long_toks[4170 + i:4171 + i], [0]), StepEntry(b, short_toks[31 + i:32 + i], [0])]).cpu()
         assert float((got[0] - ref_a[4170 + i]).abs().max()) < tol and float((got[1] - ref_b[31 + i]).abs().max()) < tol
     assert a.length == 4174 and b.length == 35
+    e.cache.check()
+
+
+def test_portions_dealt_out_differently_share_a_tape(tmp_path):
+    """Steps that agree in their tokens, entries and bounds, and in what the attention planner says its plan
+    depends on (the tile and the number of tiles), share a recorded tape however the tokens are dealt out over
+    the portions: the tile lists and the entries' starts are data, not shapes.  Four such steps in a row, the last
+    two from the tape, against the plain implementation."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "A")
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["A"]
+    e = Engine.from_folder(folder, "float32", SchedulerConfig(num_kv_blocks=3 * (832 // ps + 2), kv_block_size=ps, max_batch_requests=4))
+    e.use_graphs = False
+    toks = {r: traces.random_tokens(cfg["vocab_size"], 800, seed=30 + i) for i, r in enumerate("abx")}
+    ref = {r: plain.forward(cfg, w, t) for r, t in toks.items()}
+    seqs = {r: e.open(r) for r in toks}
+    fed = {}
+    for r, n in (("a", 520), ("b", 520), ("x", 20)):      # far enough in that the block tables keep their width
+        e.step([StepEntry(seqs[r], toks[r][:n], [])])
+        fed[r] = n
+    tol = F32_TOL * max(1.0, max(float(v.abs().max()) for v in ref.values()))
+    for na, nb in ((70, 60), (10, 100), (128, 50), (64, 65)):          # 128 + 64, 64 + 128, 128 + 64, 64 + 128 tokens as run
+        plan = [("a", na), ("b", nb), ("x", 1)]
+        got = e.step([StepEntry(seqs[r], toks[r][fed[r]:fed[r] + n], [n - 1]) for r, n in plan]).cpu()
+        for row, (r, n) in enumerate(plan):
+            fed[r] += n
+            assert float((got[row] - ref[r][fed[r] - 1]).abs().max()) < tol, (plan, r)
+    mixed = [k for k in e._prompt_graphs if k[1] > 0]
+    assert len(mixed) == 1 and mixed[0][2] == 192 and e.tape_runs >= 2, (mixed, e.tape_runs)
+    # a step with another number of tokens is another shape
+    e.step([StepEntry(seqs["a"], toks["a"][fed["a"]:fed["a"] + 6], [5]), StepEntry(seqs["x"], toks["x"][fed["x"]:fed["x"] + 1], [0])])
+    assert len([k for k in e._prompt_graphs if k[1] > 0]) == 2
+    e.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_fewer_and_fewer_requests_share_a_shape(tmp_path, dtype):
+    """Requests end one by one: steps of 7, 6 and 5 decoding requests all run as 8 entries (the rest belong to no
+    request), so they share one recorded shape; every request's logits are the plain implementation's, and the
+    pages of a request that ended serve a new one."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    from zedinfer_amd.engine.engine import decode_entries_at_least
+    assert [decode_entries_at_least(n) for n in (1, 2, 3, 5, 9, 16, 17, 33, 64, 65, 100, 256)] == \
+        [1, 2, 4, 8, 16, 16, 32, 48, 64, 96, 128, 256]
+    store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "C", dtype=store, std=tiny_configs.SHARP_STD)
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["C"]
+    e = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=8 * (64 // ps + 1), kv_block_size=ps, max_batch_requests=8))
+    e.use_graphs = False
+    names = list("abcdefg")
+    toks = {r: traces.random_tokens(cfg["vocab_size"], 40, seed=40 + i) for i, r in enumerate(names + ["h"])}
+    ref = {r: plain.forward(cfg, w, t) for r, t in toks.items()}
+    seqs, fed = {}, {}
+
+    def prefill(r, n):
+        seqs[r] = e.open(r)
+        e.step([StepEntry(seqs[r], toks[r][:n], [])])
+        fed[r] = n
+
+    def decode(rs):
+        got = e.step([StepEntry(seqs[r], toks[r][fed[r]:fed[r] + 1], [0]) for r in rs]).cpu()
+        assert got.shape[0] == len(rs)
+        for row, r in enumerate(rs):
+            d = (got[row] - ref[r][fed[r]]).abs()
+            scale = float(ref[r].abs().max())
+            if dtype == "float32":
+                assert float(d.max()) < F32_TOL * max(1.0, scale), (rs, r)
+            else:
+                assert bf16_within(float(d.max()), float(d.mean()), scale), (rs, r)
+            fed[r] += 1
+
+    for i, r in enumerate(names):
+        prefill(r, 5 + i)
+    live = list(names)
+    for _ in range(3):
+        for _ in range(3):
+            decode(live)
+        e.close(seqs.pop(live.pop(1)))
+    assert len(live) == 4
+    shapes = [k for k in e._graphs]
+    assert len(shapes) == 1 and shapes[0][0] == 8, shapes
+    assert e.tape_runs >= 6
+    prefill("h", 9)                                     # takes pages that were given back
+    for _ in range(4):
+        decode(live + ["h"])
+    assert len(e._graphs) == 1
+    decode(live)                                        # four requests: a shape of its own
+    assert sorted(k[0] for k in e._graphs) == [4, 8]
     e.cache.check()

@@ -243,18 +243,22 @@ class DecodeImage:
     change, and a block table row when its sequence took or gave back a page: ``refresh`` rewrites
     just those in place instead of packing everything anew (and the arrays of planners that do not say
     ``fixed_for_single_tokens``).  The layout is the one ``build_device_batch`` makes for the same
-    entries and table widths."""
+    entries and table widths.  ``pad_entries`` / ``pad_rows``: entries that belong to no request and wanted
+    rows behind the real ones, as in ``build_device_batch``; they stay as they were made."""
 
     def __init__(self, entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int, device: torch.device,
                  staging: StagingRing, widths: Sequence[int], static: Optional[torch.Tensor],
-                 planners: Sequence[StepPlanner] = (), position_axes: int = 1, bound_single: int = 0):
+                 planners: Sequence[StepPlanner] = (), position_axes: int = 1, bound_single: int = 0,
+                 pad_entries: int = 0, pad_rows: int = 0):
         self.cache, self.vocab_size, self.staging, self.static = cache, vocab_size, staging, static
         self.widths = tuple(int(w) for w in widths)
         self.planners, self.axes, self.bound_single = tuple(planners), int(position_axes), int(bound_single)
         self.batch = build_device_batch(entries, cache, vocab_size, device, staging, widths, static,
-                                        planners=planners, position_axes=position_axes, bound_single=bound_single)
+                                        planners=planners, position_axes=position_axes, bound_single=bound_single,
+                                        pad_entries=pad_entries, pad_rows=pad_rows)
         self.static = self.batch.device_image       # the buffer given, or the one this step made
-        E, R = len(entries), self.batch.num_logit_rows
+        self.real = len(entries)                    # the entries of requests come first
+        E, R = len(entries) + int(pad_entries), self.batch.num_logit_rows
         self.seqs = [e.seq for e in entries]
         self.wants = tuple(len(e.want) for e in entries)
         self.versions = [e.seq.version for e in entries]
@@ -273,7 +277,8 @@ class DecodeImage:
         self.image = np.empty(max(self.total, 1), dtype=np.int32)
         self.image[:self.total] = self.batch.host_image
         self.page_sizes = [g.page_size for g in cache.groups]
-        self.rows = np.arange(E)
+        self.entries_made = E
+        self.rows = np.arange(self.real)
 
     def piece(self, i: int) -> np.ndarray:
         return self.image[self.offsets[i]:self.offsets[i + 1]]
@@ -289,18 +294,18 @@ class DecodeImage:
 
     def refresh(self, entries: Sequence[StepEntry]) -> DeviceBatch:
         """The image for this step (``matches(entries)`` holds), copied to the device buffer."""
-        E = len(entries)
+        E, made = len(entries), self.entries_made
         toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=E)
         if toks.min() < 0 or toks.max() >= self.vocab_size:
             bad = toks[(toks < 0) | (toks >= self.vocab_size)][0]
             raise ValueError(f"token id {int(bad)} is outside the vocabulary of {self.vocab_size}")
         pos = np.fromiter((s.length for s in self.seqs), dtype=np.int32, count=E)
-        self.piece(0)[:] = toks
-        self.piece(1)[:] = pos
-        self.piece(6)[:] = pos
+        self.piece(0)[:E] = toks
+        self.piece(1)[:E] = pos
+        self.piece(6)[:E] = pos
         G = len(self.widths)
         for g, w in enumerate(self.widths):
-            table = self.piece(FIXED_PIECES + 1 + 2 * g).reshape(E, w)
+            table = self.piece(FIXED_PIECES + 1 + 2 * g).reshape(made, w)
             for i, s in enumerate(self.seqs):
                 if s.version != self.versions[i]:
                     pg = s.pages[g]
@@ -312,15 +317,16 @@ class DecodeImage:
             pages = table[self.rows, pos // ps]
             if (pages < 0).any():
                 raise RuntimeError("a decoded token's position has no page")
-            self.piece(FIXED_PIECES + 2 * g)[:] = pages * ps + pos % ps
+            self.piece(FIXED_PIECES + 2 * g)[:E] = pages * ps + pos % ps
         if self.axes > 1:
-            self.piece(FIXED_PIECES + 2 * G)[:] = np.repeat(pos, self.axes)
+            self.piece(FIXED_PIECES + 2 * G)[:E * self.axes] = np.repeat(pos, self.axes)
         for i, s in enumerate(self.seqs):
             self.versions[i] = s.version
         moving = [pl for pl in self.planners if not pl.fixed_for_single_tokens]
         if moving:
-            hb = HostBatch(num_tokens=E, num_entries=E, entry_start=self.batch.host_start,
-                           entry_len=self.batch.host_len, entry_past=pos, single_tokens=True,
+            past = pos if made == E else np.concatenate([pos, np.zeros(made - E, dtype=np.int32)])
+            hb = HostBatch(num_tokens=made, num_entries=made, entry_start=self.batch.host_start,
+                           entry_len=self.batch.host_len, entry_past=past, single_tokens=True,
                            bound_single=self.bound_single)
             for pl in moving:
                 plan = pl.plan(hb)
@@ -336,5 +342,5 @@ class DecodeImage:
         host.numpy()[:] = self.image[:self.total]
         self.static[:self.total].copy_(host, non_blocking=True)
         self.staging.copied()
-        self.batch.host_past = pos
+        self.batch.host_past = pos if made == E else np.concatenate([pos, np.zeros(made - E, dtype=np.int32)])
         return self.batch

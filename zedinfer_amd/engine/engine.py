@@ -79,6 +79,7 @@ class Engine:
         self.tape_runs = 0
         self.graph_max_entries = 256     # measured: 128 requests decode 77% faster as a graph, 256 37%
         self.graph_limit = 48
+        self.graph_after = int(os.environ.get("ZEDINFER_GRAPH_AFTER", "6"))   # steps of a kind before it is captured
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.graph_replays = 0
         # A step that is one portion of one prompt, alone or beside single decoded tokens, has the portion
@@ -226,7 +227,14 @@ class Engine:
         only: the first step of a kind runs eagerly and is captured, later ones replay the graph
         after the step's index arrays have been copied into the graph's buffer."""
         E = len(entries)
-        R = sum(len(e.want) for e in entries)
+        wanted = R = sum(len(e.want) for e in entries)
+        more_entries = 0
+        if self.padding_safe and (self.use_graphs or self.use_tapes):
+            # the number of requests moves (they end one by one): entries that belong to no request bring it to
+            # one of few numbers, a row wanted of each, so that the kinds of steps are few
+            more_entries = decode_entries_at_least(E) - E
+            E += more_entries
+            R = E if wanted else 0
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
         # a bound, the same for many steps, of the tokens any sequence holds after this step: the
@@ -244,20 +252,26 @@ class Engine:
             batch = dg.image.refresh(entries)      # the same sequences go on: only what changed is rewritten
         else:
             dg.image = DecodeImage(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
-                                   planners=self.planners, position_axes=self.position_axes, bound_single=bound)
+                                   planners=self.planners, position_axes=self.position_axes, bound_single=bound,
+                                   pad_entries=more_entries, pad_rows=R - wanted)
             dg.buffer = dg.image.static         # the first step's buffer serves all later ones of the shape
             batch = dg.image.batch
         if token_source is not None:
-            batch.token_ids.copy_(token_source, non_blocking=True)
+            batch.token_ids[:len(entries)].copy_(token_source, non_blocking=True)
+        logits = self._decode_step(dg, batch)
+        return logits[:wanted] if (logits is not None and R != wanted) else logits      # the requests' rows come first
+
+    def _decode_step(self, dg: "_DecodeGraph", batch) -> Optional[torch.Tensor]:
         if dg.graph is not None:
             dg.graph.replay()
             self.graph_replays += 1
             return dg.logits
-        if not self.use_graphs:
-            return self._run_or_replay(dg, batch)
-        logits = self.model.run(batch, self.memories)      # allocates every workspace; its result is this step's
-        if dg.warm:
-            # the second step of this kind: capture (nothing runs), to be replayed from the third on
+        # the first step of a kind runs part by part (it allocates every workspace), the second is recorded as a
+        # tape, and a kind that keeps coming is captured as a graph (capturing costs about ten steps: kinds that
+        # come a few times only, as while a batch of requests ends one by one, stay with their tape)
+        logits = self._run_or_replay(dg, batch)
+        dg.seen += 1
+        if self.use_graphs and dg.seen >= (self.graph_after if self.use_tapes and not dg.no_tape else 2):
             torch.cuda.synchronize(self.device)
             first = logits.clone() if logits is not None else None
             g = torch.cuda.CUDAGraph()
@@ -265,26 +279,28 @@ class Engine:
                 dg.logits = self.model.run(batch, self.memories)
             dg.graph = g
             return first
-        dg.warm = True
         return logits
 
     def _run_or_replay(self, dg: "_DecodeGraph", batch) -> Optional[torch.Tensor]:
-        """A step of a shape that has no graph: from the shape's tape when it has one, else part by part, and
-        then (once the workspaces have their sizes: not at the shape's first step, which may still allocate)
-        recorded as its tape.  The batch lives in the shape's own buffer, as for a graph."""
+        """A step of a shape that has no graph: from the shape's tape when it has one, else part by part, recorded
+        as its tape on the way.  A recording during which device memory was taken is dropped (the memory would be
+        another's at the next run): that is the rule at a shape's first step when workspaces still grow, and the
+        step is then recorded again the next time; a second such recording marks the shape as one that cannot be
+        taped.  The batch lives in the shape's own buffer, as for a graph."""
         if dg.tape is not None:
             dg.tape.run()
             self.tape_runs += 1
             return dg.logits
-        if not self.use_tapes or dg.no_tape or not dg.ran:
+        if not self.use_tapes or dg.no_tape:
             dg.ran = True
             return self.model.run(batch, self.memories)
         with Recording(self.device) as rec:
             logits = self.model.run(batch, self.memories)
         if rec.allocations:
-            dg.no_tape = True       # memory taken during the step would be another's at the next
+            dg.no_tape = dg.ran       # at the first step workspaces may still get their sizes
         else:
             dg.tape, dg.logits = rec.tape(), logits
+        dg.ran = True
         return logits
 
 
@@ -353,9 +369,11 @@ class Engine:
         long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions) + more_tokens, 2048)
         short_bucket = _bucket_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
         singles = len(entries) - len(portions) + more_entries
-        # everything the launches' sizes depend on: the portions' sizes one by one (the planners cut each into
-        # tiles by rules of their own), not their sum
-        key = (E, singles, sizes, R, widths, long_bucket, short_bucket)
+        # everything the launches' sizes depend on: the tokens of the step, and what of the portions' sizes one by
+        # one the planners say their plans depend on (tiles are cut portion by portion, by rules of their own)
+        entry_lens = sizes + (1,) * singles
+        shapes = tuple(pl.shape(entry_lens, short_bucket if singles else 0, long_bucket) for pl in self.planners)
+        key = (E, singles, padded, shapes, R, widths, long_bucket, short_bucket)
         dg = self._prompt_graphs.pop(key, None)
         if dg is not None:
             self._prompt_graphs[key] = dg       # used last: the last to go
@@ -393,7 +411,6 @@ class _DecodeGraph:
         self.buffer: Optional[torch.Tensor] = None      # the device buffer of the step's index arrays
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
-        self.warm = False
         self.seen = 0
         self.ran = False                                # a step of the shape has run part by part
         self.tape = None                                # the library calls of one step of the shape
@@ -429,6 +446,15 @@ def many_rows_step_sizes(most_tokens: int, step: int = Engine.PROMPT_GRAPH_STEP,
         s = _many_rows_spacing(n - 1, step)
         n = (n - 1) // s * s
     return sizes
+
+
+def decode_entries_at_least(entries: int) -> int:
+    """The number of entries a step of ``entries`` decoding requests is run with: a power of two up to 16 (one
+    tile of rows of the few-rows kernels), then a multiple of 16 up to 64 and of 32 beyond."""
+    if entries <= 16:
+        return _pow2_at_least(entries)
+    step = 16 if entries <= 64 else 32
+    return -(-entries // step) * step
 
 
 def _bucket_at_least(n: int, floor: int = 1) -> int:

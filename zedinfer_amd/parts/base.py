@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import os
 from dataclasses import dataclass, field
-from typing import Callable, Dict, Optional, Tuple
+from typing import Callable, Dict, Optional, Sequence, Tuple
 
 import torch
 
@@ -236,6 +236,13 @@ class StepPlanner:
 
     def plan(self, hb: HostBatch) -> StepPlan:
         raise NotImplementedError
+
+    def shape(self, entry_lens: Sequence[int], bound_single: int, bound_multi: int) -> tuple:
+        """Everything of the entries' token counts (as the step runs them, padding included) that the sizes of
+        this planner's arrays and launches depend on, beyond their number and their sum: steps that agree in it
+        (and in the bounds, the number of entries and of tokens) can share a recorded graph or tape.  The default
+        is the counts themselves; a planner whose plan depends on less says so."""
+        return tuple(sorted(int(n) for n in entry_lens))
 
 
 class Mixer(Part):

@@ -62,13 +62,7 @@ class AttentionPlanner(StepPlanner):
                             hb.bound_multi if several else 0, 1)
         if long_idx.size and hb.bound_multi:
             max_long = hb.bound_multi
-        tile, alone = LONG_TILE, False
-        if self.wide_tile > LONG_TILE and long_idx.size:
-            wide = int(sum(-(-int(n) // self.wide_tile) for n in lens[~short]))
-            groups = wide * -(-max_long // self.CUT_KEYS) * self.heads
-            if groups >= self.FILL:
-                tile = self.wide_tile
-                alone = groups >= self.FILL_ALONE
+        tile, alone = self._tile([int(n) for n in lens[~short]], max_long)
         tiles = [(int(past[i]) + off + min(tile, int(lens[i]) - off), i, off)
                  for i in range(hb.num_entries) if not short[i] for off in range(0, int(lens[i]), tile)]
         tiles.sort(key=lambda t: -t[0])
@@ -78,6 +72,26 @@ class AttentionPlanner(StepPlanner):
                     "tile_off": np.array([t[2] for t in tiles], dtype=np.int32)},
             sizes={"num_short": int(short_idx.size), "num_long": int(long_idx.size), "num_tiles": len(tiles),
                    "tile": tile, "alone": alone, "max_short_keys": max_short, "max_long_keys": max_long})
+
+
+    def _tile(self, long_lens, max_long: int):
+        """(queries a tile, workgroups of four wavefronts) for portions of these many tokens whose keys are bounded
+        by ``max_long``: the wide tile when that many workgroups still fill the chip."""
+        tile, alone = LONG_TILE, False
+        if self.wide_tile > LONG_TILE and long_lens:
+            wide = int(sum(-(-int(n) // self.wide_tile) for n in long_lens))
+            groups = wide * -(-max_long // self.CUT_KEYS) * self.heads
+            if groups >= self.FILL:
+                tile = self.wide_tile
+                alone = groups >= self.FILL_ALONE
+        return tile, alone
+
+    def shape(self, entry_lens, bound_single: int, bound_multi: int) -> tuple:
+        """The tile, and how many tiles and short tokens there are: how the tokens are dealt out over the portions
+        matters no further (tiles of 64 queries: not at all, for portions that are multiples of 64)."""
+        long_lens = [int(n) for n in entry_lens if n > SHORT_ENTRY]
+        tile, alone = self._tile(long_lens, int(bound_multi))
+        return (tile, alone, sum(-(-n // tile) for n in long_lens), sum(int(n) for n in entry_lens if n <= SHORT_ENTRY))
 
 
 _PLANNERS: Dict[tuple, AttentionPlanner] = {}
