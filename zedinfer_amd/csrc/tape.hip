@@ -88,6 +88,24 @@ extern "C" int zi_tape_record(void* tape, const char* name, const int64_t* words
     return zi_fail("tape_record: %s is not an entry point that a tape can hold", name);
 }
 
+// Append `calls` calls at once: their names one after the other, each ended by a zero byte; counts[i] argument
+// words of call i, all words in one row.  Nothing is appended when one of them is refused.
+extern "C" int zi_tape_record_many(void* tape, const char* names, const int* counts, const int64_t* words, int calls) {
+    ZI_REQUIRE(tape && names && counts && (words || calls == 0) && calls >= 0, "tape_record_many: null argument");
+    Tape* t = static_cast<Tape*>(tape);
+    const size_t had_calls = t->calls.size(), had_words = t->words.size();
+    for (int i = 0; i < calls; ++i) {
+        if (zi_tape_record(tape, names, words, counts[i]) != 0) {
+            t->calls.resize(had_calls);
+            t->words.resize(had_words);
+            return 1;
+        }
+        names += strlen(names) + 1;
+        words += counts[i];
+    }
+    return 0;
+}
+
 // Make every recorded call again, in order.  Stops at the first that fails and returns what it returned
 // (its message is the one zi_last_error() gives); `done`, when not null, receives the number of calls made.
 extern "C" int zi_tape_run(const void* tape, int* done) {

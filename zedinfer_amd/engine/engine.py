@@ -367,7 +367,9 @@ class Engine:
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
         long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions) + more_tokens, 2048)
-        short_bucket = _bucket_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
+        # (a power of two here: beside portions of prompts the decoding requests' attention is a small part of the
+        # step, and every further value of the bound is a further kind of step)
+        short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
         singles = len(entries) - len(portions) + more_entries
         # everything the launches' sizes depend on: the tokens of the step, and what of the portions' sizes one by
         # one the planners say their plans depend on (tiles are cut portion by portion, by rules of their own)

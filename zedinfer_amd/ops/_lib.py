@@ -56,6 +56,7 @@ _PROTOTYPES = {
     "zi_argmax": [P, P, P, I, I, I, L, P, L, P],
     "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],
     "zi_tape_record": [P, c_char_p, P, I],
+    "zi_tape_record_many": [P, c_char_p, P, P, I],
     "zi_tape_run": [P, P],
     "zi_tape_length": [P],
 }

@@ -28,10 +28,14 @@ class Tape:
         self._handle = ctypes.c_void_p(lib.zi_tape_new())
         if not self._handle:
             raise _lib.KernelLibraryError("no memory for a tape")
+        words, counts = [], []
         for name, args in calls:
-            words = _lib.argument_words(name, args)
-            arr = (ctypes.c_int64 * len(words))(*words)
-            _lib.call("zi_tape_record", self._handle, name.encode(), ctypes.cast(arr, ctypes.c_void_p), len(words))
+            w = _lib.argument_words(name, args)
+            words += w
+            counts.append(len(w))
+        names = b"".join(name.encode() + b"\0" for name, _ in calls)
+        _lib.call("zi_tape_record_many", self._handle, names, (ctypes.c_int * len(counts))(*counts),
+                  (ctypes.c_int64 * len(words))(*words), len(calls))
         self.length = len(calls)
 
     def run(self) -> None:
