@@ -238,23 +238,6 @@ def test_no_batch_ahead_when_the_results_could_change_it():
         commit(c, first)
         a.cancelled = cancel
         assert s.schedule_ahead(first) is None
-    # a prompt that is only partly in
-    s, c = make(max_batch_tokens=8, max_prefill_tokens=8)
-    a, b = req(3, max_new=8), req(12, max_new=8)
-    s.submit(a)
-    s.submit(b)
-    first = s.schedule()            # a whole, 5 tokens of b
-    assert first.prefill_chunk_sizes == [3, 5]
-    commit(c, first)
-    assert s.schedule_ahead(first) is None
-    # a waiting prompt that could be admitted now
-    s, c = make()
-    a = req(3, max_new=8)
-    s.submit(a)
-    first = s.schedule()
-    commit(c, first)
-    s.submit(req(3, max_new=8))
-    assert s.schedule_ahead(first) is None
     # no page for the next token
     s, c = make(pages=2, page_size=4, generation_reserve=1)
     a = req(8, max_new=8)
@@ -263,6 +246,111 @@ def test_no_batch_ahead_when_the_results_could_change_it():
     commit(c, first)
     assert s.schedule_ahead(first) is None
     c.check()
+
+
+def test_batch_ahead_takes_the_prompts_that_the_next_step_would():
+    """The batch ahead holds, beside the decoding requests, the portions of prompts that ``schedule()`` would take
+    after the running step: a prompt that is partly in goes on, a waiting prompt that fits is admitted, and a step
+    that samples nothing (a portion in the middle of a prompt) has a batch ahead too."""
+    # a prompt that is only partly in
+    s, c = make(max_batch_tokens=8, max_prefill_tokens=8)
+    a, b = req(3, max_new=8), req(12, max_new=8)
+    s.submit(a)
+    s.submit(b)
+    first = s.schedule()            # a whole, 5 tokens of b
+    assert first.prefill_chunk_sizes == [3, 5]
+    commit(c, first)
+    ahead = s.schedule_ahead(first)
+    assert ahead.decode_requests == [a] and ahead.prefill_requests == [b] and ahead.tokens_on_device
+    assert ahead.prefill_chunk_starts == [5] and ahead.prefill_chunk_sizes == [7] and ahead.sampled_requests() == [a, b]
+    commit(c, ahead)
+    s.process_results(first, [7])
+    s.process_results(ahead, [8, 9])
+    assert a.output_ids == [7, 8] and b.output_ids == [9] and b.phase == RequestPhase.DECODE
+    c.check()
+    # a waiting prompt that can be admitted now
+    s, c = make()
+    a, b = req(3, max_new=8), req(4, max_new=8)
+    s.submit(a)
+    first = s.schedule()
+    commit(c, first)
+    s.submit(b)
+    ahead = s.schedule_ahead(first)
+    assert ahead.decode_requests == [a] and ahead.prefill_requests == [b] and ahead.prefill_chunk_sizes == [4]
+    # a portion in the middle of a prompt: nothing is sampled, the next portion is known all the same
+    s, c = make(max_batch_tokens=8, max_prefill_tokens=8)
+    a = req(20, max_new=8)
+    s.submit(a)
+    first = s.schedule()
+    assert first.prefill_chunk_sizes == [8] and not first.sampled_requests()
+    commit(c, first)
+    ahead = s.schedule_ahead(first)
+    assert ahead.prefill_chunk_starts == [8] and ahead.prefill_chunk_sizes == [8] and not ahead.decode_requests
+    commit(c, ahead)
+    s.process_results(first, [])
+    s.process_results(ahead, [])
+    last = s.schedule()
+    assert last.prefill_chunk_starts == [16] and last.prefill_chunk_sizes == [4] and last.sampled_requests() == [a]
+    c.check()
+
+
+def test_requests_get_the_same_tokens_with_and_without_batches_ahead():
+    """A random workload through the scheduler twice, once with every batch that can be made ahead made ahead (as
+    the serving loop does), once without: prompts cut into portions, requests that end by length and on stop
+    tokens, few pages.  The 'model' gives request r its k-th token as a function of (r, k) alone, so every
+    request must get the same output either way; the cache's books must balance all along."""
+    import random
+
+    def run(ahead_on, seed):
+        rng = random.Random(seed)
+        s, c = make(pages=rng.choice([24, 40, 64]), page_size=4, max_batch_tokens=rng.choice([6, 12, 40]),
+                    max_prefill_tokens=rng.choice([4, 8, 32]), max_batch_requests=rng.choice([2, 3, 8]),
+                    generation_reserve=4)
+        everyone = [req(rng.randint(1, 30), max_new=rng.randint(1, 12)) for _ in range(10)]
+        late = everyone[7:]
+        for r in everyone[:7]:
+            s.submit(r)
+        names = {id(r): i for i, r in enumerate(everyone)}
+
+        def token(r):
+            v = (names[id(r)] * 31 + len(r.output_ids) * 7) % 101
+            return 99 if v % 17 == 0 else v            # now and then the stop token
+
+        flight, steps, mixed_ahead = None, 0, 0
+        while s.has_work() or flight is not None or late:
+            steps += 1
+            assert steps < 2000
+            if late and (steps in (3, 9, 15) or not (s.has_work() or flight is not None)):
+                s.submit(late.pop(0))
+            if flight is None:
+                batch = s.schedule()
+                if batch.empty():
+                    continue
+                commit(c, batch)
+            else:
+                batch, flight = flight, None
+            if ahead_on:
+                nxt = s.schedule_ahead(batch)
+                if nxt is not None:
+                    commit(c, nxt)
+                    flight = nxt
+                    mixed_ahead += bool(nxt.prefill_requests)
+            s.process_results(batch, [token(r) for r in batch.sampled_requests()])
+            if flight is not None and not flight.prefill_requests and all(r.done for r in flight.decode_requests):
+                flight = None
+            c.check()
+        assert not c.live and not late
+        return [(r.finish_reason, r.error, list(r.result.output_ids) if r.result else None) for r in everyone], mixed_ahead
+
+    mixed, reasons = 0, set()
+    for seed in range(24):
+        with_ahead, mixed_ahead = run(True, seed)
+        without, _ = run(False, seed)
+        assert with_ahead == without, seed
+        mixed += mixed_ahead
+        reasons |= {r[0] for r in without}
+    assert mixed > 20                                   # batches ahead with portions of prompts were among them
+    assert reasons >= {"stop", "length"}
 
 
 def test_batch_ahead_while_the_head_of_the_queue_cannot_enter():

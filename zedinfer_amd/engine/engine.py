@@ -184,16 +184,16 @@ class Engine:
         a view of a workspace that the next step overwrites.  Raises OutOfPages, with no
         request's length changed, when the pool cannot hold the new tokens.
 
-        ``token_source``: an int32 device tensor [entries].  Every entry then brings one token whose
-        value is read from there on the device (``tokens`` holds a placeholder), so that a step can be
-        queued before the host has seen what the step before it sampled."""
+        ``token_source``: an int32 device tensor [k], k <= entries.  The first k entries then bring one token
+        each whose value is read from there on the device (``tokens`` holds a placeholder), so that a step can
+        be queued before the host has seen what the step before it sampled."""
         single = all(len(e.tokens) == 1 for e in entries)
         if token_source is not None:
-            if not single:
-                raise ValueError("tokens can come from the device only when every entry brings one token")
-            if (token_source.dtype != torch.int32 or token_source.device != self.device
-                    or token_source.shape != (len(entries),)):
-                raise ValueError(f"token_source must be an int32 tensor [{len(entries)}] on {self.device}")
+            k = token_source.shape[0] if token_source.dim() == 1 else -1
+            if token_source.dtype != torch.int32 or token_source.device != self.device or not (0 < k <= len(entries)):
+                raise ValueError(f"token_source must be an int32 tensor of at most {len(entries)} entries on {self.device}")
+            if any(len(e.tokens) != 1 for e in entries[:k]):
+                raise ValueError("tokens can come from the device only for entries that bring one token")
         grown = []
         try:
             for e in entries:
@@ -206,13 +206,13 @@ class Engine:
             raise
         if (self.use_graphs or self.use_tapes) and 0 < len(entries) <= self.graph_max_entries and single:
             logits = self._graph_step(entries, token_source)
-        elif (self.use_graphs or self.use_tapes) and token_source is None and self._one_portion(entries):
-            logits = self._prompt_graph_step(entries)
+        elif (self.use_graphs or self.use_tapes) and self._one_portion(entries):
+            logits = self._prompt_graph_step(entries, token_source)
         else:
             batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging,
                                        planners=self.planners, position_axes=self.position_axes)
-            if token_source is not None:
-                batch.token_ids.copy_(token_source, non_blocking=True)
+            if token_source is not None:        # the entries' tokens lie in their order: the first k are the first k tokens
+                batch.token_ids[:token_source.shape[0]].copy_(token_source, non_blocking=True)
             logits = self.model.run(batch, self.memories)
         for e in entries:
             self.cache.commit(e.seq, e.seq.length + len(e.tokens))
@@ -257,7 +257,7 @@ class Engine:
             dg.buffer = dg.image.static         # the first step's buffer serves all later ones of the shape
             batch = dg.image.batch
         if token_source is not None:
-            batch.token_ids[:len(entries)].copy_(token_source, non_blocking=True)
+            batch.token_ids[:token_source.shape[0]].copy_(token_source, non_blocking=True)
         logits = self._decode_step(dg, batch)
         return logits[:wanted] if (logits is not None and R != wanted) else logits      # the requests' rows come first
 
@@ -336,7 +336,8 @@ class Engine:
         # many very short portions would be padded to many times their tokens: such a step runs as it is
         return 0 < total <= most and total <= 4 * real + self.PROMPT_GRAPH_STEP and len(entries) <= self.graph_max_entries
 
-    def _prompt_graph_step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+    def _prompt_graph_step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None
+                           ) -> Optional[torch.Tensor]:
         """A step of portions of prompts (entries of several tokens) beside single decoded tokens,
         with every portion run as if it brought a multiple of PROMPT_GRAPH_STEP tokens (see
         ``build_device_batch``): the first step of a kind runs eagerly, the second is captured, later
@@ -388,6 +389,8 @@ class Engine:
                                    planners=self.planners, position_axes=self.position_axes,
                                    bound_single=short_bucket if singles else 0, bound_multi=long_bucket)
         dg.buffer = batch.device_image          # the first step's buffer serves all later ones of the shape
+        if token_source is not None:
+            batch.token_ids[:token_source.shape[0]].copy_(token_source, non_blocking=True)
         if dg.graph is not None:
             dg.graph.replay()
             self.prompt_graph_replays += 1

@@ -153,72 +153,73 @@ class Scheduler:
                 batch.decode_requests.append(req)
                 budget -= 1
             self.active = [r for r in self.active if not r.done]
-            # 2. prompts, from the head of the queue
-            prefill_budget = min(budget, self.config.max_prefill_tokens)
-            while self.waiting and prefill_budget > 0:
-                req = self.waiting[0]
-                if len(self.active) + len([r for r in batch.prefill_requests if r not in self.active]) \
-                        >= self.config.max_batch_requests:
-                    break
-                if req.seq is None:
-                    reserve = self._reserve(req)
-                    if not self.cache.can_open(reserve):
-                        msg = (f"Cannot admit request {req.request_id}: prompt={len(req.input_ids)} tokens, "
-                               f"reserve={reserve} tokens, free pages="
-                               f"{[g.pool.uncommitted for g in self.cache.groups]}, "
-                               f"free slots={self.cache.slots.num_free}")
-                        req.admission_warned = True
-                        if batch.empty() and not self.active:
-                            self.waiting.popleft()
-                            self._fail(req, msg)
-                            continue
-                        break
-                    try:
-                        req.seq = self.cache.open(req.request_id, reserve)
-                    except (OutOfPages, OutOfSlots) as e:
+            self._schedule_prompts(batch, budget)
+        return batch
+
+    def _schedule_prompts(self, batch: ScheduledBatch, budget: int) -> None:
+        """The second half of a step's batch: portions of prompts, from the head of the queue, under what the
+        decoding requests left of the token budget.  The caller holds the lock."""
+        prefill_budget = min(budget, self.config.max_prefill_tokens)
+        while self.waiting and prefill_budget > 0:
+            req = self.waiting[0]
+            if len(self.active) + len([r for r in batch.prefill_requests if r not in self.active]) \
+                    >= self.config.max_batch_requests:
+                break
+            if req.seq is None:
+                reserve = self._reserve(req)
+                if not self.cache.can_open(reserve):
+                    msg = (f"Cannot admit request {req.request_id}: prompt={len(req.input_ids)} tokens, "
+                           f"reserve={reserve} tokens, free pages="
+                           f"{[g.pool.uncommitted for g in self.cache.groups]}, "
+                           f"free slots={self.cache.slots.num_free}")
+                    req.admission_warned = True
+                    if batch.empty() and not self.active:
                         self.waiting.popleft()
-                        self._fail(req, f"Cannot allocate KV cache for request {req.request_id}: {e}")
+                        self._fail(req, msg)
                         continue
-                remaining = len(req.input_ids) - req.prefill_progress
-                chunk = min(remaining, prefill_budget)
+                    break
                 try:
-                    self.cache.ensure(req.seq, req.seq.length + chunk)
-                except OutOfPages as e:
+                    req.seq = self.cache.open(req.request_id, reserve)
+                except (OutOfPages, OutOfSlots) as e:
                     self.waiting.popleft()
                     self._fail(req, f"Cannot allocate KV cache for request {req.request_id}: {e}")
                     continue
-                batch.prefill_requests.append(req)
-                batch.prefill_chunk_starts.append(req.prefill_progress)
-                batch.prefill_chunk_sizes.append(chunk)
-                prefill_budget -= chunk
-                req.prefill_progress += chunk
-                req.phase = RequestPhase.PREFILL
-                if req.prefill_progress >= len(req.input_ids):
-                    self.active.append(self.waiting.popleft())
-                else:
-                    break
-        return batch
+            remaining = len(req.input_ids) - req.prefill_progress
+            chunk = min(remaining, prefill_budget)
+            try:
+                self.cache.ensure(req.seq, req.seq.length + chunk)
+            except OutOfPages as e:
+                self.waiting.popleft()
+                self._fail(req, f"Cannot allocate KV cache for request {req.request_id}: {e}")
+                continue
+            batch.prefill_requests.append(req)
+            batch.prefill_chunk_starts.append(req.prefill_progress)
+            batch.prefill_chunk_sizes.append(chunk)
+            prefill_budget -= chunk
+            req.prefill_progress += chunk
+            req.phase = RequestPhase.PREFILL
+            if req.prefill_progress >= len(req.input_ids):
+                self.active.append(self.waiting.popleft())
+            else:
+                break
 
     def schedule_ahead(self, batch: ScheduledBatch) -> Optional[ScheduledBatch]:
         """The batch after ``batch``, made while ``batch`` still runs, or None when it cannot be known
         yet.  It can when the results of ``batch`` will change nothing but the tokens: the requests it
-        samples for are all that run, none of them reaches its length with this token, is cancelled or
-        needs its history for sampling, and ``schedule()`` would not admit a prompt now.  A request that
-        ends on a stop token in ``batch`` has one token too many computed; ``process_results`` drops it.
-        A waiting prompt that only a request's end makes room for enters one step later than it
-        would without looking ahead."""
+        samples for are all that run, and none of them reaches its length with this token, is cancelled or
+        needs its history for sampling.  Every such request then decodes in the next step, whatever its token
+        (read on the device), and the prompts' portions beside them are what ``schedule()`` would take: lengths
+        and pages are booked when a step is queued, not when it ends.  A request that ends on a stop token in
+        ``batch`` has one token too many computed; ``process_results`` drops it.  A waiting prompt that only a
+        request's end makes room for enters one step later than it would without looking ahead."""
         with self._lock:
             sampled = batch.sampled_requests()
-            if not sampled or len(sampled) != len(self.active) or any(a is not b for a, b in zip(self.active, sampled)):
+            if len(sampled) != len(self.active) or any(a is not b for a, b in zip(self.active, sampled)):
+                return None
+            if not sampled and not self.waiting:
                 return None
             if len(sampled) > self.config.max_batch_tokens:
                 return None
-            if self.waiting:
-                head = self.waiting[0]
-                if head.seq is not None:
-                    return None         # a prompt is partly in: its next portion belongs to the next step
-                if len(self.active) < self.config.max_batch_requests and self.cache.can_open(self._reserve(head)):
-                    return None
             for r in sampled:
                 made = (r.generated_count if r.phase == RequestPhase.DECODE else 0) + 1
                 if r.done or r.cancelled or made >= r.config.max_new_tokens:
@@ -230,7 +231,9 @@ class Scheduler:
                     self.cache.ensure(r.seq, r.seq.length + 1)
             except OutOfPages:
                 return None             # the ordinary step decides who fails
-            return ScheduledBatch(decode_requests=list(sampled), tokens_on_device=True)
+            ahead = ScheduledBatch(decode_requests=list(sampled), tokens_on_device=True)
+            self._schedule_prompts(ahead, self.config.max_batch_tokens - len(sampled))
+            return None if ahead.empty() else ahead
 
     # ---- after the step ------------------------------------------------------------------
     def process_results(self, batch: ScheduledBatch, tokens: Sequence[int]) -> None:

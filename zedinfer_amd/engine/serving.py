@@ -36,8 +36,8 @@ class _Flight:
 
 
 class ServingLoop:
-    """``look_ahead``: while a decode step runs, the next one is queued behind it with its tokens read
-    on the device from what the running step samples, so the device does not wait for the host between
+    """``look_ahead``: while a step runs, the next one is queued behind it with its decoding requests' tokens
+    read on the device from what the running step samples, so the device does not wait for the host between
     steps.  The tokens a request gets are the same either way (``Scheduler.schedule_ahead`` says when the
     next batch is known early).  The reference's loop waits for every step's tokens before it schedules
     the next (src/zedinfer/serving_loop.cpp:330-408)."""
@@ -98,7 +98,7 @@ class ServingLoop:
             if flight is None:
                 return True
         batch = flight.batch
-        if self.look_ahead and flight.tokens_dev is not None:
+        if self.look_ahead:
             ahead = self.scheduler.schedule_ahead(batch)
             if ahead is not None:
                 self._flight = self._launch(ahead, flight.tokens_dev)
@@ -120,7 +120,8 @@ class ServingLoop:
         for r in batch.decode_requests:
             r.stats.decode_time_ms += ms / n_dec if not n_pre else ms * 0.5 / n_dec
         self.scheduler.process_results(batch, tokens)
-        if self._flight is not None and all(r.done for r in self._flight.batch.decode_requests):
+        if (self._flight is not None and not self._flight.batch.prefill_requests
+                and all(r.done for r in self._flight.batch.decode_requests)):
             self._flight = None         # everything the step ahead computes for has ended
         return True
 
