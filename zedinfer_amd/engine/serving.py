@@ -107,6 +107,10 @@ class ServingLoop:
             tokens = flight.wait()
         except Exception as e:  # noqa: BLE001
             self.scheduler.fail_batch(batch, f"step failed: {type(e).__name__}: {e}")
+            if self._flight is not None:
+                # the step queued behind it may carry portions of other requests' prompts: what it computed for
+                # them is not to be trusted either, and its tokens will not be read
+                self.scheduler.fail_batch(self._flight.batch, f"step failed: {type(e).__name__}: {e}")
             self._flight = None
             return True
         now = time.perf_counter()
