@@ -123,8 +123,8 @@ def test_stop_token_ends_generation(tiny):
 
 
 def test_steps_queued_ahead_give_the_same_tokens(tiny):
-    """Decode steps that are queued before the step before them has finished (their tokens are read on
-    the device) against a loop that waits for every step: requests of different lengths, greedy and
+    """Steps that are queued before the step before them has finished (their decoding requests' tokens are read
+    on the device; portions of prompts ride along) against a loop that waits for every step: requests of different lengths, greedy and
     sampled, one that ends on a stop token while a step ahead already computes for it, one that arrives
     while the others decode, and prompts that enter in portions.  Every request gets the same tokens and
     the same reason to end, and no page is lost."""
@@ -154,13 +154,13 @@ def test_steps_queued_ahead_give_the_same_tokens(tiny):
         assert all(r.done and not r.error for r in reqs)
         ie.engine.cache.check()
         assert not ie.engine.cache.live
-        return [(r.result.output_ids, r.result.finish_reason) for r in reqs], loop.steps_ahead
+        return [(r.result.output_ids, r.result.finish_reason) for r in reqs], (loop.steps_ahead, loop.prompt_steps_ahead)
 
     free, _ = run(False, [])
     stop = free[1][0][11]           # a token the second request makes on its way
-    want, none_ahead = run(False, [stop])
-    got, ahead = run(True, [stop])
-    assert none_ahead == 0 and ahead > 10
+    want, (none_ahead, _) = run(False, [stop])
+    got, (ahead, with_prompts) = run(True, [stop])
+    assert none_ahead == 0 and ahead > 10 and with_prompts > 0
     assert want[1][1] == "stop" and len(want[1][0]) <= 12
     assert got == want
 

@@ -50,6 +50,7 @@ class ServingLoop:
         self.look_ahead = os.environ.get("ZEDINFER_DISABLE_LOOKAHEAD", "0") in ("", "0") if look_ahead is None \
             else bool(look_ahead)
         self.steps_ahead = 0            # steps that were queued before the one before them had finished
+        self.prompt_steps_ahead = 0     # those of them that carried portions of prompts
         self._flight: Optional[_Flight] = None
         self._token_ring = StagingRing(engine.device)
         self._last_results = 0.0
@@ -103,6 +104,7 @@ class ServingLoop:
             if ahead is not None:
                 self._flight = self._launch(ahead, flight.tokens_dev)
                 self.steps_ahead += self._flight is not None
+                self.prompt_steps_ahead += self._flight is not None and bool(ahead.prefill_requests)
         try:
             tokens = flight.wait()
         except Exception as e:  # noqa: BLE001
