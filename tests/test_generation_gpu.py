@@ -165,6 +165,45 @@ def test_steps_queued_ahead_give_the_same_tokens(tiny):
     assert got == want
 
 
+@pytest.mark.parametrize("seed", range(5))
+def test_random_workloads_get_the_same_tokens_with_steps_queued_ahead(tiny, seed):
+    """Random requests (prompts from 1 to 200 tokens that enter in portions, greedy and sampled, some that end on
+    stop tokens, arriving while others run, few pages so that some wait) through a loop that queues steps ahead and
+    one that waits for every step, in 32 bits, where a token's logits do not depend on what else is in its step:
+    the same tokens and reasons to end for everyone, and no page lost."""
+    import random
+    from zedinfer_amd import GenerationConfig, InferenceEngine, InferenceRequest, SchedulerConfig
+    from zedinfer_amd.engine import ServingLoop
+    V = tiny["cfg"]["vocab_size"]
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    rng = random.Random(seed)
+    lens = [rng.choice([1, 5, 20, 64, 65, 130, 200]) for _ in range(9)]
+    prompts = [traces.random_tokens(V, n, seed=seed * 50 + i) for i, n in enumerate(lens)]
+    cfgs = [dict(max_new_tokens=rng.randint(1, 30), ignore_eos=rng.random() < 0.7, temperature=rng.choice([0.0, 0.0, 0.8]),
+                 top_k=rng.choice([0, 10]), seed=rng.randint(1, 99)) for _ in lens]
+    arrive = sorted(rng.randrange(0, 25) for _ in lens)
+    sched = dict(num_kv_blocks=rng.choice([60, 90, 200]) * 16 // ps, kv_block_size=ps, max_batch_requests=rng.choice([2, 4, 8]),
+                 max_prefill_tokens=rng.choice([24, 64, 512]), max_batch_tokens=rng.choice([72, 128, 520]), generation_reserve=32)
+    outs, ahead = [], None
+    for look_ahead in (False, True):
+        ie = InferenceEngine.create(tiny["folder"], "float32", SchedulerConfig(**sched))
+        loop = ServingLoop(ie.engine, [7, 11, 13], look_ahead=look_ahead)
+        reqs, step, todo = [], 0, list(zip(arrive, prompts, cfgs))
+        while todo or loop.scheduler.has_work():
+            while todo and todo[0][0] <= step:
+                _, p, c = todo.pop(0)
+                reqs.append(loop.submit_async(InferenceRequest(p, GenerationConfig(**c))))
+            loop.step()
+            step += 1
+            assert step < 5000
+        ie.engine.cache.check()
+        assert not ie.engine.cache.live
+        outs.append([(r.error, r.result.finish_reason if r.result else None, r.result.output_ids if r.result else None)
+                     for r in reqs])
+        ahead = loop.steps_ahead
+    assert ahead > 0 and outs[0] == outs[1]
+
+
 def test_steps_queued_ahead_without_graphs(tiny, monkeypatch):
     """The same with decode steps launched kernel by kernel (no graphs): the tokens of a step queued
     ahead are copied into the step's batch on the device."""
