@@ -485,3 +485,16 @@ def test_sizes_at_which_a_serving_engine_measures_its_choices():
     for n in range(128, 20001, 7):
         up = many_rows_size_at_least(n)
         assert up in sizes and n <= up <= n + max(63, n // 32), n
+    # what an engine measures by default: the sizes of its steps with prompt portions, and of its pure decode steps
+    # of more than 64 requests
+    from zedinfer_amd.engine import InferenceEngine
+    from zedinfer_amd.engine.engine import decode_entries_at_least
+    few = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=520, max_prefill_tokens=512))
+    assert few == [640, 576, 512, 448, 384, 320, 256, 192, 128]     # 520 tokens, rounded up, and one more size
+    many = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=200, max_batch_tokens=2248, max_prefill_tokens=2048))
+    assert many[0] == 2368 and many[-3:] == [160, 128, 96] and 224 in many and len(many) == len(set(many))
+    for e in range(65, 201):
+        assert decode_entries_at_least(e) in many
+    long = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=16392, max_prefill_tokens=16384,
+                                                                 max_seq_len=32768))
+    assert long[:4] == [16896, 16384, 8448, 8192] and long[-1] == 128

@@ -17,7 +17,7 @@ import torch
 from ..config import SchedulerConfig
 from ..ops.staging import StagingRing
 from ..sampling.sampler import Sampler
-from .engine import Engine, many_rows_size_at_least, many_rows_step_sizes
+from .engine import Engine, decode_entries_at_least, many_rows_size_at_least, many_rows_step_sizes
 from .request import GenerationConfig, GenerationResult, InferenceRequest
 from .scheduler import ScheduledBatch, Scheduler
 
@@ -162,6 +162,22 @@ class InferenceEngine:
 
     WARM_UP_EVERY_SIZE_UP_TO = 8192     # rows; measuring every size of longer steps would take minutes
 
+    @classmethod
+    def default_warm_up_sizes(cls, sched: SchedulerConfig, most_entries: int = 256) -> List[int]:
+        """The numbers of rows that the steps of an engine with these limits come in, largest first: every size
+        a step with portions of prompts can bring (``many_rows_step_sizes``) up to WARM_UP_EVERY_SIZE_UP_TO rows, of
+        longer steps the two that recur (a full portion alone and beside decoding requests), and the sizes of pure
+        decode steps of more requests than the few-rows kernels take (``decode_entries_at_least``)."""
+        step = Engine.PROMPT_GRAPH_STEP
+        # a portion and the decoding entries beside it are rounded up: one more size
+        most = min(sched.max_batch_tokens, sched.max_prefill_tokens + sched.max_batch_requests)
+        sizes = many_rows_step_sizes(min(most, cls.WARM_UP_EVERY_SIZE_UP_TO) + step)
+        if most > cls.WARM_UP_EVERY_SIZE_UP_TO:
+            sizes += [many_rows_size_at_least(sched.max_prefill_tokens),
+                      many_rows_size_at_least(min(most, sched.max_prefill_tokens + step) + step)]
+        sizes += [decode_entries_at_least(e) for e in range(65, min(sched.max_batch_requests, most_entries) + 1)]
+        return sorted(set(sizes), reverse=True)
+
     def __init__(self, engine: Engine, warm_up_sizes: Optional[Sequence[int]] = None):
         """``warm_up_sizes``: the numbers of rows to measure the parts' choices for (None: every size a step with
         prompt portions can bring under the scheduler's limits; empty: none)."""
@@ -176,16 +192,8 @@ class InferenceEngine:
         # src/zedinfer/engine.cpp:506)
         if (os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and "ZEDINFER_DISABLE_WARMUP" not in os.environ
                 and engine.device.type == "cuda"):
-            sched = engine.sched
-            most = min(sched.max_batch_tokens, sched.max_prefill_tokens + sched.max_batch_requests)
-            if warm_up_sizes is None:       # a portion and the decoding entries are rounded up: one more size
-                step = Engine.PROMPT_GRAPH_STEP
-                warm_up_sizes = many_rows_step_sizes(min(most, self.WARM_UP_EVERY_SIZE_UP_TO) + step)
-                if most > self.WARM_UP_EVERY_SIZE_UP_TO:
-                    # of longer steps only the ones that recur: a full portion, alone and beside decoding requests
-                    full = sorted({many_rows_size_at_least(sched.max_prefill_tokens),
-                                   many_rows_size_at_least(min(most, sched.max_prefill_tokens + step) + step)}, reverse=True)
-                    warm_up_sizes = [n for n in full if n > warm_up_sizes[0]] + warm_up_sizes
+            if warm_up_sizes is None:
+                warm_up_sizes = self.default_warm_up_sizes(engine.sched, engine.graph_max_entries)
             engine.warm_up(list(warm_up_sizes))
         # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
         # taken out of the garbage collector's passes, a full collection in the middle of serving costs
