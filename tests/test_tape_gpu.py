@@ -308,3 +308,42 @@ def test_decode_steps_of_fewer_and_fewer_requests_share_a_shape(tmp_path, dtype)
     decode(live)                                        # four requests: a shape of its own
     assert sorted(k[0] for k in e._graphs) == [4, 8]
     e.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_decode_steps_that_want_some_rows_only(tmp_path, dtype, graphs):
+    """Four requests decode; which of them want their logits changes from step to step (all, two of them, another
+    two, one, none, all again).  Steps that want every row pick no rows at all, the others do: they are different
+    kinds of steps although they have as many entries and, padded, as many wanted rows, and each wanted row is its
+    own request's whichever kind ran before."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "A", dtype=store, std=tiny_configs.SHARP_STD)
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["A"]
+    e = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=4 * (64 // ps + 1), kv_block_size=ps, max_batch_requests=4))
+    e.use_graphs, e.graph_after = graphs, 2
+    names = list("abcd")
+    toks = {r: traces.random_tokens(cfg["vocab_size"], 48, seed=70 + i) for i, r in enumerate(names)}
+    ref = {r: plain.forward(cfg, w, t) for r, t in toks.items()}
+    seqs, fed = {}, {}
+    for i, r in enumerate(names):
+        seqs[r] = e.open(r)
+        e.step([StepEntry(seqs[r], toks[r][:4 + i], [])])
+        fed[r] = 4 + i
+    patterns = ["abcd", "abcd", "ac", "ac", "bd", "abcd", "c", "", "ac", "abd", "abcd", "bd", "bd", "bd", "abcd"]
+    for wanting in patterns:
+        got = e.step([StepEntry(seqs[r], toks[r][fed[r]:fed[r] + 1], [0] if r in wanting else []) for r in names])
+        assert (got is None) == (not wanting) and (got is None or got.shape[0] == len(wanting))
+        for row, r in enumerate(wanting):
+            d = (got[row].cpu() - ref[r][fed[r]]).abs()
+            scale = float(ref[r].abs().max())
+            if dtype == "float32":
+                assert float(d.max()) < F32_TOL * max(1.0, scale), (wanting, r)
+            else:
+                assert bf16_within(float(d.max()), float(d.mean()), scale), (wanting, r)
+        for r in names:
+            fed[r] += 1
+    assert e.tape_runs + e.graph_replays > 0 and (e.graph_replays > 0) == graphs

@@ -240,7 +240,9 @@ class Engine:
         # a bound, the same for many steps, of the tokens any sequence holds after this step: the
         # mixers' planners size their launches by it
         bound = _bucket_at_least(max(e.seq.length for e in entries) + 1, 256)
-        key = (E, R, widths, bound)
+        # (whether every token's row is wanted, in order, decides if the model picks rows at all: such steps and
+        # steps that want some rows only, or rows of padding entries, are different kinds)
+        key = (E, R, widths, bound, wanted == E)
         dg = self._graphs.pop(key, None)
         if dg is not None:
             self._graphs[key] = dg              # used last: the last to go
