@@ -81,15 +81,17 @@ def check(tiny, dtype, steps, outputs):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("shape", ["whole", "last32", "portions", "mixed"])
+@pytest.mark.parametrize("shape", ["whole", "last32", "portions", "mixed", "mixed_few_wanted"])
 def test_engine_matches_plain(tiny, dtype, shape):
     steps = {"whole": traces.whole, "last32": traces.last_decoded, "portions": traces.portions,
-             "mixed": traces.mixed}[shape](tiny["requests"])
+             "mixed": traces.mixed,
+             "mixed_few_wanted": lambda reqs: traces.few_wanted(traces.mixed(reqs, decode_tail=24, seed=3), seed=3)
+             }[shape](tiny["requests"])
     ps = tiny_configs.PAGE_SIZES[tiny["name"]]
     pages = traces.max_live_tokens(steps) // ps      # as few pages as the replay tool would have
     engine = make_engine(tiny, dtype, pages)
     out = traces.run_in_process(engine, steps)
-    if shape == "mixed":
+    if shape.startswith("mixed"):
         # pages were given back and taken again: more pages handed out than the pool has
         assert all(g.pool.takes > g.pool.total for g in engine.cache.groups)
     check(tiny, dtype, steps, out)

@@ -92,6 +92,17 @@ def mixed(requests, max_live=4, seed=0, decode_tail=12, max_portion=24):
     return steps
 
 
+def few_wanted(steps, seed=0, none=0.15):
+    """The same steps with the logits of at most the last token of each entry wanted, and of some entries none:
+    which rows a step wants then changes from step to step among steps of the same entries."""
+    rng = random.Random(seed)
+    out = []
+    for st in steps:
+        entries = [dict(e, want=[] if rng.random() < none else [len(e["tokens"]) - 1]) for e in st["entries"]]
+        out.append(dict(st, entries=entries))
+    return out
+
+
 def max_live_tokens(steps, round_to=64):
     """The largest sum over live requests of their token counts rounded up, at any step."""
     held, best = {}, 0
