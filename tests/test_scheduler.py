@@ -498,3 +498,24 @@ def test_sizes_at_which_a_serving_engine_measures_its_choices():
     long = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=16392, max_prefill_tokens=16384,
                                                                  max_seq_len=32768))
     assert long[:4] == [16896, 16384, 8448, 8192] and long[-1] == 128
+
+
+def test_a_recorded_shape_refuses_a_step_that_plans_differently():
+    """A shape that has been recorded (tape or graph) keeps the launch sizes and the sizes of the index arrays that
+    the mixers' planners gave its first step; a later step of the shape whose plan differs (a planner whose
+    ``shape`` does not name all that its plan depends on) raises instead of running the wrong launches."""
+    import numpy as np
+    from types import SimpleNamespace
+    from zedinfer_amd.engine.engine import Engine, _DecodeGraph
+    from zedinfer_amd.parts.base import StepPlan
+
+    def batch(tiles, n):
+        return SimpleNamespace(plans={("attention", 16): StepPlan(arrays={"tile_entry": np.zeros(n, np.int32)},
+                                                                  sizes={"num_tiles": tiles, "tile": 64})})
+    dg = _DecodeGraph()
+    Engine._same_plans(dg, batch(3, 3))
+    Engine._same_plans(dg, batch(3, 3))
+    with pytest.raises(RuntimeError, match="plans its launches differently"):
+        Engine._same_plans(dg, batch(4, 3))
+    with pytest.raises(RuntimeError, match="plans its launches differently"):
+        Engine._same_plans(dg, batch(3, 5))

@@ -289,6 +289,7 @@ class Engine:
         another's at the next run): that is the rule at a shape's first step when workspaces still grow, and the
         step is then recorded again the next time; a second such recording marks the shape as one that cannot be
         taped.  The batch lives in the shape's own buffer, as for a graph."""
+        self._same_plans(dg, batch)
         if dg.tape is not None:
             dg.tape.run()
             self.tape_runs += 1
@@ -305,6 +306,17 @@ class Engine:
         dg.ran = True
         return logits
 
+
+    @staticmethod
+    def _same_plans(dg: "_DecodeGraph", batch) -> None:
+        """A recorded step fixes its launches: the sizes that the mixers' planners gave its first step must be what
+        they give every later step of the shape (``StepPlanner.shape`` has to name all that they depend on)."""
+        planned = {key: (tuple(sorted(plan.sizes.items())), tuple((name, int(a.size)) for name, a in plan.arrays.items()))
+                   for key, plan in batch.plans.items()}
+        if dg.planned is None:
+            dg.planned = planned
+        elif planned != dg.planned:
+            raise RuntimeError(f"a step of a recorded shape plans its launches differently: {planned} against {dg.planned}")
 
     def _drop_oldest(self, graphs: Dict[tuple, "_DecodeGraph"]) -> None:
         """Forget the first graph of the dictionary.  One that was recorded may still be running, and with
@@ -394,6 +406,7 @@ class Engine:
         if token_source is not None:
             batch.token_ids[:token_source.shape[0]].copy_(token_source, non_blocking=True)
         if dg.graph is not None:
+            self._same_plans(dg, batch)
             dg.graph.replay()
             self.prompt_graph_replays += 1
             return dg.logits[:wanted] if wanted else None
@@ -422,6 +435,7 @@ class _DecodeGraph:
         self.ran = False                                # a step of the shape has run part by part
         self.tape = None                                # the library calls of one step of the shape
         self.no_tape = False                            # a step of the shape cannot be recorded
+        self.planned = None                             # the sizes the planners gave the shape's first step
         self.image: Optional[DecodeImage] = None
 
 
