@@ -1,4 +1,4 @@
-// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for 1..64 rows of x: the decode-time products, bound by the one
+// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for 1..128 rows of x: the decode-time products, bound by the one
 // pass over the weights (the entry points are in gemm_skinny.hip).
 //
 // A workgroup of four to eight wavefronts owns 16 weight rows a wavefront and a range of k.  It walks its
@@ -41,6 +41,73 @@ union gm_pack {
 __device__ __forceinline__ gm_u32x4_t gm_keep(gm_u32x4_t v, bool keep) {
     const unsigned mask = 0u - (unsigned)keep;
     return v & mask;
+}
+
+// What a wavefront does with its sums: C[n = n0 + j*4 + e][m = t*16 + r] in acc[t][e].
+template <int MT>
+__device__ __forceinline__ void gm_epilogue(const gm_f32x4_t (&acc)[MT], void* __restrict__ out, int mode, int out_f32,
+                                            const zi_bf16* __restrict__ bias, int M, int N, int64_t ldo, int split,
+                                            int n0, int r, int j, int vec_out) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        gm_f32x4_t s = acc[t];
+        const int m = t * 16 + r;
+        if (mode == GM_MODE_SWIGLU) {
+            // lanes j = 0,1 hold gate rows j*4 + e, lanes j = 2,3 the up rows of the same columns
+            gm_f32x4_t up;
+            up[0] = __shfl_xor(s[0], 32, ZI_WAVE); up[1] = __shfl_xor(s[1], 32, ZI_WAVE);
+            up[2] = __shfl_xor(s[2], 32, ZI_WAVE); up[3] = __shfl_xor(s[3], 32, ZI_WAVE);
+            if (j >= 2 || m >= M || n0 >= N) continue;
+            const int col = (n0 / 16) * 8 + j * 4;     // N / 2 columns of output; N % 16 == 0
+            float act[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) act[e] = up[e] * (s[e] / (1.f + expf(-s[e])));
+            zi_bf16* dst = (zi_bf16*)out + (int64_t)m * ldo + col;
+            if (vec_out) {
+                uint2 pk;
+                pk.x = zi_pack_bf16x2(act[0], act[1]);
+                pk.y = zi_pack_bf16x2(act[2], act[3]);
+                *reinterpret_cast<uint2*>(dst) = pk;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) zi_store(dst + e, act[e]);
+            }
+            continue;
+        }
+        if (m >= M) continue;
+        const int nb = n0 + j * 4;
+        if (nb + 3 < N && vec_out) {
+            if (mode == GM_MODE_PARTIAL) {
+                *reinterpret_cast<gm_f32x4_t*>((float*)out + ((int64_t)split * M + m) * N + nb) = s;
+            } else {
+                if (bias) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) s[e] += zi_load(bias + nb + e);
+                }
+                if (out_f32) {
+                    *reinterpret_cast<gm_f32x4_t*>((float*)out + (int64_t)m * ldo + nb) = s;
+                } else {
+                    uint2 pk;
+                    pk.x = zi_pack_bf16x2(s[0], s[1]);
+                    pk.y = zi_pack_bf16x2(s[2], s[3]);
+                    *reinterpret_cast<uint2*>((zi_bf16*)out + (int64_t)m * ldo + nb) = pk;
+                }
+            }
+            continue;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = nb + e;
+            if (n >= N) continue;
+            if (mode == GM_MODE_PARTIAL) {
+                ((float*)out)[((int64_t)split * M + m) * N + n] = s[e];
+            } else {
+                const float v = s[e] + (bias ? zi_load(bias + n) : 0.f);
+                if (out_f32) ((float*)out)[(int64_t)m * ldo + n] = v;
+                else zi_store((zi_bf16*)out + (int64_t)m * ldo + n, v);
+            }
+        }
+    }
 }
 
 template <int MT, int GM_RING, int GM_WAVES>
@@ -173,67 +240,124 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
             default: if (GM_RING > 3) ending(std::integral_constant<int, 3>{}, kb0); break;
         }
     }
-    // C[n = n0 + j*4 + e][m = t*16 + r]
+    gm_epilogue<MT>(acc, out, mode, out_f32, bias, M, N, ldo, split, n0, r, j, vec_out);
+}
+
+// The same product for 65 .. 128 rows of x (MT = 5 .. 8 tiles of 16 rows): one pass over the weights where two
+// launches of the kernel above would make two, and where the library's products of so few rows stay far from the
+// weights' stream.  The registers that the kernel above spends on rings of x and on all of a block's x operands
+// do not stretch to eight tiles, so here a block's x is requested one step ahead only (it comes from the cache;
+// the weights keep their ring of three), it lies in LDS once (two barriers a block instead of one: 32 KB for
+// 128 rows, and with the wavefronts' weight tiles that is the 64 KB a workgroup may declare), and the x operands
+// are read a k-step at a time, just before their matrix instructions.  The cut, the order of the sums and the
+// epilogues are the kernel's above: a row's result does not depend on which of the two kernels makes it.
+template <int MT, int GM_WAVES>
+__global__ void __launch_bounds__(GM_WAVES* ZI_WAVE)
+gemm_wide_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __restrict__ x,
+                 const zi_bf16* __restrict__ w, const zi_bf16* __restrict__ bias, int M, int N, int K, int64_t ldx,
+                 int64_t ldw, int64_t ldo, int kb_per_split, int vec_out) {
+    constexpr int RING = 3;
+    __shared__ __attribute__((aligned(16))) uint16_t xs[MT * 16 * GM_XS];
+    __shared__ __attribute__((aligned(16))) uint16_t wt[GM_WAVES][16 * GM_XS];
+    const int tid = threadIdx.x, lane = tid & (ZI_WAVE - 1), wave = tid / ZI_WAVE;
+    const int r = lane & 15, j = lane >> 4;
+    const int split = blockIdx.y;
+    const int kb_total = (K + GM_KB - 1) / GM_KB;
+    const int kb_lo = split * kb_per_split;
+    const int kb_hi = (kb_lo + kb_per_split < kb_total) ? kb_lo + kb_per_split : kb_total;
+    const int n0 = (blockIdx.x * GM_WAVES + wave) * 16;
+    const int wq = lane & 15;
+    const zi_bf16* wrow[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const int n = n0 + c * 4 + j;
+        wrow[c] = w + (int64_t)(n < N ? n : N - 1) * ldw;
+    }
+    uint16_t* const wt_w = &wt[wave][0];
+    const int srow = (tid % GM_STAGERS) / 16, spc = tid % 16;
+    const bool stager = tid < GM_STAGERS;
+    gm_u32x4_t ring[RING][4], xnext[MT];
+    const zi_bf16* xrow[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-        gm_f32x4_t s = acc[t];
-        const int m = t * 16 + r;
-        if (mode == GM_MODE_SWIGLU) {
-            // lanes j = 0,1 hold gate rows j*4 + e, lanes j = 2,3 the up rows of the same columns
-            gm_f32x4_t up;
-            up[0] = __shfl_xor(s[0], 32, ZI_WAVE); up[1] = __shfl_xor(s[1], 32, ZI_WAVE);
-            up[2] = __shfl_xor(s[2], 32, ZI_WAVE); up[3] = __shfl_xor(s[3], 32, ZI_WAVE);
-            if (j >= 2 || m >= M || n0 >= N) continue;
-            const int col = (n0 / 16) * 8 + j * 4;     // N / 2 columns of output; N % 16 == 0
-            float act[4];
+        const int m = t * 16 + srow;
+        xrow[t] = x + (int64_t)(m < M ? m : M - 1) * ldx;
+    }
+    // a block's x is requested before the weights that are requested in the same step: loads return in order,
+    // and x is wanted first.  The block index is clamped: the last step asks for its own block again.
+    auto fetch_x = [&](int kb) __attribute__((always_inline)) {
+        const int k0 = (kb < kb_hi ? kb : kb_hi - 1) * GM_KB;
+        const int kx = k0 + spc * 8 < K ? k0 + spc * 8 : K - 8;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) act[e] = up[e] * (s[e] / (1.f + expf(-s[e])));
-            zi_bf16* dst = (zi_bf16*)out + (int64_t)m * ldo + col;
-            if (vec_out) {
-                uint2 pk;
-                pk.x = zi_pack_bf16x2(act[0], act[1]);
-                pk.y = zi_pack_bf16x2(act[2], act[3]);
-                *reinterpret_cast<uint2*>(dst) = pk;
-            } else {
+        for (int t = 0; t < MT; ++t) xnext[t] = *reinterpret_cast<const gm_u32x4_t*>(xrow[t] + kx);
+    };
+    auto fetch_w = [&](const int slot, int kb) __attribute__((always_inline)) {
+        const int k = kb * GM_KB + wq * 8;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) zi_store(dst + e, act[e]);
-            }
-            continue;
+        for (int c = 0; c < 4; ++c) ring[slot][c] = *reinterpret_cast<const gm_u32x4_t*>(wrow[c] + (k < K ? k : K - 8));
+    };
+    auto stash = [&]() __attribute__((always_inline)) {
+        if (GM_WAVES * ZI_WAVE > GM_STAGERS && !stager) return;
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+            *reinterpret_cast<gm_u32x4_t*>(&xs[(t * 16 + srow) * GM_XS + (spc ^ srow) * 8]) = xnext[t];
+    };
+    gm_f32x4_t acc[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[t] = gm_f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto step = [&](const int slot, int kb, const bool request) __attribute__((always_inline)) {
+        fetch_x(kb + 1);
+        if (request) fetch_w((slot + RING - 1) % RING, kb + RING - 1);
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            *reinterpret_cast<gm_u32x4_t*>(wt_w + (c * 4 + j) * GM_XS + (wq ^ (c * 4 + j)) * 8) =
+                gm_keep(ring[slot][c], kb * GM_KB + wq * 8 < K);
+        gm_pack a[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) a[c].u = *reinterpret_cast<const gm_u32x4_t*>(wt_w + r * GM_XS + ((c * 4 + j) ^ r) * 8);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            gm_pack bb[MT];
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                bb[t].u = *reinterpret_cast<const gm_u32x4_t*>(&xs[(t * 16 + r) * GM_XS + ((c * 4 + j) ^ r) * 8]);
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[c].b, bb[t].b, acc[t], 0, 0, 0);
         }
-        if (m >= M) continue;
-        const int nb = n0 + j * 4;
-        if (nb + 3 < N && vec_out) {
-            if (mode == GM_MODE_PARTIAL) {
-                *reinterpret_cast<gm_f32x4_t*>((float*)out + ((int64_t)split * M + m) * N + nb) = s;
-            } else {
-                if (bias) {
+        __syncthreads();        // every wavefront has read this block's x
+        stash();                // the next block's (after the last block: something nobody reads)
+        __syncthreads();
+    };
+    auto ending = [&](auto left_c, int kb0) __attribute__((always_inline)) {
+        constexpr int LEFT = decltype(left_c)::value;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) s[e] += zi_load(bias + nb + e);
-                }
-                if (out_f32) {
-                    *reinterpret_cast<gm_f32x4_t*>((float*)out + (int64_t)m * ldo + nb) = s;
-                } else {
-                    uint2 pk;
-                    pk.x = zi_pack_bf16x2(s[0], s[1]);
-                    pk.y = zi_pack_bf16x2(s[2], s[3]);
-                    *reinterpret_cast<uint2*>((zi_bf16*)out + (int64_t)m * ldo + nb) = pk;
-                }
-            }
-            continue;
-        }
+        for (int i = 0; i < LEFT + RING - 1; ++i) step(i % RING, kb0 + i, i < LEFT);
+    };
+    fetch_x(kb_lo);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int n = nb + e;
-            if (n >= N) continue;
-            if (mode == GM_MODE_PARTIAL) {
-                ((float*)out)[((int64_t)split * M + m) * N + n] = s[e];
-            } else {
-                const float v = s[e] + (bias ? zi_load(bias + n) : 0.f);
-                if (out_f32) ((float*)out)[(int64_t)m * ldo + n] = v;
-                else zi_store((zi_bf16*)out + (int64_t)m * ldo + n, v);
-            }
+    for (int b = 0; b < RING - 1; ++b) fetch_w(b, kb_lo + b < kb_hi ? kb_lo + b : kb_hi - 1);
+    stash();
+    __syncthreads();
+    int kb0 = kb_lo;
+    for (; kb0 + 2 * RING - 1 <= kb_hi; kb0 += RING) {
+#pragma unroll
+        for (int b = 0; b < RING; ++b) step(b, kb0 + b, true);
+    }
+    const int left = kb_hi - kb0 - (RING - 1);
+    if (left < 0) {
+#pragma unroll
+        for (int b = 0; b < RING - 1; ++b)
+            if (kb0 + b < kb_hi) step(b, kb0 + b, false);
+    } else {
+        switch (left) {
+            case 0: ending(std::integral_constant<int, 0>{}, kb0); break;
+            case 1: ending(std::integral_constant<int, 1>{}, kb0); break;
+            default: ending(std::integral_constant<int, 2>{}, kb0); break;
         }
     }
+    gm_epilogue<MT>(acc, out, mode, out_f32, bias, M, N, ldo, split, n0, r, j, vec_out);
 }
 
 // How the product with a weight matrix [N, K] is cut: wavefronts a workgroup (16 weight rows each), splits
@@ -292,13 +416,30 @@ int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const
         case 7: ZI_GM2(MT, 7); break;           \
         default: ZI_GM2(MT, 8); break;          \
     }
+#define ZI_GW2(MT, WV)                                                                                         \
+    gemm_wide_kernel<MT, WV><<<grid, WV * ZI_WAVE, 0, stream>>>(out, mode, out_f32, x, w, bias, M, N, K, ldx, ldw, ldo, \
+                                                               per, vec_out)
+#define ZI_GW(MT)                               \
+    switch (waves) {                            \
+        case 4: ZI_GW2(MT, 4); break;           \
+        case 5: ZI_GW2(MT, 5); break;           \
+        case 6: ZI_GW2(MT, 6); break;           \
+        case 7: ZI_GW2(MT, 7); break;           \
+        default: ZI_GW2(MT, 8); break;          \
+    }
     switch (mt) {
         case 1: ZI_GM(1); break;
         case 2: ZI_GM(2); break;
         case 3: ZI_GM(3); break;
-        default: ZI_GM(4); break;
+        case 4: ZI_GM(4); break;
+        case 5: ZI_GW(5); break;
+        case 6: ZI_GW(6); break;
+        case 7: ZI_GW(7); break;
+        default: ZI_GW(8); break;
     }
 #undef ZI_GM
 #undef ZI_GM2
+#undef ZI_GW
+#undef ZI_GW2
     return zi_check_launch("gemm_mid");
 }

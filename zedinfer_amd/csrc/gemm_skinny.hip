@@ -1,4 +1,4 @@
-// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for up to 64 rows of x: the decode-time matrix products, bound by the
+// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for up to 128 rows of x: the decode-time matrix products, bound by the
 // one pass over the weights.  This file holds their entry points, the cut's bookkeeping and the kernel that
 // adds partial sums; the product kernel is in gemm_mid.hip (it stages x in LDS, a workgroup's wavefronts
 // take 16 weight rows each, and the cut over workgroups is balanced over the compute units).
@@ -37,7 +37,7 @@ __global__ void gemm_skinny_reduce_kernel(void* __restrict__ out, int out_f32, c
 }
 
 extern "C" int zi_gemm_skinny_supported(int M, int N, int K, int64_t ldx, int64_t ldw) {
-    return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
+    return M >= 1 && M <= 128 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
 }
 
 // The product kernel (gemm_mid.hip): its cut and its launch.
@@ -68,7 +68,7 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
                               int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, float* workspace,
                               int64_t workspace_floats, hipStream_t stream) {
     ZI_REQUIRE(zi_gemm_skinny_supported(M, N, K, ldx, ldw),
-               "gemm_skinny: unsupported sizes M=%d N=%d K=%d (1 <= M <= 64, K and row strides multiples of 8)", M, N, K);
+               "gemm_skinny: unsupported sizes M=%d N=%d K=%d (1 <= M <= 128, K and row strides multiples of 8)", M, N, K);
     ZI_REQUIRE(out_dt == ZI_F32 || out_dt == ZI_BF16, "gemm_skinny: unknown output dtype %d", out_dt);
     ZI_REQUIRE(mode >= 0 && mode <= 2, "gemm_skinny: unknown mode %d", mode);
     ZI_REQUIRE(ldx >= K && ldw >= K, "gemm_skinny: leading dimension too small");

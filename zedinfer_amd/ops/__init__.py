@@ -14,7 +14,8 @@ from .functional import (add, add_rms_norm, argmax, attention, attention_decode,
                          has_cuda, has_gpu, linear, linear_choose, linear_splits, linear_sums,
                          linear_sums_supported, linear_swiglu, linear_swiglu_supported,
                          linear_transposed, linear_tune, reduce_sums, rms_norm, rope, rope_inv_freq,
-                         rope_kv_store, rope_kv_store_sums, rope_table, sample, swiglu, swiglu_t)
+                         rope_kv_store, rope_kv_store_sums, rope_table, sample, swiglu, swiglu_t,
+                         FEW_ROWS, SUMS_MAX_ROWS)
 from ._lib import KernelLibraryError, library_path, load
 
 __all__ = [
@@ -26,5 +27,5 @@ __all__ = [
     "linear", "linear_choose", "linear_splits", "linear_sums", "linear_sums_supported", "linear_swiglu",
     "linear_swiglu_supported", "linear_transposed", "linear_tune", "reduce_sums", "rms_norm", "rope",
     "rope_inv_freq", "rope_kv_store", "rope_kv_store_sums", "rope_table", "sample", "swiglu", "swiglu_t",
-    "KernelLibraryError", "library_path", "load",
+    "KernelLibraryError", "library_path", "load", "FEW_ROWS", "SUMS_MAX_ROWS",
 ]

@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_float, c_int, c_void_p
 from typing import Optional, Tuple
 
@@ -785,11 +786,13 @@ def linear_choose(x: torch.Tensor, weight: torch.Tensor, which: int, bias: Optio
               M if transposed else N, LIBRARY_WORKSPACE_BYTES, int(which))
 
 
-def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether ``linear_sums`` takes this product: bfloat16, at most FEW_ROWS rows."""
+def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor, most_rows: Optional[int] = None) -> bool:
+    """Whether ``linear_sums`` takes this product: bfloat16, at most SUMS_MAX_ROWS rows (or ``most_rows``,
+    if that is fewer)."""
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.dim() != 2 or weight.dim() != 2:
         return False
-    if not (0 < x.shape[0] <= FEW_ROWS) or x.shape[1] != weight.shape[1]:
+    most = SUMS_MAX_ROWS if most_rows is None else min(int(most_rows), SUMS_MAX_ROWS)
+    if not (0 < x.shape[0] <= most) or x.shape[1] != weight.shape[1]:
         return False
     if (x.shape[1] > 1 and x.stride(1) != 1) or (weight.shape[1] > 1 and weight.stride(1) != 1):
         return False
@@ -802,11 +805,11 @@ def linear_splits(M: int, N: int, K: int) -> int:
 
 
 def linear_sums(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x[M,K] . weight[N,K]^T for M <= FEW_ROWS as float32 partial sums [S, M, N], S =
+    """x[M,K] . weight[N,K]^T for M <= SUMS_MAX_ROWS as float32 partial sums [S, M, N], S =
     ``linear_splits(M, N, K)``, without bias: the consumer adds them in rising order."""
     _gpu("linear_sums", x, weight, out)
     if not linear_sums_supported(x, weight):
-        raise ValueError(f"linear_sums: needs bfloat16 x and weight, at most {FEW_ROWS} rows, 16-byte aligned rows")
+        raise ValueError(f"linear_sums: needs bfloat16 x and weight, at most {SUMS_MAX_ROWS} rows, 16-byte aligned rows")
     M, K = x.shape
     N = weight.shape[0]
     S = linear_splits(M, N, K)
@@ -820,7 +823,7 @@ def linear_sums(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tenso
 
 
 def linear_swiglu_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    return (linear_sums_supported(x, weight) and weight.shape[0] % 16 == 0
+    return (linear_sums_supported(x, weight, FEW_ROWS) and weight.shape[0] % 16 == 0
             and linear_splits(x.shape[0], weight.shape[0], weight.shape[1]) == 1)
 
 
@@ -860,8 +863,15 @@ def reduce_sums(sums: torch.Tensor, bias: Optional[torch.Tensor] = None, out: Op
     return out
 
 
-SKINNY_MAX_ROWS = 64   # rows the few-rows kernels take in one launch
+SKINNY_MAX_ROWS = 64   # rows ``linear`` gives the few-rows kernels in one launch
 FEW_ROWS = 64          # up to here they beat the library product: the weights stream once, x stays on the chip
+# Products that leave partial sums (q/k/v, output, down: few weight rows, k cut over workgroups) go to the
+# few-rows kernel up to this many rows: measured at 128 rows with the weights coming from memory, 1.5B sizes,
+# 6.2 / 5.6 / 17.5 us against the library's 9.7 / 8.1 / 24.5; 7B sizes 20 / 16 / 55 against 20 / 16 / 92.  The
+# gate/up product with its activation does not (37 against 24 + 5 us at the 1.5B sizes: every wavefront reads
+# all of x from LDS for its 16 weight rows, and with 128 rows those reads bound it): FEW_ROWS stays its limit.
+# (ZEDINFER_SUMS_MAX_ROWS=64 gives such products of more than 64 rows back to the library.)
+SUMS_MAX_ROWS = max(FEW_ROWS, min(128, int(os.environ.get("ZEDINFER_SUMS_MAX_ROWS", "128") or 128)))
 _WORKSPACES = {}
 _OUTGROWN_WORKSPACES: list = []
 

@@ -132,7 +132,7 @@ class SwiGLU(FeedForward):
         act = self.rt.buffer("ffn_act", (n, I))
         if self.interleave and ops.linear_swiglu_supported(x, self.gate_up):
             ops.linear_swiglu(x, self.gate_up, out=act)
-        elif self.interleave and ops.linear_sums_supported(x, self.gate_up):
+        elif self.interleave and ops.linear_sums_supported(x, self.gate_up, ops.FEW_ROWS):
             S = ops.linear_splits(n, 2 * I, self.hidden)
             sums = ops.linear_sums(x, self.gate_up, out=self.rt.buffer("ffn_gate_up_sums", (S, n, 2 * I), torch.float32))
             ops.swiglu(sums, out=act, interleave=self.interleave)
