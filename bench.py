@@ -9,7 +9,7 @@ A step is one decode step of the serving loop (schedule, model, sampling) with `
 requests that each hold a 2,048-token prompt.  Prints ONE JSON line.  Besides the decode speed it
 reports a 2,048-token prefill (tokens a second and the fraction of the bf16 matrix peak), the
 decode step against the HBM roofline (bytes that must be read: every weight once and the cache of
-the live requests), decode at batch 1 and 64, and (under "further") the same architecture at the
+the live requests), decode at batch 1, 64, 128 and 256, and (under "further") the same architecture at the
 Qwen2.5-7B sizes: decode at batch 8 and 64 requests batched continuously.  Weights are seeded random, token ids seeded
 uniform random in [100, vocab-100] as in the reference's own benchmark
 (reference: src/zedinfer/profiler.cpp:79-84, docs/perf/benchmark_v0.1.0.md:3-11).
@@ -268,7 +268,7 @@ def main():
     ap.add_argument("--mix", type=int, default=0, metavar="R",
                     help="instead: continuous batching of R requests, prompts uniform in [128, 4096], 256 greedy "
                          "tokens each, prompts cut at 2,048 tokens a step")
-    ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 / 128 / 256 points")
     ap.add_argument("--no-further", action="store_true", help="skip the figures at the 7B and 32B sizes")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
@@ -352,7 +352,7 @@ def main():
                           "frac": round(fl / (pms / 1000.0) / MFMA_PEAK[args.dtype], 4)}
         points = {}
         per_token = 2 * args.layers * cfg.num_key_value_heads * cfg.head_dim * el      # cache bytes of one token
-        for b, st in ((1, min(args.steps, 64)), (64, min(args.steps, 32)), (256, min(args.steps, 16))):
+        for b, st in ((1, min(args.steps, 64)), (64, min(args.steps, 32)), (128, min(args.steps, 24)), (256, min(args.steps, 16))):
             gc.collect()
             torch.cuda.empty_cache()
             tokens = args.prompt_len + args.warmup + args.steps + 2 * b + 64
