@@ -106,6 +106,19 @@ def test_replay_tool(tiny, dtype, tmp_path):
     check(tiny, dtype, steps, out)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16ws"])
+def test_replay_tool_when_few_rows_are_wanted(tiny, dtype, tmp_path):
+    """A mixed trace with a long decoding tail in which every entry wants the logits of its last token at most
+    and some want none, through bin/trace_run: steps that write nothing still print their `done` line, and the
+    files of the others hold the wanted rows only."""
+    steps = traces.few_wanted(traces.mixed(tiny["requests"], seed=7, decode_tail=20), seed=7, none=0.25)
+    assert any(not any(e["want"] for e in st["entries"]) for st in steps)       # a step that wants nothing
+    folder, engine_dtype, _ = variant(tiny, dtype)
+    out = traces.run_tool(folder, engine_dtype, steps, str(tmp_path / "out"), traces.max_live_tokens(steps))
+    assert sorted(out) == [st["step"] for st in steps if any(e["want"] for e in st["entries"])]
+    check(tiny, dtype, steps, out)
+
+
 @pytest.mark.parametrize("how", ["options", "trace"])
 def test_replay_tool_with_the_configuration_s_own_pages(tiny, how, tmp_path):
     """The pool geometry given to the tool, on the command line or as the trace's first line: the page
