@@ -333,9 +333,11 @@ def test_decode_steps_that_want_some_rows_only(tmp_path, dtype, graphs):
         seqs[r] = e.open(r)
         e.step([StepEntry(seqs[r], toks[r][:4 + i], [])])
         fed[r] = 4 + i
-    patterns = ["abcd", "abcd", "ac", "ac", "bd", "abcd", "c", "", "ac", "abd", "abcd", "bd", "bd", "bd", "abcd"]
+    # (a name twice: the request asks for its one row twice, and a step may then want more rows than it has entries)
+    patterns = ["abcd", "abcd", "ac", "ac", "bd", "abcd", "c", "", "ac", "abd", "abcd", "bd", "bd", "bd", "abcd",
+                "aabbcd", "aabbcd", "aaccd", "abcd", "bbbb", "bbbb"]
     for wanting in patterns:
-        got = e.step([StepEntry(seqs[r], toks[r][fed[r]:fed[r] + 1], [0] if r in wanting else []) for r in names])
+        got = e.step([StepEntry(seqs[r], toks[r][fed[r]:fed[r] + 1], [0] * wanting.count(r)) for r in names])
         assert (got is None) == (not wanting) and (got is None or got.shape[0] == len(wanting))
         for row, r in enumerate(wanting):
             d = (got[row].cpu() - ref[r][fed[r]]).abs()

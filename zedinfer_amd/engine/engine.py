@@ -234,7 +234,8 @@ class Engine:
             # one of few numbers, a row wanted of each, so that the kinds of steps are few
             more_entries = decode_entries_at_least(E) - E
             E += more_entries
-            R = E if wanted else 0
+            # (an entry may name its one token several times: more rows than entries are left as they are)
+            R = E if 0 < wanted <= E else wanted
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
         # a bound, the same for many steps, of the tokens any sequence holds after this step: the
@@ -242,7 +243,8 @@ class Engine:
         bound = _bucket_at_least(max(e.seq.length for e in entries) + 1, 256)
         # (whether every token's row is wanted, in order, decides if the model picks rows at all: such steps and
         # steps that want some rows only, or rows of padding entries, are different kinds)
-        key = (E, R, widths, bound, wanted == E)
+        every_row = more_entries == 0 and all(len(e.want) == 1 for e in entries)
+        key = (E, R, widths, bound, every_row)
         dg = self._graphs.pop(key, None)
         if dg is not None:
             self._graphs[key] = dg              # used last: the last to go
