@@ -97,6 +97,28 @@ def test_engine_matches_plain(tiny, dtype, shape):
     check(tiny, dtype, steps, out)
 
 
+@pytest.mark.parametrize("dtype", ["float32s", "bfloat16ws"])
+@pytest.mark.parametrize("seed,max_live", [(1, 4), (2, 4), (3, 9)])
+def test_random_steps_match_plain(tiny, dtype, seed, max_live):
+    """Mixed steps of up to ``max_live`` requests with the wanted places of every entry drawn at random (all, the
+    last, none, a few in any order and perhaps twice) and the entries of a step shuffled: which kind of step the
+    engine makes of each (recorded, padded, part by part) follows from that, and every wanted row is the plain
+    implementation's."""
+    import random
+    rng = random.Random(seed)
+    steps = traces.random_wanted(traces.mixed(tiny["requests"], max_live=max_live, seed=seed,
+                                              decode_tail=rng.choice([3, 12, 40]), max_portion=rng.choice([24, 70, 150])), seed=seed)
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    folder, engine_dtype, _ = variant(tiny, dtype)
+    engine = Engine.from_folder(folder, engine_dtype, SchedulerConfig(num_kv_blocks=traces.max_live_tokens(steps, round_to=ps) // ps + 1,
+                                                                      kv_block_size=ps, max_batch_requests=max_live))
+    engine.graph_after = 2
+    out = traces.run_in_process(engine, steps)
+    check(tiny, dtype, steps, out)
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16", "bfloat16w", "bfloat16ws"])
 def test_replay_tool(tiny, dtype, tmp_path):
     """The same mixed trace through bin/trace_run as a child process."""

@@ -103,6 +103,23 @@ def few_wanted(steps, seed=0, none=0.15):
     return out
 
 
+def random_wanted(steps, seed=0):
+    """The same steps with wanted places drawn at random for every entry (all of them, the last one, none, or a
+    few in any order, a place perhaps twice) and the entries of a step in a random order."""
+    rng = random.Random(seed)
+    out = []
+    for st in steps:
+        entries = []
+        for e in st["entries"]:
+            n, c = len(e["tokens"]), rng.random()
+            want = list(range(n)) if c < 0.25 else [n - 1] if c < 0.6 else [] if c < 0.75 else \
+                [rng.randrange(n) for _ in range(rng.randint(1, 4))]
+            entries.append(dict(e, want=want))
+        rng.shuffle(entries)
+        out.append(dict(st, entries=entries))
+    return out
+
+
 def max_live_tokens(steps, round_to=64):
     """The largest sum over live requests of their token counts rounded up, at any step."""
     held, best = {}, 0
