@@ -492,7 +492,7 @@ def test_sizes_at_which_a_serving_engine_measures_its_choices():
     few = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=520, max_prefill_tokens=512))
     assert few == [640, 576, 512, 448, 384, 320, 256, 192, 128]     # 520 tokens, rounded up, and one more size
     many = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=200, max_batch_tokens=2248, max_prefill_tokens=2048))
-    assert many[0] == 2368 and many[-3:] == [160, 128, 96] and 224 in many and len(many) == len(set(many))
+    assert many[0] == 2368 and many[-4:] == [128, 112, 96, 80] and 224 in many and 160 in many and len(many) == len(set(many))
     for e in range(65, 201):
         assert decode_entries_at_least(e) in many
     long = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=16392, max_prefill_tokens=16384,

@@ -260,8 +260,8 @@ def test_decode_steps_of_fewer_and_fewer_requests_share_a_shape(tmp_path, dtype)
     from zedinfer_amd.config import SchedulerConfig
     from zedinfer_amd.engine import Engine, StepEntry
     from zedinfer_amd.engine.engine import decode_entries_at_least
-    assert [decode_entries_at_least(n) for n in (1, 2, 3, 5, 9, 16, 17, 33, 64, 65, 100, 256)] == \
-        [1, 2, 4, 8, 16, 16, 32, 48, 64, 96, 128, 256]
+    assert [decode_entries_at_least(n) for n in (1, 2, 3, 5, 9, 16, 17, 33, 64, 65, 100, 128, 129, 256)] == \
+        [1, 2, 4, 8, 16, 16, 32, 48, 64, 80, 112, 128, 160, 256]
     store = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     folder = tiny_configs.write_tiny(str(tmp_path / "m"), "C", dtype=store, std=tiny_configs.SHARP_STD)
     cfg, w = plain.load_folder(folder)

@@ -473,10 +473,11 @@ def many_rows_step_sizes(most_tokens: int, step: int = Engine.PROMPT_GRAPH_STEP,
 
 def decode_entries_at_least(entries: int) -> int:
     """The number of entries a step of ``entries`` decoding requests is run with: a power of two up to 16 (one
-    tile of rows of the few-rows kernels), then a multiple of 16 up to 64 and of 32 beyond."""
+    tile of rows of the few-rows kernels), then a multiple of 16 up to 128 (what those kernels take) and of 32
+    beyond."""
     if entries <= 16:
         return _pow2_at_least(entries)
-    step = 16 if entries <= 64 else 32
+    step = 16 if entries <= 128 else 32
     return -(-entries // step) * step
 
 
