@@ -642,6 +642,16 @@ def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatc
     last = both([("b", 1)])[0]
     ref = plain.forward(tiny["cfg"], tiny16["weights"], toks["b"][:fed["b"]])
     assert float((last[0].cpu() - ref[fed["b"] - 1]).abs().max()) < 0.06 * float(ref.abs().max())
+    # a launch of more workgroups (tokens x key/value heads x chunks of the keys) than the limit takes the
+    # separate kernels: with the limit below this step's launch nothing is fused, and the logits agree as before
+    nkv = tiny["cfg"]["num_key_value_heads"]
+    assert 3 * nkv * ops.attention_decode_chunks(256) <= Attention.FUSED_DECODE_MAX_WORKGROUPS == 512
+    monkeypatch.setattr(Attention, "FUSED_DECODE_MAX_WORKGROUPS", 3 * nkv - 1)
+    before = calls["fused"]
+    both([("a", 1), ("b", 1), ("c", 1)])
+    assert calls["fused"] == before
+    both([("b", 1)])
+    assert calls["fused"] == before + layers
 
 
 @pytest.mark.parametrize("requests", [20, 70, 136])

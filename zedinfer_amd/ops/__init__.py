@@ -5,7 +5,8 @@ then launches on torch's current stream.  The op-level names follow the
 reference's Python module (reference: python/bindings/zedinfer_ops.cpp:257-291:
 add, argmax, embedding, linear, rms_norm, rope, swiglu).
 """
-from .functional import (add, add_rms_norm, argmax, attention, attention_decode, attention_decode_fused,
+from .functional import (add, add_rms_norm, argmax, attention, attention_decode, attention_decode_chunks,
+                         attention_decode_fused,
                          attention_decode_fused_supported, attention_decode_project,
                          attention_decode_project_splits, attention_decode_project_supported,
                          attention_decode_supported, attention_decode_workspace, attention_prefill,
@@ -19,7 +20,7 @@ from .functional import (add, add_rms_norm, argmax, attention, attention_decode,
 from ._lib import KernelLibraryError, library_path, load
 
 __all__ = [
-    "add", "add_rms_norm", "argmax", "attention", "attention_decode", "attention_decode_fused",
+    "add", "add_rms_norm", "argmax", "attention", "attention_decode", "attention_decode_chunks", "attention_decode_fused",
     "attention_decode_fused_supported", "attention_decode_project", "attention_decode_project_splits",
     "attention_decode_project_supported", "attention_decode_supported", "attention_decode_workspace",
     "attention_prefill", "attention_prefill_supported", "attention_prefill_tile", "attention_prefill_variant",

@@ -387,6 +387,12 @@ def attention_decode_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, pa
     return bool(_lib.load().zi_attention_decode_supported(_CODES[dtype], nh, nkv, d, page_size))
 
 
+def attention_decode_chunks(max_keys: int) -> int:
+    """Chunks of the keys that the decode attention launches for every token and key/value head when no token
+    sees more than ``max_keys`` keys."""
+    return int(_lib.load().zi_attention_decode_chunks(int(max_keys)))
+
+
 def attention_decode_workspace(tokens: int, nh: int, d: int) -> int:
     """Floats of workspace for the chunk partials of ``tokens`` tokens."""
     return tokens * nh * DECODE_MAX_CHUNKS * (d + 2)

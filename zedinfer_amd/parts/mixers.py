@@ -127,6 +127,13 @@ class Attention(Mixer):
     # 256 keys), which costs more than the separate rotary kernel once many tokens decode together:
     # measured faster at 1 and 8 tokens, slower at 64.
     FUSED_DECODE_MAX_TOKENS = 16
+    # ... and once the launch (tokens x key/value heads x chunks of the keys) is more workgroups than the chip
+    # holds at a time (two a compute unit): the workgroups of a second round pay the three dependent trips to
+    # memory that come before their keys once more.  Measured at the 1.5B sizes, fused against separate kernels:
+    # 8 tokens at 2,048 keys (176 workgroups) 1.47 against 1.54 ms a step, 12 at 4,096 (456) 1.72 against 1.76;
+    # 8 at 8,192 (656) 1.98 against 1.87, 16 at 8,192 (1,312) 2.43 against 2.21; the 7B and 32B sizes turn over
+    # between 352 and 704 workgroups as well.
+    FUSED_DECODE_MAX_WORKGROUPS = 512
     # The one-kernel decode path leaves its chunks unmerged and the output projection merges them as it
     # loads its operand: one launch less a layer.  That kernel does not stream a large weight as well as
     # the plain product does (measured: 6.9 against 4.4 + 3.7 us with 4.7 MB of weight, 31.7 against
@@ -296,6 +303,8 @@ class Attention(Mixer):
         ps = memory.k.shape[2]
         max_keys = batch.plans[self.plan_key].sizes["max_short_keys"]
         if not ops.attention_decode_fused_supported(memory.k.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
+            return None
+        if n * self.nkv * ops.attention_decode_chunks(max_keys) > self.FUSED_DECODE_MAX_WORKGROUPS:
             return None
         ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
         # every entry brings one token: token t is of entry t
