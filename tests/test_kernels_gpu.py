@@ -768,6 +768,34 @@ def test_attention_prefill_bound_too_low_shows(ops):
     assert ops.attention_prefill_workspace(T, nh, d, 2048) == 0 and ops.attention_prefill_workspace(T, nh, d, 2049) > 0
 
 
+@pytest.mark.parametrize("nh,nkv,d,T,tile,cuts", [(14, 2, 64, 7000, 128, 1), (6, 1, 64, 16500, 128, 2), (12, 2, 128, 8200, 64, 1)])
+def test_attention_prefill_with_the_cut_of_long_prompts(ops, nh, nkv, d, T, tile, cuts):
+    """A launch of 768 tiles x heads or more whose queries see more than 6,144 keys cuts its tiles every 16,384 keys,
+    not every 2,048: one workgroup walks up to 16,384 keys (its block table entries staged in turns), no workspace
+    is needed up to there and two cuts are merged beyond.  Rows at the cuts' edges and elsewhere against a float32
+    reference; a launch of fewer tiles over the same keys keeps the short cut."""
+    dtype, ps = torch.bfloat16, 16
+    k, v = rnd(T, nkv, d, dtype=dtype, seed=1), rnd(T, nkv, d, dtype=dtype, seed=2)
+    kc, vc, table = make_paged(k, v, ps, T // ps + 2)
+    q = rnd(T, nh, d, dtype=dtype, seed=3)
+    te, to = prefill_tiles([(0, T, 0)], tile)
+    assert te.numel() * nh >= 768
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    scale = 1 / math.sqrt(d)
+    need = ops.attention_prefill_workspace(T, nh, d, T, 0, te.numel())
+    assert (need == 0) == (cuts == 1) and ops.attention_prefill_workspace(T, nh, d, T, 0, 10) > need
+    out = ops.attention_prefill(q.view(T, nh * d), kc, vc, te, to, dev([0]), dev([T]), dev([0]), table[None].contiguous(),
+                                nh, nkv, d, scale, max_keys=T, tile=tile)
+    rows = sorted({0, 1, 63, 64, 2047, 2048, 2049, 6143, 6144, 6145, T // 2, T - 129, T - 1, 16383, 16384, 16385} & set(range(T)))
+    G = nh // nkv
+    for r in rows:
+        kk, vv = k[:r + 1].float(), v[:r + 1].float()                      # [keys, nkv, d]
+        for h in range(nh):
+            p = torch.softmax((kk[:, h // G] @ q[r, h].float()) * scale, 0)
+            ref = p @ vv[:, h // G]
+            torch.testing.assert_close(out.view(T, nh, d)[r, h].float(), ref, atol=2e-2, rtol=2e-2)
+
+
 def test_attention_prefill_far_key_stands_out(ops):
     """One far key among a thousand is made to dominate one query of a late tile."""
     nh, nkv, d, ps, T = 4, 1, 64, 16, 1100

@@ -269,3 +269,36 @@ def test_prefill_walk_of_a_long_prompt_and_what_is_broken(model, tile):
     assert rc != 0 and "page entry" in err
     rc, err, stats = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, 2, tile=tile)    # sized for fewer cuts
     assert rc == 0 and stats[2] == plan.sizes["num_tiles"]
+
+
+@pytest.mark.parametrize("tile", [64, 128, -128])
+def test_prefill_walk_with_the_cut_of_long_prompts(model, tile):
+    """Launches of 768 tiles x heads and more whose queries see more than 6,144 keys cut their tiles every 16,384
+    keys instead of every 2,048 (they fill the chip without cuts, and every cut costs a merge): a portion behind 17,000 tokens walks its
+    keys in two cuts, every (query, key) pair once, its block table entries within what the kernel stages; a
+    portion behind 7,000 in one, with no workspace."""
+    m = CacheManager({0: KVCacheRequest("full", 2, 32)}, {}, 2300, 8, 2, torch.bfloat16, None, max_step_tokens=2048)
+    assert model.pm_prefill_chunk_for(6144, 5000) == 2048 and model.pm_prefill_chunk_for(6145, 768) == 16384
+    assert model.pm_prefill_chunk_for(30000, 767) == 2048
+    for past, cuts in ((17000, 2), (7000, 1)):
+        s = m.open(f"long{past}")
+        m.ensure(s, past)
+        m.commit(s, past)
+        m.ensure(s, past + 300)
+        hb = HostBatch(300, 1, np.array([0], dtype=np.int32), np.array([300], dtype=np.int32),
+                       np.array([past], dtype=np.int32), False)
+        planner = AttentionPlanner(abs(tile), heads=4)
+        planner.FILL = 1
+        planner.FILL_ALONE = 1 if tile < 0 else 10 ** 9
+        plan = planner.plan(hb)
+        tables = padded_tables([s], 0, pow2(len(s.pages[0]), 8))
+        keys = plan.sizes["max_long_keys"]
+        before = model.pm_set_prefill_chunk(model.pm_prefill_chunk_for(keys, 1000))       # as in a launch of many tiles
+        try:
+            assert before == 2048 and model.pm_prefill_chunks(keys) == cuts
+            rc, err, stats = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, 0, cuts, tile=tile)
+        finally:
+            model.pm_set_prefill_chunk(before)
+        assert rc == 0, err
+        assert stats[0] == sum(past + i + 1 for i in range(300)) and stats[1] == (300 * 4 * cuts if cuts > 1 else 0)
+        m.close(s)

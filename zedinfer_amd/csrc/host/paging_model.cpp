@@ -159,6 +159,16 @@ extern "C" int pm_check_decode(int n_idx, const int* tok_index, const int* tok_s
 // stats[0] = (query, key) pairs covered, stats[1] = workspace slots written, stats[2] = tiles given NaN.
 // `entry_real` (or null): the tokens of each entry that are its own; the rest are padding, whose queries'
 // results nobody reads and whose keys are nowhere: they are checked for bounds only.
+// The keys between the cuts of a tile, as the caller of the kernels chooses them for its launch
+// (zi_pf_chunk_for): ZI_PF_CHUNK unless set otherwise.  Returns what it was.
+static int pm_pf_chunk = ZI_PF_CHUNK;
+extern "C" int pm_set_prefill_chunk(int chunk) {
+    const int before = pm_pf_chunk;
+    if (chunk == ZI_PF_CHUNK || chunk == ZI_PF_CHUNK_LONG) pm_pf_chunk = chunk;
+    return before;
+}
+extern "C" int pm_prefill_chunk_for(int max_keys, int groups) { return zi_pf_chunk_for(max_keys, groups); }
+
 extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int* tile_off, const int* entry_start,
                                 const int* entry_len, const int* entry_past, const int* entry_real, int num_entries,
                                 const int* block_tables,
@@ -185,7 +195,7 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
         PM_CHECK(start + off + count <= rows, "prefill: tile %d covers rows up to %d of %d", tile, start + off + count, rows);
         const int* bt = block_tables + (int64_t)e * max_pages;
         const int pos0 = past + off;
-        const PfCut whole = zi_pf_cut(pos0, count, window, 0);
+        const PfCut whole = zi_pf_cut(pos0, count, window, 0, pm_pf_chunk);
         if (whole.nc > max_chunks) {
             ++stats[2];
             continue;
@@ -193,13 +203,13 @@ extern "C" int pm_check_prefill(int num_tiles, const int* tile_entry, const int*
         // pairs[q][key - lo_tile]: times the (query, key) pair was covered
         std::vector<std::vector<int>> pairs(count, std::vector<int>(whole.kmax - whole.lo_tile + 1, 0));
         for (int cut_i = 0; cut_i < whole.nc; ++cut_i) {
-            const PfCut cut = zi_pf_cut(pos0, count, window, cut_i);
+            const PfCut cut = zi_pf_cut(pos0, count, window, cut_i, pm_pf_chunk);
             PM_CHECK(cut.live, "prefill: tile %d has %d cuts but cut %d does not exist", tile, whole.nc, cut_i);
-            PM_CHECK(cut.kb_begin % ZI_PF_BS == 0 && cut.kb_begin <= cut.khi && cut.khi - cut.kb_begin < ZI_PF_CHUNK,
+            PM_CHECK(cut.kb_begin % ZI_PF_BS == 0 && cut.kb_begin <= cut.khi && cut.khi - cut.kb_begin < pm_pf_chunk,
                      "prefill: cut %d of tile %d walks [%d, %d]", cut_i, tile, cut.kb_begin, cut.khi);
             // the block table entries the workgroup copies to LDS
             const int pi_first = cut.kb_begin >> ps_shift, n_entries = (cut.khi >> ps_shift) - pi_first + 1;
-            PM_CHECK(n_entries <= ZI_PF_CHUNK / 8 + 8 && n_entries <= 8 * 64, "prefill: %d block table entries for one cut",
+            PM_CHECK(n_entries <= ZI_PF_CHUNK_LONG / 8 + 8, "prefill: %d block table entries for one cut",
                      n_entries);
             for (int kb = cut.kb_begin; kb <= cut.khi; kb += BS) {
                 for (int k = 0; k < BS; ++k) {
@@ -305,4 +315,4 @@ extern "C" int pm_decode_chunks(int keys) {
     if (keys + 7 > ZI_DEC_CHUNK * ZI_DEC_MAXC) return ZI_DEC_MAXC;
     return dec_split(keys - 1 + 7, 0).count;
 }
-extern "C" int pm_prefill_chunks(int keys) { return ((keys < 1 ? 1 : keys) + ZI_PF_CHUNK - 1) / ZI_PF_CHUNK; }
+extern "C" int pm_prefill_chunks(int keys) { return ((keys < 1 ? 1 : keys) + pm_pf_chunk - 1) / pm_pf_chunk; }

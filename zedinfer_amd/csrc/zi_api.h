@@ -34,7 +34,7 @@ int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_
     kcache, const void* vcache, const int32_t* tile_entry, const int32_t* tile_off, const int32_t* entry_start, const
     int32_t* entry_len, const int32_t* entry_past, const int32_t* block_tables, int max_pages, int num_pages, int nh,
     int nkv, int d, int page_size, int window, float scale, int rows, int max_chunks, float* workspace, int64_t
-    workspace_floats, int tile, int alone, hipStream_t stream);
+    workspace_floats, int tile, int alone, int chunk_keys, hipStream_t stream);
 // elementwise.hip
 int zi_embedding(void* out, int out_dt, const void* table, int table_dt, const int32_t* ids, int n, int hidden, int
     vocab, hipStream_t stream);

@@ -110,28 +110,36 @@ ZI_HD int64_t zi_dec_part_slot(int token_index, int nh, int head, int chunk) {
 // ---- prompt attention: the cut of one tile's keys ---------------------------------------------------
 #define ZI_PF_BM 64          // queries of a tile
 #define ZI_PF_BS 128         // keys of a block
-#define ZI_PF_CHUNK 2048     // keys one workgroup walks at most
+#define ZI_PF_CHUNK 2048     // keys one workgroup walks at most: the cut of launches over few keys
+#define ZI_PF_CHUNK_LONG 16384      // the cut of launches whose queries see more than ZI_PF_LONG_FROM keys and that have
+#define ZI_PF_LONG_FROM 6144        // ZI_PF_LONG_GROUPS workgroups (tiles x heads) without any cut: those fill the chip as
+#define ZI_PF_LONG_GROUPS 768       // they are, and every cut costs a merge
 #define ZI_PF_MAXC 64        // most cuts of one tile
 
+// The cut of a launch of `groups` tiles x heads none of whose queries sees more than max_keys keys.
+ZI_HD int zi_pf_chunk_for(int max_keys, int groups) {
+    return (max_keys > ZI_PF_LONG_FROM && groups >= ZI_PF_LONG_GROUPS) ? ZI_PF_CHUNK_LONG : ZI_PF_CHUNK;
+}
+
 // A tile of `count` queries whose first sits at position pos0 sees keys [lo_tile, kmax].  Its walk starts at
-// kb_first (a multiple of the block) and is cut at absolute multiples of ZI_PF_CHUNK into nc cuts, the first
+// kb_first (a multiple of the block) and is cut at absolute multiples of `chunk` into nc cuts, the first
 // being cut c0 of the sequence; cut number `cut` (0-based within the tile) walks [kb_begin, khi].
 struct PfCut {
     int kmax, lo_tile, kb_first, c0, nc;
     int live;              // this cut exists
     int kb_begin, khi;
 };
-ZI_HD PfCut zi_pf_cut(int pos0, int count, int window, int cut) {
+ZI_HD PfCut zi_pf_cut(int pos0, int count, int window, int cut, int chunk = ZI_PF_CHUNK) {
     PfCut t;
     t.kmax = pos0 + count - 1;
     t.lo_tile = (window > 0 && pos0 - window + 1 > 0) ? pos0 - window + 1 : 0;
     t.kb_first = (t.lo_tile / ZI_PF_BS) * ZI_PF_BS;
-    t.c0 = t.kb_first / ZI_PF_CHUNK;
-    t.nc = t.kmax / ZI_PF_CHUNK - t.c0 + 1;
+    t.c0 = t.kb_first / chunk;
+    t.nc = t.kmax / chunk - t.c0 + 1;
     const int c = t.c0 + cut;
-    t.live = c * ZI_PF_CHUNK <= t.kmax;
-    t.kb_begin = (c * ZI_PF_CHUNK > t.kb_first) ? c * ZI_PF_CHUNK : t.kb_first;
-    t.khi = ((c + 1) * ZI_PF_CHUNK - 1 < t.kmax) ? (c + 1) * ZI_PF_CHUNK - 1 : t.kmax;
+    t.live = c * chunk <= t.kmax;
+    t.kb_begin = (c * chunk > t.kb_first) ? c * chunk : t.kb_first;
+    t.khi = ((c + 1) * chunk - 1 < t.kmax) ? (c + 1) * chunk - 1 : t.kmax;
     return t;
 }
 ZI_HD int64_t zi_pf_workspace_floats(int rows, int nh, int d, int max_chunks) {

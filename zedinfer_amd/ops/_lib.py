@@ -38,7 +38,8 @@ _PROTOTYPES = {
     "zi_attention_decode_project_heads": [I],
     "zi_rope_table": [P, P, P, I, I, P],
     "zi_attention_decode_chunks": [I],
-    "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, I, P],
+    "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, I, I, P],
+    "zi_attention_prefill_chunk_keys_for": [I, I],
     "zi_attention_prefill_chunks": [I],
     "zi_attention_prefill_variant": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],

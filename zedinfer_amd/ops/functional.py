@@ -589,17 +589,24 @@ def attention_prefill_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, p
     return bool(_lib.load().zi_attention_prefill_supported(_CODES[dtype], nh, nkv, d, page_size))
 
 
-def attention_prefill_workspace(rows: int, nh: int, d: int, max_keys: int, window: int = 0) -> int:
-    """float32 entries of workspace ``attention_prefill`` needs for ``rows`` query rows of which none sees
-    more than ``max_keys`` keys (0: none)."""
+def attention_prefill_workspace(rows: int, nh: int, d: int, max_keys: int, window: int = 0, num_tiles: int = 0) -> int:
+    """float32 entries of workspace ``attention_prefill`` needs for ``rows`` query rows in ``num_tiles`` tiles of
+    which none sees more than ``max_keys`` keys (0: none)."""
     lib = _lib.load()
-    return int(lib.zi_attention_prefill_workspace(int(rows), nh, d, _prefill_chunks(max_keys, window)))
+    return int(lib.zi_attention_prefill_workspace(int(rows), nh, d, _prefill_cut(max_keys, window, int(num_tiles) * nh)[1]))
 
 
-def _prefill_chunks(max_keys: int, window: int) -> int:
+def _prefill_cut(max_keys: int, window: int, groups: int) -> Tuple[int, int]:
+    """(keys between cuts, most cuts of a tile) of a prompt attention launch of ``groups`` tiles x heads none of
+    whose queries sees more than ``max_keys`` keys: the cut is the library's choice (longer when there are tiles
+    enough to fill the chip without cuts: every cut costs a merge)."""
+    max_keys = max(int(max_keys), 1)
     if window > 0:      # a windowed tile's keys span at most the window, a tile and a block, from anywhere in a cut
-        max_keys = min(max_keys, window + PREFILL_TILE_MAX + 128) + int(_lib.load().zi_attention_prefill_chunk_keys()) - 1
-    return int(_lib.load().zi_attention_prefill_chunks(int(max_keys)))
+        max_keys = min(max_keys, window + PREFILL_TILE_MAX + 128)
+    chunk = int(_lib.load().zi_attention_prefill_chunk_keys_for(max_keys, int(groups)))
+    if window > 0:
+        max_keys += chunk - 1
+    return chunk, -(-max_keys // chunk)
 
 
 def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tile_entry: torch.Tensor,
@@ -648,7 +655,7 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
         raise ValueError("attention_prefill: out has the wrong shape or dtype")
     if max_keys <= 0:
         max_keys = block_tables.shape[1] * ps      # no bound given: what the block tables could hold
-    max_chunks = _prefill_chunks(int(max_keys), int(window))
+    chunk_keys, max_chunks = _prefill_cut(int(max_keys), int(window), num_tiles * nh)
     need = int(_lib.load().zi_attention_prefill_workspace(n, nh, d, max_chunks))
     if need:
         if workspace is None:
@@ -659,7 +666,7 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
               _p(vcache), _p(tile_entry), _p(tile_off), _p(entry_start), _p(entry_len), _p(entry_past),
               _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), n,
               max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, int(tile), int(bool(alone)),
-              _stream())
+              chunk_keys, _stream())
     return out
 
 

@@ -212,7 +212,8 @@ class Attention(Mixer):
         elif n_long > 0:
             if ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
                 max_keys = plan.sizes["max_long_keys"]
-                need = ops.attention_prefill_workspace(q.shape[0], self.nh, self.d, max_keys, self.window)
+                need = ops.attention_prefill_workspace(q.shape[0], self.nh, self.d, max_keys, self.window,
+                                                       plan.sizes["num_tiles"])
                 ws = self.rt.buffer("attn_prompt_split", (need,), torch.float32) if need else None
                 ops.attention_prefill(q, memory.k, memory.v, plan.dev["tile_entry"], plan.dev["tile_off"],
                                       batch.entry_start, batch.entry_len, batch.entry_past, view.block_tables, self.nh,
