@@ -247,8 +247,8 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
 // launches of the kernel above would make two, and where the library's products of so few rows stay far from the
 // weights' stream.  The registers that the kernel above spends on rings of x and on all of a block's x operands
 // do not stretch to eight tiles, so here a block's x is requested one step ahead only (it comes from the cache;
-// the weights keep their ring of three), it lies in LDS once (two barriers a block instead of one: 32 KB for
-// 128 rows, and with the wavefronts' weight tiles that is the 64 KB a workgroup may declare), and the x operands
+// the weights keep their ring of three), it lies in LDS once (two barriers a block instead of one; a second
+// buffer for it, 96 KB of LDS in all, was measured and changed nothing), and the x operands
 // are read a k-step at a time, just before their matrix instructions.  The cut, the order of the sums and the
 // epilogues are the kernel's above: a row's result does not depend on which of the two kernels makes it.
 template <int MT, int GM_WAVES>
