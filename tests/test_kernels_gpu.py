@@ -768,8 +768,9 @@ def test_attention_prefill_bound_too_low_shows(ops):
     assert ops.attention_prefill_workspace(T, nh, d, 2048) == 0 and ops.attention_prefill_workspace(T, nh, d, 2049) > 0
 
 
-@pytest.mark.parametrize("nh,nkv,d,T,tile,cuts", [(14, 2, 64, 7000, 128, 1), (6, 1, 64, 16500, 128, 2), (12, 2, 128, 8200, 64, 1)])
-def test_attention_prefill_with_the_cut_of_long_prompts(ops, nh, nkv, d, T, tile, cuts):
+@pytest.mark.parametrize("nh,nkv,d,T,tile,cuts,window", [(14, 2, 64, 7000, 128, 1, 0), (6, 1, 64, 16500, 128, 2, 0),
+                                                         (12, 2, 128, 8200, 64, 1, 0), (6, 2, 64, 17000, 128, 2, 7000)])
+def test_attention_prefill_with_the_cut_of_long_prompts(ops, nh, nkv, d, T, tile, cuts, window):
     """A launch of 768 tiles x heads or more whose queries see more than 6,144 keys cuts its tiles every 16,384 keys,
     not every 2,048: one workgroup walks up to 16,384 keys (its block table entries staged in turns), no workspace
     is needed up to there and two cuts are merged beyond.  Rows at the cuts' edges and elsewhere against a float32
@@ -782,14 +783,15 @@ def test_attention_prefill_with_the_cut_of_long_prompts(ops, nh, nkv, d, T, tile
     assert te.numel() * nh >= 768
     dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
     scale = 1 / math.sqrt(d)
-    need = ops.attention_prefill_workspace(T, nh, d, T, 0, te.numel())
-    assert (need == 0) == (cuts == 1) and ops.attention_prefill_workspace(T, nh, d, T, 0, 10) > need
+    need = ops.attention_prefill_workspace(T, nh, d, T, window, te.numel())
+    assert (need == 0) == (cuts == 1) and ops.attention_prefill_workspace(T, nh, d, T, window, 10) > need
     out = ops.attention_prefill(q.view(T, nh * d), kc, vc, te, to, dev([0]), dev([T]), dev([0]), table[None].contiguous(),
-                                nh, nkv, d, scale, max_keys=T, tile=tile)
+                                nh, nkv, d, scale, window, max_keys=T, tile=tile)
     rows = sorted({0, 1, 63, 64, 2047, 2048, 2049, 6143, 6144, 6145, T // 2, T - 129, T - 1, 16383, 16384, 16385} & set(range(T)))
     G = nh // nkv
     for r in rows:
-        kk, vv = k[:r + 1].float(), v[:r + 1].float()                      # [keys, nkv, d]
+        lo = max(0, r - window + 1) if window else 0                       # a window of w keys: positions r-w+1 .. r
+        kk, vv = k[lo:r + 1].float(), v[lo:r + 1].float()                  # [keys, nkv, d]
         for h in range(nh):
             p = torch.softmax((kk[:, h // G] @ q[r, h].float()) * scale, 0)
             ref = p @ vv[:, h // G]
