@@ -301,4 +301,14 @@ def test_prefill_walk_with_the_cut_of_long_prompts(model, tile):
             model.pm_set_prefill_chunk(before)
         assert rc == 0, err
         assert stats[0] == sum(past + i + 1 for i in range(300)) and stats[1] == (300 * 4 * cuts if cuts > 1 else 0)
+        if past == 17000:
+            # the same portion with a window of 7,000 keys: every tile's keys lie across the cut at 16,384
+            window = 7000
+            before = model.pm_set_prefill_chunk(16384)
+            try:
+                rc, err, stats = prefill(model, plan, hb, None, tables, m.num_pages, 4, 2, 32, 8, window, 2, tile=tile)
+            finally:
+                model.pm_set_prefill_chunk(before)
+            assert rc == 0, err
+            assert stats[0] == 300 * window and stats[1] == 300 * 4 * 2
         m.close(s)
