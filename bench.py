@@ -114,6 +114,37 @@ def measure_decode(engine_factory, batch, steps, warmup, vocab, prompt_len=PROMP
     return batch * steps / dt, dt / steps * 1000.0, (ctx0 + ctx1) / 2.0
 
 
+def decode_point(engine_factory, shape, layers, batch, steps, warmup, prompt_len, el, warm_up_sizes=None):
+    """A decode measurement as a record: tokens a second, ms a step, and the step against the HBM roofline."""
+    tps, ms_step, ctx_mid = measure_decode(engine_factory, batch, steps, warmup, shape["vocab_size"], prompt_len,
+                                           warm_up_sizes=warm_up_sizes)
+    achieved = decode_bytes(shape, layers, batch, ctx_mid, el) / (ms_step / 1000.0) / 1e9
+    return {"value": round(tps, 2), "unit": "tok/s", "ms_per_step": round(ms_step, 4), "batch": batch, "seq_len": prompt_len,
+            "steps": steps, "roofline_achieved_gbs": round(achieved, 1), "roofline_frac": round(achieved / HBM_PEAK_GBS, 4)}
+
+
+def long_context_points(base_engine, shape, layers, el, args, contexts=(16384, 32768), batch=8):
+    """Decode at batch 8 with prompts of 16,384 and 32,768 tokens (the cache of the live requests is then most of
+    what a step reads), on another cache pool of an engine that holds the weights already."""
+    import torch
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine.engine import many_rows_size_at_least
+    out = {}
+    steps, warm = min(args.steps, 32), min(args.warmup, 8)
+    for ctx in contexts:
+        gc.collect()
+        torch.cuda.empty_cache()
+        tokens = ctx + warm + steps + 2 * batch + 64
+
+        def make():
+            return base_engine().with_cache(SchedulerConfig(
+                num_kv_blocks=batch * (-(-tokens // 16)) + 16, kv_block_size=16, max_batch_requests=batch,
+                max_batch_tokens=ctx + batch, max_prefill_tokens=ctx, max_seq_len=2 * ctx))
+        out[f"decode_b{batch}_ctx{ctx}"] = decode_point(make, shape, layers, batch, steps, warm, ctx, el,
+                                                         warm_up_sizes=[many_rows_size_at_least(ctx + 64), ctx])
+    return out
+
+
 def measure_mix(engine_factory, requests, vocab, new_tokens=256, lo=128, hi=4096):
     """Continuous batching: `requests` prompts of lengths uniform in [lo, hi], all queued at once,
     `new_tokens` greedy tokens each; generated tokens a second over the whole run, prompt tokens a
@@ -196,6 +227,7 @@ def further_7b(args):
         sched = SchedulerConfig(num_kv_blocks=64 * (-(-(4096 + 256 + 64) // 16)) + 16, kv_block_size=16,
                                 max_batch_requests=64, max_batch_tokens=2048 + 64, max_prefill_tokens=2048, max_seq_len=8192)
         return holder["e"].with_cache(sched)
+    res["long_context"] = long_context_points(lambda: holder["e"], shape, L, el, args)
     gen, pre, secs, ptoks = measure_mix(mix_engine, 64, cfg.vocab_size)
     res["mix64"] = {"value": round(gen, 1), "unit": "generated tok/s", "requests": 64, "prompt_tokens": ptoks,
                     "prompt_lens": "uniform 128..4096", "new_tokens_each": 256, "prefill_chunk": 2048,
@@ -204,9 +236,9 @@ def further_7b(args):
 
 
 def further_32b(args):
-    """Decode at batch 8 and 1 with 8,192-token prompts and the prefill of one 16,384-token prompt in one step, at
+    """Decode at batch 8, 1 and 64 with 8,192-token prompts and the prefill of one 16,384-token prompt in one step, at
     the Qwen2.5-32B sizes (64 layers, 65 GB of weights; batch 64 holds 139 GB of keys and values and takes half a
-    minute to prefill: `--shape 32B --batch 64 --prompt-len 8192` measures it)."""
+    minute to prefill; reference method: examples/batch_bench.cpp:101-180)."""
     import torch
     from zedinfer_amd.config import Qwen2Config, SchedulerConfig
     from zedinfer_amd.engine import Engine
@@ -241,6 +273,18 @@ def further_32b(args):
         max_batch_tokens=prompt + 1, max_prefill_tokens=prompt, max_seq_len=2 * prompt)), 1, steps, warm, cfg.vocab_size,
         prompt, warm_up_sizes=[prompt])
     res["decode_b1"] = {"value": round(one, 2), "unit": "tok/s", "seq_len": prompt}
+    gc.collect()
+    torch.cuda.empty_cache()
+    many, st64 = 64, min(args.steps, 16)
+    tokens64 = prompt + warm + st64 + 2 * many + 64
+    if many * tokens64 * 2 * L * cfg.num_key_value_heads * cfg.head_dim * el <= 0.9 * torch.cuda.mem_get_info()[0]:
+        res["decode_b64"] = decode_point(lambda: holder["e"].with_cache(SchedulerConfig(
+            num_kv_blocks=many * (-(-tokens64 // 16)) + 16, kv_block_size=16, max_batch_requests=many,
+            max_batch_tokens=prompt + many, max_prefill_tokens=prompt, max_seq_len=2 * prompt)), shape, L, many, st64, warm,
+            prompt, el, warm_up_sizes=[many_rows_size_at_least(prompt + 64), prompt, many])
+    else:
+        res["decode_b64"] = None        # the requests' keys and values do not fit beside the weights
+    gc.collect()
     torch.cuda.empty_cache()
 
     def prefill_engine():
@@ -367,6 +411,8 @@ def main():
         short = measure_prefill(factory(1, 128), V, tokens=128, warm=2)
         points["prefill_128"] = round(128 / short * 1000.0, 1)
         out["points"] = points
+        if not args.no_further:
+            out["long_context"] = long_context_points(lambda: weights_cache["w"], shape, args.layers, el, args)
         if args.shape == "1.5B" and args.layers == FULL_LAYERS and not args.no_further:
             # the same architecture at the Qwen2.5-7B sizes: decode at batch 8 and the continuous-batching mix
             weights_cache.clear()

@@ -40,6 +40,21 @@ def test_missing_and_bad_keys():
         Qwen2Config.from_dict(dict(tiny_configs.TINY_A, rms_norm_eps=0.0))
 
 
+def test_another_activation_is_refused_and_rope_scaling_is_said(capsys):
+    # the reference reads hidden_act and computes SiLU whatever it says (base.cpp:686,
+    # transformer_forward.cpp:128-137); rope_scaling is not among the keys it parses (base.cpp:683-720)
+    with pytest.raises(ConfigError, match="hidden_act 'gelu'"):
+        Qwen2Config.from_dict(dict(tiny_configs.TINY_A, hidden_act="gelu"))
+    assert Qwen2Config.from_dict(dict(tiny_configs.TINY_A, hidden_act="silu")).hidden_act == "silu"
+    capsys.readouterr()
+    Qwen2Config.from_dict(dict(tiny_configs.TINY_A))
+    assert "rope_scaling" not in capsys.readouterr().err
+    cfg = Qwen2Config.from_dict(dict(tiny_configs.TINY_A, rope_scaling={"type": "yarn", "factor": 4.0}))
+    said = capsys.readouterr().err
+    assert "rope_scaling" in said and "ignored" in said
+    assert cfg.rope_theta == Qwen2Config.from_dict(dict(tiny_configs.TINY_A)).rope_theta
+
+
 def test_registry(tmp_path):
     assert "Qwen2ForCausalLM" in registered_architectures()
     assert find_architecture({"architectures": ["Qwen2ForCausalLM"]}).name == "Qwen2ForCausalLM"

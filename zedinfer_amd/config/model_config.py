@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import json
 import os
+import sys
 from dataclasses import dataclass, asdict
 from typing import Any, Dict, Mapping, Tuple
 
@@ -71,6 +72,18 @@ class ModelConfig:
         eos_ids = tuple(int(e) for e in eos) if isinstance(eos, (list, tuple)) else (int(eos),)
         nh = _as_int(d, "num_attention_heads")
         hidden = _as_int(d, "hidden_size")
+        # The reference reads hidden_act (base.cpp:686) and computes SiLU whatever it says
+        # (transformer_forward.cpp:128-137); a checkpoint trained with another activation would run and be
+        # silently something else, so it is refused here.
+        act = str(d.get("hidden_act") or "silu")
+        if act != "silu":
+            raise ConfigError(f"config.json: hidden_act '{act}' is not supported: the feed-forward computes 'silu'")
+        # rope_scaling is not among the keys the reference parses (base.cpp:683-720): positions rotate by
+        # rope_theta alone.  Said once, so that a long-context variant is not taken for what its config says.
+        if d.get("rope_scaling") is not None:
+            print("zedinfer_amd: config.json has 'rope_scaling'; it is ignored, as the reference ignores it "
+                  "(src/frontend/models/base.cpp:683-720 does not parse it): angles come from rope_theta alone",
+                  file=sys.stderr, flush=True)
         head_dim = int(d.get("head_dim") or 0)
         if head_dim == 0:
             if nh <= 0 or hidden % nh:
@@ -81,7 +94,7 @@ class ModelConfig:
         return dict(
             architectures=tuple(d.get("architectures") or ()),
             model_type=str(d.get("model_type") or "unknown"),
-            hidden_act=str(d.get("hidden_act") or "silu"),
+            hidden_act=act,
             torch_dtype=str(d.get("torch_dtype") or "bfloat16"),
             bos_token_id=int(d.get("bos_token_id", 151643)),
             eos_token_ids=eos_ids,
