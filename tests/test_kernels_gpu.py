@@ -822,6 +822,78 @@ def test_attention_prefill_far_key_stands_out(ops):
         assert (diff < 2e-2) == seen, (window, diff)
 
 
+def plant_far_key(q, k, who, head, far, d, seed):
+    """Make key ``far`` dominate query (who, head): the query is drawn anew at full width, the key points along it
+    with a score of 60 after the scale."""
+    q[who, head] = rnd(d, seed=seed)
+    k[far, 0] = q[who, head] * 60.0 / q[who, head].norm() ** 2 * math.sqrt(d)
+
+
+@pytest.mark.parametrize("alone", [False, True])
+def test_attention_prefill_long_cut_far_keys_stand_out(ops, alone):
+    """The cut every 16,384 keys with single keys that dominate: a key of the first cut seen from the second (the
+    two cuts are merged), keys just below and just above the cut's edge, and with a window across the edge one key
+    inside it and one outside.  With keys and queries of unit width the softmax over thousands of keys is so flat
+    that a lost block of 128 keys moves the output by less than the tolerance; a dominating key that is lost, or
+    seen where it must not be, moves it by its whole size."""
+    nh, nkv, d, ps, T, tile = 6, 1, 64, 16, 17000, 128
+    dtype = torch.bfloat16
+    k, v = rnd(T, nkv, d, seed=1) * 0.1, rnd(T, nkv, d, seed=2)
+    q = rnd(T, nh, d, seed=3) * 0.1
+    # (query row, head, far key)
+    plants = [(16900, 0, 37), (16700, 1, 16383), (16800, 2, 16384), (16390, 3, 16389), (16500, 4, 2047), (9000, 5, 8191)]
+    for i, (who, h, far) in enumerate(plants):
+        plant_far_key(q, k, who, h, far, d, seed=20 + i)
+    k, v, q = k.to(dtype), v.to(dtype), q.to(dtype)
+    kc, vc, table = make_paged(k, v, ps, T // ps + 2)
+    te, to = prefill_tiles([(0, T, 0)], tile)
+    assert te.numel() * nh >= 768 and ops.attention_prefill_workspace(T, nh, d, T, 0, te.numel()) > 0     # two long cuts
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    scale = 1 / math.sqrt(d)
+    out = ops.attention_prefill(q.view(T, nh * d), kc, vc, te, to, dev([0]), dev([T]), dev([0]), table[None].contiguous(),
+                                nh, nkv, d, scale, max_keys=T, tile=tile, alone=alone).view(T, nh, d)
+    for who, h, far in plants:
+        torch.testing.assert_close(out[who, h].float(), v[far, 0].float(), atol=2e-2, rtol=2e-2,
+                                   msg=lambda m: f"query {who} head {h} far key {far}: {m}")
+    # a window of 600 keys across the 16,384 edge: the key inside it is seen, the one just outside is not
+    window = 600
+    inside, outside = (16700, 1, 16383), (16900, 0, 16900 - window)
+    k2 = k.float()
+    plant_far_key(q, k2, outside[0], outside[1], outside[2], d, seed=40)      # q keeps its type: rounded on assignment
+    k2 = k2.to(dtype)
+    kc2, vc2, table2 = make_paged(k2, v, ps, T // ps + 2)
+    o = ops.attention_prefill(q.view(T, nh * d), kc2, vc2, te, to, dev([0]), dev([T]), dev([0]), table2[None].contiguous(),
+                              nh, nkv, d, scale, window, max_keys=T, tile=tile, alone=alone).view(T, nh, d)
+    torch.testing.assert_close(o[inside[0], inside[1]].float(), v[inside[2], 0].float(), atol=2e-2, rtol=2e-2)
+    assert float((o[outside[0], outside[1]].float() - v[outside[2], 0].float()).abs().max()) > 0.5
+    o = ops.attention_prefill(q.view(T, nh * d), kc2, vc2, te, to, dev([0]), dev([T]), dev([0]), table2[None].contiguous(),
+                              nh, nkv, d, scale, window + 1, max_keys=T, tile=tile, alone=alone).view(T, nh, d)
+    torch.testing.assert_close(o[outside[0], outside[1]].float(), v[outside[2], 0].float(), atol=2e-2, rtol=2e-2)
+
+
+def test_attention_prefill_short_cut_far_keys_stand_out(ops):
+    """The cut every 2,048 keys (a launch of few tiles): dominating keys just below and just above the edges at
+    2,048 and 4,096, seen from queries of a later cut, with both tile sizes."""
+    nh, nkv, d, ps, T = 3, 1, 128, 16, 4500
+    dtype = torch.bfloat16
+    k, v = rnd(T, nkv, d, seed=1) * 0.1, rnd(T, nkv, d, seed=2)
+    q = rnd(T, nh, d, seed=3) * 0.1
+    plants = [(4400, 0, 2047), (4300, 1, 2048), (4499, 2, 4095), (4200, 2, 4096), (2100, 1, 5), (2050, 0, 2049)]
+    for i, (who, h, far) in enumerate(plants):
+        plant_far_key(q, k, who, h, far, d, seed=60 + i)
+    k, v, q = k.to(dtype), v.to(dtype), q.to(dtype)
+    kc, vc, table = make_paged(k, v, ps, T // ps + 2)
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    for tile in (64, 128):
+        te, to = prefill_tiles([(0, T, 0)], tile)
+        assert ops.attention_prefill_workspace(T, nh, d, T, 0, te.numel()) > 0
+        out = ops.attention_prefill(q.view(T, nh * d), kc, vc, te, to, dev([0]), dev([T]), dev([0]),
+                                    table[None].contiguous(), nh, nkv, d, 1 / math.sqrt(d), max_keys=T, tile=tile).view(T, nh, d)
+        for who, h, far in plants:
+            torch.testing.assert_close(out[who, h].float(), v[far, 0].float(), atol=2e-2, rtol=2e-2,
+                                       msg=lambda m: f"tile {tile} query {who} head {h} far key {far}: {m}")
+
+
 def test_attention_prefill_refuses_other_shapes(ops):
     assert not ops.attention_prefill_supported(torch.float32, 12, 2, 128, 16)
     assert not ops.attention_prefill_supported(torch.bfloat16, 12, 2, 256, 16)

@@ -5,6 +5,8 @@ length; the float32 path is checked against it at short lengths by the other tes
 import pytest
 import torch
 
+from tolerances import sharp_std
+
 pytestmark = pytest.mark.gpu
 
 
@@ -20,8 +22,9 @@ def test_long_context_serving_kernels_agree_with_the_float32_path(tmp_path):
         torch_dtype="bfloat16", eos_token_id=2002, hidden_size=512, intermediate_size=1408, num_attention_heads=8,
         num_key_value_heads=2, head_dim=128, tie_word_embeddings=True))
     folder = str(tmp_path / "long")
+    # sharp weights: attention is peaked, so a lost or doubled run of keys moves the logits beyond the tolerance
     write_model_folder(folder, cfg, expected_weights(qwen2_forward_config(cfg)), seed=3, dtype=torch.bfloat16,
-                       noisy_norms=True)
+                       noisy_norms=True, std=sharp_std(cfg.hidden_size))
     T, decoded = 20000, 40
     toks = torch.randint(0, 2002, (T + decoded,), generator=torch.Generator().manual_seed(0)).tolist()
     outs = {}
@@ -62,7 +65,7 @@ def test_a_long_prompt_in_one_step_agrees_with_the_float32_path(tmp_path):
         num_key_value_heads=2, head_dim=128, tie_word_embeddings=True))
     folder = str(tmp_path / "long")
     write_model_folder(folder, cfg, expected_weights(qwen2_forward_config(cfg)), seed=4, dtype=torch.bfloat16,
-                       noisy_norms=True)
+                       noisy_norms=True, std=sharp_std(cfg.hidden_size))
     T, more = 13000, 700
     toks = torch.randint(0, 2002, (T + more,), generator=torch.Generator().manual_seed(1)).tolist()
     want = [0, 1, 2047, 2048, 6143, 6144, 9999, T - 1]
