@@ -298,6 +298,82 @@ def further_32b(args):
     return res
 
 
+STAMP_NAMES = {0: "start", 1: "normed", 2: "q/k/v product done", 3: "at barrier 1", 4: "past barrier 1",
+               5: "attention done, at barrier 2", 6: "past barrier 2", 13: "attention's output in LDS",
+               7: "output product done, at barrier 3", 8: "past barrier 3", 12: "normed residual in LDS",
+               9: "gate/up done, at barrier 4", 10: "past barrier 4", 14: "activation in LDS", 11: "end"}
+STAMP_ORDER = [0, 1, 2, 3, 4, 5, 6, 13, 7, 8, 12, 9, 10, 14, 11]
+
+
+def resident_layer_probe(args, shape):
+    """Times ops.decode_layer (one launch a decoder layer) alone: `layers` layers of distinct random weights, one
+    launch each, replayed as a graph, for `batch` requests at position `prompt_len`.  A library built with
+    -DDL_TIMING also leaves the clock at the phases of the last launch; their spread over the workgroups is printed
+    to stderr."""
+    import math
+
+    import torch
+    from zedinfer_amd import ops
+    n, ctx, L = args.batch, args.prompt_len, args.layers
+    H, I = shape["hidden_size"], shape["intermediate_size"]
+    nh, nkv = shape["num_attention_heads"], shape["num_key_value_heads"]
+    d, ps, bt, dev = H // nh, 16, torch.bfloat16, "cuda"
+    Qd, KVd = nh * d, nkv * d
+    max_keys = ctx + 64
+    if not ops.decode_layer_supported(bt, n, H, I, nh, nkv, d, d, ps, max_keys, 0):
+        print(json.dumps({"resident_layer": None, "why": "the kernel does not take this shape"}))
+        return 0
+    W = [dict(wqkv=torch.randn(Qd + 2 * KVd, H, device=dev, dtype=bt) * 0.02, bias=torch.randn(Qd + 2 * KVd, device=dev, dtype=bt) * 0.1,
+              wo=torch.randn(H, Qd, device=dev, dtype=bt) * 0.02, wgu=torch.randn(2 * I, H, device=dev, dtype=bt) * 0.02,
+              wd=torch.randn(H, I, device=dev, dtype=bt) * 0.01, g=torch.ones(H, device=dev, dtype=bt)) for _ in range(L)]
+    pages_each = -(-(ctx + 64) // ps)
+    num_pages = n * pages_each + 1
+    caches = [(torch.randn(num_pages, nkv, ps, d, device=dev, dtype=bt), torch.randn(num_pages, nkv, d, ps, device=dev, dtype=bt))
+              for _ in range(L)]
+    table = (torch.arange(n * pages_each, dtype=torch.int32).view(n, pages_each) + 1).to(dev)
+    pos = torch.full((n,), ctx, dtype=torch.int32, device=dev)
+    slots = (table[:, ctx // ps].long() * ps + ctx % ps).to(torch.int32)
+    ws = torch.empty(ops.decode_layer_workspace(n, H, I, nh, nkv, d, max_keys, 0), dtype=torch.uint8, device=dev)
+    words = ops.decode_layer_sync_words()
+    sync = torch.zeros(words, dtype=torch.int32, device=dev)
+    err = torch.zeros(1, dtype=torch.int32).pin_memory()
+    rope = ops.rope_table(pos, ops.rope_inv_freq(d, shape["rope_theta"], torch.device(dev)))
+    resid = torch.randn(n, H, device=dev)
+
+    def step():
+        for w, (kc, vc) in zip(W, caches):
+            ops.decode_layer(resid, w["g"], w["g"], 1e-6, 1e-6, False, w["wqkv"], w["bias"], w["wo"], w["wgu"], w["wd"], rope,
+                             slots, kc, vc, pos, table, nh, nkv, d, 1 / math.sqrt(d), max_keys, 0, ws, sync, err)
+    step()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        step()
+    for _ in range(max(args.warmup, 1)):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        g.replay()
+    torch.cuda.synchronize()
+    us = (time.perf_counter() - t0) / args.steps * 1e6
+    weights = L * 2 * ((Qd + 2 * KVd) * H + H * Qd + 3 * I * H)
+    cache = L * n * ctx * 2 * KVd * 2
+    print(json.dumps({"resident_layer": {"us_per_layer": round(us / L, 2), "us_per_step": round(us, 1), "layers": L,
+                                         "batch": n, "context": ctx, "shape": args.shape,
+                                         "GB/s": round((weights + cache) / us / 1e3, 1), "wait_ran_out": int(err[0])}}))
+    stamps = ops.decode_layer_stamps()
+    if stamps:
+        st = sync[words - 256 * 2 * stamps:].view(torch.int64).view(256, stamps).cpu().double()
+        rel = (st - st[:, 0].min()) / 100.0           # the clock runs at 100 MHz: microseconds
+        for i in STAMP_ORDER:
+            col = rel[:, i][st[:, i] > 0]
+            if col.numel():
+                print(f"{STAMP_NAMES[i]:36s} first {col.min():7.2f}  median {col.median():7.2f}  last {col.max():7.2f} us",
+                      file=sys.stderr)
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -316,6 +392,8 @@ def main():
     ap.add_argument("--no-further", action="store_true", help="skip the figures at the 7B and 32B sizes")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
+    ap.add_argument("--resident-layer", action="store_true",
+                    help="instead: time the one-launch decoder layer (ops.decode_layer) alone, --layers launches a step")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -330,6 +408,8 @@ def main():
         args.layers = full_layers
     shape = dict(SHAPE, **SHAPES[args.shape])
     shape["num_hidden_layers"] = args.layers
+    if args.resident_layer:
+        return resident_layer_probe(args, shape)
     cfg = Qwen2Config.from_dict(shape)
     el = 2 if args.dtype == "bf16" else 4
     weights_cache = {}

@@ -32,6 +32,8 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-unknown-warning-option",
 ]
+# More flags for hipcc from the environment (a probe build, e.g. -DDL_TIMING); they go into the library's hash.
+FLAGS += os.environ.get("ZEDINFER_AMD_EXTRA_FLAGS", "").split()
 # The library matrix product (gemm_lt.hip) is hipBLASLt's.
 LINK_LIBS = ["-lhipblaslt"]
 

@@ -35,6 +35,13 @@ int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_
     int32_t* entry_len, const int32_t* entry_past, const int32_t* block_tables, int max_pages, int num_pages, int nh,
     int nkv, int d, int page_size, int window, float scale, int rows, int max_chunks, float* workspace, int64_t
     workspace_floats, int tile, int alone, int chunk_keys, hipStream_t stream);
+// decode_layer.hip
+int zi_decode_layer(float* resid, int n, int H, int I, const void* norm1, const void* norm2, int norm_dt, float eps1,
+    float eps2, int add_one, const void* wqkv, int64_t ld_qkv, const void* bias, int bias_dt, const void* wo, int64_t
+    ld_o, const void* wgu, int64_t ld_gu, const void* wd, int64_t ld_d, int dt, const float* table, int rot, const
+    int32_t* slots, int64_t cache_slots, void* kcache, void* vcache, const int32_t* tok_pos, const int32_t*
+    block_tables, int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window, float scale, int
+    max_keys, void* workspace, int64_t workspace_bytes, uint32_t* sync, int* err, int spin_limit, hipStream_t stream);
 // elementwise.hip
 int zi_embedding(void* out, int out_dt, const void* table, int table_dt, const int32_t* ids, int n, int hidden, int
     vocab, hipStream_t stream);
@@ -97,6 +104,7 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_attention_decode_project) \
     X(zi_attention_generic) \
     X(zi_attention_prefill) \
+    X(zi_decode_layer) \
     X(zi_embedding) \
     X(zi_gather_rows) \
     X(zi_add) \

@@ -37,6 +37,11 @@ _PROTOTYPES = {
     "zi_attention_decode_project_supported": [I, I, I, I, L],
     "zi_attention_decode_project_heads": [I],
     "zi_rope_table": [P, P, P, I, I, P],
+    "zi_decode_layer": [P, I, I, I, P, P, I, F, F, I, P, L, P, I, P, L, P, L, P, L, I, P, I, P, L, P, P, P, P, I, I, I, I,
+                        I, I, I, F, I, P, L, P, P, I, P],
+    "zi_decode_layer_supported": [I, I, I, I, I, I, I, I, I, I, I],
+    "zi_decode_layer_sync_words": [],
+    "zi_decode_layer_stamps": [],
     "zi_attention_decode_chunks": [I],
     "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, I, I, P],
     "zi_attention_prefill_chunk_keys_for": [I, I],
@@ -99,6 +104,8 @@ def load() -> ctypes.CDLL:
         lib.zi_gemm_skinny_workspace.restype = c_int64
         lib.zi_attention_prefill_workspace.argtypes = [I, I, I, I]
         lib.zi_attention_prefill_workspace.restype = c_int64
+        lib.zi_decode_layer_workspace.argtypes = [I, I, I, I, I, I, I, I]
+        lib.zi_decode_layer_workspace.restype = c_int64
         lib.zi_argmax_workspace.argtypes = [I, I]
         lib.zi_argmax_workspace.restype = c_int64
         lib.zi_tape_new.argtypes = []

@@ -562,6 +562,99 @@ def attention_decode_project(workspace: torch.Tensor, weight: torch.Tensor, tok_
     return out
 
 
+DECODE_LAYER_SPIN_LIMIT = 400000      # polls of a barrier inside the resident layer kernel before it gives up (about 0.2 s)
+
+
+def decode_layer_sync_words() -> int:
+    """int32 words of synchronisation state the resident layer kernel needs (zeroed once, shared by every call)."""
+    return int(_lib.load().zi_decode_layer_sync_words())
+
+
+def decode_layer_stamps() -> int:
+    """Clock stamps a workgroup of the resident layer kernel leaves per launch behind the synchronisation words:
+    32 in a library built with -DDL_TIMING (a probe for tuning), 0 in the product's."""
+    return int(_lib.load().zi_decode_layer_stamps())
+
+
+def decode_layer_supported(dtype: torch.dtype, n: int, hidden: int, inter: int, nh: int, nkv: int, d: int, rot: int,
+                           page_size: int, max_keys: int, window: int = 0) -> bool:
+    """Whether ``decode_layer`` takes a step of ``n`` single tokens of these sizes on the current device."""
+    if dtype not in _CODES:
+        return False
+    return bool(_lib.load().zi_decode_layer_supported(_CODES[dtype], int(n), int(hidden), int(inter), int(nh), int(nkv),
+                                                       int(d), int(rot), int(page_size), int(max_keys), int(window)))
+
+
+def decode_layer_workspace(n: int, hidden: int, inter: int, nh: int, nkv: int, d: int, max_keys: int,
+                           window: int = 0) -> int:
+    """Bytes of workspace ``decode_layer`` needs for these sizes."""
+    need = int(_lib.load().zi_decode_layer_workspace(int(n), int(hidden), int(inter), int(nh), int(nkv), int(d),
+                                                     int(max_keys), int(window)))
+    if need < 0:
+        raise _lib.KernelLibraryError(_lib.load().zi_last_error().decode("utf-8", "replace"))
+    return need
+
+
+def decode_layer(resid: torch.Tensor, norm1: torch.Tensor, norm2: torch.Tensor, eps1: float, eps2: float, add_one: bool,
+                 wqkv: torch.Tensor, bias: Optional[torch.Tensor], wo: torch.Tensor, wgu: torch.Tensor, wd: torch.Tensor,
+                 table: Optional[torch.Tensor], slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+                 tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
+                 max_keys: int, window: int, workspace: torch.Tensor, sync: torch.Tensor, err: torch.Tensor,
+                 spin_limit: int = DECODE_LAYER_SPIN_LIMIT) -> torch.Tensor:
+    """One pre-norm decoder layer (attention with a split-half rotation, SwiGLU feed-forward, RMS norms) for
+    n <= 16 tokens that are each the only one of their sequence in the step, in one launch of resident
+    workgroups: ``resid`` [n, hidden] float32 is replaced by the layer's output and the tokens' new keys and
+    values are stored at ``slots``.  ``wgu`` [2I, hidden] holds gate and up rows alternating in blocks of 8;
+    ``table`` [n, pairs, 2] are the step's (cos, sin) from ``rope_table`` (None: no rotation).  ``sync``
+    (``decode_layer_sync_words()`` zeroed int32 words on the device) is shared by every call; ``err`` is one
+    int32 word of pinned host memory which the kernel sets when one of its waits ran out: the step's result is
+    then garbage (NaN), and ``sync`` must be zeroed before the next call."""
+    _gpu("decode_layer", resid, norm1, norm2, wqkv, bias, wo, wgu, wd, table, slots, kcache, vcache, tok_pos,
+         block_tables, workspace, sync)
+    if resid.dim() != 2 or resid.dtype != torch.float32 or not resid.is_contiguous():
+        raise ValueError("decode_layer: resid must be a contiguous float32 [n, hidden] tensor")
+    n, H = resid.shape
+    for name, w in (("wqkv", wqkv), ("wo", wo), ("wgu", wgu), ("wd", wd)):
+        if w.dim() != 2 or w.dtype != torch.bfloat16 or w.stride(1) != 1:
+            raise ValueError(f"decode_layer: {name} must be a bfloat16 matrix with dense rows")
+    Qd, KVd = nh * d, nkv * d
+    inter = wd.shape[1]
+    if (tuple(wqkv.shape) != (Qd + 2 * KVd, H) or tuple(wo.shape) != (H, Qd) or tuple(wgu.shape) != (2 * inter, H)
+            or wd.shape[0] != H):
+        raise ValueError(f"decode_layer: weight shapes {tuple(wqkv.shape)}, {tuple(wo.shape)}, {tuple(wgu.shape)}, "
+                         f"{tuple(wd.shape)} do not fit hidden {H}, heads {nh}/{nkv} of {d}")
+    for name, g in (("norm1", norm1), ("norm2", norm2)):
+        if g.dim() != 1 or g.numel() != H or not g.is_contiguous() or g.dtype != norm1.dtype:
+            raise ValueError(f"decode_layer: {name} must hold {H} gains of one type")
+    if bias is not None and (bias.dim() != 1 or bias.numel() != Qd + 2 * KVd or not bias.is_contiguous()):
+        raise ValueError(f"decode_layer: bias must hold {Qd + 2 * KVd} values")
+    pages, ps = _check_cache(kcache, vcache, nkv, d, torch.bfloat16, "decode_layer")
+    _i32(tok_pos, "decode_layer tok_pos", n)
+    _i32(slots, "decode_layer slots", n)
+    if block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous() \
+            or block_tables.shape[0] < n:
+        raise ValueError(f"decode_layer: block_tables must be a contiguous int32 [>= {n}, max_pages] tensor")
+    rot = 0
+    if table is not None:
+        if table.dim() != 3 or table.shape[0] != n or table.shape[2] != 2 or table.dtype != torch.float32 \
+                or not table.is_contiguous():
+            raise ValueError(f"decode_layer: table must be a contiguous float32 [{n}, pairs, 2] tensor")
+        rot = 2 * table.shape[1]
+    if sync.dtype != torch.int32 or sync.numel() < decode_layer_sync_words() or not sync.is_contiguous():
+        raise ValueError("decode_layer: sync must hold decode_layer_sync_words() int32 words")
+    if err.dtype != torch.int32 or err.numel() < 1 or err.is_cuda or not err.is_pinned():
+        raise ValueError("decode_layer: err must be an int32 word of pinned host memory")
+    if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+        raise ValueError("decode_layer: workspace must be a contiguous uint8 tensor")
+    _lib.call("zi_decode_layer", _p(resid), n, H, inter, _p(norm1), _p(norm2), _code(norm1, "decode_layer gains"),
+              c_float(eps1), c_float(eps2), int(bool(add_one)), _p(wqkv), wqkv.stride(0), _p(bias),
+              _code(bias, "decode_layer bias") if bias is not None else 0, _p(wo), wo.stride(0), _p(wgu), wgu.stride(0),
+              _p(wd), wd.stride(0), BF16, _p(table), rot, _p(slots), pages * ps, _p(kcache), _p(vcache), _p(tok_pos),
+              _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), c_float(scale), int(max_keys),
+              _p(workspace), workspace.numel(), _p(sync), c_void_p(err.data_ptr()), int(spin_limit), _stream())
+    return resid
+
+
 def attention_prefill_variant(variant: int = -1) -> int:
     """Which prompt-attention kernel head sizes 64 and 128 take: 1 (the default) loads keys and values
     straight into LDS, 0 stages them through registers like the other head sizes; both give the same
