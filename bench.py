@@ -128,7 +128,7 @@ def long_context_points(base_engine, shape, layers, el, args, contexts=(16384, 3
     what a step reads), on another cache pool of an engine that holds the weights already."""
     import torch
     from zedinfer_amd.config import SchedulerConfig
-    from zedinfer_amd.engine.engine import many_rows_size_at_least
+    from zedinfer_amd.parts.rows import many_rows as many_rows_size_at_least
     out = {}
     steps, warm = min(args.steps, 32), min(args.warmup, 8)
     for ctx in contexts:
@@ -177,8 +177,7 @@ def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT, warm=1):
     eng = engine_factory()
     # which of two equivalent orientations the library's gate/up product takes at this many rows is
     # measured here, before the clock starts, and reported with the result
-    from zedinfer_amd.engine.engine import many_rows_size_at_least
-    rows = many_rows_size_at_least(tokens)      # the step runs padded to this many rows
+    rows = eng.model.step_rows(tokens, "mixed")      # the step runs padded to this many rows
     CHOICES.update({" ".join(str(x) for x in k): v for k, v in eng.warm_up([rows]).items()
                     if len(k) > 1 and k[1] == rows})          # this step's own; a serving engine holds one set a size
     rng = random.Random(77)
@@ -255,7 +254,7 @@ def further_32b(args):
         holder["e"] = Engine.from_config(cfg, "Qwen2ForCausalLM", args.dtype, seed=0, sched=sched)
         return holder["e"]
     # the prompts enter whole, alone or beside the requests that decode already: the two sizes of such steps
-    from zedinfer_amd.engine.engine import many_rows_size_at_least
+    from zedinfer_amd.parts.rows import many_rows as many_rows_size_at_least
     tps, ms_step, ctx_mid = measure_decode(decode_engine, batch, steps, warm, cfg.vocab_size, prompt,
                                            warm_up_sizes=[many_rows_size_at_least(prompt + 64), prompt])
     need = decode_bytes(shape, L, batch, ctx_mid, el)

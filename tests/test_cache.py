@@ -6,13 +6,13 @@ import pytest
 import torch
 
 from zedinfer_amd.cache import CacheManager, IdPool, OutOfPages, OutOfSlots, PagePool
-from zedinfer_amd.parts import KVCacheRequest
+from zedinfer_amd.parts.mixers import attention_cache_request
 
 
 def manager(pages=12, page_size=4, requests=4, window=0, max_step_tokens=8):
-    kv = {0: KVCacheRequest("full", 2, 16), 1: KVCacheRequest("full", 2, 16)}
+    kv = {0: attention_cache_request("full", 2, 16), 1: attention_cache_request("full", 2, 16)}
     if window:
-        kv[2] = KVCacheRequest("window", 1, 32, window)
+        kv[2] = attention_cache_request("window", 1, 32, window)
     return CacheManager(kv, {}, pages, page_size, requests, torch.float32, None, max_step_tokens)
 
 

@@ -574,7 +574,7 @@ def test_steps_of_many_rows_come_in_the_sizes_the_warm_up_measured(tmp_path):
     decoding entries filled up to a multiple of 64, so every such step's rows are among the measured sizes; the
     tokens are the plain implementation's."""
     from zedinfer_amd import GenerationConfig, InferenceEngine, SchedulerConfig
-    from zedinfer_amd.engine.engine import many_rows_step_sizes
+    from zedinfer_amd.parts.rows import sizes_between
     folder = tiny_configs.write_tiny(str(tmp_path / "m"), "B", dtype=torch.bfloat16, std=tiny_configs.SHARP_STD)
     cfg, w = plain.load_folder(folder)
     ps = tiny_configs.PAGE_SIZES["B"]
@@ -582,7 +582,7 @@ def test_steps_of_many_rows_come_in_the_sizes_the_warm_up_measured(tmp_path):
                                                                     max_prefill_tokens=192, max_batch_tokens=256))
     eng = ie.engine
     measured = {k[1] for k in eng.rt.choices if k[0] == "library_product"}
-    assert measured == set(many_rows_step_sizes(192 + 4 + 64)) == {320, 256, 192, 128}
+    assert measured == set(sizes_between(eng.model.step_rows, "mixed", 128, 192 + 4 + 64)) == {320, 256, 192, 128}
     prompts = [traces.random_tokens(cfg["vocab_size"], n, seed=70 + i) for i, n in enumerate([250, 200, 130, 70])]
     results = ie.generate(prompts, GenerationConfig(max_new_tokens=12, ignore_eos=True))
     mixed = [k for k in eng._prompt_graphs if k[1] > 0]             # (entries, decoding entries, tokens of the portions, ...)

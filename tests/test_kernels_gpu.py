@@ -224,7 +224,7 @@ def test_rope_kv_store(ops, dtype):
     q_ref = torch_rope(q.float().reshape(n, nh, d), pos, theta)
     k_ref = torch_rope(k.float().reshape(n, nkv, d), pos, theta)
     v_ref = v.clone().reshape(n, nkv, d)
-    ops.rope_kv_store(q, k, v, pos, slots, ops.rope_inv_freq(d, theta, "cuda"), kc, vc, nh, nkv, d)
+    ops.rope_kv_store(q, k, v, ops.rope_table(pos, ops.rope_inv_freq(d, theta, "cuda")), slots, kc, vc, nh, nkv, d)
     torch.testing.assert_close(q.float().reshape(n, nh, d), q_ref, **tol(dtype, 5e-4, 2e-2))
     for t in range(n):
         p, o = int(slots[t]) // ps, int(slots[t]) % ps
@@ -252,7 +252,7 @@ def test_rope_kv_store_many_tokens(ops, nh, nkv, d, rot, ps, layout):
         slots = torch.arange(n, dtype=torch.int32) + (0 if layout == "runs" else 3)
     slots[17] = -1
     slots = slots.cuda()
-    inv = ops.rope_inv_freq(rot, theta, "cuda") if rot else None
+    table = ops.rope_table(pos, ops.rope_inv_freq(rot, theta, "cuda")) if rot else None      # the step's (cos, sin)
 
     def run(step):
         qq = qkv.clone()
@@ -260,8 +260,8 @@ def test_rope_kv_store_many_tokens(ops, nh, nkv, d, rot, ps, layout):
         vc = torch.full((pages, nkv, d, ps), 3.0, dtype=dtype, device="cuda")
         for a in range(0, n, step):
             b = min(n, a + step)
-            ops.rope_kv_store(qq[a:b, :nh * d], qq[a:b, nh * d:(nh + nkv) * d], qq[a:b, (nh + nkv) * d:], pos[a:b],
-                              slots[a:b], inv, kc, vc, nh, nkv, d)
+            ops.rope_kv_store(qq[a:b, :nh * d], qq[a:b, nh * d:(nh + nkv) * d], qq[a:b, (nh + nkv) * d:],
+                              table[a:b] if rot else None, slots[a:b], kc, vc, nh, nkv, d)
         return qq[:, :nh * d], kc, vc
 
     q1, kc1, vc1 = run(n)       # one call: the kernel for many tokens
@@ -272,7 +272,7 @@ def test_rope_kv_store_many_tokens(ops, nh, nkv, d, rot, ps, layout):
     assert int((vc1 != 3.0).any(1).any(1).sum()) == n - 1      # every token's slot but the one out of range
     # queries only
     q3 = qkv.clone()
-    ops.rope_kv_store(q3[:, :nh * d], None, None, pos, None, inv, None, None, nh, nkv, d)
+    ops.rope_kv_store(q3[:, :nh * d], None, None, table, None, None, None, nh, nkv, d)
     assert torch.equal(q3[:, :nh * d], q1) and torch.equal(q3[:, nh * d:], qkv[:, nh * d:])
 
 
@@ -484,7 +484,8 @@ def test_attention_decode_fused(ops, nh, nkv, d, ps, lens, window, S, bias_dtype
     # the two kernels
     kc1, vc1 = kc.clone(), vc.clone()
     q = torch.empty(B, nh * d, dtype=dtype, device="cuda")
-    ops.rope_kv_store_sums(sums, bias, q, pos, slots, inv_freq, kc1, vc1, nh, nkv, d)
+    ops.rope_kv_store_sums(sums, bias, q, ops.rope_table(pos, inv_freq) if inv_freq is not None else None, slots, kc1,
+                           vc1, nh, nkv, d)
     ref = ops.attention_decode(q, kc1, vc1, seq, pos, bt, nh, nkv, d, scale, T, window)
     # the one kernel
     kc2, vc2 = kc.clone(), vc.clone()
@@ -986,7 +987,8 @@ def test_rope_kv_store_sums(ops, dtype, with_bias):
     kc = torch.zeros(pages, nkv, ps, d, dtype=dtype, device="cuda")
     vc = torch.zeros(pages, nkv, d, ps, dtype=dtype, device="cuda")
     q_out = torch.empty(n, nh * d, dtype=dtype, device="cuda")
-    ops.rope_kv_store_sums(sums, bias, q_out, pos, slots, ops.rope_inv_freq(d, theta, "cuda"), kc, vc, nh, nkv, d)
+    table = ops.rope_table(pos, ops.rope_inv_freq(d, theta, "cuda"))
+    ops.rope_kv_store_sums(sums, bias, q_out, table, slots, kc, vc, nh, nkv, d)
     q_ref = torch_rope(q.reshape(n, nh, d), pos, theta)
     k_ref = torch_rope(k.reshape(n, nkv, d), pos, theta)
     torch.testing.assert_close(q_out.float().reshape(n, nh, d), q_ref, **tol(dtype, 5e-4, 3e-2))
@@ -996,5 +998,5 @@ def test_rope_kv_store_sums(ops, dtype, with_bias):
         torch.testing.assert_close(vc[p, :, :, o].float(), v[t].reshape(nkv, d), **tol(dtype, 1e-6, 2e-2))
     # queries alone (a layer that reads another layer's cache)
     q2 = torch.empty_like(q_out)
-    ops.rope_kv_store_sums(sums, bias, q2, pos, None, ops.rope_inv_freq(d, theta, "cuda"), None, None, nh, nkv, d)
+    ops.rope_kv_store_sums(sums, bias, q2, table, None, None, None, nh, nkv, d)
     assert torch.equal(q2, q_out)

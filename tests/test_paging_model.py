@@ -17,7 +17,8 @@ import pytest
 import torch
 
 from zedinfer_amd.cache import CacheManager, OutOfPages
-from zedinfer_amd.parts import HostBatch, KVCacheRequest
+from zedinfer_amd.parts import HostBatch
+from zedinfer_amd.parts.mixers import attention_cache_request
 from zedinfer_amd.parts.mixers import AttentionPlanner
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -72,9 +73,9 @@ def decode(pm, pos, tables, num_pages, nh, nkv, d, ps, window, max_chunks, slots
 def traffic(seed, window, pages=48, ps=16, requests=6):
     """A cache manager after random opens, growth and closes; returns it with its live sequences."""
     rng = random.Random(seed)
-    kv = {0: KVCacheRequest("full", 2, 32)}
+    kv = {0: attention_cache_request("full", 2, 32)}
     if window:
-        kv[1] = KVCacheRequest("window", 2, 32, window)
+        kv[1] = attention_cache_request("window", 2, 32, window)
     m = CacheManager(kv, {}, pages, ps, requests, torch.bfloat16, None, max_step_tokens=64)
     live = []
     for step in range(60):
@@ -148,7 +149,7 @@ def test_decode_walk_under_random_traffic(model, seed, window):
 
 
 def test_decode_walk_reports_what_is_broken(model):
-    m = CacheManager({0: KVCacheRequest("full", 2, 32)}, {}, 64, 16, 4, torch.bfloat16, None, max_step_tokens=64)
+    m = CacheManager({0: attention_cache_request("full", 2, 32)}, {}, 64, 16, 4, torch.bfloat16, None, max_step_tokens=64)
     live = [m.open("a"), m.open("b")]
     for s, n in zip(live, (700, 40)):
         m.ensure(s, n)
@@ -243,7 +244,7 @@ def test_prefill_walk_under_random_traffic(model, seed, window, tile):
 def test_prefill_walk_of_a_long_prompt_and_what_is_broken(model, tile):
     """One portion that continues a long sequence: its tiles are cut along the keys every 2,048, and the cuts'
     partial results have places of their own in the workspace."""
-    m = CacheManager({0: KVCacheRequest("full", 2, 32)}, {}, 700, 8, 2, torch.bfloat16, None, max_step_tokens=2048)
+    m = CacheManager({0: attention_cache_request("full", 2, 32)}, {}, 700, 8, 2, torch.bfloat16, None, max_step_tokens=2048)
     s = m.open("long")
     m.ensure(s, 4100)
     m.commit(s, 4100)
@@ -277,7 +278,7 @@ def test_prefill_walk_with_the_cut_of_long_prompts(model, tile):
     keys instead of every 2,048 (they fill the chip without cuts, and every cut costs a merge): a portion behind 17,000 tokens walks its
     keys in two cuts, every (query, key) pair once, its block table entries within what the kernel stages; a
     portion behind 7,000 in one, with no workspace."""
-    m = CacheManager({0: KVCacheRequest("full", 2, 32)}, {}, 2300, 8, 2, torch.bfloat16, None, max_step_tokens=2048)
+    m = CacheManager({0: attention_cache_request("full", 2, 32)}, {}, 2300, 8, 2, torch.bfloat16, None, max_step_tokens=2048)
     assert model.pm_prefill_chunk_for(6144, 5000) == 2048 and model.pm_prefill_chunk_for(6145, 768) == 16384
     assert model.pm_prefill_chunk_for(30000, 767) == 2048
     for past, cuts in ((17000, 2), (7000, 1)):

@@ -198,30 +198,51 @@ def test_embedding_and_head_parts(dtype):
 # ---- position encoding ------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("rotary_dim", [48, 16])
-def test_rope_part_rotates_queries_and_stores_keys(dtype, rotary_dim):
-    from zedinfer_amd.parts import POSITION_ENCODINGS, LayerMemory
+def test_rope_part_encodes_and_hands_over_the_table_the_store_kernel_takes(dtype, rotary_dim):
+    """The encoding alone: ``encode`` turns q and k in place; ``step_table`` gives the step's (cos, sin), with which
+    the store kernel (the attention's fast path) turns q in place and puts the turned k and the raw v into a cache."""
+    from types import SimpleNamespace
+    from zedinfer_amd import ops
+    from zedinfer_amd.parts import POSITION_ENCODINGS
     n, nh, nkv, d, ps, pages, theta = 6, 4, 2, 48, 8, 5, 3e4
     part = POSITION_ENCODINGS.get("rope_neox")(spec("rope_neox", {"head_dim": d, "theta": theta,
                                                                    "rotary_dim": rotary_dim}), {}, runtime(dtype))
     qkv = rnd(n, (nh + 2 * nkv) * d, seed=1).to(dtype).cuda()
+    qkv2 = qkv.clone()
     q, k, v = qkv[:, :nh * d], qkv[:, nh * d:(nh + nkv) * d], qkv[:, (nh + nkv) * d:]
     q0, k0, v0 = q.float().cpu().clone(), k.float().cpu().clone(), v.clone()
     pos = torch.arange(20, 20 + n, dtype=torch.int32, device="cuda")
     slots = torch.tensor([3, 9, 17, 39, 0, 8], dtype=torch.int32, device="cuda")
-    mem = LayerMemory(group=0, k=torch.zeros(pages, nkv, ps, d, dtype=dtype, device="cuda"),
-                      v=torch.zeros(pages, nkv, d, ps, dtype=dtype, device="cuda"))
-    part.rotate_and_store(q, k, v, pos, slots, mem, nh, nkv, d)
 
     def ref(x, heads):
         x = x.view(n, heads, d).clone()
         x[..., :rotary_dim] = plain.rope_neox(x[..., :rotary_dim].contiguous(), pos.long().cpu(), theta)
         return x
+    part.encode(q, k, pos, nh, nkv, d)
     torch.testing.assert_close(q.float().cpu().view(n, nh, d), ref(q0, nh), **tol(dtype, 5e-4, 2e-2))
-    kr = ref(k0, nkv)
+    torch.testing.assert_close(k.float().cpu().view(n, nkv, d), ref(k0, nkv), **tol(dtype, 5e-4, 2e-2))
+    assert torch.equal(v, v0)
+    # the table, and the kernel that turns and stores by it
+    batch = SimpleNamespace(shared={}, num_tokens=n, positions=pos)
+    table = part.step_table(batch)
+    assert tuple(table.shape) == (n, rotary_dim // 2, 2) and part.step_table(batch) is table      # once a step
+    q2, k2, v2 = qkv2[:, :nh * d], qkv2[:, nh * d:(nh + nkv) * d], qkv2[:, (nh + nkv) * d:]
+    kc = torch.zeros(pages, nkv, ps, d, dtype=dtype, device="cuda")
+    vc = torch.zeros(pages, nkv, d, ps, dtype=dtype, device="cuda")
+    ops.rope_kv_store(q2, k2, v2, table, slots, kc, vc, nh, nkv, d)
+    assert torch.equal(q2, q)                        # the same turn, bit for bit
+    assert torch.equal(k2.float().cpu(), k0.to(dtype).float())      # k itself is left as it was
     for t in range(n):
         p, o = int(slots[t]) // ps, int(slots[t]) % ps
-        torch.testing.assert_close(mem.k[p, :, o].float().cpu(), kr[t], **tol(dtype, 5e-4, 2e-2))
-        assert torch.equal(mem.v[p, :, :, o], v0[t].view(nkv, d))
+        torch.testing.assert_close(kc[p, :, o].float(), k[t].view(nkv, d).float(), **tol(dtype, 1e-6, 1e-2))
+        assert torch.equal(vc[p, :, :, o], v0[t].view(nkv, d))
+    # keys and values that are encoded already are stored as they are
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ops.kv_store(k, v, slots, kc2, vc2, nkv, d)
+    assert torch.equal(vc2, vc)
+    for t in range(n):
+        p, o = int(slots[t]) // ps, int(slots[t]) % ps
+        assert torch.equal(kc2[p, :, o], k[t].view(nkv, d))
 
 
 # ---- mixer ------------------------------------------------------------------------------------
@@ -442,7 +463,7 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
     requests = {f"t{i}": traces.random_tokens(TOY["vocab_size"], n, seed=40 + i) for i, n in enumerate([37, 64, 9, 50, 23])}
     ref = {rid: toy_plain_forward(pcfg, w, toks) for rid, toks in requests.items()}
     engine = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=24, kv_block_size=8, max_batch_requests=4))
-    assert len(engine.cache.state) == 2 and len(engine.cache.k) == 1     # two stateful layers, one with a cache
+    assert len(engine.cache.state) == 2 and len(engine.cache.tensors) == 1     # two stateful layers, one with a cache
     for make in (traces.whole, traces.portions, traces.mixed):
         steps = make(requests)
         out = traces.run_in_process(engine, steps)
@@ -578,11 +599,9 @@ def _define_toy_routed():
             a, b = t[..., 0], t[..., 1]
             return torch.stack([a * c - b * s, b * c + a * s], dim=-1).view(x.shape[0], heads * d).to(x.dtype)
 
-        def rotate_and_store(self, q, k, v, positions, slots, memory, nh, nkv, d):
+        def encode(self, q, k, positions, nh, nkv, d):
             q.copy_(self.turn(q, positions, nh, d))
-            if memory.writes:
-                kk = self.turn(k, positions, nkv, d)
-                ops.rope_kv_store(q, kk, v.contiguous(), positions, slots, None, memory.k, memory.v, nh, nkv, d)
+            k.copy_(self.turn(k, positions, nkv, d))
 
     @dataclass(frozen=True)
     class ToyRoutedConfig(ModelConfig):
@@ -687,8 +706,8 @@ def toy_routed_plain_forward(cfg, w, ids):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16w"])
 def test_toy_architecture_with_routing_pairs_rotation_and_a_shared_cache(tmp_path, dtype):
     """float32, and bfloat16 with a bfloat16 checkpoint: there the attention takes the few-rows products and
-    their partial sums, the position encoding (which offers no table of angles) gets them through the
-    default of its base class, and the layer that reads another layer's cache stores nothing."""
+    their partial sums, the position encoding (which offers no table of angles) gets q and k once the attention
+    has added the sums up, and the layer that reads another layer's cache stores nothing."""
     _define_toy_routed()
     from zedinfer_amd.config import SchedulerConfig, load_config
     from zedinfer_amd.engine import Engine
@@ -710,7 +729,7 @@ def test_toy_architecture_with_routing_pairs_rotation_and_a_shared_cache(tmp_pat
     ref = {rid: toy_routed_plain_forward(pcfg, w, toks) for rid, toks in requests.items()}
     engine = Engine.from_folder(folder, "float32" if dtype == "float32" else "bfloat16",
                                 SchedulerConfig(num_kv_blocks=32, kv_block_size=8, max_batch_requests=4))
-    assert len(engine.cache.k) == 3          # four runs of layers, three caches
+    assert len(engine.cache.tensors) == 3          # four runs of layers, three caches
     for make in (traces.whole, traces.last_decoded, traces.mixed):
         steps = make(requests)
         out = traces.run_in_process(engine, steps)
@@ -760,12 +779,9 @@ def _define_toy_two_axes():
             a, b = t[..., :half], t[..., half:]
             return torch.cat([a * c - b * s, b * c + a * s], dim=-1).view(x.shape[0], heads * d).to(x.dtype)
 
-        def rotate_and_store(self, q, k, v, positions, slots, memory, nh, nkv, d):
+        def encode(self, q, k, positions, nh, nkv, d):
             q.copy_(self.turn(q, positions, nh, d))
-            if memory.writes:
-                kk = self.turn(k, positions, nkv, d)
-                ops.rope_kv_store(q, kk, v.contiguous(), positions[:, 0].contiguous(), slots, None, memory.k,
-                                  memory.v, nh, nkv, d)
+            k.copy_(self.turn(k, positions, nkv, d))
 
     def forward_config(cfg) -> ModelForwardConfig:
         H, nh, nkv, d = cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim

@@ -103,7 +103,8 @@ def test_rotation_store_and_attention(ops, ref, dtype, nh, nkv, d, rot, ps, wind
     ref.kv_store(kc_ref, vc_ref, k_ref, v.reshape(n, nkv, d), slots)
     kc = torch.full((num_pages, nkv, ps, d), float("nan"), dtype=dtype, device="cuda")
     vc = torch.full((num_pages, nkv, d, ps), float("nan"), dtype=dtype, device="cuda")
-    ops.rope_kv_store(q, k, v, pos.cuda(), slots.cuda(), ops.rope_inv_freq(rot, theta, "cuda"), kc, vc, nh, nkv, d)
+    ops.rope_kv_store(q, k, v, ops.rope_table(pos.cuda(), ops.rope_inv_freq(rot, theta, "cuda")), slots.cuda(), kc, vc,
+                      nh, nkv, d)
     close(q.reshape(n, nh, d), q_ref, dtype, f32=5e-4)
     stored = ~torch.isnan(kc_ref)
     assert torch.equal(torch.isnan(kc).cpu(), ~stored) and torch.equal(torch.isnan(vc).cpu(), torch.isnan(vc_ref))

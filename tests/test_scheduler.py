@@ -7,12 +7,12 @@ from zedinfer_amd.cache import CacheManager
 from zedinfer_amd.config import SchedulerConfig
 from zedinfer_amd.engine.request import GenerationConfig, InferenceRequest, RequestPhase, resolve_max_new_tokens
 from zedinfer_amd.engine.scheduler import QueueFull, Scheduler
-from zedinfer_amd.parts import KVCacheRequest
+from zedinfer_amd.parts.mixers import attention_cache_request
 
 
 def make(pages=64, page_size=4, **kw):
     cfg = SchedulerConfig(num_kv_blocks=pages, kv_block_size=page_size, **kw)
-    cache = CacheManager({0: KVCacheRequest("full", 1, 16)}, {}, pages, page_size, cfg.max_batch_requests,
+    cache = CacheManager({0: attention_cache_request("full", 1, 16)}, {}, pages, page_size, cfg.max_batch_requests,
                          torch.float32, None, cfg.max_batch_tokens)
     return Scheduler(cfg, cache, stop_token_ids=[99]), cache
 
@@ -438,7 +438,7 @@ def test_default_sampling_from_the_model_folder(tmp_path, monkeypatch):
 def test_requests_without_sampling_options_take_the_default():
     from zedinfer_amd.sampling import SamplingParams
     cfg = SchedulerConfig(num_kv_blocks=16, kv_block_size=4)
-    cache = CacheManager({0: KVCacheRequest("full", 1, 16)}, {}, 16, 4, cfg.max_batch_requests, torch.float32, None,
+    cache = CacheManager({0: attention_cache_request("full", 1, 16)}, {}, 16, 4, cfg.max_batch_requests, torch.float32, None,
                          cfg.max_batch_tokens)
     s = Scheduler(cfg, cache, default_sampling=SamplingParams(temperature=0.6, top_k=20, seed=7))
     plain_req, own, greedy, seeded = req(3), req(3, temperature=0.9), req(3, use_argmax=True), req(3, seed=11)
@@ -474,8 +474,13 @@ def test_sizes_at_which_a_serving_engine_measures_its_choices():
     """The multiples of the step that portions of prompts are padded to, from 128 rows to the most a step can
     bring, largest first; beyond 4,096 rows they lie further apart (32 an octave), and every number of rows has
     one at most a 32nd above it."""
-    from zedinfer_amd.engine.engine import Engine, many_rows_size_at_least, many_rows_step_sizes
-    assert Engine.PROMPT_GRAPH_STEP == 64
+    from zedinfer_amd.parts.rows import PORTION_ROWS, ProductRows, few_rows_entries, sizes_between
+    from zedinfer_amd.parts.rows import many_rows as many_rows_size_at_least
+
+    def many_rows_step_sizes(most):
+        return sizes_between(ProductRows.step_rows, "mixed", 128, most)
+    assert PORTION_ROWS == 64
+    assert [ProductRows.step_rows(n, "portion") for n in (2, 64, 65, 200)] == [64, 64, 128, 256]
     assert many_rows_step_sizes(300) == [320, 256, 192, 128]
     assert many_rows_step_sizes(2112) == list(range(2112, 127, -64))
     assert many_rows_step_sizes(64) == [] and many_rows_step_sizes(100) == [128]
@@ -488,16 +493,39 @@ def test_sizes_at_which_a_serving_engine_measures_its_choices():
     # what an engine measures by default: the sizes of its steps with prompt portions, and of its pure decode steps
     # of more than 64 requests
     from zedinfer_amd.engine import InferenceEngine
-    from zedinfer_amd.engine.engine import decode_entries_at_least
-    few = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=520, max_prefill_tokens=512))
-    assert few == [640, 576, 512, 448, 384, 320, 256, 192, 128]     # 520 tokens, rounded up, and one more size
-    many = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=200, max_batch_tokens=2248, max_prefill_tokens=2048))
-    assert many[0] == 2368 and many[-4:] == [128, 112, 96, 80] and 224 in many and 160 in many and len(many) == len(set(many))
-    for e in range(65, 201):
+    decode_entries_at_least, rows = few_rows_entries, ProductRows.step_rows      # what a model of such parts answers
+    few = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=520, max_prefill_tokens=512), rows)
+    # 520 tokens, rounded up, and one more size; then the decode steps of up to 8 requests
+    assert few == [640, 576, 512, 448, 384, 320, 256, 192, 128, 64, 8, 4, 2, 1]
+    many = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=200, max_batch_tokens=2248, max_prefill_tokens=2048), rows)
+    assert many[0] == 2368 and [m for m in many if 64 < m <= 128] == [128, 112, 96, 80] and 224 in many and 160 in many
+    assert len(many) == len(set(many)) and many[-8:] == [64, 48, 32, 16, 8, 4, 2, 1]
+    for e in range(1, 201):
         assert decode_entries_at_least(e) in many
     long = InferenceEngine.default_warm_up_sizes(SchedulerConfig(max_batch_requests=8, max_batch_tokens=16392, max_prefill_tokens=16384,
-                                                                 max_seq_len=32768))
-    assert long[:4] == [16896, 16384, 8448, 8192] and long[-1] == 128
+                                                                 max_seq_len=32768), rows)
+    assert long[:4] == [16896, 16384, 8448, 8192] and long[-5:] == [64, 8, 4, 2, 1]
+
+    # a part that wants other numbers has its say: the model takes the least number that every part accepts
+    from types import SimpleNamespace
+    from zedinfer_amd.models.model import DecoderModel
+    from zedinfer_amd.parts import Part
+
+    class Tens(Part):
+        def __init__(self):
+            pass
+
+        def step_rows(self, n, kind):
+            return -(-n // 10) * 10
+
+    class Products(Part):
+        def __init__(self):
+            pass
+        step_rows = staticmethod(ProductRows.step_rows)
+    model = SimpleNamespace(_row_parts=[Tens(), Products()], _step_rows={})
+    assert DecoderModel.step_rows(model, 3, "decode") == 80          # the first multiple of 10 among 4, 8, 16, 32, 48, 64, 80
+    assert DecoderModel.step_rows(model, 65, "portion") == 320       # ... and among the multiples of 64
+    assert DecoderModel.step_rows(SimpleNamespace(_row_parts=[], _step_rows={}), 7, "decode") == 7
 
 
 def test_a_recorded_shape_refuses_a_step_that_plans_differently():

@@ -193,7 +193,7 @@ def test_a_large_step_is_brought_up_to_a_measured_size(tmp_path):
     implementation's."""
     from zedinfer_amd.config import SchedulerConfig
     from zedinfer_amd.engine import Engine, StepEntry
-    from zedinfer_amd.engine.engine import many_rows_size_at_least
+    from zedinfer_amd.parts.rows import many_rows as many_rows_size_at_least
     assert [many_rows_size_at_least(n) for n in (4096, 4097, 4288, 8192, 8200)] == [4096, 4224, 4352, 8192, 8448]
     folder = tiny_configs.write_tiny(str(tmp_path / "m"), "A")
     cfg, w = plain.load_folder(folder)
@@ -259,7 +259,7 @@ def test_decode_steps_of_fewer_and_fewer_requests_share_a_shape(tmp_path, dtype)
     pages of a request that ended serve a new one."""
     from zedinfer_amd.config import SchedulerConfig
     from zedinfer_amd.engine import Engine, StepEntry
-    from zedinfer_amd.engine.engine import decode_entries_at_least
+    from zedinfer_amd.parts.rows import few_rows_entries as decode_entries_at_least
     assert [decode_entries_at_least(n) for n in (1, 2, 3, 5, 9, 16, 17, 33, 64, 65, 100, 128, 129, 256)] == \
         [1, 2, 4, 8, 16, 16, 32, 48, 64, 80, 112, 128, 160, 256]
     store = torch.bfloat16 if dtype == "bfloat16" else torch.float32

@@ -7,11 +7,11 @@ each request its own block table per group; all caches of a group share the
 page ids, so one table serves every layer of the group (the reference keeps a
 page list per layer, reference: src/backend/kvcache/block_pool.hpp:73-103).
 Pages go back to the pool when the request ends, or, in a window group, as soon
-as no later token can see them.  A page holds ``page_size`` tokens of one layer:
-keys as [kv_head][slot][head_dim], values transposed as [kv_head][head_dim][slot]
-(reference layout [slot][kv_head][head_dim], block_pool.hpp:16-25; here one head's
-keys are contiguous, and so is a run of positions of one value dimension, which is
-the order the matrix cores read P.V in).
+as no later token can see them.  A page holds ``page_size`` tokens of one layer,
+in the tensors the layer's mixer asked for (``KVCacheRequest.tensors``: names,
+shapes of one page, types): the manager allocates them and hands them over by
+name and knows nothing of what they hold (the reference's page is keys and values
+as [slot][kv_head][head_dim], block_pool.hpp:16-25).
 
 Admission works on promises: ``open`` promises a sequence the pages its prompt
 and a reserve of generated tokens need (reference: prompt + min(max_new, 256),
@@ -40,7 +40,7 @@ class CacheGroup:
     window: int                    # 0 for full
     page_size: int
     pool: PagePool
-    caches: Dict[int, Tuple[int, int]] = field(default_factory=dict)   # cache id -> (kv heads, head_dim)
+    caches: Dict[int, KVCacheRequest] = field(default_factory=dict)    # cache id -> what its layer asked for
 
     def pages_for(self, tokens: int) -> int:
         return (tokens + self.page_size - 1) // self.page_size
@@ -110,20 +110,18 @@ class CacheManager:
                 keys[key] = len(self.groups)
                 self.groups.append(CacheGroup(rq.kind, key[1], self.page_size, PagePool(self.num_pages)))
             g = keys[key]
-            self.groups[g].caches[cid] = (rq.num_kv_heads, rq.head_dim)
+            self.groups[g].caches[cid] = rq
             self.group_of_cache[cid] = g
         self.slots = IdPool(self.max_requests, "state slot")
         self.live: Dict[object, SequenceCache] = {}
-        self.k: Dict[int, torch.Tensor] = {}
-        self.v: Dict[int, torch.Tensor] = {}
+        self.tensors: Dict[int, Dict[str, torch.Tensor]] = {}      # cache id -> name -> [pages, *page shape]
         self.state: Dict[int, torch.Tensor] = {}
         self.state_requests = dict(state_requests)
         if self.device is not None:
             for cid, rq in kv_requests.items():
-                self.k[cid] = torch.zeros((self.num_pages, rq.num_kv_heads, self.page_size, rq.head_dim),
-                                          dtype=dtype, device=self.device)
-                self.v[cid] = torch.zeros((self.num_pages, rq.num_kv_heads, rq.head_dim, self.page_size),
-                                          dtype=dtype, device=self.device)
+                self.tensors[cid] = {name: torch.zeros((self.num_pages,) + pt.page_shape(self.page_size),
+                                                       dtype=pt.dtype or dtype, device=self.device)
+                                     for name, pt in rq.tensors}
             for cid, sr in state_requests.items():
                 self.state[cid] = torch.zeros((self.max_requests,) + tuple(sr.shape), dtype=sr.dtype,
                                               device=self.device)
@@ -131,16 +129,22 @@ class CacheManager:
     # ---- sizes -------------------------------------------------------------------
     @staticmethod
     def bytes_per_page(kv_requests: Dict[int, KVCacheRequest], page_size: int, dtype: torch.dtype) -> int:
-        """Device bytes one page id costs over all caches (keys and values)."""
-        el = torch.empty((), dtype=dtype).element_size()
-        return sum(2 * page_size * r.num_kv_heads * r.head_dim * el for r in kv_requests.values())
+        """Device bytes one page id costs over all caches."""
+        total = 0
+        for r in kv_requests.values():
+            for _, pt in r.tensors:
+                n = 1
+                for s in pt.page_shape(page_size):
+                    n *= s
+                total += n * torch.empty((), dtype=pt.dtype or dtype).element_size()
+        return total
 
     def memories(self, schedule: Sequence[ScheduleStep]) -> List[LayerMemory]:
         out = []
         for st in schedule:
             g = self.group_of_cache.get(st.cache, -1)
-            out.append(LayerMemory(group=g, k=self.k.get(st.cache), v=self.v.get(st.cache),
-                                   writes=st.writes_cache, state=self.state.get(st.cache)))
+            out.append(LayerMemory(group=g, tensors=self.tensors.get(st.cache, {}), writes=st.writes_cache,
+                                   state=self.state.get(st.cache)))
         return out
 
     # ---- admission ---------------------------------------------------------------

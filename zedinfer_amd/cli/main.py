@@ -79,8 +79,7 @@ def _engine(args, step_tokens: Optional[List[int]] = None):
              eng.cache.num_pages, eng.cache.page_size)
     sizes = None
     if step_tokens is not None:
-        from ..engine.engine import many_rows_size_at_least
-        sizes = sorted({many_rows_size_at_least(n) for n in step_tokens if n > Engine.PROMPT_GRAPH_STEP}, reverse=True)
+        sizes = sorted({eng.model.step_rows(n, "mixed") for n in step_tokens if n > 1}, reverse=True)
     ie = InferenceEngine(eng, warm_up_sizes=sizes)
     log.debug("choices made at warm-up: %s", eng.rt.choices)
     return ie

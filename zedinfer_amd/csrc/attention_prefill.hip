@@ -821,6 +821,22 @@ extern "C" int zi_attention_prefill_chunk_keys() { return PF_CHUNK; }
 // 16.6 against 17.6; at the 32B sizes 16,384 tokens 1,036 against 985 ms.
 extern "C" int zi_attention_prefill_chunk_keys_for(int max_keys, int groups) { return zi_pf_chunk_for(max_keys, groups); }
 
+// The smallest tile of queries (every head size takes it).
+extern "C" int zi_attention_prefill_tile_min() { return PF_BM; }
+
+// How a launch of `groups` tiles x heads is cut when no query sees more than `max_keys` keys (position + 1) and
+// a query sees `window` keys at most (0: all): the keys between cuts go to *chunk_keys, the cuts a tile can
+// have are returned; both go to zi_attention_prefill, and the cuts size its workspace.  A windowed tile's keys
+// span at most the window, the widest tile and a block, from anywhere in a cut.
+extern "C" int zi_attention_prefill_cuts(int max_keys, int window, int groups, int* chunk_keys) {
+    if (max_keys < 1) max_keys = 1;
+    if (window > 0 && max_keys > window + 2 * PF_BM + PF_BS) max_keys = window + 2 * PF_BM + PF_BS;
+    const int chunk = zi_pf_chunk_for(max_keys, groups);
+    if (window > 0) max_keys += chunk - 1;
+    if (chunk_keys) *chunk_keys = chunk;
+    return (max_keys + chunk - 1) / chunk;
+}
+
 // Tile i covers the queries [tile_off[i], tile_off[i] + tile) of entry tile_entry[i] (fewer at the
 // entry's end; `tile` is 64, or 128 for head sizes 64 and 128); entry e brings entry_len[e] tokens that start at row entry_start[e] of q and at
 // position entry_past[e] of its sequence, whose block table is row e of block_tables.  `alone` (head sizes 64 and

@@ -5,7 +5,9 @@
 //   angle = float(pos) * inv_freq[k]          (float32; inv_freq[k] = theta^(-2k/R), made on the host)
 //   out[k]       = a cos(angle) - b sin(angle)
 //   out[k + R/2] = b cos(angle) + a sin(angle)     with a = in[k], b = in[k + R/2]
-// (reference: src/backend/ops/rope/cpu/rope_cpu.cpp:33,47-52,62-65).  Queries are
+// (reference: src/backend/ops/rope/cpu/rope_cpu.cpp:33,47-52,62-65).  The kernels that store take the step's
+// (cos, sin) of every (token, k) as a table [n][R/2][2] (zi_rope_table makes it once per step, every layer
+// reads it): whoever encodes positions decides the angles, the store only turns by them.  Queries are
 // rotated in place; keys are rotated on their way into the cache, values copied
 // (reference: K is stored after rotation, V raw, src/frontend/models/transformer_forward.cpp:99-104).
 //
@@ -20,19 +22,17 @@
 
 template <typename T>
 __global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
-                                     int64_t ldq, int64_t ldk, int64_t ldv, const int32_t* __restrict__ pos,
-                                     const int32_t* __restrict__ slots, const float* __restrict__ inv_freq,
-                                     T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int d,
-                                     int rot, int page_size, int write_kv, int64_t cache_slots) {
+                                     int64_t ldq, int64_t ldk, int64_t ldv, const int32_t* __restrict__ slots,
+                                     const float2* __restrict__ table, T* __restrict__ kcache,
+                                     T* __restrict__ vcache, int nh, int nkv, int d, int rot, int page_size,
+                                     int write_kv, int64_t cache_slots) {
     extern __shared__ float cs[];  // cos[rot/2], sin[rot/2]
     const int64_t t = blockIdx.x;
     const int half = rot / 2;
-    const float p = (float)pos[t];
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
-        float s, c;
-        sincosf(p * inv_freq[i], &s, &c);
-        cs[i] = c;
-        cs[half + i] = s;
+        const float2 e = table[t * half + i];
+        cs[i] = e.x;
+        cs[half + i] = e.y;
     }
     __syncthreads();
     // queries, in place
@@ -78,9 +78,8 @@ __global__ void rope_kv_store_kernel(T* __restrict__ q, const T* __restrict__ k,
 #define RKT_TOKENS 8
 __global__ void __launch_bounds__(256)
 rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k, const zi_bf16* __restrict__ v,
-                          int64_t ldq, int64_t ldk, int64_t ldv, const int32_t* __restrict__ pos,
-                          const int32_t* __restrict__ slots, const float* __restrict__ inv_freq,
-                          zi_bf16* __restrict__ kcache, zi_bf16* __restrict__ vcache, int n, int nh, int nkv, int d,
+                          int64_t ldq, int64_t ldk, int64_t ldv, const int32_t* __restrict__ slots,
+                          const float2* __restrict__ table, zi_bf16* __restrict__ kcache, zi_bf16* __restrict__ vcache, int n, int nh, int nkv, int d,
                           int rot, int page_size, int write_kv, int64_t cache_slots) {
     extern __shared__ __attribute__((aligned(16))) unsigned char rkt_lds[];
     const int half = rot / 2, kvd = nkv * d;
@@ -90,10 +89,9 @@ rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k
     const int nt = (n - t0 < RKT_TOKENS) ? n - t0 : RKT_TOKENS;
     for (int i = tid; i < nt * half; i += 256) {
         const int tt = i / half, jj = i % half;
-        float sn, c;
-        sincosf((float)pos[t0 + tt] * inv_freq[jj], &sn, &c);
-        cs[tt * rot + jj] = c;
-        cs[tt * rot + half + jj] = sn;
+        const float2 e = table[(int64_t)(t0 + tt) * half + jj];
+        cs[tt * rot + jj] = e.x;
+        cs[tt * rot + half + jj] = e.y;
     }
     if (write_kv)
         for (int i = tid; i < nt * (kvd / 8); i += 256) {
@@ -192,7 +190,7 @@ rope_kv_store_tile_kernel(zi_bf16* __restrict__ q, const zi_bf16* __restrict__ k
 #define ROPE_MANY_TOKENS 1024
 
 extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, int n, int64_t ldq, int64_t ldk,
-                                int64_t ldv, const int32_t* pos, const int32_t* slots, const float* inv_freq,
+                                int64_t ldv, const int32_t* slots, const float* table,
                                 void* kcache, void* vcache, int64_t cache_slots, int nh, int nkv, int d, int rot,
                                 int page_size, int write_kv, hipStream_t stream) {
     ZI_REQUIRE(n >= 0 && nh > 0 && nkv >= 0 && d > 0, "rope_kv_store: bad sizes");
@@ -205,23 +203,25 @@ extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, i
         ZI_REQUIRE(k && v && kcache && vcache && slots, "rope_kv_store: null cache or key/value pointer");
     }
     ZI_REQUIRE(rot * sizeof(float) <= 48 * 1024, "rope_kv_store: rotary dims %d too large", rot);
+    ZI_REQUIRE(rot == 0 || (table && ((uintptr_t)table % 8) == 0), "rope_kv_store: no table of angles");
     if (n == 0) return 0;
+    const float2* tb = reinterpret_cast<const float2*>(table);
     {
         // the tile kernel: bfloat16, rows and pointers that allow 16-byte pieces, eight rotated dims on one side
         const bool al = ((uintptr_t)q % 16) == 0 && ldq % 8 == 0 && d % 8 == 0 && (rot / 2) % 8 == 0 &&
                         (!write_kv || (((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0 && ((uintptr_t)kcache % 16) == 0 &&
                                        ((uintptr_t)vcache % 16) == 0 && ldk % 8 == 0 && ldv % 8 == 0 && page_size % 8 == 0));
         const size_t lds = (size_t)RKT_TOKENS * rot * sizeof(float) + (write_kv ? (size_t)RKT_TOKENS * nkv * d * 2 : 0);
-        if (dt == ZI_BF16 && n >= ROPE_MANY_TOKENS && al && lds <= 48 * 1024 && (rot == 0 || inv_freq)) {
+        if (dt == ZI_BF16 && n >= ROPE_MANY_TOKENS && al && lds <= 48 * 1024) {
             rope_kv_store_tile_kernel<<<(n + RKT_TOKENS - 1) / RKT_TOKENS, 256, lds, stream>>>(
-                (zi_bf16*)q, (const zi_bf16*)k, (const zi_bf16*)v, ldq, ldk, ldv, pos, slots, inv_freq, (zi_bf16*)kcache,
+                (zi_bf16*)q, (const zi_bf16*)k, (const zi_bf16*)v, ldq, ldk, ldv, slots, tb, (zi_bf16*)kcache,
                 (zi_bf16*)vcache, n, nh, nkv, d, rot, page_size, write_kv, cache_slots);
             return zi_check_launch("rope_kv_store");
         }
     }
     ZI_DISPATCH_DTYPE(dt, T, {
         rope_kv_store_kernel<T><<<n, 256, rot * sizeof(float), stream>>>(
-            (T*)q, (const T*)k, (const T*)v, ldq, ldk, ldv, pos, slots, inv_freq, (T*)kcache, (T*)vcache, nh, nkv, d,
+            (T*)q, (const T*)k, (const T*)v, ldq, ldk, ldv, slots, tb, (T*)kcache, (T*)vcache, nh, nkv, d,
             rot, page_size, write_kv, cache_slots);
     });
     return zi_check_launch("rope_kv_store");
@@ -232,16 +232,16 @@ extern "C" int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, i
 // part + s * split_stride + t * ldp.  The splits are added in rising order, the bias is added, and
 // the row is rotated from float32: q goes to q_out (rounded once), k and v into the cache.
 // One wavefront per (token, head): blockIdx.y < nh is a query head, the others are key heads, which
-// bring their value head along.  A lane owns the pairs (j, j + rot/2) it rotates and computes their
-// angle itself, so nothing is shared and nothing waits at a barrier.  SP is the number of splits
+// bring their value head along.  A lane owns the pairs (j, j + rot/2) it rotates and reads their
+// (cos, sin) itself, so nothing is shared and nothing waits at a barrier.  SP is the number of splits
 // rounded up to a power of two: that many loads are issued at once per value.
 template <typename T, typename TB, int SP>
 __global__ void __launch_bounds__(ZI_WAVE)
 rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __restrict__ part, int splits,
                            int64_t split_stride, int64_t ldp, const TB* __restrict__ bias,
-                           const int32_t* __restrict__ pos, const int32_t* __restrict__ slots,
-                           const float* __restrict__ inv_freq, T* __restrict__ kcache, T* __restrict__ vcache, int nh,
-                           int nkv, int d, int rot, int page_size, int64_t cache_slots) {
+                           const int32_t* __restrict__ slots, const float2* __restrict__ table,
+                           T* __restrict__ kcache, T* __restrict__ vcache, int nh, int nkv, int d, int rot,
+                           int page_size, int64_t cache_slots) {
     const int64_t t = blockIdx.x;
     const int hs = blockIdx.y, lane = threadIdx.x;
     const int half = rot / 2;
@@ -249,7 +249,6 @@ rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __re
     const bool is_q = hs < nh;
     const int g = hs - nh;
     const int col0 = is_q ? hs * d : qd + g * d;
-    const float p = (float)pos[t];
     const float* pr = part + t * ldp;
     auto value = [&](int col) {
         float v[SP];
@@ -275,10 +274,9 @@ rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __re
     }
     for (int j = lane; j < half; j += ZI_WAVE) {
         const float a = value(col0 + j), b = value(col0 + j + half);
-        float sn, cs;
-        sincosf(p * inv_freq[j], &sn, &cs);
-        zi_store(dst + j, a * cs - b * sn);
-        zi_store(dst + j + half, b * cs + a * sn);
+        const float2 e = table[t * half + j];
+        zi_store(dst + j, a * e.x - b * e.y);
+        zi_store(dst + j + half, b * e.x + a * e.y);
     }
     for (int j = rot + lane; j < d; j += ZI_WAVE) zi_store(dst + j, value(col0 + j));
     if (store_v)
@@ -287,7 +285,7 @@ rope_kv_store_split_kernel(T* __restrict__ q_out, int64_t ldq, const float* __re
 
 extern "C" int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const float* part, int splits,
                                       int64_t split_stride, int64_t ldp, const void* bias, int bias_dt, int n,
-                                      const int32_t* pos, const int32_t* slots, const float* inv_freq, void* kcache,
+                                      const int32_t* slots, const float* table, void* kcache,
                                       void* vcache, int64_t cache_slots, int nh, int nkv, int d, int rot,
                                       int page_size, int write_kv, hipStream_t stream) {
     ZI_REQUIRE(n >= 0 && nh > 0 && nkv >= 0 && d > 0, "rope_kv_store_split: bad sizes");
@@ -297,7 +295,7 @@ extern "C" int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const fl
     ZI_REQUIRE(ldq >= (int64_t)nh * d && ldp >= width, "rope_kv_store_split: row stride too small");
     ZI_REQUIRE(splits >= 1 && (splits == 1 || split_stride >= (int64_t)n * ldp),
                "rope_kv_store_split: bad partial sums (splits %d, stride %lld)", splits, (long long)split_stride);
-    ZI_REQUIRE(rot == 0 || inv_freq, "rope_kv_store_split: no frequency table");
+    ZI_REQUIRE(rot == 0 || (table && ((uintptr_t)table % 8) == 0), "rope_kv_store_split: no table of angles");
     if (write_kv) {
         ZI_REQUIRE(page_size > 0 && cache_slots > 0 && cache_slots % page_size == 0,
                    "rope_kv_store_split: cache of %lld slots is not a whole number of pages of %d", (long long)cache_slots,
@@ -311,7 +309,8 @@ extern "C" int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const fl
     const dim3 grid(n, nh + (write_kv ? nkv : 0));
 #define ZI_RKS(SP)                                                                                                  \
     rope_kv_store_split_kernel<T, TB, SP><<<grid, ZI_WAVE, 0, stream>>>(                                            \
-        (T*)q_out, ldq, part, splits, split_stride, ldp, (const TB*)bias, pos, slots, inv_freq, (T*)kcache, (T*)vcache, \
+        (T*)q_out, ldq, part, splits, split_stride, ldp, (const TB*)bias, slots, reinterpret_cast<const float2*>(table), \
+        (T*)kcache, (T*)vcache, \
         nh, nkv, d, rot, page_size, cache_slots)
     ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(bias_dt, TB, {
         if (splits <= 1) ZI_RKS(1);

@@ -76,13 +76,12 @@ int zi_add_rmsnorm(void* out, int out_dt, float* resid, const void* delta, int d
     split_stride, const void* w, int w_dt, int n, int hidden, float eps, int add_one, hipStream_t stream);
 // rope_kv.hip
 int zi_rope_kv_store(void* q, const void* k, const void* v, int dt, int n, int64_t ldq, int64_t ldk, int64_t ldv,
-    const int32_t* pos, const int32_t* slots, const float* inv_freq, void* kcache, void* vcache, int64_t cache_slots,
-    int nh, int nkv, int d, int rot, int page_size, int write_kv, hipStream_t stream);
+    const int32_t* slots, const float* table, void* kcache, void* vcache, int64_t cache_slots, int nh, int nkv, int d,
+    int rot, int page_size, int write_kv, hipStream_t stream);
 // rope_kv.hip
 int zi_rope_kv_store_split(void* q_out, int dt, int64_t ldq, const float* part, int splits, int64_t split_stride,
-    int64_t ldp, const void* bias, int bias_dt, int n, const int32_t* pos, const int32_t* slots, const float*
-    inv_freq, void* kcache, void* vcache, int64_t cache_slots, int nh, int nkv, int d, int rot, int page_size, int
-    write_kv, hipStream_t stream);
+    int64_t ldp, const void* bias, int bias_dt, int n, const int32_t* slots, const float* table, void* kcache, void*
+    vcache, int64_t cache_slots, int nh, int nkv, int d, int rot, int page_size, int write_kv, hipStream_t stream);
 // rope_kv.hip
 int zi_rope(void* out, const void* in, int dt, int n, int64_t ld_in, int64_t ld_out, const int32_t* pos, const float*
     inv_freq, int nh, int d, int rot, hipStream_t stream);

@@ -86,13 +86,13 @@ FIXED_PIECES = 8      # token ids, positions, tok_seq, logit rows, entry start /
 def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_size: int,
                        device: torch.device, staging: Optional[StagingRing] = None,
                        table_widths: Optional[Sequence[int]] = None,
-                       static: Optional[torch.Tensor] = None, pad_to: int = 0, pad_entries: int = 0,
+                       static: Optional[torch.Tensor] = None, pad_to=None, pad_entries: int = 0,
                        pad_rows: int = 0, pad_more: int = 0, planners: Sequence[StepPlanner] = (), position_axes: int = 1,
                        bound_single: int = 0, bound_multi: int = 0) -> DeviceBatch:
     """Check the entries, then pack every index array into one host buffer and copy it over once.
 
-    ``pad_to``: every entry that brings more than one token is run as if it brought a multiple of that
-    many.  The tokens past its own are token 0 at the positions that follow; they have no place in the cache
+    ``pad_to``: a function of a number of tokens; every entry that brings more than one token is run as if it
+    brought ``pad_to(tokens)``.  The tokens past its own are token 0 at the positions that follow; they have no place in the cache
     (slot -1: nothing is stored for them) and no real token sees them, so they change nothing but the
     shapes, which then recur from step to step.  ``pad_more``: that many more such tokens behind the longest
     entry's.  ``pad_entries`` adds that many entries of one token that
@@ -132,7 +132,9 @@ def build_device_batch(entries: Sequence[StepEntry], cache: CacheManager, vocab_
     lens = lens + [1] * int(pad_entries)
     real = list(lens)
     if pad_to:
-        lens = [-(-n // int(pad_to)) * int(pad_to) if n > 1 else n for n in lens]
+        lens = [int(pad_to(n)) if n > 1 else n for n in lens]
+        if any(a < b for a, b in zip(lens, real)):
+            raise ValueError("padding cannot take tokens away")
     if pad_more:
         longest = max(range(len(lens)), key=lambda i: lens[i])
         if lens[longest] <= 1:

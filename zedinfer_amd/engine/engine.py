@@ -10,7 +10,7 @@ block tables before the run and commits the new lengths after it.
 from __future__ import annotations
 
 import os
-from typing import Dict, List, Optional, Sequence
+from typing import Dict, Optional, Sequence
 
 import torch
 
@@ -83,7 +83,7 @@ class Engine:
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.graph_replays = 0
         # A step that is one portion of one prompt, alone or beside single decoded tokens, has the portion
-        # padded to the next multiple of PROMPT_GRAPH_STEP tokens and is captured too (launching a step
+        # padded to a number of tokens that the model's parts choose (``step_rows``) and is captured too (launching a step
         # kernel by kernel costs the host about 5 ms, more than the GPU needs for a short prompt), one graph
         # per (entries, padded tokens, wanted rows, table widths, attention launch sizes).  Portions of
         # more tokens are bound by the GPU and run as they are.
@@ -232,7 +232,7 @@ class Engine:
         if self.padding_safe and (self.use_graphs or self.use_tapes):
             # the number of requests moves (they end one by one): entries that belong to no request bring it to
             # one of few numbers, a row wanted of each, so that the kinds of steps are few
-            more_entries = decode_entries_at_least(E) - E
+            more_entries = self.model.step_rows(E, "decode") - E
             E += more_entries
             # (an entry may name its one token several times: more rows than entries are left as they are)
             R = E if 0 < wanted <= E else wanted
@@ -327,8 +327,11 @@ class Engine:
         if dg.graph is not None:
             torch.cuda.synchronize(self.device)
 
-    # ---- one portion of one prompt as a graph -------------------------------------------
-    PROMPT_GRAPH_STEP = 64
+    # ---- portions of prompts as graphs and tapes -------------------------------------------
+    def portion_rows(self, tokens: int) -> int:
+        """The tokens a portion of ``tokens`` tokens is run with when the step is padded (the parts' choice)."""
+        return self.model.step_rows(tokens, "portion")
+
     # padded tokens of the portions of a step that is still padded and run from a tape (a step of many tokens does
     # not need the tape, the GPU takes far longer than the host, but its padded rows are a size whose library
     # products can have been measured)
@@ -346,44 +349,42 @@ class Engine:
             if len(e.want) > 1 or e.positions is not None:
                 return False
             if n > 1:
-                total += -(-n // self.PROMPT_GRAPH_STEP) * self.PROMPT_GRAPH_STEP
+                total += self.portion_rows(n)
                 real += n
         most = max(self.prompt_graph_max_tokens if self.use_graphs else 0, self.TAPE_MAX_TOKENS if self.use_tapes else 0)
         # many very short portions would be padded to many times their tokens: such a step runs as it is
-        return 0 < total <= most and total <= 4 * real + self.PROMPT_GRAPH_STEP and len(entries) <= self.graph_max_entries
+        return 0 < total <= most and total <= 4 * real + self.portion_rows(2) and len(entries) <= self.graph_max_entries
 
     def _prompt_graph_step(self, entries: Sequence[StepEntry], token_source: Optional[torch.Tensor] = None
                            ) -> Optional[torch.Tensor]:
         """A step of portions of prompts (entries of several tokens) beside single decoded tokens,
-        with every portion run as if it brought a multiple of PROMPT_GRAPH_STEP tokens (see
+        with every portion run as if it brought the number of tokens the model's parts round it up to (see
         ``build_device_batch``): the first step of a kind runs eagerly, the second is captured, later
         ones replay."""
-        step = self.PROMPT_GRAPH_STEP
         portions = [e for e in entries if len(e.tokens) > 1]
-        sizes = tuple(sorted(-(-len(e.tokens) // step) * step for e in portions))     # tokens of the portions, padded
+        sizes = tuple(sorted(self.portion_rows(len(e.tokens)) for e in portions))     # tokens of the portions, padded
         padded = sum(sizes)
         wanted = sum(len(e.want) for e in entries)
         E, R, more_entries = len(entries), wanted, 0
         if E > 1:
             # the numbers of portions and of decoding requests move from step to step: the decoding entries are
-            # brought to a multiple of PROMPT_GRAPH_STEP with entries that belong to no request, and a row is
-            # wanted of every entry.  The step's rows are then a multiple of that step as well: fewer shapes, and
-            # the many-rows products come in the numbers of rows that a warm-up has measured
-            # (``many_rows_step_sizes``).
+            # brought to a number the parts choose with entries that belong to no request, and a row is wanted of
+            # every entry: fewer shapes, and the step's rows are among the numbers that a warm-up has measured
+            # the parts' choices for (``InferenceEngine.default_warm_up_sizes``).
             decoding = E - len(portions)
-            more_entries = -(-decoding // step) * step - decoding
+            more_entries = self.model.step_rows(decoding, "beside") - decoding if decoding else 0
             E += more_entries
             R = E
-        # beyond 4,096 rows the measured sizes lie further apart: the step is brought up to the next one with
-        # more padding behind its longest portion (at most a 32nd more rows)
+        # the parts may want the whole step's rows rounded up further (measured sizes lie further apart for large
+        # steps): more padding behind the longest portion
         rows = padded + (E - len(portions))
-        more_tokens = many_rows_size_at_least(rows) - rows
+        more_tokens = self.model.step_rows(rows, "mixed") - rows
         if more_tokens:
             sizes = tuple(sorted(sizes[:-1] + (sizes[-1] + more_tokens,)))
             padded += more_tokens
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
-        long_bucket = _pow2_at_least(max(e.seq.length + -(-len(e.tokens) // step) * step for e in portions) + more_tokens, 2048)
+        long_bucket = _pow2_at_least(max(e.seq.length + self.portion_rows(len(e.tokens)) for e in portions) + more_tokens, 2048)
         # (a power of two here: beside portions of prompts the decoding requests' attention is a small part of the
         # step, and every further value of the bound is a further kind of step)
         short_bucket = _pow2_at_least(max([e.seq.length + 1 for e in entries if len(e.tokens) == 1], default=0), 256)
@@ -401,7 +402,7 @@ class Engine:
                 self._drop_oldest(self._prompt_graphs)
             dg = self._prompt_graphs[key] = _DecodeGraph()
         batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging, widths, dg.buffer,
-                                   pad_to=step, pad_more=more_tokens, pad_entries=more_entries, pad_rows=R - wanted,
+                                   pad_to=self.portion_rows, pad_more=more_tokens, pad_entries=more_entries, pad_rows=R - wanted,
                                    planners=self.planners, position_axes=self.position_axes,
                                    bound_single=short_bucket if singles else 0, bound_multi=long_bucket)
         dg.buffer = batch.device_image          # the first step's buffer serves all later ones of the shape
@@ -439,46 +440,6 @@ class _DecodeGraph:
         self.no_tape = False                            # a step of the shape cannot be recorded
         self.planned = None                             # the sizes the planners gave the shape's first step
         self.image: Optional[DecodeImage] = None
-
-
-def _many_rows_spacing(rows: int, step: int) -> int:
-    top, s = 64 * step, step
-    while rows > top:
-        top, s = 2 * top, 2 * s
-    return s
-
-
-def many_rows_size_at_least(rows: int, step: int = Engine.PROMPT_GRAPH_STEP) -> int:
-    """The number of rows a step of ``rows`` rows is run with: the next multiple of ``step`` up to 4,096 rows, of
-    2 x ``step`` up to 8,192, of 4 x ``step`` up to 16,384 and so on (32 sizes an octave: measuring every size
-    when an engine is made stays affordable, and a step gets at most a 32nd more rows)."""
-    rows = max(int(rows), 1)
-    s = _many_rows_spacing(rows, step)
-    return -(-rows // s) * s
-
-
-def many_rows_step_sizes(most_tokens: int, step: int = Engine.PROMPT_GRAPH_STEP, least: int = 128) -> List[int]:
-    """The numbers of rows that steps with portions of prompts come in, up to ``most_tokens`` tokens a step:
-    portions are run as multiples of ``step`` tokens, decoding entries beside them in multiples of ``step``, and
-    large steps are brought up to sizes further apart (``Engine._prompt_graph_step``,
-    ``many_rows_size_at_least``).  From ``least`` rows on: fewer go to the few-rows kernels or are not worth
-    measuring.  Largest first: workspaces get their final sizes at once."""
-    sizes, n = [], many_rows_size_at_least(most_tokens, step)
-    while n >= least:
-        sizes.append(n)
-        s = _many_rows_spacing(n - 1, step)
-        n = (n - 1) // s * s
-    return sizes
-
-
-def decode_entries_at_least(entries: int) -> int:
-    """The number of entries a step of ``entries`` decoding requests is run with: a power of two up to 16 (one
-    tile of rows of the few-rows kernels), then a multiple of 16 up to 128 (what those kernels take) and of 32
-    beyond."""
-    if entries <= 16:
-        return _pow2_at_least(entries)
-    step = 16 if entries <= 128 else 32
-    return -(-entries // step) * step
 
 
 def _bucket_at_least(n: int, floor: int = 1) -> int:

@@ -17,7 +17,8 @@ import torch
 from ..config import SchedulerConfig
 from ..ops.staging import StagingRing
 from ..sampling.sampler import Sampler
-from .engine import Engine, decode_entries_at_least, many_rows_size_at_least, many_rows_step_sizes
+from ..parts.rows import sizes_between
+from .engine import Engine
 from .request import GenerationConfig, GenerationResult, InferenceRequest
 from .scheduler import ScheduledBatch, Scheduler
 
@@ -163,19 +164,20 @@ class InferenceEngine:
     WARM_UP_EVERY_SIZE_UP_TO = 8192     # rows; measuring every size of longer steps would take minutes
 
     @classmethod
-    def default_warm_up_sizes(cls, sched: SchedulerConfig, most_entries: int = 256) -> List[int]:
-        """The numbers of rows that the steps of an engine with these limits come in, largest first: every size
-        a step with portions of prompts can bring (``many_rows_step_sizes``) up to WARM_UP_EVERY_SIZE_UP_TO rows, of
-        longer steps the two that recur (a full portion alone and beside decoding requests), and the sizes of pure
-        decode steps of more requests than the few-rows kernels take (``decode_entries_at_least``)."""
-        step = Engine.PROMPT_GRAPH_STEP
-        # a portion and the decoding entries beside it are rounded up: one more size
+    def default_warm_up_sizes(cls, sched: SchedulerConfig, step_rows, most_entries: int = 256) -> List[int]:
+        """The numbers of rows that the padded steps of an engine with these limits come in, largest first.
+        ``step_rows(rows, kind)`` is the model's (``DecoderModel.step_rows``: the parts say which numbers of rows
+        steps are run with).  Every size a step with portions of prompts can bring up to WARM_UP_EVERY_SIZE_UP_TO
+        rows, of longer steps the two that recur (a full portion alone and beside decoding requests), and the
+        sizes of pure decode steps.  What, if anything, is measured at a size is each part's business
+        (``Part.tune``)."""
+        beside = step_rows(1, "beside")         # decoding entries beside a portion are rounded up: one more size
         most = min(sched.max_batch_tokens, sched.max_prefill_tokens + sched.max_batch_requests)
-        sizes = many_rows_step_sizes(min(most, cls.WARM_UP_EVERY_SIZE_UP_TO) + step)
+        sizes = sizes_between(step_rows, "mixed", step_rows(2, "portion"), min(most, cls.WARM_UP_EVERY_SIZE_UP_TO) + beside)
         if most > cls.WARM_UP_EVERY_SIZE_UP_TO:
-            sizes += [many_rows_size_at_least(sched.max_prefill_tokens),
-                      many_rows_size_at_least(min(most, sched.max_prefill_tokens + step) + step)]
-        sizes += [decode_entries_at_least(e) for e in range(65, min(sched.max_batch_requests, most_entries) + 1)]
+            sizes += [step_rows(sched.max_prefill_tokens, "mixed"),
+                      step_rows(min(most, sched.max_prefill_tokens + beside) + beside, "mixed")]
+        sizes += sizes_between(step_rows, "decode", 1, min(sched.max_batch_requests, most_entries))
         return sorted(set(sizes), reverse=True)
 
     def __init__(self, engine: Engine, warm_up_sizes: Optional[Sequence[int]] = None):
@@ -186,14 +188,13 @@ class InferenceEngine:
         # The products' algorithms (and other choices of the parts) for steps of many rows are measured now, once
         # (ZEDINFER_WARM_UP=0: the defaults), at every number of rows that steps with portions of prompts come
         # in: the library's first proposal for a shape can be a third slower than what timing finds, and what
-        # timing finds for one number of rows does not carry over to its neighbours (measured; see
-        # ``many_rows_step_sizes``).
+        # timing finds for one number of rows does not carry over to its neighbours (measured).
         # (the reference's own switch for its warm-up is honoured too: ZEDINFER_DISABLE_WARMUP set,
         # src/zedinfer/engine.cpp:506)
         if (os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and "ZEDINFER_DISABLE_WARMUP" not in os.environ
                 and engine.device.type == "cuda"):
             if warm_up_sizes is None:
-                warm_up_sizes = self.default_warm_up_sizes(engine.sched, engine.graph_max_entries)
+                warm_up_sizes = self.default_warm_up_sizes(engine.sched, engine.model.step_rows, engine.graph_max_entries)
             engine.warm_up(list(warm_up_sizes))
         # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
         # taken out of the garbage collector's passes, a full collection in the middle of serving costs

@@ -82,6 +82,9 @@ class DecoderModel:
         self.parts += [self.embedding, self.final_norm, self.lm_head]
         self.vocab_size = fc.vocab_size
         self.hidden_size = fc.hidden_size
+        # the parts that have a say in the numbers of rows steps are padded to
+        self._row_parts = [p for p in self.parts if getattr(type(p), "step_rows", Part.step_rows) is not Part.step_rows]
+        self._step_rows: Dict[tuple, int] = {}
 
     # ---- what the cache manager has to provide ------------------------------
     def cache_requests(self) -> Dict[int, KVCacheRequest]:
@@ -91,8 +94,8 @@ class DecoderModel:
             req = self.blocks[st.layer].mixer.cache_request()
             if req is None:
                 continue
-            if st.cache in out and (out[st.cache].num_kv_heads, out[st.cache].head_dim) != (req.num_kv_heads, req.head_dim):
-                raise ValueError(f"cache {st.cache} is shared by layers with different key/value shapes")
+            if st.cache in out and out[st.cache].tensors != req.tensors:
+                raise ValueError(f"cache {st.cache} is shared by layers that keep different tensors in a page")
             if st.writes_cache or st.cache not in out:
                 out[st.cache] = req
         return out
@@ -113,6 +116,25 @@ class DecoderModel:
             if pl is not None and pl.key not in out:
                 out[pl.key] = pl
         return tuple(out.values())
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        """The number of rows (``Part.step_rows`` says of what, by ``kind``) a step of ``rows`` is run with when it
+        is padded: the least number from ``rows`` on that every part accepts."""
+        key = (int(rows), kind)
+        found = self._step_rows.get(key)
+        if found is None:
+            r = max(int(rows), 1)
+            for _ in range(64):
+                nxt = max(int(p.step_rows(r, kind)) for p in self._row_parts) if self._row_parts else r
+                if nxt < r:
+                    raise ValueError(f"a part wants a step of {r} rows run with fewer ({nxt})")
+                if nxt == r:
+                    break
+                r = nxt
+            else:
+                raise ValueError(f"the parts do not agree on a number of rows for a step of {rows} ({kind})")
+            found = self._step_rows[key] = r
+        return found
 
     def position_axes(self) -> int:
         """The axes the step's positions need: the most any position encoding of the model reads."""

@@ -10,9 +10,9 @@ from .functional import (add, add_rms_norm, argmax, attention, attention_decode,
                          attention_decode_fused_supported, attention_decode_project,
                          attention_decode_project_splits, attention_decode_project_supported,
                          attention_decode_supported, attention_decode_workspace, attention_prefill,
-                         attention_prefill_supported, attention_prefill_tile, attention_prefill_variant,
+                         attention_prefill_supported, attention_prefill_tile, attention_prefill_tile_min, attention_prefill_variant,
                          attention_prefill_workspace, decode_layer, decode_layer_stamps, decode_layer_supported, decode_layer_sync_words,
-                         decode_layer_workspace, device_synchronize, embedding, gather_rows,
+                         decode_layer_workspace, device_synchronize, embedding, gather_rows, kv_store,
                          has_cuda, has_gpu, linear, linear_choose, linear_splits, linear_sums,
                          linear_sums_supported, linear_swiglu, linear_swiglu_supported,
                          linear_transposed, linear_tune, reduce_sums, rms_norm, rope, rope_inv_freq,
@@ -25,9 +25,9 @@ __all__ = [
     "add", "add_rms_norm", "argmax", "attention", "attention_decode", "attention_decode_chunks", "attention_decode_fused",
     "attention_decode_fused_supported", "attention_decode_project", "attention_decode_project_splits",
     "attention_decode_project_supported", "attention_decode_supported", "attention_decode_workspace",
-    "attention_prefill", "attention_prefill_supported", "attention_prefill_tile", "attention_prefill_variant",
+    "attention_prefill", "attention_prefill_supported", "attention_prefill_tile", "attention_prefill_tile_min", "attention_prefill_variant",
     "attention_prefill_workspace", "decode_layer", "decode_layer_stamps", "decode_layer_supported", "decode_layer_sync_words",
-    "decode_layer_workspace", "device_synchronize", "embedding", "gather_rows", "has_cuda", "has_gpu",
+    "decode_layer_workspace", "device_synchronize", "embedding", "gather_rows", "has_cuda", "kv_store", "has_gpu",
     "linear", "linear_choose", "linear_splits", "linear_sums", "linear_sums_supported", "linear_swiglu",
     "linear_swiglu_supported", "linear_transposed", "linear_tune", "reduce_sums", "rms_norm", "rope",
     "rope_inv_freq", "rope_kv_store", "rope_kv_store_sums", "rope_table", "sample", "swiglu", "swiglu_t",

@@ -25,7 +25,7 @@ _PROTOTYPES = {
     "zi_swiglu_t": [P, P, I, I, I, L, P],
     "zi_rmsnorm": [P, I, P, I, P, I, I, I, L, L, F, I, P],
     "zi_add_rmsnorm": [P, I, P, P, I, I, L, P, I, I, I, F, I, P],
-    "zi_rope_kv_store": [P, P, P, I, I, L, L, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
+    "zi_rope_kv_store": [P, P, P, I, I, L, L, L, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_rope": [P, P, I, I, L, L, P, P, I, I, I, P],
     "zi_attention_generic": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P],
     "zi_attention_decode": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P],
@@ -45,6 +45,8 @@ _PROTOTYPES = {
     "zi_attention_decode_chunks": [I],
     "zi_attention_prefill": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, I, I, P],
     "zi_attention_prefill_chunk_keys_for": [I, I],
+    "zi_attention_prefill_cuts": [I, I, I, P],
+    "zi_attention_prefill_tile_min": [],
     "zi_attention_prefill_chunks": [I],
     "zi_attention_prefill_variant": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],
@@ -57,7 +59,7 @@ _PROTOTYPES = {
     "zi_gemm_lt_tune": [P, I, P, P, P, I, L, L, L, L, L, L, P, L, I, I, P, P, P, P],
     "zi_gemm_lt_choose": [I, I, I, L, L, L, L, L, L, L, I],
     "zi_reduce_splits": [P, I, P, P, I, I, L, I, P],
-    "zi_rope_kv_store_split": [P, I, L, P, I, L, L, P, I, I, P, P, P, P, P, L, I, I, I, I, I, I, P],
+    "zi_rope_kv_store_split": [P, I, L, P, I, L, L, P, I, I, P, P, P, P, L, I, I, I, I, I, I, P],
     "zi_gemm_skinny_supported": [I, I, I, L, L],
     "zi_argmax": [P, P, P, I, I, I, L, P, L, P],
     "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],
@@ -102,6 +104,8 @@ def load() -> ctypes.CDLL:
             fn.restype = c_int
         lib.zi_gemm_skinny_workspace.argtypes = [I, I, I]
         lib.zi_gemm_skinny_workspace.restype = c_int64
+        lib.zi_attention_decode_workspace.argtypes = [I, I, I]
+        lib.zi_attention_decode_workspace.restype = c_int64
         lib.zi_attention_prefill_workspace.argtypes = [I, I, I, I]
         lib.zi_attention_prefill_workspace.restype = c_int64
         lib.zi_decode_layer_workspace.argtypes = [I, I, I, I, I, I, I, I]

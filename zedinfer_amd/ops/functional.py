@@ -266,18 +266,27 @@ def _check_cache(kcache: torch.Tensor, vcache: torch.Tensor, nkv: int, d: int, d
     return pages, ps
 
 
-def rope_kv_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], pos: torch.Tensor,
-                  slots: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor], kcache: Optional[torch.Tensor],
-                  vcache: Optional[torch.Tensor], nh: int, nkv: int, d: int) -> None:
-    """Rotate q [n, nh*d] in place; rotate k and copy v [n, nkv*d] into the cache at ``slots``.
-    q, k and v may be column slices of one tensor.  With ``k`` None nothing is stored;
-    with ``inv_freq`` None nothing is rotated."""
-    _gpu("rope_kv_store", q, k, v, pos, slots, inv_freq, kcache, vcache)
+def _angle_table(table: Optional[torch.Tensor], n: int, d: int, what: str) -> int:
+    """Checks a step's table of (cos, sin) [n, R/2, 2] and returns R, the rotated dims (0 without a table)."""
+    if table is None:
+        return 0
+    if (table.dim() != 3 or table.shape[0] != n or table.shape[2] != 2 or table.dtype != torch.float32
+            or not table.is_contiguous() or 2 * table.shape[1] > d):
+        raise ValueError(f"{what}: the table of angles must be a contiguous float32 [{n}, R/2, 2] tensor with R <= {d}")
+    return 2 * int(table.shape[1])
+
+
+def rope_kv_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], table: Optional[torch.Tensor],
+                  slots: Optional[torch.Tensor], kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor],
+                  nh: int, nkv: int, d: int) -> None:
+    """Rotate q [n, nh*d] in place by the step's ``table`` of (cos, sin) [n, R/2, 2] (``rope_table``); rotate k
+    and copy v [n, nkv*d] into the cache at ``slots``.  q, k and v may be column slices of one tensor.  With
+    ``k`` None nothing is stored; with ``table`` None nothing is rotated."""
+    _gpu("rope_kv_store", q, k, v, table, slots, kcache, vcache)
     ldq, wq = _rows(q, "rope_kv_store q")
     n = q.shape[0]
     if wq != nh * d:
         raise ValueError(f"rope_kv_store: q has width {wq}, expected {nh}*{d}")
-    _i32(pos, "rope_kv_store positions", n)
     write = k is not None
     ldk = ldv = 0
     pages = ps = 0
@@ -288,25 +297,24 @@ def rope_kv_store(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
             raise ValueError("rope_kv_store: k and v must be [n, kv_heads*head_dim] of q's dtype")
         pages, ps = _check_cache(kcache, vcache, nkv, d, q.dtype, "rope_kv_store")
         _i32(slots, "rope_kv_store slots", n)
-    if inv_freq is not None:
-        rot = 2 * inv_freq.numel()
-        if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous() or rot > d:
-            raise ValueError("rope_kv_store: inv_freq must be float32 with at most head_dim/2 entries")
-    else:
-        rot = 0
-    _lib.call("zi_rope_kv_store", _p(q), _p(k), _p(v), _code(q, "rope_kv_store"), n, ldq, ldk, ldv, _p(pos),
-              _p(slots), _p(inv_freq), _p(kcache), _p(vcache), pages * ps, nh, nkv, d, rot, max(ps, 1), int(write),
-              _stream())
+    rot = _angle_table(table, n, d, "rope_kv_store")
+    _lib.call("zi_rope_kv_store", _p(q), _p(k), _p(v), _code(q, "rope_kv_store"), n, ldq, ldk, ldv, _p(slots), _p(table),
+              _p(kcache), _p(vcache), pages * ps, nh, nkv, d, rot, max(ps, 1), int(write), _stream())
 
 
-def rope_kv_store_sums(sums: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.Tensor, pos: torch.Tensor,
-                       slots: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
-                       kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], nh: int, nkv: int, d: int
-                       ) -> None:
+def kv_store(k: torch.Tensor, v: torch.Tensor, slots: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor,
+             nkv: int, d: int) -> None:
+    """Copy keys and values [n, nkv*d] (already encoded) into the cache at ``slots``."""
+    rope_kv_store(k, k, v, None, slots, kcache, vcache, nkv, nkv, d)
+
+
+def rope_kv_store_sums(sums: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.Tensor,
+                       table: Optional[torch.Tensor], slots: Optional[torch.Tensor], kcache: Optional[torch.Tensor],
+                       vcache: Optional[torch.Tensor], nh: int, nkv: int, d: int) -> None:
     """The same from the float32 partial sums [S, n, nh*d + 2*nkv*d] of one fused q/k/v projection:
     adds the splits in rising order and the bias, rotates, writes q to ``q_out`` [n, nh*d] and k, v
     into the cache.  With ``kcache`` None only q is made (the sums may then be [S, n, nh*d])."""
-    _gpu("rope_kv_store_sums", sums, bias, q_out, pos, slots, inv_freq, kcache, vcache)
+    _gpu("rope_kv_store_sums", sums, bias, q_out, table, slots, kcache, vcache)
     if sums.dim() != 3 or sums.dtype != torch.float32 or not sums.is_contiguous():
         raise ValueError("rope_kv_store_sums: sums must be a contiguous float32 [S, n, width] tensor")
     S, n, width = sums.shape
@@ -319,20 +327,14 @@ def rope_kv_store_sums(sums: torch.Tensor, bias: Optional[torch.Tensor], q_out: 
     ldq, wq = _rows(q_out, "rope_kv_store_sums q_out")
     if q_out.shape[0] != n or wq != nh * d:
         raise ValueError(f"rope_kv_store_sums: q_out must be [{n}, {nh * d}]")
-    _i32(pos, "rope_kv_store_sums positions", n)
     pages = ps = 0
     if write:
         pages, ps = _check_cache(kcache, vcache, nkv, d, q_out.dtype, "rope_kv_store_sums")
         _i32(slots, "rope_kv_store_sums slots", n)
-    rot = 0
-    if inv_freq is not None:
-        rot = 2 * inv_freq.numel()
-        if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous() or rot > d:
-            raise ValueError("rope_kv_store_sums: inv_freq must be float32 with at most head_dim/2 entries")
+    rot = _angle_table(table, n, d, "rope_kv_store_sums")
     _lib.call("zi_rope_kv_store_split", _p(q_out), _code(q_out, "rope_kv_store_sums"), ldq, _p(sums), S, n * width,
-              width, _p(bias), _code(bias, "rope_kv_store_sums bias") if bias is not None else F32, n, _p(pos),
-              _p(slots), _p(inv_freq), _p(kcache), _p(vcache), pages * ps, nh, nkv, d, rot, max(ps, 1), int(write),
-              _stream())
+              width, _p(bias), _code(bias, "rope_kv_store_sums bias") if bias is not None else F32, n, _p(slots),
+              _p(table), _p(kcache), _p(vcache), pages * ps, nh, nkv, d, rot, max(ps, 1), int(write), _stream())
 
 
 def _attention_args(what, q, kcache, vcache, tok_seq, tok_pos, block_tables, nh, nkv, d, tok_index, out):
@@ -378,7 +380,6 @@ def attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_s
     return out
 
 
-DECODE_MAX_CHUNKS = 64
 
 
 def attention_decode_supported(dtype: torch.dtype, nh: int, nkv: int, d: int, page_size: int) -> bool:
@@ -395,7 +396,7 @@ def attention_decode_chunks(max_keys: int) -> int:
 
 def attention_decode_workspace(tokens: int, nh: int, d: int) -> int:
     """Floats of workspace for the chunk partials of ``tokens`` tokens."""
-    return tokens * nh * DECODE_MAX_CHUNKS * (d + 2)
+    return int(_lib.load().zi_attention_decode_workspace(int(tokens), int(nh), int(d)))
 
 
 def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
@@ -662,16 +663,17 @@ def attention_prefill_variant(variant: int = -1) -> int:
     return int(_lib.load().zi_attention_prefill_variant(int(variant)))
 
 
-PREFILL_TILE = 64     # queries one workgroup of the prompt kernel takes, at least
-PREFILL_TILE_MAX = 128
+def attention_prefill_tile_min() -> int:
+    """Queries of the smallest tile of ``attention_prefill`` (every head size takes it)."""
+    return int(_lib.load().zi_attention_prefill_tile_min())
 
 
 def attention_prefill_tile(dtype: torch.dtype, d: int) -> int:
-    """Queries of a tile of ``attention_prefill`` for this head size: 64, or 128 where the kernel that loads keys
-    and values straight into LDS serves (a staged block then serves twice the queries).  The caller cuts its
-    entries into tiles of this many queries."""
+    """Queries of the widest tile of ``attention_prefill`` for this head size: the smallest, or twice that where
+    the kernel that loads keys and values straight into LDS serves (a staged block then serves twice the
+    queries).  The caller cuts its entries into tiles of this many queries."""
     if dtype not in _CODES:
-        return PREFILL_TILE
+        return attention_prefill_tile_min()
     return int(_lib.load().zi_attention_prefill_tile(_CODES[dtype], int(d)))
 
 
@@ -693,27 +695,23 @@ def _prefill_cut(max_keys: int, window: int, groups: int) -> Tuple[int, int]:
     """(keys between cuts, most cuts of a tile) of a prompt attention launch of ``groups`` tiles x heads none of
     whose queries sees more than ``max_keys`` keys: the cut is the library's choice (longer when there are tiles
     enough to fill the chip without cuts: every cut costs a merge)."""
-    max_keys = max(int(max_keys), 1)
-    if window > 0:      # a windowed tile's keys span at most the window, a tile and a block, from anywhere in a cut
-        max_keys = min(max_keys, window + PREFILL_TILE_MAX + 128)
-    chunk = int(_lib.load().zi_attention_prefill_chunk_keys_for(max_keys, int(groups)))
-    if window > 0:
-        max_keys += chunk - 1
-    return chunk, -(-max_keys // chunk)
+    chunk = c_int(0)
+    cuts = int(_lib.load().zi_attention_prefill_cuts(max(int(max_keys), 1), int(window), int(groups), ctypes.byref(chunk)))
+    return chunk.value, cuts
 
 
 def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tile_entry: torch.Tensor,
                       tile_off: torch.Tensor, entry_start: torch.Tensor, entry_len: torch.Tensor,
                       entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, out: Optional[torch.Tensor] = None, max_keys: int = 0,
-                      workspace: Optional[torch.Tensor] = None, tile: int = PREFILL_TILE, alone: bool = False) -> torch.Tensor:
+                      workspace: Optional[torch.Tensor] = None, tile: int = 0, alone: bool = False) -> torch.Tensor:
     """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
     of 16 up to 128, page size a power of two from 8).
 
     Entry e brings ``entry_len[e]`` tokens, rows ``entry_start[e]...`` of q, that continue a sequence
     holding ``entry_past[e]`` tokens whose block table is row e of ``block_tables``.  Tile i covers the
-    queries [tile_off[i], tile_off[i] + tile) of entry ``tile_entry[i]`` (``tile``: 64, or what
-    ``attention_prefill_tile`` says for the head size); rows of ``out`` that no tile covers are left alone.  ``max_keys`` is an upper bound, known on the host, of the keys any query
+    queries [tile_off[i], tile_off[i] + tile) of entry ``tile_entry[i]`` (``tile``: 0 for the smallest,
+    ``attention_prefill_tile_min()``, or what ``attention_prefill_tile`` says for the head size); rows of ``out`` that no tile covers are left alone.  ``max_keys`` is an upper bound, known on the host, of the keys any query
     sees (its position + 1; 0: what the block tables could hold): tiles that see more than 2,048 keys are
     cut over several workgroups and merged, which needs ``workspace`` (``attention_prefill_workspace``
     entries of float32; allocated here when not given).  A bound that is too low leaves NaN in the rows
@@ -737,9 +735,10 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
     if (block_tables.dim() != 2 or block_tables.dtype != torch.int32 or not block_tables.is_contiguous()
             or block_tables.shape[0] < E):
         raise ValueError("attention_prefill: block_tables must be a contiguous int32 [entries, max_pages] tensor")
-    if tile not in (PREFILL_TILE, attention_prefill_tile(q.dtype, d)):
+    tile = int(tile) or attention_prefill_tile_min()
+    if tile not in (attention_prefill_tile_min(), attention_prefill_tile(q.dtype, d)):
         raise ValueError(f"attention_prefill: tiles of {tile} queries are not taken for head size {d}")
-    if alone and attention_prefill_tile(q.dtype, d) == PREFILL_TILE:
+    if alone and attention_prefill_tile(q.dtype, d) == attention_prefill_tile_min():
         raise ValueError(f"attention_prefill: workgroups of four wavefronts are not made for head size {d}")
     if out is None:
         out = torch.empty((n, nh * d), dtype=q.dtype, device=q.device)

@@ -130,15 +130,31 @@ register_embedding = EMBEDDINGS.register
 register_head = HEADS.register
 
 
+PAGE = -1      # in the shape of a page tensor: where the number of tokens a page holds goes
+
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One tensor a mixer keeps per page of the cache: ``shape`` is that of one page, with PAGE where the page
+    size goes (the cache manager knows it, the mixer need not); ``dtype`` None is the engine's activation type."""
+
+    shape: Tuple[int, ...]
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        return tuple(int(page_size) if s == PAGE else int(s) for s in self.shape)
+
+
 @dataclass(frozen=True)
 class KVCacheRequest:
-    """What a mixer needs from the paged cache: keys of all positions ("full") or of the
-    last ``window`` positions ("window"), for ``num_kv_heads`` heads of ``head_dim``."""
+    """What a mixer needs from the paged cache: pages for all positions ("full") or for the last ``window``
+    positions ("window"), and in every page the named ``tensors`` (name, PageTensor).  The cache manager
+    allocates [pages, *page shape] for each and hands them to the mixer's runs by name
+    (``LayerMemory.tensors``); what they hold and how they are laid out is the mixer's business."""
 
     kind: str
-    num_kv_heads: int
-    head_dim: int
     window: int = 0
+    tensors: Tuple[Tuple[str, PageTensor], ...] = ()
 
 
 @dataclass(frozen=True)
@@ -154,8 +170,7 @@ class LayerMemory:
     """What the cache manager binds to one run of a layer."""
 
     group: int = -1                       # cache group whose slots and block tables apply
-    k: Optional[torch.Tensor] = None      # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None      # [pages, kv_heads, head_dim, page_size] (transposed)
+    tensors: Dict[str, torch.Tensor] = field(default_factory=dict)   # name -> [pages, *page shape], as requested
     writes: bool = True
     state: Optional[torch.Tensor] = None  # [slots, *StateRequest.shape]
 
@@ -188,6 +203,18 @@ class Part:
         """Measure, outside of any step, which of several equivalent ways is faster for steps of
         ``num_tokens`` tokens and record the decision in ``rt.choices`` (``Engine.warm_up`` calls this).
         ``forward`` only reads ``rt.choices``; without an entry it takes a fixed default."""
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        """The number of rows, at least ``rows``, that this part wants a step to be run with when the engine may
+        pad it (so that the kinds of steps are few and recur, and so that the part's kernels meet numbers of
+        rows they are built or were measured for).  ``kind`` says what is counted:
+        "decode"  the entries of a step in which every entry brings one token;
+        "portion" the tokens of one portion of a prompt;
+        "beside"  the entries of one token beside portions of prompts;
+        "mixed"   all rows of a step with portions.
+        The engine takes the least number every part of the model accepts (``DecoderModel.step_rows``).  The
+        default accepts every number."""
+        return int(rows)
 
 
 @dataclass
@@ -299,19 +326,16 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
-    """Encodes positions into queries and keys on their way into the cache.
+    """Encodes positions into queries and keys.  It transforms; what is stored where is the mixer's business.
 
-    ``rotate_and_store`` encodes q [n, nh*d] in place and stores the encoded k and the raw v
-    [n, nkv*d] at ``slots`` of ``memory``'s cache (nothing is stored when ``memory.writes`` is
-    False).  ``rotate_and_store_sums`` does the same from the float32 partial sums [S, n,
-    nh*d + 2*nkv*d] of a fused q/k/v projection plus its bias, and writes q to ``q_out``; the
-    default adds the sums up and calls ``rotate_and_store``.
+    ``encode(q, k, positions, nh, nkv, d)`` encodes q [n, nh*d] and k [n, nkv*d] in place (either may be a
+    column slice of a wider tensor).
 
-    ``step_table(batch)`` lets a mixer fold the encoding into a kernel of its own: an encoding that
+    ``step_table(batch)`` lets a mixer fold the encoding into kernels of its own: an encoding that
     is a rotation of pairs (k, k + R/2) of the first R dims of every head returns the step's angles
     as a float32 tensor [n, R/2, 2] of (cos, sin), computed once per step and kept in
     ``batch.shared``; an encoding that does nothing returns the string "none"; every other encoding
-    returns None (the default), and the mixer calls ``rotate_and_store*``.
+    returns None (the default), and the mixer calls ``encode``.
 
     ``positions`` is what the step gives for each token: int32 [n], the token's index in its sequence,
     when ``position_axes`` is 1; with more axes int32 [n, position_axes], every axis the index in the
@@ -322,17 +346,8 @@ class PositionEncoding(Part):
     def step_table(self, batch):
         return None
 
-    def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
+    def encode(self, q, k, positions, nh: int, nkv: int, d: int) -> None:
         raise NotImplementedError
-
-    def rotate_and_store_sums(self, sums, bias, q_out, positions, slots, memory: LayerMemory, nh: int, nkv: int,
-                              d: int) -> None:
-        from .. import ops
-        qkv = ops.reduce_sums(sums, bias, out_dtype=q_out.dtype)
-        qd, kvd = nh * d, nkv * d
-        q, k, v = qkv[:, :qd], qkv[:, qd:qd + kvd], qkv[:, qd + kvd:]
-        self.rotate_and_store(q, k, v, positions, slots, memory, nh, nkv, d)
-        q_out.copy_(q)
 
 
 class Block:

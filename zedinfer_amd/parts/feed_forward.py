@@ -10,6 +10,7 @@ from .. import ops
 from ..config.forward_config import PartSpec
 from ..weights.loader import WeightSpec
 from .base import FeedForward, Runtime, register_feed_forward
+from .rows import ProductRows
 
 
 def stack_rows(tensors):
@@ -82,6 +83,9 @@ class SwiGLU(FeedForward):
             if wins:
                 return self._gate_up_transposed(x, act)
         return self._gate_up_straight(x, act)
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
 
     def tune(self, num_tokens: int) -> None:
         """For steps of ``num_tokens`` rows: the library's algorithms for the gate/up and down products, then the

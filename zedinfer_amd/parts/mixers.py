@@ -10,8 +10,9 @@ import torch
 from .. import ops
 from ..config.forward_config import PartSpec
 from ..weights.loader import WeightSpec
-from .base import (HostBatch, KVCacheRequest, LayerMemory, Mixer, POSITION_ENCODINGS, Runtime, StepPlan, StepPlanner,
-                   register_mixer)
+from .base import (PAGE, HostBatch, KVCacheRequest, LayerMemory, Mixer, PageTensor, POSITION_ENCODINGS, Runtime, StepPlan,
+                   StepPlanner, register_mixer)
+from .rows import ProductRows
 from .feed_forward import stack_rows
 
 SHORT_ENTRY = 4     # entries of up to this many tokens are attended token by token, split over the keys
@@ -95,6 +96,14 @@ class AttentionPlanner(StepPlanner):
 
 
 _PLANNERS: Dict[tuple, AttentionPlanner] = {}
+
+
+def attention_cache_request(kind: str, num_kv_heads: int, head_dim: int, window: int = 0) -> KVCacheRequest:
+    """What the attention kernels keep in a page: keys as [kv_head][slot][head_dim], values transposed as
+    [kv_head][head_dim][slot] (a run of positions of one value dim is contiguous, which is the order the matrix
+    cores read P.V in)."""
+    return KVCacheRequest(kind, int(window), (("k", PageTensor((int(num_kv_heads), PAGE, int(head_dim)))),
+                                              ("v", PageTensor((int(num_kv_heads), int(head_dim), PAGE)))))
 
 
 def attention_planner(wide_tile: int, heads: int) -> AttentionPlanner:
@@ -195,12 +204,12 @@ class Attention(Mixer):
         """Tokens of short entries (decoded tokens) go to the kernel that splits one query's keys over
         many wavefronts, longer portions to the matrix-core prompt kernel; every shape those kernels do
         not take goes to the plain one."""
-        args = (memory.k, memory.v, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
-                self.scale)
+        kc, vc = memory.tensors["k"], memory.tensors["v"]
+        args = (kc, vc, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale)
         plan = batch.plans[self.plan_key]
         n_short, n_long, N = plan.sizes["num_short"], plan.sizes["num_long"], batch.num_tokens
         if n_short:
-            if ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
+            if ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, kc.shape[2]):
                 ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n_short, self.nh, self.d),),
                                     torch.float32)
                 ops.attention_decode(q, *args, plan.sizes["max_short_keys"], self.window, out=att,
@@ -210,12 +219,12 @@ class Attention(Mixer):
         if n_long < 0:
             ops.attention(q, *args, self.window, out=att)
         elif n_long > 0:
-            if ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, memory.k.shape[2]):
+            if ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, kc.shape[2]):
                 max_keys = plan.sizes["max_long_keys"]
                 need = ops.attention_prefill_workspace(q.shape[0], self.nh, self.d, max_keys, self.window,
                                                        plan.sizes["num_tiles"])
                 ws = self.rt.buffer("attn_prompt_split", (need,), torch.float32) if need else None
-                ops.attention_prefill(q, memory.k, memory.v, plan.dev["tile_entry"], plan.dev["tile_off"],
+                ops.attention_prefill(q, kc, vc, plan.dev["tile_entry"], plan.dev["tile_off"],
                                       batch.entry_start, batch.entry_len, batch.entry_past, view.block_tables, self.nh,
                                       self.nkv, self.d, self.scale, self.window, out=att, max_keys=max_keys,
                                       workspace=ws, tile=plan.sizes["tile"], alone=plan.sizes["alone"])
@@ -231,7 +240,47 @@ class Attention(Mixer):
         return batch.position_ids if self.position.position_axes > 1 else batch.positions
 
     def cache_request(self) -> Optional[KVCacheRequest]:
-        return KVCacheRequest("window" if self.window > 0 else "full", self.nkv, self.d, self.window)
+        return attention_cache_request("window" if self.window > 0 else "full", self.nkv, self.d, self.window)
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        """The projections are few-rows products up to a number of rows and the library's beyond; portions are cut
+        into tiles of LONG_TILE queries (PORTION_ROWS is a multiple)."""
+        return ProductRows.step_rows(rows, kind)
+
+    def encode_and_store(self, q, k, v, batch, view, memory: LayerMemory) -> None:
+        """Queries and keys get their positions, keys and values go into the cache (when this run writes it).  An
+        encoding that hands over the step's table of angles (or says that it does nothing) is folded into the
+        kernel that stores; any other transforms q and k itself first."""
+        table = self.position.step_table(batch)
+        if table is None:
+            self.position.encode(q, k, self.positions_of(batch), self.nh, self.nkv, self.d)
+            if memory.writes:
+                ops.kv_store(k, v, view.slots, memory.tensors["k"], memory.tensors["v"], self.nkv, self.d)
+            return
+        angles = None if isinstance(table, str) else table
+        if memory.writes:
+            ops.rope_kv_store(q, k, v, angles, view.slots, memory.tensors["k"], memory.tensors["v"], self.nh, self.nkv,
+                              self.d)
+        elif angles is not None:
+            ops.rope_kv_store(q, None, None, angles, None, None, None, self.nh, self.nkv, self.d)
+
+    def encode_and_store_sums(self, sums, q_out, batch, view, memory: LayerMemory) -> None:
+        """The same from the float32 partial sums [S, n, Qd + 2 KVd] of the fused projection (the bias is added
+        here); the encoded queries go to ``q_out``."""
+        table = self.position.step_table(batch)
+        if table is None:
+            qkv = ops.reduce_sums(sums, self.bias, out_dtype=q_out.dtype,
+                                  out=self.rt.buffer("attn_qkv", (sums.shape[1], self.qd + 2 * self.kvd)))
+            q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
+            self.encode_and_store(q, k, v, batch, view, memory)
+            q_out.copy_(q)
+            return
+        angles = None if isinstance(table, str) else table
+        if memory.writes:
+            ops.rope_kv_store_sums(sums, self.bias, q_out, angles, view.slots, memory.tensors["k"], memory.tensors["v"],
+                                   self.nh, self.nkv, self.d)
+        else:
+            ops.rope_kv_store_sums(sums, self.bias, q_out, angles, None, None, None, self.nh, self.nkv, self.d)
 
     def forward(self, x: torch.Tensor, batch, memory: LayerMemory) -> torch.Tensor:
         n = x.shape[0]
@@ -244,8 +293,7 @@ class Attention(Mixer):
             # every head is a row of head_dim values: normed in place
             ops.rms_norm(q.view(n * self.nh, self.d), self.q_norm, self.qk_norm_eps, out=q.view(n * self.nh, self.d))
             ops.rms_norm(k.view(n * self.nkv, self.d), self.k_norm, self.qk_norm_eps, out=k.view(n * self.nkv, self.d))
-            self.position.rotate_and_store(q, k, v, self.positions_of(batch), view.slots, memory, self.nh, self.nkv,
-                                           self.d)
+            self.encode_and_store(q, k, v, batch, view, memory)
         elif self.qkv is not None and ops.linear_sums_supported(x, self.qkv):
             # few rows: the projection leaves float32 partial sums; the rotary kernel adds them and the bias
             S = ops.linear_splits(n, self.qkv.shape[0], self.hidden)
@@ -255,8 +303,7 @@ class Attention(Mixer):
             if out is not None:
                 return out
             q = self.rt.buffer("attn_q", (n, self.qd))
-            self.position.rotate_and_store_sums(sums, self.bias, q, self.positions_of(batch), view.slots, memory, self.nh,
-                                                self.nkv, self.d)
+            self.encode_and_store_sums(sums, q, batch, view, memory)
         else:
             qkv = self.rt.buffer("attn_qkv", (n, self.qd + 2 * self.kvd))
             q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
@@ -265,8 +312,7 @@ class Attention(Mixer):
             else:
                 for dst, m, b in zip((q, k, v), self.mats, self.biases or (None, None, None)):
                     ops.linear(x, m, b, out=dst)
-            self.position.rotate_and_store(q, k, v, self.positions_of(batch), view.slots, memory, self.nh, self.nkv,
-                                           self.d)
+            self.encode_and_store(q, k, v, batch, view, memory)
         att = self.rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
         return self.project(att, n)
@@ -301,16 +347,16 @@ class Attention(Mixer):
             return None
         rot = 0 if isinstance(table, str) else 2 * table.shape[1]
         S, n, width = sums.shape
-        ps = memory.k.shape[2]
+        kc, vc = memory.tensors["k"], memory.tensors["v"]
+        ps = kc.shape[2]
         max_keys = batch.plans[self.plan_key].sizes["max_short_keys"]
-        if not ops.attention_decode_fused_supported(memory.k.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
+        if not ops.attention_decode_fused_supported(kc.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
             return None
         if n * self.nkv * ops.attention_decode_chunks(max_keys) > self.FUSED_DECODE_MAX_WORKGROUPS:
             return None
         ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
         # every entry brings one token: token t is of entry t
-        args = (sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None, memory.k, memory.v,
-                None, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale,
+        args = (sums, self.bias, None if rot == 0 else table, view.slots if memory.writes else None, kc, vc, None, batch.positions, view.block_tables, self.nh, self.nkv, self.d, self.scale,
                 max_keys, self.window)
         if (self.o.numel() * self.o.element_size() <= self.PROJECT_FROM_CHUNKS_MAX_BYTES
                 and ops.attention_decode_project_supported(self.o, n, self.nh, self.d)):

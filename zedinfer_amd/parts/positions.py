@@ -1,5 +1,4 @@
-"""Position encodings.  They act where queries and keys leave the projection:
-queries are encoded in place, keys on their way into the paged cache."""
+"""Position encodings.  They act where queries and keys leave the projection; the mixer stores what they made."""
 from __future__ import annotations
 
 from typing import Dict
@@ -8,7 +7,7 @@ import torch
 
 from .. import ops
 from ..config.forward_config import PartSpec
-from .base import LayerMemory, PositionEncoding, Runtime, register_position_encoding
+from .base import PositionEncoding, Runtime, register_position_encoding
 
 
 @register_position_encoding("rope_neox")
@@ -39,18 +38,11 @@ class RopeNeox(PositionEncoding):
             table = batch.shared[key] = ops.rope_table(batch.positions, self.inv_freq, out=out)
         return table
 
-    def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
-        if memory.writes:
-            ops.rope_kv_store(q, k, v, positions, slots, self.inv_freq, memory.k, memory.v, nh, nkv, d)
-        else:
-            ops.rope_kv_store(q, None, None, positions, None, self.inv_freq, None, None, nh, nkv, d)
-
-    def rotate_and_store_sums(self, sums, bias, q_out, positions, slots, memory: LayerMemory, nh: int, nkv: int,
-                              d: int) -> None:
-        if memory.writes:
-            ops.rope_kv_store_sums(sums, bias, q_out, positions, slots, self.inv_freq, memory.k, memory.v, nh, nkv, d)
-        else:
-            ops.rope_kv_store_sums(sums, bias, q_out, positions, None, self.inv_freq, None, None, nh, nkv, d)
+    def encode(self, q, k, positions, nh: int, nkv: int, d: int) -> None:
+        """(A mixer that takes ``step_table`` does not come here.)"""
+        table = ops.rope_table(positions, self.inv_freq)
+        ops.rope_kv_store(q, None, None, table, None, None, None, nh, nkv, d)
+        ops.rope_kv_store(k, None, None, table, None, None, None, nkv, nkv, d)
 
 
 @register_position_encoding("none")
@@ -63,13 +55,5 @@ class NoPosition(PositionEncoding):
     def step_table(self, batch):
         return "none"
 
-    def rotate_and_store(self, q, k, v, positions, slots, memory: LayerMemory, nh: int, nkv: int, d: int) -> None:
-        if memory.writes:
-            ops.rope_kv_store(q, k, v, positions, slots, None, memory.k, memory.v, nh, nkv, d)
-
-    def rotate_and_store_sums(self, sums, bias, q_out, positions, slots, memory: LayerMemory, nh: int, nkv: int,
-                              d: int) -> None:
-        if memory.writes:
-            ops.rope_kv_store_sums(sums, bias, q_out, positions, slots, None, memory.k, memory.v, nh, nkv, d)
-        else:
-            ops.rope_kv_store_sums(sums, bias, q_out, positions, None, None, None, None, nh, nkv, d)
+    def encode(self, q, k, positions, nh: int, nkv: int, d: int) -> None:
+        pass
