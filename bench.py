@@ -490,16 +490,27 @@ def main():
         short = measure_prefill(factory(1, 128), V, tokens=128, warm=2)
         points["prefill_128"] = round(128 / short * 1000.0, 1)
         out["points"] = points
+        def flat(prefix, results):
+            """Further measurements as flat numbers of `points` (what is deeper is lost in the record)."""
+            for name, r in results.items():
+                if isinstance(r, dict) and "value" in r:
+                    points[prefix + name] = r["value"]
+                    if "roofline_frac" in r:
+                        points[prefix + name + "_roofline_frac"] = r["roofline_frac"]
         if not args.no_further:
             out["long_context"] = long_context_points(lambda: weights_cache["w"], shape, args.layers, el, args)
+            flat("", out["long_context"])
         if args.shape == "1.5B" and args.layers == FULL_LAYERS and not args.no_further:
             # the same architecture at the Qwen2.5-7B sizes: decode at batch 8 and the continuous-batching mix
             weights_cache.clear()
             torch.cuda.empty_cache()
             out["further"] = further_7b(args)
+            flat("7b_", out["further"].get("long_context", {}))
+            flat("7b_", {k: v for k, v in out["further"].items() if k != "long_context"})
             gc.collect()
             torch.cuda.empty_cache()
             out["further_32b"] = further_32b(args)
+            flat("32b_", out["further_32b"])
     out["choices"] = CHOICES
     print(json.dumps(out))
     return 0

@@ -645,7 +645,7 @@ def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatc
     # a launch of more workgroups (tokens x key/value heads x chunks of the keys) than the limit takes the
     # separate kernels: with the limit below this step's launch nothing is fused, and the logits agree as before
     nkv = tiny["cfg"]["num_key_value_heads"]
-    assert 3 * nkv * ops.attention_decode_chunks(256) <= Attention.FUSED_DECODE_MAX_WORKGROUPS == 512
+    assert 3 * nkv * ops.attention_decode_chunks(256) <= Attention.FUSED_DECODE_WORKGROUPS_PER_UNIT * ops.compute_units() == 512
     monkeypatch.setattr(Attention, "FUSED_DECODE_MAX_WORKGROUPS", 3 * nkv - 1)
     before = calls["fused"]
     both([("a", 1), ("b", 1), ("c", 1)])

@@ -166,6 +166,49 @@ def test_a_step_that_allocates_is_not_taped(tmp_path, monkeypatch):
     assert e.tape_runs == 0 and any(dg.no_tape for dg in e._graphs.values())
 
 
+def test_a_step_with_work_that_is_no_library_call_is_not_taped(tmp_path, monkeypatch):
+    """A part that does device work through a torch operator that takes no memory (against what ``tape_safe``
+    promises) leaves nothing on the tape for it.  A new tape is therefore run once on its own step, from workspaces
+    made NaN, and must repeat the step's logits: this one does not, the shape is marked, and its steps go on part
+    by part with the right results.  Without the part's extra work the same steps do run from tapes."""
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    from zedinfer_amd.parts.norms import RMSNorm
+    folder = tiny_configs.write_tiny(str(tmp_path / "m"), "A")
+    cfg, w = plain.load_folder(folder)
+    ps = tiny_configs.PAGE_SIZES["A"]
+    toks = traces.random_tokens(cfg["vocab_size"], 40, seed=2)
+
+    def run(engine):
+        engine.use_graphs = False
+        seq = engine.open("r")
+        rows = [engine.step([StepEntry(seq, toks[:8], [7])]).cpu()]
+        for i in range(8, 40):
+            rows.append(engine.step([StepEntry(seq, toks[i:i + 1], [0])]).cpu())
+        engine.close(seq)
+        return torch.cat(rows)
+
+    sched = SchedulerConfig(num_kv_blocks=64, kv_block_size=ps, max_batch_requests=4)
+    plain_engine = Engine.from_folder(folder, "float32", sched)
+    straight = run(plain_engine)
+    assert plain_engine.tape_runs > 20
+    from zedinfer_amd import ops
+
+    def through_a_copy(self, resid, delta):
+        """The library's norm into another workspace, then a torch copy into the one the next part reads: the copy
+        takes no memory and is on no tape, so a replay would leave the last step's rows there."""
+        out = self.rt.buffer("norm_out", (resid.shape[0], self.dim), self.rt.dtype)
+        tmp = self.rt.buffer("norm_elsewhere", (resid.shape[0], self.dim), self.rt.dtype)
+        ops.add_rms_norm(resid, delta, self.weight, self.eps, out=tmp, add_one=self.add_one)
+        out.copy_(tmp)
+        return out
+    monkeypatch.setattr(RMSNorm, "add_forward", through_a_copy)
+    e = Engine.from_folder(folder, "float32", sched)
+    got = run(e)
+    assert torch.equal(got, straight)
+    assert e.tape_runs == 0 and all(dg.no_tape for dg in e._graphs.values())
+
+
 def test_generation_from_tapes_alone(tmp_path, monkeypatch):
     """The serving loop (continuous batching, chunked prefill, steps queued ahead) with graphs switched off: the
     recurring steps run from tapes, and every request gets the plain implementation's greedy tokens."""

@@ -819,7 +819,7 @@ extern "C" int zi_attention_prefill_chunk_keys() { return PF_CHUNK; }
 // it to zi_attention_prefill.  Measured at the 1.5B sizes (12 heads), one prompt in one step, cut every 2,048
 // against no cut: 16,384 tokens (1,536 groups) 83.7 against 78.0 ms, 8,192 (768) 33.3 against 32.3, 4,096 (384)
 // 16.6 against 17.6; at the 32B sizes 16,384 tokens 1,036 against 985 ms.
-extern "C" int zi_attention_prefill_chunk_keys_for(int max_keys, int groups) { return zi_pf_chunk_for(max_keys, groups); }
+extern "C" int zi_attention_prefill_chunk_keys_for(int max_keys, int groups) { return zi_pf_chunk_for(max_keys, groups, zi_compute_units()); }
 
 // The smallest tile of queries (every head size takes it).
 extern "C" int zi_attention_prefill_tile_min() { return PF_BM; }
@@ -831,7 +831,7 @@ extern "C" int zi_attention_prefill_tile_min() { return PF_BM; }
 extern "C" int zi_attention_prefill_cuts(int max_keys, int window, int groups, int* chunk_keys) {
     if (max_keys < 1) max_keys = 1;
     if (window > 0 && max_keys > window + 2 * PF_BM + PF_BS) max_keys = window + 2 * PF_BM + PF_BS;
-    const int chunk = zi_pf_chunk_for(max_keys, groups);
+    const int chunk = zi_pf_chunk_for(max_keys, groups, zi_compute_units());
     if (window > 0) max_keys += chunk - 1;
     if (chunk_keys) *chunk_keys = chunk;
     return (max_keys + chunk - 1) / chunk;

@@ -25,7 +25,6 @@ typedef __attribute__((ext_vector_type(4))) unsigned gm_u32x4_t;
 #define GM_STAGERS 256      // threads that stage the block's x slice (the first four wavefronts)
 #define GM_KB 128
 #define GM_XS GM_KB         // LDS row stride, in elements: rows of 16 pieces of 16 bytes, piece c of row r at place c xor (r mod 16)
-#define GM_CUS 256          // compute units the cut is balanced over
 
 #define GM_MODE_PLAIN 0
 #define GM_MODE_PARTIAL 1
@@ -377,7 +376,8 @@ void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split, int* waves) 
     const int kb_total = (K + GM_KB - 1) / GM_KB;
     int64_t best_cost = -1;
     int best_s = 1, best_w = GM_MIN_WAVES, best_per = kb_total;
-    const bool many = (tiles + GM_MIN_WAVES - 1) / GM_MIN_WAVES > 4 * GM_CUS;
+    const int cus = zi_compute_units();          // the cut is balanced over the device's compute units
+    const bool many = (tiles + GM_MIN_WAVES - 1) / GM_MIN_WAVES > 4 * cus;
     for (int w = GM_MIN_WAVES; w <= (many ? GM_MIN_WAVES : GM_MAX_WAVES); ++w) {
         const int groups = (tiles + w - 1) / w;
         for (int s0 = 1; s0 <= (many ? 1 : 16) && s0 <= (kb_total > 1 ? kb_total / 2 : 1); ++s0) {
@@ -385,7 +385,7 @@ void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split, int* waves) 
             const int s = (kb_total + per - 1) / per;
             if (s != s0) continue;      // the same cut under another name
             const int64_t wgs = (int64_t)groups * s;
-            const int64_t rounds = (wgs + GM_CUS - 1) / GM_CUS;
+            const int64_t rounds = (wgs + cus - 1) / cus;
             const int64_t cost = rounds * ((int64_t)w * per + 10);
             if (best_cost < 0 || cost < best_cost || (cost == best_cost && s < best_s)) {
                 best_cost = cost; best_s = s; best_w = w; best_per = per;

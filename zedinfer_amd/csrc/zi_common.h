@@ -84,6 +84,8 @@ __device__ __forceinline__ float zi_block_max(float v, float* scratch) {
 // Every entry point returns 0 on success.  On failure it returns non-zero and
 // leaves a message that zi_last_error() hands out.
 extern "C" const char* zi_last_error();
+#define ZI_DEFAULT_COMPUTE_UNITS 256      // an MI355X
+extern "C" int zi_compute_units();
 int zi_fail(const char* fmt, ...);
 int zi_check_launch(const char* what);
 

@@ -112,13 +112,13 @@ ZI_HD int64_t zi_dec_part_slot(int token_index, int nh, int head, int chunk) {
 #define ZI_PF_BS 128         // keys of a block
 #define ZI_PF_CHUNK 2048     // keys one workgroup walks at most: the cut of launches over few keys
 #define ZI_PF_CHUNK_LONG 16384      // the cut of launches whose queries see more than ZI_PF_LONG_FROM keys and that have
-#define ZI_PF_LONG_FROM 6144        // ZI_PF_LONG_GROUPS workgroups (tiles x heads) without any cut: those fill the chip as
-#define ZI_PF_LONG_GROUPS 768       // they are, and every cut costs a merge
+#define ZI_PF_LONG_FROM 6144        // ZI_PF_LONG_GROUPS_PER_CU workgroups (tiles x heads) a compute unit without any cut: those
+#define ZI_PF_LONG_GROUPS_PER_CU 3  // fill the chip as they are, and every cut costs a merge (768 on 256 units)
 #define ZI_PF_MAXC 64        // most cuts of one tile
 
 // The cut of a launch of `groups` tiles x heads none of whose queries sees more than max_keys keys.
-ZI_HD int zi_pf_chunk_for(int max_keys, int groups) {
-    return (max_keys > ZI_PF_LONG_FROM && groups >= ZI_PF_LONG_GROUPS) ? ZI_PF_CHUNK_LONG : ZI_PF_CHUNK;
+ZI_HD int zi_pf_chunk_for(int max_keys, int groups, int compute_units = 256) {
+    return (max_keys > ZI_PF_LONG_FROM && groups >= ZI_PF_LONG_GROUPS_PER_CU * compute_units) ? ZI_PF_CHUNK_LONG : ZI_PF_CHUNK;
 }
 
 // A tile of `count` queries whose first sits at position pos0 sees keys [lo_tile, kmax].  Its walk starts at

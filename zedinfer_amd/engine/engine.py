@@ -200,20 +200,24 @@ class Engine:
                 growth = self.cache.ensure(e.seq, e.seq.length + len(e.tokens))
                 if growth is not NO_GROWTH:
                     grown.append((e.seq, growth))
-        except Exception:
-            for seq, growth in reversed(grown):      # nothing of a step that cannot run stays
+            if (self.use_graphs or self.use_tapes) and 0 < len(entries) <= self.graph_max_entries and single:
+                logits = self._graph_step(entries, token_source)
+            elif (self.use_graphs or self.use_tapes) and self._one_portion(entries):
+                logits = self._prompt_graph_step(entries, token_source)
+            else:
+                batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging,
+                                           planners=self.planners, position_axes=self.position_axes)
+                if token_source is not None:        # the entries' tokens lie in their order: the first k are the first k tokens
+                    batch.token_ids[:token_source.shape[0]].copy_(token_source, non_blocking=True)
+                logits = self.model.run(batch, self.memories)
+        except BaseException:
+            # nothing of a step that did not run to its end stays: the pages and promises it took go back, no
+            # length has changed (what a step that failed half-way wrote lies beyond every length)
+            for seq, growth in reversed(grown):
                 self.cache.undo(seq, growth)
+            for dg in self._graphs.values():       # a host image may have been rewritten half-way: made again next time
+                dg.image = None
             raise
-        if (self.use_graphs or self.use_tapes) and 0 < len(entries) <= self.graph_max_entries and single:
-            logits = self._graph_step(entries, token_source)
-        elif (self.use_graphs or self.use_tapes) and self._one_portion(entries):
-            logits = self._prompt_graph_step(entries, token_source)
-        else:
-            batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging,
-                                       planners=self.planners, position_axes=self.position_axes)
-            if token_source is not None:        # the entries' tokens lie in their order: the first k are the first k tokens
-                batch.token_ids[:token_source.shape[0]].copy_(token_source, non_blocking=True)
-            logits = self.model.run(batch, self.memories)
         for e in entries:
             self.cache.commit(e.seq, e.seq.length + len(e.tokens))
         self.steps_run += 1
@@ -304,9 +308,37 @@ class Engine:
         if rec.allocations:
             dg.no_tape = dg.ran       # at the first step workspaces may still get their sizes
         else:
-            dg.tape, dg.logits = rec.tape(), logits
+            tape = rec.tape()
+            if tape is None:
+                dg.no_tape = True
+            elif self._tape_repeats_the_step(tape, logits):
+                dg.tape, dg.logits = tape, logits
+            else:
+                dg.no_tape = True
+                logits = self.model.run(batch, self.memories)     # what the failed replay left in cache and workspaces is made again
         dg.ran = True
         return logits
+
+    def _tape_repeats_the_step(self, tape, logits: Optional[torch.Tensor]) -> bool:
+        """A new tape is run once, right after the step it was recorded from and on the same inputs, with every
+        floating-point workspace of the runtime (the logits among them) made NaN before, and must leave the same
+        logits bit for bit: device work that is no call into the kernel library (a torch operator in a part that
+        says ``tape_safe``) is not on the tape, its result would be stale at every replay, and here it is NaN.  A
+        model with state per request is not run twice (the second run would advance the state): its tapes are
+        trusted as before."""
+        if logits is None or self.model.state_requests():
+            return True
+        first = logits.clone()
+        self.rt.poison()
+        logits.fill_(float("nan"))
+        tape.run()
+        same = bool(torch.equal(first, logits))
+        if not same:
+            import logging
+            logging.getLogger("zedinfer_amd").warning(
+                "a recorded step does not repeat its logits: some device work of the model is not a call into the "
+                "kernel library; steps of this shape run part by part")
+        return same
 
 
     @staticmethod

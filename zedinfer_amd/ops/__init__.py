@@ -11,7 +11,7 @@ from .functional import (add, add_rms_norm, argmax, attention, attention_decode,
                          attention_decode_project_splits, attention_decode_project_supported,
                          attention_decode_supported, attention_decode_workspace, attention_prefill,
                          attention_prefill_supported, attention_prefill_tile, attention_prefill_tile_min, attention_prefill_variant,
-                         attention_prefill_workspace, decode_layer, decode_layer_stamps, decode_layer_supported, decode_layer_sync_words,
+                         attention_prefill_workspace, compute_units, decode_layer, decode_layer_stamps, decode_layer_supported, decode_layer_sync_words,
                          decode_layer_workspace, device_synchronize, embedding, gather_rows, kv_store,
                          has_cuda, has_gpu, linear, linear_choose, linear_splits, linear_sums,
                          linear_sums_supported, linear_swiglu, linear_swiglu_supported,
@@ -26,7 +26,7 @@ __all__ = [
     "attention_decode_fused_supported", "attention_decode_project", "attention_decode_project_splits",
     "attention_decode_project_supported", "attention_decode_supported", "attention_decode_workspace",
     "attention_prefill", "attention_prefill_supported", "attention_prefill_tile", "attention_prefill_tile_min", "attention_prefill_variant",
-    "attention_prefill_workspace", "decode_layer", "decode_layer_stamps", "decode_layer_supported", "decode_layer_sync_words",
+    "attention_prefill_workspace", "compute_units", "decode_layer", "decode_layer_stamps", "decode_layer_supported", "decode_layer_sync_words",
     "decode_layer_workspace", "device_synchronize", "embedding", "gather_rows", "has_cuda", "kv_store", "has_gpu",
     "linear", "linear_choose", "linear_splits", "linear_sums", "linear_sums_supported", "linear_swiglu",
     "linear_swiglu_supported", "linear_transposed", "linear_tune", "reduce_sums", "rms_norm", "rope",

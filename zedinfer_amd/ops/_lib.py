@@ -47,6 +47,7 @@ _PROTOTYPES = {
     "zi_attention_prefill_chunk_keys_for": [I, I],
     "zi_attention_prefill_cuts": [I, I, I, P],
     "zi_attention_prefill_tile_min": [],
+    "zi_compute_units": [],
     "zi_attention_prefill_chunks": [I],
     "zi_attention_prefill_variant": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],

@@ -663,6 +663,12 @@ def attention_prefill_variant(variant: int = -1) -> int:
     return int(_lib.load().zi_attention_prefill_variant(int(variant)))
 
 
+def compute_units() -> int:
+    """Compute units of the current device: what the kernels' cuts and the parts' tile choices are balanced over
+    (256 when there is no device to ask)."""
+    return int(_lib.load().zi_compute_units())
+
+
 def attention_prefill_tile_min() -> int:
     """Queries of the smallest tile of ``attention_prefill`` (every head size takes it)."""
     return int(_lib.load().zi_attention_prefill_tile_min())

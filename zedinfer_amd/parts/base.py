@@ -84,6 +84,13 @@ class Runtime:
         view = self._views[vkey] = buf[:n].view(tuple(shape))
         return view
 
+    def poison(self) -> None:
+        """Make every floating-point workspace NaN (a check that a replay writes all it reads; integer workspaces
+        may hold indices and are left alone)."""
+        for buf in self._buffers.values():
+            if buf.dtype.is_floating_point:
+                buf.fill_(float("nan"))
+
     def outgrown_bytes(self) -> int:
         """Bytes of allocations that were outgrown and are kept for graphs captured before."""
         return sum(b.numel() * b.element_size() for b in self._outgrown)

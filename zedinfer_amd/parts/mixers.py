@@ -39,13 +39,17 @@ class AttentionPlanner(StepPlanner):
     bound of the keys a token of either kind sees (its position + 1), which sizes the launches."""
 
     fixed_for_single_tokens = True
-    FILL = 384          # workgroups of wide tiles from which they pay (one and a half a compute unit)
-    FILL_ALONE = 768    # and from which workgroups of four wavefronts, two to a compute unit, pay (``alone``)
+    # Workgroups of wide tiles from which they pay: one and a half a compute unit (384 on the 256 of an MI355X);
+    # and from which workgroups of four wavefronts, two to a compute unit, pay (``alone``): three a compute unit.
+    # FILL / FILL_ALONE, when set, stand for the products (tests set them).
+    FILL_PER_UNIT, FILL_ALONE_PER_UNIT = 1.5, 3.0
+    FILL = FILL_ALONE = None
     CUT_KEYS = 2048     # a tile's keys are cut over several workgroups every so many
 
     def __init__(self, wide_tile: int = LONG_TILE, heads: int = 1):
         self.wide_tile, self.heads = int(wide_tile), int(heads)
         self.key = ("attention", SHORT_ENTRY, self.wide_tile, self.heads)
+        self.units = compute_units()
 
     def plan(self, hb: HostBatch) -> StepPlan:
         lens, past = hb.entry_len, hb.entry_past
@@ -82,9 +86,9 @@ class AttentionPlanner(StepPlanner):
         if self.wide_tile > LONG_TILE and long_lens:
             wide = int(sum(-(-int(n) // self.wide_tile) for n in long_lens))
             groups = wide * -(-max_long // self.CUT_KEYS) * self.heads
-            if groups >= self.FILL:
+            if groups >= (self.FILL if self.FILL is not None else self.FILL_PER_UNIT * self.units):
                 tile = self.wide_tile
-                alone = groups >= self.FILL_ALONE
+                alone = groups >= (self.FILL_ALONE if self.FILL_ALONE is not None else self.FILL_ALONE_PER_UNIT * self.units)
         return tile, alone
 
     def shape(self, entry_lens, bound_single: int, bound_multi: int) -> tuple:
@@ -96,6 +100,11 @@ class AttentionPlanner(StepPlanner):
 
 
 _PLANNERS: Dict[tuple, AttentionPlanner] = {}
+
+
+def compute_units() -> int:
+    """The device's compute units (an MI355X's 256 where no device can be asked: planning on the host alone)."""
+    return ops.compute_units() if torch.cuda.is_available() else 256
 
 
 def attention_cache_request(kind: str, num_kv_heads: int, head_dim: int, window: int = 0) -> KVCacheRequest:
@@ -137,12 +146,14 @@ class Attention(Mixer):
     # measured faster at 1 and 8 tokens, slower at 64.
     FUSED_DECODE_MAX_TOKENS = 16
     # ... and once the launch (tokens x key/value heads x chunks of the keys) is more workgroups than the chip
-    # holds at a time (two a compute unit): the workgroups of a second round pay the three dependent trips to
+    # holds at a time (two a compute unit, FUSED_DECODE_WORKGROUPS_PER_UNIT; FUSED_DECODE_MAX_WORKGROUPS, when set,
+    # stands for the product): the workgroups of a second round pay the three dependent trips to
     # memory that come before their keys once more.  Measured at the 1.5B sizes, fused against separate kernels:
     # 8 tokens at 2,048 keys (176 workgroups) 1.47 against 1.54 ms a step, 12 at 4,096 (456) 1.72 against 1.76;
     # 8 at 8,192 (656) 1.98 against 1.87, 16 at 8,192 (1,312) 2.43 against 2.21; the 7B and 32B sizes turn over
     # between 352 and 704 workgroups as well.
-    FUSED_DECODE_MAX_WORKGROUPS = 512
+    FUSED_DECODE_WORKGROUPS_PER_UNIT = 2
+    FUSED_DECODE_MAX_WORKGROUPS = None
     # The one-kernel decode path leaves its chunks unmerged and the output projection merges them as it
     # loads its operand: one launch less a layer.  That kernel does not stream a large weight as well as
     # the plain product does (measured: 6.9 against 4.4 + 3.7 us with 4.7 MB of weight, 31.7 against
@@ -352,7 +363,10 @@ class Attention(Mixer):
         max_keys = batch.plans[self.plan_key].sizes["max_short_keys"]
         if not ops.attention_decode_fused_supported(kc.dtype, self.nh, self.nkv, self.d, ps, rot, S, width, n):
             return None
-        if n * self.nkv * ops.attention_decode_chunks(max_keys) > self.FUSED_DECODE_MAX_WORKGROUPS:
+        most = self.FUSED_DECODE_MAX_WORKGROUPS
+        if most is None:
+            most = self.FUSED_DECODE_WORKGROUPS_PER_UNIT * compute_units()
+        if n * self.nkv * ops.attention_decode_chunks(max_keys) > most:
             return None
         ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
         # every entry brings one token: token t is of entry t
