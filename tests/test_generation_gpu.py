@@ -569,17 +569,19 @@ def test_graphs_that_are_dropped_and_recorded_again(tiny):
 
 
 def test_steps_of_many_rows_come_in_the_sizes_the_warm_up_measured(tmp_path):
-    """A serving engine on bfloat16 weights measures the library's algorithms for its many-rows products at every
-    multiple of 64 rows a step can bring; portions of prompts beside decoding requests then run with their
-    decoding entries filled up to a multiple of 64, so every such step's rows are among the measured sizes; the
-    tokens are the plain implementation's."""
+    """A serving engine on bfloat16 weights that is told to measure everything at once measures the library's algorithms for its many-rows
+    products at every multiple of 64 rows a step can bring; portions of prompts beside decoding requests then run
+    with their decoding entries filled up to a multiple of 64, so every such step's rows are among the measured
+    sizes; the tokens are the plain implementation's.  Left to itself an engine measures nothing when it is made
+    and every size when its first step is about to run."""
     from zedinfer_amd import GenerationConfig, InferenceEngine, SchedulerConfig
     from zedinfer_amd.parts.rows import sizes_between
     folder = tiny_configs.write_tiny(str(tmp_path / "m"), "B", dtype=torch.bfloat16, std=tiny_configs.SHARP_STD)
     cfg, w = plain.load_folder(folder)
     ps = tiny_configs.PAGE_SIZES["B"]
-    ie = InferenceEngine.create(folder, "bfloat16", SchedulerConfig(num_kv_blocks=160, kv_block_size=ps, max_batch_requests=4,
-                                                                    max_prefill_tokens=192, max_batch_tokens=256))
+    sched = SchedulerConfig(num_kv_blocks=160, kv_block_size=ps, max_batch_requests=4, max_prefill_tokens=192,
+                            max_batch_tokens=256)
+    ie = InferenceEngine.create(folder, "bfloat16", sched, warm_up_sizes="all")
     eng = ie.engine
     measured = {k[1] for k in eng.rt.choices if k[0] == "library_product"}
     assert measured == set(sizes_between(eng.model.step_rows, "mixed", 128, 192 + 4 + 64)) == {320, 256, 192, 128}
@@ -595,6 +597,14 @@ def test_steps_of_many_rows_come_in_the_sizes_the_warm_up_measured(tmp_path):
         taken = ref[torch.arange(12), torch.tensor(res.output_ids)]
         assert bool((taken >= ref.max(dim=1).values - 0.06 * float(ref.abs().max())).all()), (taken, ref.max(dim=1).values)
     eng.cache.check()
+    # left to itself: nothing when it is made, the sizes of the steps that came afterwards, and the same tokens
+    lazy = InferenceEngine.create(folder, "bfloat16", sched)
+    assert lazy.engine.tune_when_scheduled and not [k for k in lazy.engine.rt.choices if k[0] == "library_product"]
+    again = lazy.generate(prompts, GenerationConfig(max_new_tokens=12, ignore_eos=True))
+    came = {k[1] for k in lazy.engine.rt.choices if k[0] == "library_product"}
+    ran = {k[2] + k[1] for k in lazy.engine._prompt_graphs}
+    assert came and came <= measured and {r for r in ran if r > 64} <= came, (came, ran)
+    assert [r.output_ids for r in again] == [r.output_ids for r in results]
 
 
 def test_one_kernel_decode_attention_equals_the_two_kernel_path(tiny, monkeypatch, tmp_path):

@@ -80,7 +80,7 @@ def _engine(args, step_tokens: Optional[List[int]] = None):
     sizes = None
     if step_tokens is not None:
         sizes = sorted({eng.model.step_rows(n, "mixed") for n in step_tokens if n > 1}, reverse=True)
-    ie = InferenceEngine(eng, warm_up_sizes=sizes)
+    ie = InferenceEngine(eng, warm_up_sizes=sizes, freeze_gc=os.environ.get("ZEDINFER_GC_FREEZE", "1") not in ("", "0"))
     log.debug("choices made at warm-up: %s", eng.rt.choices)
     return ie
 

@@ -96,6 +96,12 @@ class Engine:
         self.planners = self.model.planners()
         self.position_axes = self.model.position_axes()
         self.padding_safe = self.model.padding_safe()
+        # The parts' choices (``Part.tune``) for a number of rows are measured the first time a step of that many
+        # rows is about to run, between steps, when this is set (``InferenceEngine`` sets it): an engine is then
+        # made at once, and a size costs its measurement when it first comes instead of every possible size
+        # costing it before the first request.
+        self.tune_when_scheduled = False
+        self._tuned_rows: set = set()
 
     # ---- construction ------------------------------------------------------------
     @classmethod
@@ -165,9 +171,15 @@ class Engine:
                 part_tune = getattr(part, "tune", None)
                 if part_tune is not None:
                     part_tune(int(n))
+        self._tuned_rows.update(int(n) for n in step_sizes)
         if step_sizes:
             torch.cuda.synchronize(self.device)
         return dict(self.rt.choices)
+
+    def _tune_if_new(self, rows: int) -> None:
+        """Before a step of ``rows`` rows runs (never inside one): the parts' choices for that many rows, once."""
+        if self.tune_when_scheduled and rows not in self._tuned_rows:
+            self.warm_up([rows])
 
     # ---- requests ------------------------------------------------------------------
     def open(self, request_id, expected_tokens: int = 0) -> SequenceCache:
@@ -205,6 +217,7 @@ class Engine:
             elif (self.use_graphs or self.use_tapes) and self._one_portion(entries):
                 logits = self._prompt_graph_step(entries, token_source)
             else:
+                self._tune_if_new(sum(len(e.tokens) for e in entries))
                 batch = build_device_batch(entries, self.cache, self.vocab_size, self.device, self.staging,
                                            planners=self.planners, position_axes=self.position_axes)
                 if token_source is not None:        # the entries' tokens lie in their order: the first k are the first k tokens
@@ -240,6 +253,7 @@ class Engine:
             E += more_entries
             # (an entry may name its one token several times: more rows than entries are left as they are)
             R = E if 0 < wanted <= E else wanted
+        self._tune_if_new(E)
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
         # a bound, the same for many steps, of the tokens any sequence holds after this step: the
@@ -414,6 +428,7 @@ class Engine:
         if more_tokens:
             sizes = tuple(sorted(sizes[:-1] + (sizes[-1] + more_tokens,)))
             padded += more_tokens
+        self._tune_if_new(rows + more_tokens)
         widths = tuple(_pow2_at_least(max(len(e.seq.pages[g]) for e in entries), 8)
                        for g in range(len(self.cache.groups)))
         long_bucket = _pow2_at_least(max(e.seq.length + self.portion_rows(len(e.tokens)) for e in portions) + more_tokens, 2048)

@@ -180,34 +180,43 @@ class InferenceEngine:
         sizes += sizes_between(step_rows, "decode", 1, min(sched.max_batch_requests, most_entries))
         return sorted(set(sizes), reverse=True)
 
-    def __init__(self, engine: Engine, warm_up_sizes: Optional[Sequence[int]] = None):
-        """``warm_up_sizes``: the numbers of rows to measure the parts' choices for (None: every size a step with
-        prompt portions can bring under the scheduler's limits; empty: none)."""
+    def __init__(self, engine: Engine, warm_up_sizes: Optional[Sequence[int]] = None, freeze_gc: Optional[bool] = None):
+        """``warm_up_sizes``: numbers of rows to measure the parts' choices for now (None: none now; every size
+        is measured when a step of that size first comes.  "all": every size a step can bring under the
+        scheduler's limits, now: minutes for a large model, and no step ever waits for a measurement).
+        ``freeze_gc``: take what the process holds by now out of the garbage collector's passes (None: what
+        ZEDINFER_GC_FREEZE says, off without it: a library should not change its host's collector; the command
+        line programs switch it on)."""
         self.engine = engine
         self._loop = ServingLoop(engine, engine.fc.eos_token_ids)
-        # The products' algorithms (and other choices of the parts) for steps of many rows are measured now, once
-        # (ZEDINFER_WARM_UP=0: the defaults), at every number of rows that steps with portions of prompts come
-        # in: the library's first proposal for a shape can be a third slower than what timing finds, and what
-        # timing finds for one number of rows does not carry over to its neighbours (measured).
-        # (the reference's own switch for its warm-up is honoured too: ZEDINFER_DISABLE_WARMUP set,
-        # src/zedinfer/engine.cpp:506)
-        if (os.environ.get("ZEDINFER_WARM_UP", "1") not in ("", "0") and "ZEDINFER_DISABLE_WARMUP" not in os.environ
-                and engine.device.type == "cuda"):
-            if warm_up_sizes is None:
+        # The products' algorithms (and other choices of the parts) for steps of many rows are measured, once for
+        # every number of rows that steps come in: the library's first proposal for a shape can be a third slower
+        # than what timing finds, and what timing finds for one number of rows does not carry over to its
+        # neighbours (measured).  By default a size is measured when its first step is about to run
+        # (``Engine.tune_when_scheduled``), between steps: making the engine takes no longer than loading the model.
+        # ZEDINFER_WARM_UP=all measures every size now, ZEDINFER_WARM_UP=0 (or the reference's own switch,
+        # ZEDINFER_DISABLE_WARMUP set, src/zedinfer/engine.cpp:506) measures nothing, ever: the defaults.
+        mode = os.environ.get("ZEDINFER_WARM_UP", "1")
+        if mode not in ("", "0") and "ZEDINFER_DISABLE_WARMUP" not in os.environ and engine.device.type == "cuda":
+            if mode == "all" or (isinstance(warm_up_sizes, str) and warm_up_sizes == "all"):
                 warm_up_sizes = self.default_warm_up_sizes(engine.sched, engine.model.step_rows, engine.graph_max_entries)
-            engine.warm_up(list(warm_up_sizes))
+            engine.tune_when_scheduled = True
+            if warm_up_sizes:
+                engine.warm_up(list(warm_up_sizes))
         # What the process holds by now (modules, the model's parts and tensors) lives as long as the engine:
         # taken out of the garbage collector's passes, a full collection in the middle of serving costs
         # little (measured: one of 50 ms among decode steps of 6.5 ms without this).
-        if os.environ.get("ZEDINFER_GC_FREEZE", "1") not in ("", "0"):
+        if freeze_gc is None:
+            freeze_gc = os.environ.get("ZEDINFER_GC_FREEZE", "0") not in ("", "0")
+        if freeze_gc:
             import gc
             gc.collect()
             gc.freeze()
 
     @classmethod
     def create(cls, model_path: str, dtype="bfloat16", scheduler_config: Optional[SchedulerConfig] = None,
-               warm_up_sizes: Optional[Sequence[int]] = None) -> "InferenceEngine":
-        return cls(Engine.from_folder(model_path, dtype, scheduler_config), warm_up_sizes)
+               warm_up_sizes: Optional[Sequence[int]] = None, freeze_gc: Optional[bool] = None) -> "InferenceEngine":
+        return cls(Engine.from_folder(model_path, dtype, scheduler_config), warm_up_sizes, freeze_gc)
 
     @property
     def default_sampling(self):
