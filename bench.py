@@ -81,7 +81,7 @@ def measure_decode(engine_factory, batch, steps, warmup, vocab, prompt_len=PROMP
     import torch
     from zedinfer_amd import GenerationConfig, InferenceRequest
     from zedinfer_amd.engine import InferenceEngine
-    ie = InferenceEngine(engine_factory(), warm_up_sizes=warm_up_sizes)
+    ie = InferenceEngine(engine_factory(), warm_up_sizes=warm_up_sizes, freeze_gc=True)
     loop = ie.serving_loop()
     rng = random.Random(1234 + batch)
     reqs = [loop.submit_async(InferenceRequest(rand_ids(rng, prompt_len, vocab),
@@ -152,7 +152,9 @@ def measure_mix(engine_factory, requests, vocab, new_tokens=256, lo=128, hi=4096
     import torch
     from zedinfer_amd import GenerationConfig, InferenceRequest
     from zedinfer_amd.engine import InferenceEngine
-    ie = InferenceEngine(engine_factory())
+    # every size's choices measured before the clock starts: the figure is a server's steady state (left to itself
+    # the engine measures a size when its first step comes, which a long run does not notice and this one would)
+    ie = InferenceEngine(engine_factory(), warm_up_sizes="all", freeze_gc=True)
     loop = ie.serving_loop()
     rng = random.Random(4321)
     warm = loop.submit_async(InferenceRequest(rand_ids(rng, hi, vocab), GenerationConfig(max_new_tokens=8, ignore_eos=True)))

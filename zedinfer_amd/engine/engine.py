@@ -102,6 +102,7 @@ class Engine:
         # costing it before the first request.
         self.tune_when_scheduled = False
         self._tuned_rows: set = set()
+        self._tapes_checked: Dict[tuple, bool] = {}     # kinds of steps whose first tape has been held against its own step: did it repeat it
 
     # ---- construction ------------------------------------------------------------
     @classmethod
@@ -325,7 +326,7 @@ class Engine:
             tape = rec.tape()
             if tape is None:
                 dg.no_tape = True
-            elif self._tape_repeats_the_step(tape, logits):
+            elif self._tape_repeats_the_step(tape, logits, batch):
                 dg.tape, dg.logits = tape, logits
             else:
                 dg.no_tape = True
@@ -333,21 +334,29 @@ class Engine:
         dg.ran = True
         return logits
 
-    def _tape_repeats_the_step(self, tape, logits: Optional[torch.Tensor]) -> bool:
+    def _tape_repeats_the_step(self, tape, logits: Optional[torch.Tensor], batch) -> bool:
         """A new tape is run once, right after the step it was recorded from and on the same inputs, with every
         floating-point workspace of the runtime (the logits among them) made NaN before, and must leave the same
         logits bit for bit: device work that is no call into the kernel library (a torch operator in a part that
         says ``tape_safe``) is not on the tape, its result would be stale at every replay, and here it is NaN.  A
         model with state per request is not run twice (the second run would advance the state): its tapes are
-        trusted as before."""
+        trusted as before.  The check costs a step; it is made for the first tape of every kind of step (single
+        tokens or portions; up to 16, 64, 128 or more rows: where the parts take different ways), not for every
+        shape."""
         if logits is None or self.model.state_requests():
             return True
+        n = batch.num_tokens
+        kind = (bool(batch.single_tokens), 0 if n <= 16 else 1 if n <= 64 else 2 if n <= 128 else 3)
+        if kind in self._tapes_checked:
+            return self._tapes_checked[kind]         # what the kind's first tape showed holds for the others
+        self._tapes_checked[kind] = True
         first = logits.clone()
         self.rt.poison()
         logits.fill_(float("nan"))
         tape.run()
         same = bool(torch.equal(first, logits))
         if not same:
+            self._tapes_checked[kind] = False
             import logging
             logging.getLogger("zedinfer_amd").warning(
                 "a recorded step does not repeat its logits: some device work of the model is not a call into the "
