@@ -364,6 +364,57 @@ def test_linear_skinny_row_does_not_depend_on_batch(ops):
                        ops.linear(x2[5:6].contiguous(), w2, out_dtype=torch.float32))
 
 
+@pytest.mark.parametrize("N,K", [(1536, 22400), (3584, 18944), (5120, 27648), (1000, 33560), (1192, 28200)])
+def test_linear_sums_of_129_to_256_rows(ops, N, K):
+    """The product for many rows (32 weight rows a wavefront): partial sums of 129 .. 256 rows against a float32
+    product, at the down projections' widths of the larger sizes and at two widths that are multiples of nothing
+    much; a row's sums do not depend on how many rows ride along (the cut of k is the weight's alone)."""
+    w = rnd(N, K, dtype=torch.bfloat16, scale=0.02, seed=2)
+    x = rnd(256, K, dtype=torch.bfloat16, seed=1)
+    ref = x.float() @ w.float().t()
+    scale = float(ref.abs().max())
+    full = None
+    for M in (129, 200, 256):
+        xm = x[:M].contiguous()
+        assert ops.linear_sums_supported(xm, w)
+        S = ops.linear_splits(M, N, K)
+        assert 1 <= S <= 16 and S == ops.linear_splits(256, N, K)
+        sums = ops.linear_sums(xm, w)
+        assert tuple(sums.shape) == (S, M, N)
+        assert float((sums.sum(0) - ref[:M]).abs().max()) <= 2e-5 * scale
+        if M == 256:
+            full = sums
+    for M in (129, 200):
+        assert torch.equal(ops.linear_sums(x[:M].contiguous(), w), full[:, :M])
+    # square and small weights stay with the library's product beyond 128 rows
+    assert not ops.linear_sums_supported(x[:200, :1536].contiguous(), rnd(1536, 1536, dtype=torch.bfloat16))
+    assert ops.linear_sums_supported(x[:128, :1536].contiguous(), rnd(1536, 1536, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("M", [65, 96, 128, 129, 200, 256])
+@pytest.mark.parametrize("I,K", [(8960, 1536), (1000, 200), (18944, 3584)])
+def test_linear_swiglu_of_65_to_256_rows(ops, M, I, K, monkeypatch):
+    """The same kernel with the SwiGLU epilogue (gate and up rows interleaved in blocks of 8), which the engine
+    does not take beyond 64 rows (the library's product and the activation's own launch are faster there): here
+    with the limit lifted, against float32."""
+    from zedinfer_amd.ops import functional
+    from zedinfer_amd.parts.feed_forward import GATE_UP_BLOCK, interleave_rows
+    monkeypatch.setattr(functional, "SWIGLU_MAX_ROWS", 256)
+    monkeypatch.setattr(functional, "SUMS_MAX_ROWS", 256)
+    gate, up = rnd(I, K, dtype=torch.bfloat16, scale=0.05, seed=3), rnd(I, K, dtype=torch.bfloat16, scale=0.05, seed=4)
+    x = rnd(M, K, dtype=torch.bfloat16, seed=5)
+    w = interleave_rows(gate, up, GATE_UP_BLOCK)
+    assert ops.linear_swiglu_supported(x, w)
+    g, u = x.float() @ gate.float().t(), x.float() @ up.float().t()
+    want = u * (g / (1 + torch.exp(-g)))
+    got = ops.linear_swiglu(x, w)
+    assert tuple(got.shape) == (M, I)
+    assert float((got.float() - want).abs().max()) <= 1e-2 * float(want.abs().max())
+    # rows do not depend on each other (from 65 rows on it is this kernel, whose sums run over k in one order)
+    if M - 3 > 64:
+        assert torch.equal(ops.linear_swiglu(x[:M - 3].contiguous(), w), got[:M - 3])
+
+
 def test_linear_f32_row_does_not_depend_on_batch(ops):
     """The float32 product sums over k in one fixed order: a row's result is bit-identical whatever M is."""
     x, w = rnd(70, 176, seed=1), rnd(130, 176, seed=2)
@@ -911,7 +962,9 @@ def test_attention_prefill_refuses_other_shapes(ops):
                                    (128, 1536, 8960), (113, 3584, 18944), (80, 48, 520)])
 def test_linear_sums(ops, M, N, K):
     bf = torch.bfloat16
-    assert ops.SUMS_MAX_ROWS == 128 and not ops.linear_sums_supported(rnd(129, K, dtype=bf), rnd(N, K, dtype=bf))
+    # beyond 128 rows only large weights with twice as many columns as rows (the other test), beyond 256 none
+    assert ops.SUMS_MAX_ROWS == 256 and not ops.linear_sums_supported(rnd(257, K, dtype=bf), rnd(N, K, dtype=bf))
+    assert ops.linear_sums_supported(rnd(129, K, dtype=bf), rnd(N, K, dtype=bf)) == (K >= 2 * N and N * K >= 1 << 25)
     assert ops.linear_sums_supported(rnd(65, K, dtype=bf), rnd(N, K, dtype=bf))
     assert not ops.linear_sums_supported(rnd(65, K, dtype=bf), rnd(N, K, dtype=bf), ops.FEW_ROWS)
     x, w = rnd(M, K, dtype=bf, seed=1), rnd(N, K, dtype=bf, scale=0.05, seed=2)

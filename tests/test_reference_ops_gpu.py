@@ -62,13 +62,15 @@ def test_embedding_norms_activation_argmax(ops, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("M,N,K", [(3, 136, 72), (40, 200, 264), (70, 152, 136), (125, 264, 520), (200, 72, 1000)])
+@pytest.mark.parametrize("M,N,K", [(3, 136, 72), (40, 200, 264), (70, 152, 136), (125, 264, 520), (200, 72, 1000),
+                                   (160, 520, 64536)])
 def test_products(ops, ref, dtype, M, N, K):
-    """1..16 rows, 17..64 rows, 65..128 rows and the library's many rows in bfloat16; the plain product in 32 bits."""
+    """1..16 rows, 17..64 rows, 65..128 rows, the library's many rows and (a weight with many more columns than
+    rows) the kernel for 129..256 rows in bfloat16; the plain product in 32 bits."""
     x, w, b = rnd(M, K, dtype=dtype, seed=1), rnd(N, K, dtype=dtype, scale=0.1, seed=2), rnd(N, dtype=dtype, seed=3)
     close(ops.linear(x, w, b), ref.linear(x, w, b), dtype)
     close(ops.linear(x, w, out_dtype=torch.float32), ref.linear(x, w), dtype, bf16=2e-3)
-    if dtype == torch.bfloat16 and M <= ops.SUMS_MAX_ROWS:
+    if dtype == torch.bfloat16 and ops.linear_sums_supported(x, w):
         # the same product as partial sums (the kernels for up to 64 and for 65..128 rows), added by the consumer
         close(ops.reduce_sums(ops.linear_sums(x, w), b, out_dtype=torch.float32), ref.linear(x, w, b), dtype, bf16=2e-3)
 

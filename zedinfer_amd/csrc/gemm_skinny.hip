@@ -1,7 +1,8 @@
-// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for up to 128 rows of x: the decode-time matrix products, bound by the
+// out[M,N] = x[M,K] . w[N,K]^T (+ bias) for up to 256 rows of x: the decode-time matrix products, bound by the
 // one pass over the weights.  This file holds their entry points, the cut's bookkeeping and the kernel that
-// adds partial sums; the product kernel is in gemm_mid.hip (it stages x in LDS, a workgroup's wavefronts
-// take 16 weight rows each, and the cut over workgroups is balanced over the compute units).
+// adds partial sums; the product kernels are in gemm_mid.hip (up to 128 rows: x staged in LDS, a workgroup's
+// wavefronts take 16 weight rows each, the cut over workgroups balanced over the compute units) and in
+// gemm_rows32.hip (more rows, and the SwiGLU epilogue from 65 rows on: 32 weight rows a wavefront).
 //
 // When the weight matrix gives too few workgroups the k dimension is cut over several of them (gridDim.y
 // "splits"); those write float32 partial sums [split][M][N] that the consumer adds in rising order (the next
@@ -36,8 +37,26 @@ __global__ void gemm_skinny_reduce_kernel(void* __restrict__ out, int out_f32, c
     else zi_store((zi_bf16*)out + (int64_t)m * ldo + n, s);
 }
 
+#define SK_MAX_ROWS 256
+#define SK_MID_MAX_ROWS 128        // up to here the kernels of gemm_mid.hip, beyond gemm_rows32.hip
+#define SK_MID_MAX_ROWS_SWIGLU 64  // ... with the SwiGLU epilogue (measured: see gemm_rows32.hip)
+
 extern "C" int zi_gemm_skinny_supported(int M, int N, int K, int64_t ldx, int64_t ldw) {
-    return M >= 1 && M <= 128 && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
+    return M >= 1 && M <= SK_MAX_ROWS && N >= 1 && K >= 8 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0;
+}
+
+// most rows the products take
+extern "C" int zi_gemm_skinny_max_rows() { return SK_MAX_ROWS; }
+
+// 1 when these kernels are the faster way to partial sums than the library's product of the same operands, as
+// measured: always up to 128 rows; beyond, for large weights with at least twice as many columns as rows (a down
+// projection: 7B sizes at 256 rows 71 against 126 us, 32B 136 against 263), not for square ones (an output
+// projection: 7B at 256 rows 24.6 against 16.9 us), and not for small ones (1.5B down at 256 rows 25.5 against
+// 31 us, which the 25 MB of partial sums that the next kernel then adds take back: the decode step of 256
+// requests got 3 % slower with it).
+extern "C" int zi_gemm_skinny_pays(int M, int N, int K) {
+    if (M <= SK_MID_MAX_ROWS) return 1;
+    return M <= SK_MAX_ROWS && (int64_t)K >= 2 * (int64_t)N && (int64_t)N * K >= ((int64_t)1 << 25);
 }
 
 // The product kernel (gemm_mid.hip): its cut and its launch.
@@ -45,12 +64,18 @@ void zi_gemm_mid_plan(int N, int K, int* splits, int* kb_per_split, int* waves);
 int zi_gemm_mid_launch(void* out, int out_f32, int mode, const zi_bf16* x, const zi_bf16* w, const zi_bf16* bias, int M,
                        int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int vec_out, hipStream_t stream);
 
-// Splits of k for a weight matrix [N, K]: the leading dimension of the partial sums.  A function of N and K
-// (M is taken for the callers' sake and checked nowhere).
+void zi_gemm_rows32_plan(int N, int K, int many_rows, int whole, int* splits, int* kb_per_split, int* waves);
+int zi_gemm_rows32_launch(void* out, int out_f32, int mode, const zi_bf16* x, const zi_bf16* w, const zi_bf16* bias, int M,
+                          int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, int vec_out, hipStream_t stream);
+
+static bool sk_rows32(int M, int mode) { return M > (mode == SK_MODE_SWIGLU ? SK_MID_MAX_ROWS_SWIGLU : SK_MID_MAX_ROWS); }
+
+// Splits of k for a weight matrix [N, K]: the leading dimension of the partial sums.  A function of N and K and
+// of which of the two kernels the rows go to (up to 128, or more).
 extern "C" int zi_gemm_skinny_splits(int M, int N, int K) {
     int s, per, waves;
-    (void)M;
-    zi_gemm_mid_plan(N, K, &s, &per, &waves);
+    if (sk_rows32(M, SK_MODE_PARTIAL)) zi_gemm_rows32_plan(N, K, M > 128, 0, &s, &per, &waves);
+    else zi_gemm_mid_plan(N, K, &s, &per, &waves);
     return s;
 }
 
@@ -68,13 +93,15 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
                               int N, int K, int64_t ldx, int64_t ldw, int64_t ldo, float* workspace,
                               int64_t workspace_floats, hipStream_t stream) {
     ZI_REQUIRE(zi_gemm_skinny_supported(M, N, K, ldx, ldw),
-               "gemm_skinny: unsupported sizes M=%d N=%d K=%d (1 <= M <= 128, K and row strides multiples of 8)", M, N, K);
+               "gemm_skinny: unsupported sizes M=%d N=%d K=%d (1 <= M <= 256, K and row strides multiples of 8)", M, N, K);
     ZI_REQUIRE(out_dt == ZI_F32 || out_dt == ZI_BF16, "gemm_skinny: unknown output dtype %d", out_dt);
     ZI_REQUIRE(mode >= 0 && mode <= 2, "gemm_skinny: unknown mode %d", mode);
     ZI_REQUIRE(ldx >= K && ldw >= K, "gemm_skinny: leading dimension too small");
     ZI_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "gemm_skinny: x and w must be 16-byte aligned");
     int splits, per, waves;
-    zi_gemm_mid_plan(N, K, &splits, &per, &waves);
+    const bool rows32 = sk_rows32(M, mode);
+    if (rows32) zi_gemm_rows32_plan(N, K, M > 128, mode == SK_MODE_SWIGLU, &splits, &per, &waves);
+    else zi_gemm_mid_plan(N, K, &splits, &per, &waves);
     void* dst = out;
     int kmode = mode;
     if (mode == SK_MODE_PLAIN) {
@@ -101,8 +128,8 @@ extern "C" int zi_gemm_skinny(void* out, int out_dt, int mode, const void* x, co
     else if (kmode == SK_MODE_SWIGLU) vec_out = ldo % 4 == 0 && ((uintptr_t)dst % 8) == 0;
     else vec_out = ldo % 4 == 0 && ((uintptr_t)dst % (out_dt == ZI_F32 ? 16 : 8)) == 0;
     const int of32 = out_dt == ZI_F32;
-    const int rc = zi_gemm_mid_launch(dst, of32, kmode, (const zi_bf16*)x, (const zi_bf16*)w, b, M, N, K, ldx, ldw, ldo,
-                                      vec_out, stream);
+    const int rc = (rows32 ? zi_gemm_rows32_launch : zi_gemm_mid_launch)(dst, of32, kmode, (const zi_bf16*)x, (const zi_bf16*)w, b,
+                                                                         M, N, K, ldx, ldw, ldo, vec_out, stream);
     if (rc) return rc;
     if (mode == SK_MODE_PLAIN && splits > 1) {
         const int64_t total = (int64_t)M * N;

@@ -48,6 +48,7 @@ _PROTOTYPES = {
     "zi_attention_prefill_cuts": [I, I, I, P],
     "zi_attention_prefill_tile_min": [],
     "zi_compute_units": [],
+    "zi_gemm_skinny_pays": [I, I, I],
     "zi_attention_prefill_chunks": [I],
     "zi_attention_prefill_variant": [I],
     "zi_attention_prefill_supported": [I, I, I, I, I],

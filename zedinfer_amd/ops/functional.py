@@ -897,17 +897,25 @@ def linear_choose(x: torch.Tensor, weight: torch.Tensor, which: int, bias: Optio
               M if transposed else N, LIBRARY_WORKSPACE_BYTES, int(which))
 
 
-def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor, most_rows: Optional[int] = None) -> bool:
-    """Whether ``linear_sums`` takes this product: bfloat16, at most SUMS_MAX_ROWS rows (or ``most_rows``,
-    if that is fewer)."""
+def _few_rows_operands(x: torch.Tensor, weight: torch.Tensor, most: int) -> bool:
+    """Operands the few-rows kernels take: bfloat16 matrices, at most ``most`` rows of x, rows they can load."""
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or x.dim() != 2 or weight.dim() != 2:
         return False
-    most = SUMS_MAX_ROWS if most_rows is None else min(int(most_rows), SUMS_MAX_ROWS)
     if not (0 < x.shape[0] <= most) or x.shape[1] != weight.shape[1]:
         return False
     if (x.shape[1] > 1 and x.stride(1) != 1) or (weight.shape[1] > 1 and weight.stride(1) != 1):
         return False
     return _skinny_ok(x, weight, x.shape[1], x.stride(0), weight.stride(0))
+
+
+def linear_sums_supported(x: torch.Tensor, weight: torch.Tensor, most_rows: Optional[int] = None) -> bool:
+    """Whether ``linear_sums`` takes this product: bfloat16, at most SUMS_MAX_ROWS rows (or ``most_rows``,
+    if that is fewer), and a shape at which the library's own product is not the faster one (the kernel
+    library says: measured)."""
+    most = SUMS_MAX_ROWS if most_rows is None else min(int(most_rows), SUMS_MAX_ROWS)
+    if not _few_rows_operands(x, weight, most):
+        return False
+    return bool(_lib.load().zi_gemm_skinny_pays(int(x.shape[0]), int(weight.shape[0]), int(weight.shape[1])))
 
 
 def linear_splits(M: int, N: int, K: int) -> int:
@@ -934,8 +942,9 @@ def linear_sums(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tenso
 
 
 def linear_swiglu_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
-    return (linear_sums_supported(x, weight, FEW_ROWS) and weight.shape[0] % 16 == 0
-            and linear_splits(x.shape[0], weight.shape[0], weight.shape[1]) == 1)
+    # (beyond 64 rows the kernel for many rows never cuts k under this epilogue)
+    return (_few_rows_operands(x, weight, SWIGLU_MAX_ROWS) and weight.shape[0] % 16 == 0
+            and (x.shape[0] > FEW_ROWS or linear_splits(x.shape[0], weight.shape[0], weight.shape[1]) == 1))
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -981,8 +990,14 @@ FEW_ROWS = 64          # up to here they beat the library product: the weights s
 # 6.2 / 5.6 / 17.5 us against the library's 9.7 / 8.1 / 24.5; 7B sizes 20 / 16 / 55 against 20 / 16 / 92.  The
 # gate/up product with its activation does not (37 against 24 + 5 us at the 1.5B sizes: every wavefront reads
 # all of x from LDS for its 16 weight rows, and with 128 rows those reads bound it): FEW_ROWS stays its limit.
+# Beyond 128 rows and up to 256 a kernel with 32 weight rows a wavefront (gemm_rows32.hip) takes the products whose
+# weights have at least twice as many columns as rows (the down projection; the library decides,
+# ``zi_gemm_skinny_pays``).  With the SwiGLU epilogue it loses to the library from 65 rows on (1.5B sizes at 128
+# rows 32.5 against 26.7 us with the activation's own launch: 560 wavefronts of 32 rows are too few for the
+# chip, and the epilogue forbids a cut of k): SWIGLU_MAX_ROWS stays at FEW_ROWS.
 # (ZEDINFER_SUMS_MAX_ROWS=64 gives such products of more than 64 rows back to the library.)
-SUMS_MAX_ROWS = max(FEW_ROWS, min(128, int(os.environ.get("ZEDINFER_SUMS_MAX_ROWS", "128") or 128)))
+SUMS_MAX_ROWS = max(FEW_ROWS, min(256, int(os.environ.get("ZEDINFER_SUMS_MAX_ROWS", "256") or 256)))
+SWIGLU_MAX_ROWS = max(FEW_ROWS, min(256, int(os.environ.get("ZEDINFER_SWIGLU_MAX_ROWS", "64") or 64)))
 _WORKSPACES = {}
 _OUTGROWN_WORKSPACES: list = []
 
