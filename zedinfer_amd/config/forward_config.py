@@ -69,16 +69,12 @@ class ModelForwardConfig:
     final_norm: PartSpec
     lm_head: PartSpec
     tie_word_embeddings: bool = False
-    # Family flags, kept for inspection (reference: forward_config.hpp:36-37).
-    qkv_bias: bool = False
-    qk_norm: bool = False
-    rope_theta: float = 10000.0
-    rms_norm_eps: float = 1e-6
-    use_sliding_window: bool = False
-    sliding_window: int = 0
-    max_window_layers: int = 0
     eos_token_ids: Tuple[int, ...] = ()
     max_position_embeddings: int = 0
+    # What the architecture wants to say about itself, for whoever inspects a model (the reference keeps family
+    # flags on its forward config: forward_config.hpp:36-37).  Nothing in the engine reads it: what a part needs
+    # is in its PartSpec.
+    family: Dict[str, Any] = field(default_factory=dict)
 
     def validate(self) -> None:
         n = len(self.layers)

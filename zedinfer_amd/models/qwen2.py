@@ -77,15 +77,11 @@ def qwen2_forward_config(cfg: Qwen2Config) -> ModelForwardConfig:
                                     "tied_to": "model.embed_tokens.weight" if cfg.tie_word_embeddings else None},
                          {"weight": "lm_head.weight"}),
         tie_word_embeddings=cfg.tie_word_embeddings,
-        qkv_bias=True,
-        qk_norm=False,
-        rope_theta=cfg.rope_theta,
-        rms_norm_eps=cfg.rms_norm_eps,
-        use_sliding_window=cfg.use_sliding_window,
-        sliding_window=cfg.sliding_window,
-        max_window_layers=cfg.max_window_layers,
         eos_token_ids=cfg.eos_token_ids,
         max_position_embeddings=cfg.max_position_embeddings,
+        family={"qkv_bias": True, "qk_norm": False, "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
+                "use_sliding_window": cfg.use_sliding_window, "sliding_window": cfg.sliding_window,
+                "max_window_layers": cfg.max_window_layers},
     )
     fc.validate()
     return fc
