@@ -887,14 +887,18 @@ def linear_tune(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
 
 
 def linear_choose(x: torch.Tensor, weight: torch.Tensor, which: int, bias: Optional[torch.Tensor] = None,
-                  transposed: bool = False, out_dtype: Optional[torch.dtype] = None) -> None:
+                  transposed: bool = False, out_dtype: Optional[torch.dtype] = None,
+                  out_stride: Optional[int] = None) -> None:
     """Fix the library's algorithm for the product of these operands to proposal ``which`` (what ``linear_tune``
-    returned in an earlier run) without timing anything."""
+    returned in an earlier run) without timing anything.  ``out_stride``: the row stride of the result the
+    product will be given when that is a slice of a wider tensor (None: a contiguous result); the stride is part
+    of what the library's plan for a shape is kept by."""
     _gpu("linear_choose", x, weight, bias)
     M, N, K = x.shape[0], weight.shape[0], x.shape[1]
     code = F32 if out_dtype == torch.float32 else BF16
+    ldo = int(out_stride) if out_stride is not None else (M if transposed else N)
     _lib.call("zi_gemm_lt_choose", code, int(bias is not None), int(transposed), M, N, K, x.stride(0), weight.stride(0),
-              M if transposed else N, LIBRARY_WORKSPACE_BYTES, int(which))
+              ldo, LIBRARY_WORKSPACE_BYTES, int(which))
 
 
 def _few_rows_operands(x: torch.Tensor, weight: torch.Tensor, most: int) -> bool:
