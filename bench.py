@@ -172,7 +172,7 @@ def measure_mix(engine_factory, requests, vocab, new_tokens=256, lo=128, hi=4096
     return requests * new_tokens / dt, sum(lens) / dt, dt, sum(lens)
 
 
-def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT, warm=1):
+def measure_prefill(engine_factory, vocab, rounds=3, tokens=PROMPT, warm=2):
     import torch
     from zedinfer_amd import ops
     from zedinfer_amd.engine import StepEntry
