@@ -163,3 +163,64 @@ def test_replay_tool_with_the_configuration_s_own_pages(tiny, how, tmp_path):
     assert f"{need // ps} pages of {ps} tokens" in said and "up to 4 live requests" in said
     groups = re.findall(r"cache group \d+ \(\w+\): (\d+) pages, (\d+) handed out", said)
     assert groups and all(int(total) == need // ps and int(takes) > int(total) for total, takes in groups), said
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16w"])
+def test_a_step_that_fails_leaves_nothing_behind(tiny, dtype):
+    """A step that cannot run to its end (a token the model does not have, in a prompt portion or among decoding
+    requests; pages that run out for a later entry) gives back the pages and promises it had taken, changes no
+    request's length, and the requests go on to the plain implementation's logits afterwards."""
+    from zedinfer_amd.cache import OutOfPages
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine, StepEntry
+    folder, edtype, ref = variant(tiny, dtype)
+    V = tiny["cfg"]["vocab_size"]
+    ps = tiny_configs.PAGE_SIZES[tiny["name"]]
+    toks = {r: tiny["requests"][r] for r in ("r3", "r4")}           # 100 and 70 (47) tokens
+    pages = -(-len(toks["r3"]) // ps) + -(-len(toks["r4"]) // ps) + 1
+    eng = Engine.from_folder(folder, edtype, SchedulerConfig(num_kv_blocks=pages, kv_block_size=ps, max_batch_requests=3))
+    a, b = eng.open("a"), eng.open("b")
+    fed = {"a": 0, "b": 0}
+    ids = {"a": toks["r3"], "b": toks["r4"]}
+
+    def state():
+        pool = eng.cache.groups[0].pool
+        return (a.length, b.length, list(a.pages[0]), list(b.pages[0]), list(a.promised), list(b.promised), pool.num_held,
+                pool.committed)
+
+    def good(seq, name, n):
+        out = eng.step([StepEntry(seq, ids[name][fed[name]:fed[name] + n], [n - 1])])
+        fed[name] += n
+        scale = float(ref["r3" if name == "a" else "r4"].abs().max())
+        want = ref["r3" if name == "a" else "r4"][fed[name] - 1]
+        assert float((out[0].cpu() - want).abs().max()) <= (F32_TOL if dtype == "float32" else BF16_REL_WORST) * max(scale, 1.0)
+
+    good(a, "a", 20)
+    good(b, "b", 9)
+    for _ in range(3):                       # decode steps of the two together: their shape gets a tape
+        out = eng.step([StepEntry(a, ids["a"][fed["a"]:fed["a"] + 1], [0]), StepEntry(b, ids["b"][fed["b"]:fed["b"] + 1], [0])])
+        fed["a"] += 1
+        fed["b"] += 1
+    before = state()
+    # a bad token in a portion that needs new pages, beside a decoding request
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        eng.step([StepEntry(a, ids["a"][fed["a"]:fed["a"] + 30] + [V + 5], [30]), StepEntry(b, ids["b"][fed["b"]:fed["b"] + 1], [0])])
+    assert state() == before
+    # a bad token among decoding requests of a shape that has run before
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        eng.step([StepEntry(a, [ids["a"][fed["a"]]], [0]), StepEntry(b, [-1], [0])])
+    assert state() == before
+    # pages run out for the second entry after the first has grown
+    c = eng.open("c")
+    with pytest.raises(OutOfPages):
+        eng.step([StepEntry(a, ids["a"][fed["a"]:fed["a"] + 40], [39]), StepEntry(c, list(range(1, 60 * ps)), [0])])
+    assert state() == before and c.length == 0 and not any(p >= 0 for p in c.pages[0])
+    eng.close(c)
+    eng.cache.check()
+    good(a, "a", 30)
+    good(b, "b", 1)
+    good(a, "a", 1)
+    eng.close(a)
+    eng.close(b)
+    eng.cache.check()
+    assert eng.cache.groups[0].pool.num_held == 0
