@@ -39,8 +39,11 @@ typedef __attribute__((ext_vector_type(4))) float dec_f32x4_t;
 #define DEC_WAVES ZI_DEC_WAVES
 #define DEC_BLOCK ZI_DEC_BLOCK     // keys a wavefront handles at a time
 
+typedef __attribute__((ext_vector_type(4))) uint32_t dec_u32x4_t;
+
 union dec_pack {
     uint4 u;
+    dec_u32x4_t v;
     dec_bf16x8_t b;
     uint16_t h[8];
 };
@@ -65,7 +68,7 @@ struct DecProjection {
     int write_kv;
 };
 
-template <int D, bool FUSED>
+template <int D, bool FUSED, bool VNT>
 __global__ void __launch_bounds__(DEC_WAVES* ZI_WAVE, 2)
 attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restrict__ part_o,
                         float* __restrict__ part_ml, const zi_bf16* __restrict__ q, int64_t ldq,
@@ -77,6 +80,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DT = D / 16;          // output tiles of 16 dims
+    constexpr bool WHOLE_LINES = D % 64 == 0;   // a key is whole 128-byte lines: see the loads of the keys
     __shared__ float sm[DEC_WAVES][16], sl[DEC_WAVES][16];
     __shared__ dec_f32x4_t so[DEC_WAVES][DT][ZI_WAVE];
     __shared__ uint4 sk[DK][4];        // FUSED: the token's own key, in pieces (k-step, j)
@@ -106,6 +110,11 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     int k_begin, k_end;      // the wavefront's keys; k_end is one past the last
     zi_dec_wave_keys(sp, chunk, wave, p, &k_begin, &k_end);
     const int p8 = p & ~7, pi_last = max_pages - 1;
+    // An instruction's loads of the values cover whole 128-byte lines when a page holds at most 32 tokens (sixteen
+    // dims' runs of the page's tokens lie side by side); then they go past L2 like the keys' (VNT, chosen by the
+    // launch: a branch here costs more than the loads gain).  With larger pages a dim's run is a line of which an
+    // instruction takes half (page 64, non-temporal: 148 against 125 us).
+    constexpr bool v_lines = VNT;
 
     // FUSED: eight consecutive columns of the token's projection row (splits added in rising order, then
     // the bias), and the same after the rotation of head column `hc`, dims dim0 .. dim0 + 7.  Four
@@ -270,11 +279,28 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         // on the spot, one tile after the other.
         dec_pack kop[4][DK], vop[DT][2];
         int kpage[4], kslot[4], vpage[2], vslot[2];
+        // Head sizes that are whole 128-byte lines (WHOLE_LINES): a load instruction takes eight keys' lines whole
+        // instead of sixteen keys' halves (lane (r, j): row hf * 8 + r % 8 of the tile, piece (r / 8) * 4 + j of
+        // line L), and the halves change places between lanes r and r +- 8 afterwards.  Keys and values are read
+        // once a step: whole lines can be loaded non-temporally, past L2 (halves cannot: the line's other half
+        // would come from memory again).  Decode at the 1.5B sizes, 2,100-token contexts, same box, halves and
+        // plain loads against whole lines and non-temporal loads of keys and values: batch 8 5,480 to 5,660 tok/s,
+        // batch 64 25.5k to 26.5k, batch 256 41.0k to 42.6k (values alone: 41.9k; keys alone, as halves: slower).
+        int kpage2[4][2], kslot2[4][2];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-            const ZiTablePlace at = zi_table_place(zi_dec_tile_key(base, tt, r), p, ps, ps_shift, pi_last);
-            kslot[tt] = at.slot;
-            kpage[tt] = bt[at.index];
+            if constexpr (WHOLE_LINES) {
+#pragma unroll
+                for (int hf = 0; hf < 2; ++hf) {
+                    const ZiTablePlace at = zi_table_place(zi_dec_tile_key(base, tt, hf * 8 + (r & 7)), p, ps, ps_shift, pi_last);
+                    kslot2[tt][hf] = at.slot;
+                    kpage2[tt][hf] = bt[at.index];
+                }
+            } else {
+                const ZiTablePlace at = zi_table_place(zi_dec_tile_key(base, tt, r), p, ps, ps_shift, pi_last);
+                kslot[tt] = at.slot;
+                kpage[tt] = bt[at.index];
+            }
         }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
@@ -284,18 +310,54 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         }
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
-            const int page = zi_page_or_zero(kpage[tt], num_pages);   // a window may have freed it
-            const zi_bf16* kr = kcache + zi_key_offset(page, kvh, kslot[tt], nkv, ps, D);
+            if constexpr (WHOLE_LINES) {
 #pragma unroll
-            for (int dk = 0; dk < DK; ++dk)
-                kop[tt][dk].u = *reinterpret_cast<const uint4*>(kr + ((D % 32 == 0 || dk * 32 + j * 8 < D) ? dk * 32 + j * 8 : 0));
+                for (int hf = 0; hf < 2; ++hf) {
+                    const int page = zi_page_or_zero(kpage2[tt][hf], num_pages);   // a window may have freed it
+                    const zi_bf16* kr = kcache + zi_key_offset(page, kvh, kslot2[tt][hf], nkv, ps, D) + ((r >> 3) * 4 + j) * 8;
+#pragma unroll
+                    for (int L = 0; L < DK / 2; ++L)     // kop[tt][2L + hf] for now: rows hf * 8 .. + 7, all eight pieces of line L
+                        kop[tt][2 * L + hf].v = __builtin_nontemporal_load(reinterpret_cast<const dec_u32x4_t*>(kr + L * 64));
+                }
+            } else {
+                const int page = zi_page_or_zero(kpage[tt], num_pages);   // a window may have freed it
+                const zi_bf16* kr = kcache + zi_key_offset(page, kvh, kslot[tt], nkv, ps, D);
+#pragma unroll
+                for (int dk = 0; dk < DK; ++dk)
+                    kop[tt][dk].u = *reinterpret_cast<const uint4*>(kr + ((D % 32 == 0 || dk * 32 + j * 8 < D) ? dk * 32 + j * 8 : 0));
+            }
         }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             const int page = zi_page_or_zero(vpage[b], num_pages);
             const zi_bf16* vr = vcache + zi_value_offset(page, kvh, r, vslot[b], nkv, ps, D);
+            if constexpr (v_lines) {
 #pragma unroll
-            for (int dd = 0; dd < DT; ++dd) vop[dd][b].u = *reinterpret_cast<const uint4*>(vr + (int64_t)dd * 16 * ps);
+                for (int dd = 0; dd < DT; ++dd) vop[dd][b].v = __builtin_nontemporal_load(reinterpret_cast<const dec_u32x4_t*>(vr + (int64_t)dd * 16 * ps));
+            } else {
+#pragma unroll
+                for (int dd = 0; dd < DT; ++dd) vop[dd][b].v = *reinterpret_cast<const dec_u32x4_t*>(vr + (int64_t)dd * 16 * ps);
+            }
+        }
+        if constexpr (WHOLE_LINES) {
+            // lanes r < 8 hold rows r of both loads' pieces 0..3, lanes r >= 8 rows r - 8 with pieces 4..7: k-step 2L
+            // wants row r's pieces 0..3 (lanes >= 8 take them from the second load's lanes r - 8), k-step 2L + 1
+            // pieces 4..7 (lanes < 8 take them from the first load's lanes r + 8).  A rotation by eight lanes within
+            // every row of sixteen, written to half the lanes.
+#pragma unroll
+            for (int tt = 0; tt < 4; ++tt)
+#pragma unroll
+                for (int L = 0; L < DK / 2; ++L) {
+                    const dec_u32x4_t a = kop[tt][2 * L].v, b = kop[tt][2 * L + 1].v;
+                    dec_u32x4_t lo, hi;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        lo[w] = (uint32_t)__builtin_amdgcn_update_dpp((int)a[w], (int)b[w], 0x128, 0xf, 0xc, false);
+                        hi[w] = (uint32_t)__builtin_amdgcn_update_dpp((int)b[w], (int)a[w], 0x128, 0xf, 0x3, false);
+                    }
+                    kop[tt][2 * L].v = lo;
+                    kop[tt][2 * L + 1].v = hi;
+                }
         }
         if (D % 32 != 0) {   // the padding of the last k-step must be zero: the query is, but 0 * NaN is not
             const unsigned keep = (DK - 1) * 32 + j * 8 < D ? ~0u : 0u;
@@ -664,26 +726,30 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
     const dim3 grid(max_chunks, nkv, n_idx);
     const int G = nh / nkv;
     const DecProjection none = {};
-#define ZI_DEC(DD)                                                                                                   \
+#define ZI_DEC(DD, VNT)                                                                                              \
     if (pj)                                                                                                          \
-        attention_decode_kernel<DD, true><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
+        attention_decode_kernel<DD, true, VNT><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
             max_chunks, leave_parts, *pj);                                                                                      \
     else                                                                                                             \
-        attention_decode_kernel<DD, false><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
+        attention_decode_kernel<DD, false, VNT><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
             max_chunks, leave_parts, none)
     switch (d) {
-        case 16: ZI_DEC(16); break;
-        case 32: ZI_DEC(32); break;
-        case 48: ZI_DEC(48); break;
-        case 64: ZI_DEC(64); break;
-        case 80: ZI_DEC(80); break;
-        case 96: ZI_DEC(96); break;
-        case 112: ZI_DEC(112); break;
-        default: ZI_DEC(128); break;
+        case 16: ZI_DEC(16, false); break;
+        case 32: ZI_DEC(32, false); break;
+        case 48: ZI_DEC(48, false); break;
+        case 64:
+            if (page_size <= 32) { ZI_DEC(64, true); } else { ZI_DEC(64, false); }
+            break;
+        case 80: ZI_DEC(80, false); break;
+        case 96: ZI_DEC(96, false); break;
+        case 112: ZI_DEC(112, false); break;
+        default:
+            if (page_size <= 32) { ZI_DEC(128, true); } else { ZI_DEC(128, false); }
+            break;
     }
 #undef ZI_DEC
     if (max_chunks > 1 && !leave_parts)
