@@ -449,7 +449,8 @@ def test_argmax(ops, dtype):
 @pytest.mark.parametrize("nh,nkv,d,ps,T,window", [
     (12, 2, 128, 16, 2100, 0), (12, 2, 128, 16, 70, 0), (28, 4, 128, 16, 5000, 0), (3, 1, 64, 8, 200, 0),
     (8, 1, 64, 16, 300, 37), (5, 5, 80, 32, 150, 0), (4, 2, 128, 8, 260, 100), (14, 2, 128, 16, 9, 0),
-    (12, 1, 48, 8, 700, 0), (4, 2, 16, 16, 1000, 300), (32, 2, 112, 64, 530, 0), (12, 2, 128, 16, 17000, 0)])
+    (12, 1, 48, 8, 700, 0), (4, 2, 16, 16, 1000, 300), (32, 2, 112, 64, 530, 0), (12, 2, 128, 16, 17000, 0),
+    (12, 2, 128, 64, 600, 0), (6, 2, 64, 128, 900, 250), (40, 8, 128, 32, 1300, 0)])      # pages whose value rows are longer than half a line
 def test_attention_decode(ops, nh, nkv, d, ps, T, window):
     """The split-keys kernel against the same float32 reference, with a listed subset of the tokens."""
     dtype = torch.bfloat16
@@ -519,7 +520,8 @@ FUSED_DECODE_CASES = [
     (8, 2, 48, 8, [33, 700, 256], 0, 3, torch.float32, 32),
     (4, 2, 128, 16, [500, 120, 99], 100, 5, torch.bfloat16, 128),
     (6, 3, 80, 32, [150, 64], 0, 2, torch.bfloat16, 0),
-    (12, 2, 128, 16, [17000, 300], 0, 2, torch.bfloat16, 128)]
+    (12, 2, 128, 16, [17000, 300], 0, 2, torch.bfloat16, 128),
+    (12, 2, 128, 64, [700, 64, 65, 129], 0, 2, torch.bfloat16, 128)]
 
 
 @pytest.mark.parametrize("nh,nkv,d,ps,lens,window,S,bias_dtype,rot", FUSED_DECODE_CASES)
