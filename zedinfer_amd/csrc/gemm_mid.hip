@@ -22,7 +22,6 @@ typedef __attribute__((ext_vector_type(4))) unsigned gm_u32x4_t;
 
 #define GM_MIN_WAVES 4      // wavefronts of a workgroup: 4 .. 8, 16 weight rows each
 #define GM_MAX_WAVES 8
-#define GM_STAGERS 256      // threads that stage the block's x slice (the first four wavefronts)
 #define GM_KB 128
 #define GM_XS GM_KB         // LDS row stride, in elements: rows of 16 pieces of 16 bytes, piece c of row r at place c xor (r mod 16)
 
@@ -137,30 +136,31 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
     // LDS rows are not padded but swizzled (16-byte reads in operand order then run at the full LDS rate)
     uint16_t* const wt_w = &wt[wave][0];
 
-    // what this thread stages of a block's x slice: MT pieces of 16 bytes (row srow + 16 * t, piece spc);
-    // the first GM_STAGERS threads stage, the others' loads go to the same places and are dropped
-    const int srow = (tid % GM_STAGERS) / 16, spc = tid % 16;
-    const bool stager = tid < GM_STAGERS;
+    // what this thread stages of a block's x slice: XP pieces of 16 bytes (rows srow[p], piece spc).  The slice's
+    // MT * 256 pieces are dealt out over all the workgroup's threads, a row of 16 pieces to 16 neighbours; the
+    // last round may pass the slice's end (its loads repeat the last row and go nowhere).
+    constexpr int THREADS = GM_WAVES * ZI_WAVE, XP = (MT * 256 + THREADS - 1) / THREADS;
+    const int spc = tid % 16;
+    int srow[XP];
+#pragma unroll
+    for (int p = 0; p < XP; ++p) srow[p] = p * (THREADS / 16) + tid / 16;
     // the weights of GM_RING k-blocks are in flight at once (a ring of register buffers); the x slice of
     // the next block is fetched while this one is worked on
-    gm_u32x4_t ring[GM_RING][4], xring[GM_RING][MT];
+    gm_u32x4_t ring[GM_RING][4], xring[GM_RING][XP];
     // Loads are issued without branches and their results are not touched before the products need
     // them: only then does the compiler let several blocks' loads stay in flight.  Addresses are
     // clamped into the matrices.  Rows of x past M repeat the last row and give outputs that nobody
     // stores; columns past K would count the last eight twice, so the weights are zeroed there, when
     // they are used.  A block's x is requested before its weights: loads return in order, and x, which
     // comes from the cache and is wanted a step earlier, must not queue behind weights from memory.
-    const zi_bf16* xrow[MT];
+    const zi_bf16* xrow[XP];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        const int m = t * 16 + srow;
-        xrow[t] = x + (int64_t)(m < M ? m : M - 1) * ldx;
-    }
+    for (int p = 0; p < XP; ++p) xrow[p] = x + (int64_t)(srow[p] < M ? srow[p] : M - 1) * ldx;
     auto fetch = [&](const int slot, int kb) __attribute__((always_inline)) {
         const int k0 = kb * GM_KB;
         const int kx = k0 + spc * 8 < K ? k0 + spc * 8 : K - 8;
 #pragma unroll
-        for (int t = 0; t < MT; ++t) xring[slot][t] = *reinterpret_cast<const gm_u32x4_t*>(xrow[t] + kx);
+        for (int p = 0; p < XP; ++p) xring[slot][p] = *reinterpret_cast<const gm_u32x4_t*>(xrow[p] + kx);
         const int k = k0 + wq * 8;
         // a weight is read once a step and the weights of a step are many times the caches: non-temporal loads keep
         // them out of L2 (decode at batch 8, 1.5B sizes: 5,403 to 5,518 tok/s)
@@ -168,10 +168,10 @@ gemm_mid_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* __
         for (int c = 0; c < 4; ++c) ring[slot][c] = __builtin_nontemporal_load(reinterpret_cast<const gm_u32x4_t*>(wrow[c] + (k < K ? k : K - 8)));
     };
     auto stash = [&](const int slot, int b) __attribute__((always_inline)) {
-        if (GM_WAVES * ZI_WAVE > GM_STAGERS && !stager) return;
 #pragma unroll
-        for (int t = 0; t < MT; ++t)
-            *reinterpret_cast<gm_u32x4_t*>(&xs[b][(t * 16 + srow) * GM_XS + (spc ^ srow) * 8]) = xring[slot][t];
+        for (int p = 0; p < XP; ++p)
+            if ((p + 1) * (THREADS / 16) <= MT * 16 || srow[p] < MT * 16)
+                *reinterpret_cast<gm_u32x4_t*>(&xs[b][srow[p] * GM_XS + (spc ^ (srow[p] & 15)) * 8]) = xring[slot][p];
     };
     gm_f32x4_t acc[MT];
 #pragma unroll
@@ -275,22 +275,23 @@ gemm_wide_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* _
         wrow[c] = w + (int64_t)(n < N ? n : N - 1) * ldw;
     }
     uint16_t* const wt_w = &wt[wave][0];
-    const int srow = (tid % GM_STAGERS) / 16, spc = tid % 16;
-    const bool stager = tid < GM_STAGERS;
-    gm_u32x4_t ring[RING][4], xnext[MT];
-    const zi_bf16* xrow[MT];
+    // the block's x slice is dealt out over all the workgroup's threads (see the kernel above)
+    constexpr int THREADS = GM_WAVES * ZI_WAVE, XP = (MT * 256 + THREADS - 1) / THREADS;
+    const int spc = tid % 16;
+    int srow[XP];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-        const int m = t * 16 + srow;
-        xrow[t] = x + (int64_t)(m < M ? m : M - 1) * ldx;
-    }
+    for (int p = 0; p < XP; ++p) srow[p] = p * (THREADS / 16) + tid / 16;
+    gm_u32x4_t ring[RING][4], xnext[XP];
+    const zi_bf16* xrow[XP];
+#pragma unroll
+    for (int p = 0; p < XP; ++p) xrow[p] = x + (int64_t)(srow[p] < M ? srow[p] : M - 1) * ldx;
     // a block's x is requested before the weights that are requested in the same step: loads return in order,
     // and x is wanted first.  The block index is clamped: the last step asks for its own block again.
     auto fetch_x = [&](int kb) __attribute__((always_inline)) {
         const int k0 = (kb < kb_hi ? kb : kb_hi - 1) * GM_KB;
         const int kx = k0 + spc * 8 < K ? k0 + spc * 8 : K - 8;
 #pragma unroll
-        for (int t = 0; t < MT; ++t) xnext[t] = *reinterpret_cast<const gm_u32x4_t*>(xrow[t] + kx);
+        for (int p = 0; p < XP; ++p) xnext[p] = *reinterpret_cast<const gm_u32x4_t*>(xrow[p] + kx);
     };
     auto fetch_w = [&](const int slot, int kb) __attribute__((always_inline)) {
         const int k = kb * GM_KB + wq * 8;
@@ -298,10 +299,10 @@ gemm_wide_kernel(void* __restrict__ out, int mode, int out_f32, const zi_bf16* _
         for (int c = 0; c < 4; ++c) ring[slot][c] = __builtin_nontemporal_load(reinterpret_cast<const gm_u32x4_t*>(wrow[c] + (k < K ? k : K - 8)));
     };
     auto stash = [&]() __attribute__((always_inline)) {
-        if (GM_WAVES * ZI_WAVE > GM_STAGERS && !stager) return;
 #pragma unroll
-        for (int t = 0; t < MT; ++t)
-            *reinterpret_cast<gm_u32x4_t*>(&xs[(t * 16 + srow) * GM_XS + (spc ^ srow) * 8]) = xnext[t];
+        for (int p = 0; p < XP; ++p)
+            if ((p + 1) * (THREADS / 16) <= MT * 16 || srow[p] < MT * 16)
+                *reinterpret_cast<gm_u32x4_t*>(&xs[srow[p] * GM_XS + (spc ^ (srow[p] & 15)) * 8]) = xnext[p];
     };
     gm_f32x4_t acc[MT];
 #pragma unroll
