@@ -68,7 +68,7 @@ struct DecProjection {
     int write_kv;
 };
 
-template <int D, bool FUSED, bool VNT>
+template <int D, bool FUSED, int VMODE>
 __global__ void __launch_bounds__(DEC_WAVES* ZI_WAVE, 2)
 attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restrict__ part_o,
                         float* __restrict__ part_ml, const zi_bf16* __restrict__ q, int64_t ldq,
@@ -110,11 +110,13 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
     int k_begin, k_end;      // the wavefront's keys; k_end is one past the last
     zi_dec_wave_keys(sp, chunk, wave, p, &k_begin, &k_end);
     const int p8 = p & ~7, pi_last = max_pages - 1;
-    // An instruction's loads of the values cover whole 128-byte lines when a page holds at most 32 tokens (sixteen
-    // dims' runs of the page's tokens lie side by side); then they go past L2 like the keys' (VNT, chosen by the
-    // launch: a branch here costs more than the loads gain).  With larger pages a dim's run is a line of which an
-    // instruction takes half (page 64, non-temporal: 148 against 125 us).
-    constexpr bool v_lines = VNT;
+    // How the values are loaded (VMODE, chosen by the launch: a branch here costs more than it gains).  1: pages of
+    // at most 32 tokens, where an instruction's loads cover whole 128-byte lines as they are (sixteen dims' runs of
+    // a page's tokens lie side by side): past L2, like the keys.  2: larger pages, where a dim's run of the block's
+    // 64 tokens is a line of its own: an instruction takes eight dims' whole lines (lane (r, j): dim r % 8, the
+    // eight tokens of piece (r / 8) * 4 + j) and the lanes r and r +- 8 trade halves afterwards, as for the keys;
+    // past L2 as well (as halves, non-temporal: 148 against 125 us at page 64).  0: plain loads of halves.
+    constexpr bool v_lines = VMODE == 1, v_trade = VMODE == 2;
 
     // FUSED: eight consecutive columns of the token's projection row (splits added in rising order, then
     // the bias), and the same after the rotation of head column `hc`, dims dim0 .. dim0 + 7.  Four
@@ -302,11 +304,17 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                 kpage[tt] = bt[at.index];
             }
         }
+        if constexpr (v_trade) {      // this lane's eight tokens: piece (r / 8) * 4 + j of the block
+            const ZiTablePlace at = zi_table_place(base + ((r >> 3) * 4 + j) * 8, p8, ps, ps_shift, pi_last);
+            vslot[0] = at.slot;
+            vpage[0] = bt[at.index];
+        } else {
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const ZiTablePlace at = zi_table_place(zi_dec_value_key0(base, b, j), p8, ps, ps_shift, pi_last);
-            vslot[b] = at.slot;
-            vpage[b] = bt[at.index];
+            for (int b = 0; b < 2; ++b) {
+                const ZiTablePlace at = zi_table_place(zi_dec_value_key0(base, b, j), p8, ps, ps_shift, pi_last);
+                vslot[b] = at.slot;
+                vpage[b] = bt[at.index];
+            }
         }
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
@@ -329,6 +337,13 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         }
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
+            if constexpr (v_trade) {      // vop[dd][b] for now: dims dd * 16 + b * 8 .. + 7, all 64 tokens
+                const int page = zi_page_or_zero(vpage[0], num_pages);
+                const zi_bf16* vr = vcache + zi_value_offset(page, kvh, b * 8 + (r & 7), vslot[0], nkv, ps, D);
+#pragma unroll
+                for (int dd = 0; dd < DT; ++dd) vop[dd][b].v = __builtin_nontemporal_load(reinterpret_cast<const dec_u32x4_t*>(vr + (int64_t)dd * 16 * ps));
+                continue;
+            }
             const int page = zi_page_or_zero(vpage[b], num_pages);
             const zi_bf16* vr = vcache + zi_value_offset(page, kvh, r, vslot[b], nkv, ps, D);
             if constexpr (v_lines) {
@@ -358,6 +373,20 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                     kop[tt][2 * L].v = lo;
                     kop[tt][2 * L + 1].v = hi;
                 }
+        }
+        if constexpr (v_trade) {
+#pragma unroll
+            for (int dd = 0; dd < DT; ++dd) {
+                const dec_u32x4_t a = vop[dd][0].v, b = vop[dd][1].v;
+                dec_u32x4_t lo, hi;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    lo[w] = (uint32_t)__builtin_amdgcn_update_dpp((int)a[w], (int)b[w], 0x128, 0xf, 0xc, false);
+                    hi[w] = (uint32_t)__builtin_amdgcn_update_dpp((int)b[w], (int)a[w], 0x128, 0xf, 0x3, false);
+                }
+                vop[dd][0].v = lo;
+                vop[dd][1].v = hi;
+            }
         }
         if (D % 32 != 0) {   // the padding of the last k-step must be zero: the query is, but 0 * NaN is not
             const unsigned keep = (DK - 1) * 32 + j * 8 < D ? ~0u : 0u;
@@ -726,29 +755,29 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
     const dim3 grid(max_chunks, nkv, n_idx);
     const int G = nh / nkv;
     const DecProjection none = {};
-#define ZI_DEC(DD, VNT)                                                                                              \
+#define ZI_DEC(DD, VMODE)                                                                                            \
     if (pj)                                                                                                          \
-        attention_decode_kernel<DD, true, VNT><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
+        attention_decode_kernel<DD, true, VMODE><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
             max_chunks, leave_parts, *pj);                                                                                      \
     else                                                                                                             \
-        attention_decode_kernel<DD, false, VNT><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
+        attention_decode_kernel<DD, false, VMODE><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
             max_chunks, leave_parts, none)
     switch (d) {
-        case 16: ZI_DEC(16, false); break;
-        case 32: ZI_DEC(32, false); break;
-        case 48: ZI_DEC(48, false); break;
+        case 16: ZI_DEC(16, 0); break;
+        case 32: ZI_DEC(32, 0); break;
+        case 48: ZI_DEC(48, 0); break;
         case 64:
-            if (page_size <= 32) { ZI_DEC(64, true); } else { ZI_DEC(64, false); }
+            if (page_size <= 32) { ZI_DEC(64, 1); } else { ZI_DEC(64, 2); }
             break;
-        case 80: ZI_DEC(80, false); break;
-        case 96: ZI_DEC(96, false); break;
-        case 112: ZI_DEC(112, false); break;
+        case 80: ZI_DEC(80, 0); break;
+        case 96: ZI_DEC(96, 0); break;
+        case 112: ZI_DEC(112, 0); break;
         default:
-            if (page_size <= 32) { ZI_DEC(128, true); } else { ZI_DEC(128, false); }
+            if (page_size <= 32) { ZI_DEC(128, 1); } else { ZI_DEC(128, 2); }
             break;
     }
 #undef ZI_DEC
