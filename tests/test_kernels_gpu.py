@@ -991,6 +991,23 @@ def test_linear_sums(ops, M, N, K):
         assert torch.equal(fewer[:, 16], sums[:, 16])
 
 
+@pytest.mark.parametrize("N,K", [(4120, 1024), (5456, 1024), (6168, 1024), (10256, 768), (4096, 1024)])
+@pytest.mark.parametrize("M", [17, 33, 50, 64, 65, 81, 100, 128])
+def test_linear_sums_with_workgroups_of_every_size(ops, M, N, K):
+    """Weights whose cut gives workgroups of five, six, seven, eight and four wavefronts (on 256 compute units), at
+    every number of 16-row tiles of x from two to eight: every thread of the workgroup stages its share of the
+    block's x slice, and the last round of that passes the slice's end in some of these."""
+    bf = torch.bfloat16
+    x, w = rnd(M, K, dtype=bf, seed=M), rnd(N, K, dtype=bf, scale=0.05, seed=N)
+    sums = ops.linear_sums(x, w)
+    assert sums.shape == (ops.linear_splits(M, N, K), M, N)
+    ref = x.float() @ w.float().t()
+    torch.testing.assert_close(sums.sum(0), ref, atol=2e-3, rtol=2e-3)
+    # row 16 as part of 17 rows: the same sums, whichever kernel and however many tiles
+    if M > 17:
+        assert torch.equal(ops.linear_sums(x[:17].contiguous(), w)[:, 16], sums[:, 16])
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 8960, 1536), (8, 8960, 1536), (14, 176, 64), (16, 256, 96), (2, 208, 80),
                                    (4, 18944, 3584), (64, 8960, 1536), (24, 176, 64), (50, 18944, 3584)])
 def test_linear_swiglu(ops, M, I, K):
